@@ -1,0 +1,262 @@
+"""`fp_quant::*` operators of the inference path, backed by libfpq_hip.so.
+
+Same operator names, signatures, output shapes/dtypes and fake (meta) implementations as the
+reference's QuTLASS wrappers (inference_lib/src/fp_quant/module/qutlass_ops.py:36-168), so that
+`torch.compile(..., fullgraph=True)` keeps working across them.  Differences that stay inside
+the boundary: scales are consumed row-major by the GEMMs (no per-call re-tiling), and the
+rotation matrix is recognised once (Hadamard / identity / GSR) and applied as butterflies.
+"""
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from .. import _engine
+from ..utils import FPQuantDtype  # noqa: F401  (re-exported for parity with the reference module)
+
+HAS_HIP_ENGINE = _engine.available()
+
+# zero-nibble policy used by the operators (see include/fpq.h)
+ZERO_NIBBLE_POLICY = _engine.ZERO_REFERENCE
+
+_rotation_cache: Dict[Tuple, Tuple[int, float]] = {}
+
+
+def _sylvester(g: int) -> torch.Tensor:
+    idx = torch.arange(g)
+    anded = idx[:, None] & idx[None, :]
+    pop = torch.zeros_like(anded)
+    for b in range(8):
+        pop += (anded >> b) & 1
+    return (1 - 2 * (pop & 1)).to(torch.float32)
+
+
+def classify_rotation(h: torch.Tensor) -> Tuple[int, float]:
+    """(rotation kind, norm) of a [g, g] matrix; cached per storage/version so the one
+    device->host copy it needs happens once per matrix, not per call."""
+    key = (h.data_ptr(), h._version, tuple(h.shape), h.dtype, str(h.device))
+    hit = _rotation_cache.get(key)
+    if hit is not None:
+        return hit
+    g = h.shape[0]
+    if h.dim() != 2 or h.shape[1] != g:
+        raise ValueError(f"rotation matrix must be square, got {tuple(h.shape)}")
+    hf = h.detach().to(device="cpu", dtype=torch.float32)
+    kind, norm = _engine.ROT_GENERAL, 0.0
+    if torch.equal(hf, torch.eye(g)):
+        kind, norm = _engine.ROT_IDENTITY, 1.0
+    elif g in (16, 32, 64, 128) and float(hf[0, 0]) != 0.0:
+        n = float(hf[0, 0])
+        signed = _sylvester(g) * n
+        if torch.equal(hf, signed):
+            kind, norm = _engine.ROT_HADAMARD, n
+        else:
+            changes = torch.diff(signed, dim=0).ne(0).sum(dim=0)
+            if torch.equal(hf, signed[:, torch.argsort(changes)]):
+                kind, norm = _engine.ROT_GSR, n
+    if len(_rotation_cache) > 4096:
+        _rotation_cache.clear()
+    _rotation_cache[key] = (kind, norm)
+    return kind, norm
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require_cuda(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if not t.is_cuda:
+            raise ValueError("fp_quant HIP operators need tensors on a GPU; there is no CPU path")
+
+
+def _padded(rows: int, groups: int) -> Tuple[int, int]:
+    return (rows + 127) // 128 * 128, (groups + 3) // 4 * 4
+
+
+### Forward quantization
+
+
+@torch.library.custom_op("fp_quant::fused_quantize_mx_op", mutates_args=())
+def fused_quantize_mx_op(
+    x_flat: torch.Tensor,
+    hadamard_matrix: torch.Tensor,
+    forward_method: str,
+    return_mask: bool,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    if forward_method != "abs_max":
+        raise NotImplementedError(
+            f"forward_method={forward_method!r}: this engine implements the abs_max MXFP4 quantizer only"
+        )
+    if return_mask:
+        raise NotImplementedError("clip masks are only produced by the quest method")
+    _require_cuda(x_flat, hadamard_matrix)
+    if x_flat.dtype != torch.bfloat16 or x_flat.dim() != 2:
+        raise ValueError("x_flat must be a 2-D bfloat16 tensor")
+    x = x_flat.contiguous()
+    rows, cols = x.shape
+    kind, norm = classify_rotation(hadamard_matrix)
+    g = hadamard_matrix.shape[0]
+    prow, pcol = _padded(rows, cols // 32)
+    codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=x.device)
+    scales = torch.empty(prow, pcol, dtype=torch.uint8, device=x.device)
+    h = hadamard_matrix.contiguous()
+    with torch.cuda.device(x.device):
+        st = _engine.lib().fpq_quantize_mx(
+            x.data_ptr(), rows, cols, kind, g, norm, h.data_ptr(), codes.data_ptr(),
+            scales.data_ptr(), prow, pcol, ZERO_NIBBLE_POLICY, _stream(x))
+    _engine.check(st, "fused_quantize_mx_op")
+    return codes, scales.view(torch.float8_e8m0fnu), None
+
+
+@fused_quantize_mx_op.register_fake
+def _(x_flat, hadamard_matrix, forward_method, return_mask):
+    rows, cols = x_flat.size(0), x_flat.size(1)
+    prow, pcol = _padded(rows, cols // 32)
+    codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=x_flat.device)
+    scales = torch.empty(prow, pcol, dtype=torch.float8_e8m0fnu, device=x_flat.device)
+    mask = torch.empty(rows, cols // 8, dtype=torch.uint8, device=x_flat.device) if return_mask else None
+    return codes, scales, mask
+
+
+@torch.library.custom_op("fp_quant::fused_quantize_nv_op", mutates_args=())
+def fused_quantize_nv_op(
+    x_flat: torch.Tensor,
+    hadamard_matrix: torch.Tensor,
+    global_scale: torch.Tensor,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    _require_cuda(x_flat, hadamard_matrix, global_scale)
+    if x_flat.dtype != torch.bfloat16:
+        raise ValueError("x_flat must be a bfloat16 tensor")
+    if global_scale.dtype != torch.float32 or global_scale.numel() != 1:
+        raise ValueError("global_scale must be a one-element float32 tensor")
+    x = x_flat.contiguous()
+    cols = x.shape[-1]
+    rows = x.numel() // cols if cols else 0
+    kind, norm = classify_rotation(hadamard_matrix)
+    g = hadamard_matrix.shape[0]
+    prow, pcol = _padded(rows, cols // 16)
+    codes = torch.empty(*x.shape[:-1], cols // 2, dtype=torch.uint8, device=x.device)
+    scales = torch.empty(prow, pcol, dtype=torch.uint8, device=x.device)
+    h = hadamard_matrix.contiguous()
+    gs = global_scale.contiguous()
+    with torch.cuda.device(x.device):
+        st = _engine.lib().fpq_quantize_nv(
+            x.data_ptr(), rows, cols, kind, g, norm, h.data_ptr(), gs.data_ptr(), codes.data_ptr(),
+            scales.data_ptr(), prow, pcol, ZERO_NIBBLE_POLICY, _stream(x))
+    _engine.check(st, "fused_quantize_nv_op")
+    return codes, scales.view(torch.float8_e4m3fn)
+
+
+@fused_quantize_nv_op.register_fake
+def _(x_flat, hadamard_matrix, global_scale):
+    cols = x_flat.size(-1)
+    rows = x_flat.numel() // cols
+    prow, pcol = _padded(rows, cols // 16)
+    codes = torch.empty(*x_flat.shape[:-1], cols // 2, dtype=torch.uint8, device=x_flat.device)
+    scales = torch.empty(prow, pcol, dtype=torch.float8_e4m3fn, device=x_flat.device)
+    return codes, scales
+
+
+### GEMMs
+
+
+def _gemm(entry: str, x, w, xs, ws, alpha, bias: Optional[torch.Tensor], group: int) -> torch.Tensor:
+    _require_cuda(x, w, xs, ws, alpha)
+    if x.dtype != torch.uint8 or w.dtype != torch.uint8:
+        raise ValueError("packed operands must be uint8")
+    if alpha.dtype != torch.float32 or alpha.numel() != 1:
+        raise ValueError("alpha must be a one-element float32 tensor")
+    xq = x.contiguous().view(-1, x.shape[-1])
+    wq = w.contiguous()
+    m, kb = xq.shape
+    n = wq.shape[0]
+    k = kb * 2
+    if wq.shape[1] != kb:
+        raise ValueError(f"inner dimensions differ: x has K={k}, w has K={wq.shape[1] * 2}")
+    xs_b = xs.contiguous().view(torch.uint8)
+    ws_b = ws.contiguous().view(torch.uint8)
+    xs_b = xs_b.view(-1, xs_b.shape[-1])
+    ws_b = ws_b.view(-1, ws_b.shape[-1])
+    if xs_b.shape[0] < m or ws_b.shape[0] < n or xs_b.shape[1] < k // group or ws_b.shape[1] < k // group:
+        raise ValueError("scale tensors are smaller than the operands they describe")
+    y = torch.empty(*x.shape[:-1], n, dtype=torch.bfloat16, device=x.device)
+    b_ptr = None
+    if bias is not None:
+        if bias.dtype != torch.bfloat16 or bias.numel() != n:
+            raise ValueError("bias must be a bfloat16 vector of length N")
+        bias = bias.contiguous()
+        b_ptr = bias.data_ptr()
+    a = alpha.contiguous()
+    with torch.cuda.device(x.device):
+        st = getattr(_engine.lib(), entry)(
+            xq.data_ptr(), xs_b.data_ptr(), xs_b.shape[1], wq.data_ptr(), ws_b.data_ptr(),
+            ws_b.shape[1], a.data_ptr(), b_ptr, y.data_ptr(), m, n, k, _stream(x))
+    _engine.check(st, entry)
+    return y
+
+
+@torch.library.custom_op("fp_quant::matmul_mxf4_bf16_tn_op", mutates_args=())
+def matmul_mxf4_bf16_tn_op(
+    x: torch.Tensor, w: torch.Tensor, xs: torch.Tensor, ws: torch.Tensor, alpha: torch.Tensor
+) -> torch.Tensor:
+    return _gemm("fpq_gemm_mxf4", x, w, xs, ws, alpha, None, 32)
+
+
+@matmul_mxf4_bf16_tn_op.register_fake
+def _(x, w, xs, ws, alpha):
+    return x.new_empty(*x.shape[:-1], w.shape[0], dtype=torch.bfloat16)
+
+
+@torch.library.custom_op("fp_quant::matmul_ada_mxf4_bf16_tn_op", mutates_args=())
+def matmul_ada_mxf4_bf16_tn_op(
+    x: torch.Tensor, w: torch.Tensor, xs: torch.Tensor, ws: torch.Tensor, alpha: torch.Tensor
+) -> torch.Tensor:
+    # The reference's small-M entry takes un-tiled scales; here every entry does, and the
+    # library picks the small-M kernel by shape.
+    return _gemm("fpq_gemm_mxf4", x, w, xs, ws, alpha, None, 32)
+
+
+@matmul_ada_mxf4_bf16_tn_op.register_fake
+def _(x, w, xs, ws, alpha):
+    return x.new_empty(*x.shape[:-1], w.shape[0], dtype=torch.bfloat16)
+
+
+@torch.library.custom_op("fp_quant::matmul_nvf4_bf16_tn_op", mutates_args=())
+def matmul_nvf4_bf16_tn_op(
+    x: torch.Tensor, w: torch.Tensor, xs: torch.Tensor, ws: torch.Tensor, alpha: torch.Tensor
+) -> torch.Tensor:
+    return _gemm("fpq_gemm_nvf4", x, w, xs, ws, alpha, None, 16)
+
+
+@matmul_nvf4_bf16_tn_op.register_fake
+def _(x, w, xs, ws, alpha):
+    return x.new_empty(*x.shape[:-1], w.shape[0], dtype=torch.bfloat16)
+
+
+### Fused epilogue variants (bias added inside the GEMM; not part of the reference op set)
+
+
+@torch.library.custom_op("fp_quant::matmul_mxf4_bf16_tn_bias_op", mutates_args=())
+def matmul_mxf4_bf16_tn_bias_op(
+    x: torch.Tensor, w: torch.Tensor, xs: torch.Tensor, ws: torch.Tensor, alpha: torch.Tensor,
+    bias: torch.Tensor,
+) -> torch.Tensor:
+    return _gemm("fpq_gemm_mxf4", x, w, xs, ws, alpha, bias, 32)
+
+
+@matmul_mxf4_bf16_tn_bias_op.register_fake
+def _(x, w, xs, ws, alpha, bias):
+    return x.new_empty(*x.shape[:-1], w.shape[0], dtype=torch.bfloat16)
+
+
+@torch.library.custom_op("fp_quant::matmul_nvf4_bf16_tn_bias_op", mutates_args=())
+def matmul_nvf4_bf16_tn_bias_op(
+    x: torch.Tensor, w: torch.Tensor, xs: torch.Tensor, ws: torch.Tensor, alpha: torch.Tensor,
+    bias: torch.Tensor,
+) -> torch.Tensor:
+    return _gemm("fpq_gemm_nvf4", x, w, xs, ws, alpha, bias, 16)
+
+
+@matmul_nvf4_bf16_tn_bias_op.register_fake
+def _(x, w, xs, ws, alpha, bias):
+    return x.new_empty(*x.shape[:-1], w.shape[0], dtype=torch.bfloat16)

@@ -1,0 +1,162 @@
+"""FPQuantLinear: the quantized linear layer of the inference path.
+
+Keeps the constructor, parameter/buffer names, shapes and dtypes, `pre_forward()` and the
+inference branch of `forward()` of the reference module
+(inference_lib/src/fp_quant/module/linear.py:24-368), so state dicts and loaders written for
+the reference work unchanged.  Training branches (master weights, quantized backward) and
+pseudo-quantization are not part of this engine and raise.
+"""
+import torch
+from torch import nn
+
+from ..utils import FPQuantConfig, FPQuantDtype, validate_config
+from . import hip_ops
+from .linear_fns import FPQuant4x16NoMasterFn, forward_quantize
+
+_SCALE_GROUP = {FPQuantDtype.MXFP4: 32, FPQuantDtype.NVFP4: 16}
+
+
+def _sylvester_signs(n: int) -> torch.Tensor:
+    """+-1 Sylvester-Hadamard matrix, entry (i, j) = (-1)^popcount(i & j) (== scipy.linalg.hadamard)."""
+    h = torch.ones(1, 1, dtype=torch.float64)
+    while h.shape[0] < n:
+        h = torch.cat((torch.cat((h, h), dim=1), torch.cat((h, -h), dim=1)), dim=0)
+    if h.shape[0] != n:
+        raise ValueError(f"Hadamard size must be a power of two, got {n}")
+    return h
+
+
+def get_hadamard_matrix(group_size: int, dtype: torch.dtype, device: torch.device):
+    """hadamard(g) * g**-0.5 rounded to `dtype` (linear.py:24-30)."""
+    return (_sylvester_signs(group_size) * group_size ** -0.5).to(dtype=dtype, device=device)
+
+
+def get_identity_matrix(group_size: int, dtype: torch.dtype, device: torch.device):
+    return torch.eye(group_size, dtype=dtype, device=device)
+
+
+def get_gsr_matrix(group_size: int, dtype: torch.dtype, device: torch.device):
+    """Hadamard matrix with columns sorted by their number of sign changes (linear.py:37-41)."""
+    had = get_hadamard_matrix(group_size, dtype, device)
+    order = torch.argsort(torch.diff(had, dim=0).ne(0).sum(dim=0))
+    return had[:, order].contiguous()
+
+
+_TRANSFORMS = {"hadamard": get_hadamard_matrix, "identity": get_identity_matrix, "gsr": get_gsr_matrix}
+
+
+class FPQuantLinear(nn.Module):
+    def __init__(
+        self,
+        in_features: int,
+        out_features: int,
+        config: FPQuantConfig,
+        bias: bool = True,
+        device: torch.device = None,
+        dtype: torch.dtype = None,
+    ):
+        super().__init__()
+        validate_config(config)
+        if config.pseudoquantization:
+            raise ValueError(
+                "pseudoquantization=True is not available: this engine runs real FP4 kernels only"
+            )
+        if not hip_ops.HAS_HIP_ENGINE:
+            raise ValueError(
+                "libfpq_hip.so is not built or failed to load; build it with `python fp-quant_amd/build.py`"
+            )
+        group = _SCALE_GROUP.get(config.forward_dtype)
+        if group is None:
+            raise ValueError(f"Unsupported forward dtype: {config.forward_dtype}")
+
+        factory = {"device": device, "dtype": dtype}
+        self.in_features = in_features
+        self.out_features = out_features
+        self.config = config
+        self.weight = nn.Parameter(torch.empty((out_features, in_features), **factory))
+        self.dqweight = nn.Parameter(torch.empty((out_features, in_features), **factory))
+        if bias:
+            self.bias = nn.Parameter(torch.empty(out_features, **factory))
+        else:
+            self.register_parameter("bias", None)
+
+        dev = self.weight.device
+        self.register_buffer("qweight", torch.empty(out_features, in_features // 2, dtype=torch.uint8, device=dev))
+        self.register_buffer("scales", torch.empty(out_features, in_features // group, dtype=torch.uint8, device=dev))
+        self.register_buffer("weight_global_scale", torch.empty(1, **factory))
+        self.register_buffer("act_global_scale", torch.empty(1, **factory))
+        g = config.hadamard_group_size
+        self.register_buffer("forward_hadamard_matrix", torch.empty(g, g, **factory))
+        self.register_buffer("backward_hadamard_matrix", torch.empty(g, g, **factory))
+
+    @torch.no_grad()
+    def pre_forward(self):
+        """Build the rotation and global-scale buffers and quantize `weight` into
+        `qweight`/`scales` (linear.py:154-248, real-quant branch)."""
+        cfg = self.config
+        g = cfg.hadamard_group_size
+        assert self.weight.shape[1] % g == 0, (
+            f"Weight shape must be divisible by hadamard group size: {self.weight.shape[1]} % {g} = "
+            f"{self.weight.shape[1] % g}"
+        )
+        assert self.weight.data.device.type in ("cuda", "xpu"), (
+            f"Weight must be on CUDA or XPU, but is on {self.weight.device}"
+        )
+        try:
+            make = _TRANSFORMS[cfg.transform_init]
+        except KeyError:
+            raise ValueError(f"Invalid transform init: {cfg.transform_init}") from None
+        wdtype, wdev = self.weight.dtype, self.weight.device
+        self.forward_hadamard_matrix = nn.Buffer(make(g, wdtype, wdev))
+        self.backward_hadamard_matrix = nn.Buffer(make(g, wdtype, wdev))
+
+        if cfg.forward_dtype == FPQuantDtype.MXFP4 and cfg.forward_method == "quest":
+            global_scale_val = 1.0
+        elif cfg.forward_method == "abs_max":
+            global_scale_val = 3.0  # abs-max MXFP4 carries an implicit factor 3 per operand
+        elif cfg.forward_dtype == FPQuantDtype.NVFP4:
+            global_scale_val = 10.0
+        self.weight_global_scale = nn.Buffer(torch.tensor([global_scale_val], dtype=wdtype, device=wdev))
+        self.act_global_scale = nn.Buffer(torch.tensor([global_scale_val], dtype=wdtype, device=wdev))
+
+        if cfg.store_master_weights:
+            self.qweight = None
+            self.scales = None
+            self.dqweight = None
+            return
+        weight_q, scales, _ = forward_quantize(
+            self.weight, self.forward_hadamard_matrix, self.weight_global_scale,
+            cfg.forward_dtype, cfg.forward_method,
+        )
+        group = _SCALE_GROUP[cfg.forward_dtype]
+        rows, cols = self.weight.shape[0], self.weight.shape[1] // group
+        scales = scales.view(dtype=torch.uint8)[:rows, :cols].contiguous()  # drop the op's padding
+        self.qweight = nn.Parameter(weight_q, requires_grad=False)
+        self.scales = nn.Parameter(scales, requires_grad=False)
+        self.weight = None
+        self.dqweight = None
+
+    def forward(self, x) -> torch.Tensor:
+        cfg = self.config
+        if (
+            cfg.forward_dtype in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4)
+            and cfg.backward_dtype == FPQuantDtype.BF16
+            and not cfg.store_master_weights
+            and not cfg.pseudoquantization
+        ):
+            return FPQuant4x16NoMasterFn.apply(
+                x,
+                self.qweight,
+                self.scales,
+                self.weight_global_scale,
+                self.act_global_scale,
+                self.bias,
+                self.forward_hadamard_matrix,
+                cfg.forward_dtype,
+                cfg.forward_method,
+            )
+        raise ValueError(
+            f"Forward dtype: {cfg.forward_dtype}, backward dtype: {cfg.backward_dtype}, "
+            f"store_master_weights: {cfg.store_master_weights}, pseudoquantization: "
+            f"{cfg.pseudoquantization} isn't supported yet."
+        )

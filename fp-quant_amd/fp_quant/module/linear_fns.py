@@ -1,0 +1,89 @@
+"""Forward pieces of the quantized linear: activation quantize -> W4A4 GEMM -> bias.
+
+Mirrors `forward_quantize`, `forward_gemm` and `FPQuant4x16NoMasterFn` of the reference
+(inference_lib/src/fp_quant/module/linear_fns.py:27-64, 482-534): same argument order, same
+returned tuples, same exceptions.
+"""
+from typing import Optional, Tuple
+
+import torch
+from torch.autograd import Function
+
+from ..utils import FPQuantDtype
+from .hip_ops import (
+    fused_quantize_mx_op,
+    fused_quantize_nv_op,
+    matmul_mxf4_bf16_tn_bias_op,
+    matmul_mxf4_bf16_tn_op,
+    matmul_nvf4_bf16_tn_bias_op,
+    matmul_nvf4_bf16_tn_op,
+)
+
+
+def forward_quantize(
+    x: torch.Tensor,
+    hadamard_matrix: torch.Tensor,
+    global_scale: torch.Tensor,
+    dtype: FPQuantDtype,
+    forward_method: str,
+) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """(packed codes, scales, clip mask or None) of x rotated by `hadamard_matrix`."""
+    if dtype == FPQuantDtype.MXFP4:
+        want_mask = forward_method == "quest" and x.requires_grad
+        return fused_quantize_mx_op(
+            x.to(torch.bfloat16), hadamard_matrix.to(torch.bfloat16), forward_method, want_mask
+        )
+    if dtype == FPQuantDtype.NVFP4:
+        codes, scales = fused_quantize_nv_op(
+            x.to(torch.bfloat16), hadamard_matrix.to(torch.bfloat16), global_scale.float()
+        )
+        return codes, scales, None
+    raise ValueError(f"Unsupported forward dtype: {dtype}")
+
+
+def forward_gemm(x_q, w_q, x_scales, w_scales, alpha, dtype: FPQuantDtype, bias=None):
+    """bf16(alpha * dq(x_q) @ dq(w_q).T), optionally followed by the bf16 bias add in the
+    same kernel.  The library chooses the small-M kernel by shape."""
+    if dtype == FPQuantDtype.MXFP4:
+        if bias is None:
+            return matmul_mxf4_bf16_tn_op(x_q, w_q, x_scales, w_scales, alpha.float())
+        return matmul_mxf4_bf16_tn_bias_op(x_q, w_q, x_scales, w_scales, alpha.float(), bias)
+    if dtype == FPQuantDtype.NVFP4:
+        if bias is None:
+            return matmul_nvf4_bf16_tn_op(x_q, w_q, x_scales, w_scales, alpha.float())
+        return matmul_nvf4_bf16_tn_bias_op(x_q, w_q, x_scales, w_scales, alpha.float(), bias)
+    raise ValueError(f"Unsupported dtype: {dtype}")
+
+
+class FPQuant4x16NoMasterFn(Function):
+    """Inference-only W4A4 linear on pre-quantized weights (no backward)."""
+
+    @staticmethod
+    def forward(
+        ctx,
+        x: torch.Tensor,
+        weight_q: torch.Tensor,
+        weight_scales: torch.Tensor,
+        weight_global_scale: torch.Tensor,
+        act_global_scale: torch.Tensor,
+        bias: Optional[torch.Tensor],
+        forward_hadamard_matrix: torch.Tensor,
+        dtype: FPQuantDtype,
+        forward_method: str,
+    ):
+        x_flat = x.contiguous().flatten(end_dim=-2)
+        x_q, x_scales, _ = forward_quantize(
+            x_flat, forward_hadamard_matrix, act_global_scale, dtype, forward_method
+        )
+        # evaluated in the buffers' dtype, as the reference does (bf16 buffers round 1/9)
+        alpha = 1.0 / (weight_global_scale * act_global_scale)
+        fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16) else None
+        y = forward_gemm(x_q, weight_q, x_scales, weight_scales, alpha, dtype, fused_bias)
+        y = y.unflatten(dim=0, sizes=x.shape[:-1])
+        if bias is not None and fused_bias is None:
+            y += bias
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor):
+        raise NotImplementedError("Backward pass is not implemented for FPQuant4x16NoMasterFn yet")

@@ -1,0 +1,111 @@
+/*
+ * fpq.h — C ABI of libfpq_hip.so, the MI355X (gfx950) engine behind FP-Quant's inference path.
+ *
+ * Every entry point takes raw device pointers, sizes and a HIP stream (passed as void*, 0 = the
+ * null stream), launches asynchronously on that stream and returns an int status:
+ *   0  success;  <0  invalid argument (FPQ_E_*);  >0  a hipError_t reported by the runtime.
+ * No entry point allocates device memory, synchronises the stream or keeps mutable global state;
+ * all of them may be called from any host thread.  Scalars the reference passes as one-element
+ * tensors (alpha, global scale) stay device pointers so no host sync is introduced.
+ *
+ * Each declaration cites the reference interface it stands in for (paths relative to the
+ * reference checkout, inference_lib/src/fp_quant/module/).
+ */
+#ifndef FPQ_H_
+#define FPQ_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FPQ_VERSION 1
+
+/* status codes */
+#define FPQ_OK 0
+#define FPQ_E_NULL -1        /* a required pointer is null                       */
+#define FPQ_E_SHAPE -2       /* sizes violate the divisibility rules below       */
+#define FPQ_E_ROTATION -3    /* unknown rotation kind / unsupported block size   */
+#define FPQ_E_ALIGN -4       /* a pointer is not aligned as documented           */
+#define FPQ_E_POLICY -5      /* unknown zero-nibble policy or scale layout       */
+#define FPQ_E_UNSUPPORTED -6 /* valid request this build has no kernel for       */
+
+/* rotation kinds: how the [g, g] matrix of the reference (linear.py:24-41) is applied */
+#define FPQ_ROT_HADAMARD 0 /* +-norm Sylvester matrix: fp32 radix-2 butterflies, strides 1..g/2 */
+#define FPQ_ROT_IDENTITY 1 /* no rotation                                                      */
+#define FPQ_ROT_GSR 2      /* Hadamard with sequency-ordered columns (outputs permuted)         */
+#define FPQ_ROT_GENERAL 3  /* arbitrary bf16 matrix, sequential fp32 fma accumulation           */
+
+/* zero-nibble policies: which code a value that rounds to zero gets */
+#define FPQ_ZERO_REFERENCE 0 /* always 0x8, what src/quantization/quant_ops.py:31-40 packs */
+#define FPQ_ZERO_SIGNED 1    /* sign bit of the scaled value (+0 -> 0x0, -0 -> 0x8)         */
+
+int fpq_version(void);
+
+/* Static, NUL-terminated description of a status returned by this library. */
+const char* fpq_status_string(int status);
+
+/* 1 if `device` is a gfx950 GPU this library has code for, 0 if not, <0 / >0 on error. */
+int fpq_device_supported(int device);
+
+/*
+ * Fused rotate + MXFP4 abs-max quantize.
+ * Stands in for qutlass.fusedQuantizeMx behind fused_quantize_mx_op (qutlass_ops.py:36-71,
+ * called from forward_quantize, linear_fns.py:34-41) with method "abs_max".
+ *
+ *   x            bf16 [rows, cols] row-major, 16-byte aligned; cols % max(g, 32) == 0
+ *   rot_kind/g   rotation kind and block size (g in 16/32/64/128; identity ignores g)
+ *   norm         value every Hadamard entry has in magnitude (float(H[0][0]))
+ *   h            bf16 [g, g] matrix, only read for FPQ_ROT_GENERAL (may be null otherwise)
+ *   codes        uint8 [rows, cols/2], 4-byte aligned: element 2j in the low nibble of byte j
+ *   scales       uint8 E8M0 [scale_rows, scale_stride]; entry [r, c/32]; rows >= `rows` and
+ *                columns >= cols/32 are zero-filled (the reference pads to 128 rows / 4 columns)
+ *   zero_policy  FPQ_ZERO_*
+ */
+int fpq_quantize_mx(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                    const void* h, void* codes, void* scales, int64_t scale_rows,
+                    int64_t scale_stride, int zero_policy, void* stream);
+
+/*
+ * Fused rotate + NVFP4 quantize (group 16, E4M3 scales, fp32 per-tensor multiplier).
+ * Stands in for qutlass.fusedQuantizeNv behind fused_quantize_nv_op (qutlass_ops.py:74-105).
+ *   global_scale  device pointer to one fp32 (the reference passes a 1-element tensor)
+ *   scales        uint8 E4M3 [scale_rows, scale_stride]; entry [r, c/16]; cols % max(g,16) == 0
+ */
+int fpq_quantize_nv(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                    const void* h, const float* global_scale, void* codes, void* scales,
+                    int64_t scale_rows, int64_t scale_stride, int zero_policy, void* stream);
+
+/*
+ * y[m, n] = bf16(alpha * sum_k dq(xq)[m, k] * dq(wq)[n, k]) (+ bias[n]), MXFP4 operands.
+ * Stands in for qutlass.matmul_mxf4_bf16_tn behind matmul_mxf4_bf16_tn_op and the disabled
+ * small-M matmul_ada_mxf4_bf16_tn_op (qutlass_ops.py:111-146), plus the bias add of
+ * FPQuant4x16NoMasterFn.forward (linear_fns.py:512-514).  Scales are taken row-major (the
+ * reference re-tiles them with to_blocked on every call; this engine needs no re-tiling).
+ *   xq uint8 [M, K/2], wq uint8 [N, K/2] (16-byte aligned rows: K % 32 == 0)
+ *   xs uint8 E8M0 [>=M, xs_stride], ws uint8 E8M0 [>=N, ws_stride], entry [row, k/32]
+ *   alpha device pointer to one fp32; bias bf16 [N] or null; y bf16 [M, N]
+ */
+int fpq_gemm_mxf4(const void* xq, const void* xs, int64_t xs_stride, const void* wq,
+                  const void* ws, int64_t ws_stride, const float* alpha, const void* bias,
+                  void* y, int64_t M, int64_t N, int64_t K, void* stream);
+
+/*
+ * Same contract with NVFP4 operands: E4M3 scales per 16 elements, entry [row, k/16].
+ * Stands in for qutlass.matmul_nvf4_bf16_tn behind matmul_nvf4_bf16_tn_op (qutlass_ops.py:149-168).
+ */
+int fpq_gemm_nvf4(const void* xq, const void* xs, int64_t xs_stride, const void* wq,
+                  const void* ws, int64_t ws_stride, const float* alpha, const void* bias,
+                  void* y, int64_t M, int64_t N, int64_t K, void* stream);
+
+/*
+ * Test hook: E2M1 codes of n fp32 values exactly as the quantize kernels round them
+ * (out[i] in 0..15, one byte per value).  Used to check the device rounding exhaustively.
+ */
+int fpq_test_e2m1(const float* in, uint8_t* out, int64_t n, int zero_policy, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FPQ_H_ */

@@ -1,0 +1,40 @@
+"""Thin test helper: call the C ABI of libfpq_hip.so on torch CUDA tensors."""
+import torch
+
+from fp_quant import _engine
+
+ROT = {"hadamard": _engine.ROT_HADAMARD, "identity": _engine.ROT_IDENTITY, "gsr": _engine.ROT_GSR,
+       "general": _engine.ROT_GENERAL}
+
+
+def _padded(rows, groups, pad):
+    if not pad:
+        return rows, groups
+    return (rows + 127) // 128 * 128, (groups + 3) // 4 * 4
+
+
+def quantize(x_bf16, fmt, rot="hadamard", g=128, norm=None, h=None, global_scale=None,
+             zero_policy=_engine.ZERO_REFERENCE, pad=False, fill=0xCD):
+    """Run fpq_quantize_mx / fpq_quantize_nv on `x_bf16` (CPU or CUDA); returns CPU uint8
+    (codes [R, C/2], scales [scale_rows, scale_stride]) and raises on a non-zero status."""
+    lib = _engine.lib()
+    x = x_bf16.to("cuda").contiguous()
+    rows, cols = x.shape
+    group = 32 if fmt == "mxfp4" else 16
+    srow, scol = _padded(rows, cols // group, pad)
+    codes = torch.full((rows, cols // 2), fill, dtype=torch.uint8, device="cuda")
+    scales = torch.full((srow, scol), fill, dtype=torch.uint8, device="cuda")
+    if norm is None:
+        norm = float(torch.tensor(g ** -0.5, dtype=torch.bfloat16))
+    hp = h.to("cuda").contiguous().data_ptr() if h is not None else None
+    stream = torch.cuda.current_stream().cuda_stream
+    if fmt == "mxfp4":
+        st = lib.fpq_quantize_mx(x.data_ptr(), rows, cols, ROT[rot], g, norm, hp, codes.data_ptr(),
+                                 scales.data_ptr(), srow, scol, zero_policy, stream)
+    else:
+        gs = torch.tensor([global_scale], dtype=torch.float32, device="cuda")
+        st = lib.fpq_quantize_nv(x.data_ptr(), rows, cols, ROT[rot], g, norm, hp, gs.data_ptr(),
+                                 codes.data_ptr(), scales.data_ptr(), srow, scol, zero_policy, stream)
+    _engine.check(st, "fpq_quantize")
+    torch.cuda.synchronize()
+    return codes.cpu(), scales.cpu()

@@ -1,0 +1,48 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol include/fpq.h
+declares, and rejects bad arguments before touching a device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "fpq.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fpq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported():
+    from fp_quant import _engine
+    lib = ctypes.CDLL(_engine.library_path())
+    names = _declared()
+    assert "fpq_quantize_mx" in names and "fpq_gemm_mxf4" in names
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/fpq.h but not exported"
+    assert sorted(_engine._SIGNATURES) == names
+
+
+def test_version_and_status_strings():
+    from fp_quant import _engine
+    lib = _engine.lib()
+    assert lib.fpq_version() == 1
+    assert lib.fpq_status_string(0) == b"ok"
+    for code in range(-6, 0):
+        assert len(lib.fpq_status_string(code)) > 3
+
+
+def test_argument_validation_needs_no_device():
+    from fp_quant import _engine
+    lib = _engine.lib()
+    # null pointers and bad shapes are rejected before any HIP call
+    assert lib.fpq_quantize_mx(None, 4, 128, 0, 128, 0.088, None, None, None, 4, 4, 0, None) == -1
+    assert lib.fpq_quantize_mx(16, 4, 100, 0, 128, 0.088, None, 16, 16, 4, 4, 0, None) == -2
+    assert lib.fpq_quantize_mx(16, 4, 128, 0, 48, 0.088, None, 16, 16, 4, 4, 0, None) == -3
+    assert lib.fpq_quantize_mx(8, 4, 128, 0, 128, 0.088, None, 16, 16, 4, 4, 0, None) == -4
+    assert lib.fpq_quantize_mx(16, 4, 128, 0, 128, 0.088, None, 16, 16, 4, 4, 9, None) == -5
+    assert lib.fpq_quantize_nv(16, 4, 128, 0, 16, 0.25, None, None, 16, 16, 4, 8, 0, None) == -1
+    with pytest.raises(ValueError):
+        _engine.check(-2, "x")
