@@ -38,3 +38,21 @@ def quantize(x_bf16, fmt, rot="hadamard", g=128, norm=None, h=None, global_scale
     _engine.check(st, "fpq_quantize")
     torch.cuda.synchronize()
     return codes.cpu(), scales.cpu()
+
+
+def gemm(xq, xs, wq, ws, alpha, fmt, bias=None):
+    """Run fpq_gemm_mxf4 / fpq_gemm_nvf4 on packed operands (CPU or CUDA uint8 tensors);
+    returns the bf16 [M, N] result on the CPU."""
+    lib = _engine.lib()
+    xq, xs, wq, ws = (t.to("cuda").contiguous() for t in (xq, xs, wq, ws))
+    m, n, k = xq.shape[0], wq.shape[0], xq.shape[1] * 2
+    y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    a = torch.tensor([alpha], dtype=torch.float32, device="cuda")
+    b = bias.to("cuda").contiguous() if bias is not None else None
+    fn = lib.fpq_gemm_mxf4 if fmt == "mxfp4" else lib.fpq_gemm_nvf4
+    st = fn(xq.data_ptr(), xs.data_ptr(), xs.shape[1], wq.data_ptr(), ws.data_ptr(), ws.shape[1],
+            a.data_ptr(), b.data_ptr() if b is not None else None, y.data_ptr(), m, n, k,
+            torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_gemm")
+    torch.cuda.synchronize()
+    return y.cpu()

@@ -1,0 +1,137 @@
+"""FPQuantLinear end to end on the GPU: pre_forward weight quantization, forward through the
+operators, replace helpers, torch.compile friendliness of the operators."""
+import pytest
+import torch
+from torch import nn
+
+from oracle import fpq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _cfg(fmt, g, **kw):
+    import fp_quant
+    return fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype(fmt), forward_method="abs_max",
+                                  backward_dtype=fp_quant.FPQuantDtype.BF16, hadamard_group_size=g, **kw)
+
+
+@pytest.mark.parametrize("fmt,g", [("mxfp4", 32), ("mxfp4", 128), ("nvfp4", 16), ("nvfp4", 64)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_linear_matches_oracle_pipeline(fmt, g, bias):
+    import fp_quant
+    gen = torch.Generator().manual_seed(3)
+    k, n = 512, 384
+    w = (torch.randn(n, k, generator=gen) * 0.02).to(torch.bfloat16)
+    b = torch.randn(n, generator=gen).to(torch.bfloat16) if bias else None
+    x = torch.randn(2, 9, k, generator=gen).to(torch.bfloat16)
+    lin = fp_quant.FPQuantLinear(k, n, _cfg(fmt, g), bias=bias, device="cuda", dtype=torch.bfloat16)
+    lin.weight.data = w.cuda()
+    if bias:
+        lin.bias.data = b.cuda()
+    lin.pre_forward()
+    assert lin.weight is None and lin.dqweight is None
+    assert lin.qweight.dtype == torch.uint8 and lin.qweight.shape == (n, k // 2)
+    group = 32 if fmt == "mxfp4" else 16
+    assert lin.scales.dtype == torch.uint8 and lin.scales.shape == (n, k // group)
+    # linear.py:190-200: the abs_max branch (3.0) is tested before the NVFP4 branch (10.0), and
+    # NVFP4 only validates with abs_max, so every real-quant layer gets 3.0
+    gsv = 3.0
+    assert float(lin.weight_global_scale) == gsv and float(lin.act_global_scale) == gsv
+    assert torch.equal(lin.forward_hadamard_matrix.cpu(), O.hadamard_matrix(g))
+
+    # weights: bit-exact against the oracle quantizer
+    norm = float(O.hadamard_matrix(g)[0, 0])
+    if fmt == "mxfp4":
+        wq, ws, _ = O.quantize_mx(w, O.ROT_HADAMARD, g, norm)
+        xq, xs, _ = O.quantize_mx(x.view(-1, k), O.ROT_HADAMARD, g, norm)
+    else:
+        wq, ws, _ = O.quantize_nv(w, gsv, O.ROT_HADAMARD, g, norm)
+        xq, xs, _ = O.quantize_nv(x.view(-1, k), gsv, O.ROT_HADAMARD, g, norm)
+    assert torch.equal(lin.qweight.cpu(), wq) and torch.equal(lin.scales.cpu(), ws)
+
+    y = lin(x.cuda())
+    assert y.shape == (2, 9, n) and y.dtype == torch.bfloat16
+    alpha = O.alpha_from_global_scales(lin.weight_global_scale.cpu(), lin.act_global_scale.cpu())
+    ref, mag = O.gemm_ref(xq, xs, wq, ws, alpha, fmt)
+    yb = ref.to(torch.bfloat16)
+    if bias:
+        yb = yb + b
+    got = y.cpu().view(-1, n)
+    close = (got.double() - yb.double()).abs() <= 2.0 ** -7 * yb.double().abs() + 1e-5 * mag + 1e-6
+    assert close.all()
+    # and it approximates the unquantized linear
+    dense = x.view(-1, k).double() @ w.double().T + (b.double() if bias else 0)
+    rel = (got.double() - dense).norm() / dense.norm()
+    assert rel < 0.25, rel
+
+
+def test_replace_quantize_and_skip_rule():
+    import fp_quant
+
+    class Tiny(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.body = nn.Sequential(nn.Linear(128, 256, bias=True), nn.ReLU(), nn.Linear(256, 128, bias=False))
+            self.lm_head = nn.Linear(128, 64, bias=False)
+
+        def forward(self, x):
+            return self.lm_head(self.body(x))
+
+    torch.manual_seed(0)
+    model = Tiny().to(device="cuda", dtype=torch.bfloat16)
+    x = torch.randn(4, 128, device="cuda", dtype=torch.bfloat16)
+    want = model(x)
+    out = fp_quant.replace_quantize_with_fp_quant_linear(model, _cfg("mxfp4", 128))
+    assert out is model
+    assert isinstance(model.body[0], fp_quant.FPQuantLinear) and isinstance(model.body[2], fp_quant.FPQuantLinear)
+    assert type(model.lm_head) is nn.Linear
+    keys = set(model.body[0].state_dict().keys())
+    assert keys == {"bias", "qweight", "scales", "weight_global_scale", "act_global_scale",
+                    "forward_hadamard_matrix", "backward_hadamard_matrix"}
+    got = model(x)
+    assert (got.float() - want.float()).norm() / want.float().norm() < 0.3
+
+
+def test_state_dict_roundtrip_without_pre_forward():
+    """A checkpoint written by one layer loads into a freshly replaced (never pre_forward-ed)
+    layer and gives identical outputs: what a realquant checkpoint loader relies on."""
+    import fp_quant
+    torch.manual_seed(1)
+    cfg = _cfg("nvfp4", 16)
+    src = fp_quant.FPQuantLinear(256, 128, cfg, bias=True, device="cuda", dtype=torch.bfloat16)
+    src.weight.data.normal_(0, 0.02)
+    src.bias.data.normal_()
+    src.pre_forward()
+    sd = {k: v.clone() for k, v in src.state_dict().items()}
+    dst = fp_quant.FPQuantLinear(256, 128, cfg, bias=True, device="cuda", dtype=torch.bfloat16)
+    dst.weight = None
+    dst.dqweight = None
+    dst.load_state_dict(sd)
+    x = torch.randn(7, 256, device="cuda", dtype=torch.bfloat16)
+    assert torch.equal(src(x), dst(x))
+
+
+def test_operators_have_fake_impls_and_compile():
+    from fp_quant.module import hip_ops
+    x = torch.randn(32, 256, device="cuda", dtype=torch.bfloat16)
+    h = O.hadamard_matrix(32).cuda()
+
+    def f(x):
+        q, s, _ = hip_ops.fused_quantize_mx_op(x, h, "abs_max", False)
+        return q, s
+
+    q0, s0 = f(x)
+    q1, s1 = torch.compile(f, fullgraph=True, backend="eager")(x)
+    assert torch.equal(q0, q1) and torch.equal(s0.view(torch.uint8), s1.view(torch.uint8))
+    assert s0.shape == (128, 8) and s0.dtype == torch.float8_e8m0fnu
+
+
+def test_unsupported_branches_raise():
+    import fp_quant
+    cfg = fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype.MXFP4, forward_method="abs_max",
+                                 backward_dtype=fp_quant.FPQuantDtype.MXFP4, hadamard_group_size=32)
+    lin = fp_quant.FPQuantLinear(64, 32, cfg, bias=False, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        lin(torch.zeros(1, 64, device="cuda", dtype=torch.bfloat16))
+    with pytest.raises(ValueError):
+        fp_quant.FPQuantLinear(64, 32, fp_quant.FPQuantConfig(pseudoquantization=True), device="cuda")
