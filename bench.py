@@ -99,6 +99,72 @@ def bench_quantize(torch, fmt, rows, cols, g, steps, warmup, seed):
     }
 
 
+def bench_linear(torch, fmt, m, n, k, g, steps, warmup, seed):
+    """Quantize activations + W4A4 GEMM (the body of FPQuantLinear.forward) through the C ABI.
+    Weights are quantized once outside the timed region; activations rotate through buffers."""
+    from fp_quant import _engine
+    lib = _engine.lib()
+    dev = torch.device("cuda:0")
+    group = 32 if fmt == "mxfp4" else 16
+    gen = torch.Generator().manual_seed(seed)
+    w = (torch.randn(n, k, generator=gen) * 0.02).to(torch.bfloat16).to(dev)
+    norm = float(torch.tensor(g ** -0.5, dtype=torch.bfloat16))
+    gs = torch.tensor([3.0], dtype=torch.float32, device=dev)
+    alpha = torch.tensor([float((1.0 / (torch.tensor([3.0], dtype=torch.bfloat16) ** 2)).float())],
+                         dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def quant(src, rows, codes, scales):
+        if fmt == "mxfp4":
+            return lib.fpq_quantize_mx(src, rows, k, 0, g, norm, None, codes, scales, rows, k // group, 0, stream)
+        return lib.fpq_quantize_nv(src, rows, k, 0, g, norm, None, gs.data_ptr(), codes, scales, rows,
+                                   k // group, 0, stream)
+
+    wq = torch.empty(n, k // 2, dtype=torch.uint8, device=dev)
+    ws = torch.empty(n, k // group, dtype=torch.uint8, device=dev)
+    _engine.check(quant(w.data_ptr(), n, wq.data_ptr(), ws.data_ptr()), "weight quantize")
+    n_buf = max(2, min(64, int(320e6 // max(1, m * k * 2 + m * n * 2)) + 1))
+    xs_ = [torch.randn(m, k, generator=gen).to(torch.bfloat16).to(dev) for _ in range(min(n_buf, 4))]
+    xs_ = [xs_[i % len(xs_)].clone() for i in range(n_buf)]
+    xq = [torch.empty(m, k // 2, dtype=torch.uint8, device=dev) for _ in range(n_buf)]
+    xsc = [torch.empty(m, k // group, dtype=torch.uint8, device=dev) for _ in range(n_buf)]
+    ys = [torch.empty(m, n, dtype=torch.bfloat16, device=dev) for _ in range(n_buf)]
+    gemm = lib.fpq_gemm_mxf4 if fmt == "mxfp4" else lib.fpq_gemm_nvf4
+    p = [(xs_[i].data_ptr(), xq[i].data_ptr(), xsc[i].data_ptr(), ys[i].data_ptr()) for i in range(n_buf)]
+
+    def run_linear(i):
+        a, b, c, d = p[i]
+        st = quant(a, m, b, c)
+        st = st or gemm(b, c, k // group, wq.data_ptr(), ws.data_ptr(), k // group, alpha.data_ptr(), None,
+                        d, m, n, k, stream)
+        if st != 0:
+            _engine.check(st, "bench linear")
+
+    def run_gemm(i):
+        a, b, c, d = p[i]
+        st = gemm(b, c, k // group, wq.data_ptr(), ws.data_ptr(), k // group, alpha.data_ptr(), None,
+                  d, m, n, k, stream)
+        if st != 0:
+            _engine.check(st, "bench gemm")
+
+    wall, ev = time_kernel(torch, run_linear, n_buf, steps, warmup)
+    _, ev_gemm = time_kernel(torch, run_gemm, n_buf, steps, warmup)
+    flops = 2.0 * m * n * k
+    gemm_bytes = n * k / 2 + n * k / group + m * k / 2 + m * k / group + 2.0 * m * n
+    return {
+        "workload": f"{fmt}_linear_M{m}_N{n}_K{k}_had{g}",
+        "ms_per_step": wall,
+        "linear_ms": ev,
+        "gemm_ms": ev_gemm,
+        "flops": flops,
+        "gemm_bytes": gemm_bytes,
+        "linear_tflops": flops / (ev * 1e-3) / 1e12,
+        "gemm_tflops": flops / (ev_gemm * 1e-3) / 1e12,
+        "gemm_gbps": gemm_bytes / (ev_gemm * 1e-3) / 1e9,
+        "buffers": n_buf,
+    }
+
+
 def cpu_baseline_quantize(torch, fmt, rows, cols, g, seed, sample_rows):
     """The oracle (a torch-CPU restatement of the reference's PyTorch quantizer path) timed
     on a bounded row sample of the same workload."""
@@ -127,12 +193,42 @@ def cpu_baseline_quantize(torch, fmt, rows, cols, g, seed, sample_rows):
     }
 
 
+def cpu_baseline_linear(torch, m_sample, n, k, g, seed):
+    """The oracle's MXFP4 linear (quantize activations, dequantize both operands, fp32 matmul:
+    the reference's CPU pseudo-quant path) on a bounded sample of activation rows; weights are
+    quantized once outside the timed region, as on the GPU."""
+    from oracle import fpq_oracle as O
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    gen = torch.Generator().manual_seed(seed)
+    w = (torch.randn(n, k, generator=gen) * 0.02).to(torch.bfloat16)
+    x = torch.randn(m_sample, k, generator=gen).to(torch.bfloat16)
+    wq, ws, _ = O.quantize_mx(w, O.ROT_HADAMARD, g)
+    dw = O.dequantize(wq, ws, "mxfp4").float()
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        xq, xs, _ = O.quantize_mx(x, O.ROT_HADAMARD, g)
+        dx = O.dequantize(xq, xs, "mxfp4").float()
+        y = (torch.nn.functional.linear(dx, dw) * 0.111328125).to(torch.bfloat16)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    del y
+    return {
+        "value": 2.0 * m_sample * n * k / best / 1e12,
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{m_sample} activation rows of the M=2048 N={n} K={k} MXFP4 linear (quantize + dequant + "
+                  "fp32 matmul), best of 3, torch CPU oracle",
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="nvfp4_quantize")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -151,11 +247,32 @@ def main():
     results["nvfp4_quantize"] = bench_quantize(torch, "nvfp4", 8192, 4096, 16, args.steps, args.warmup, seed=1)
     results["mxfp4_quantize"] = bench_quantize(torch, "mxfp4", 2048, 4096, 128, args.steps, args.warmup, seed=0)
 
-    head = results[args.workload]
+    linears = {}
+    for m in (2048, 128, 16, 1):
+        linears[m] = bench_linear(torch, "mxfp4", m, 14336, 4096, 128, args.steps, args.warmup, seed=2)
+    nv = bench_linear(torch, "nvfp4", 4096, 24576, 4096, 16, max(10, args.steps // 10), max(2, args.warmup // 10), seed=3)
+
+    quant = results["nvfp4_quantize"]
+    head = linears[2048]
+    kernels = {
+        k: {"workload": v["workload"], "kernel_us": round(v["kernel_ms"] * 1e3, 3),
+            "GB/s": round(v["gbps"], 2), "hbm_frac": round(v["gbps"] / HBM_PEAK_GBS, 4)}
+        for k, v in results.items()
+    }
+    for m, v in linears.items():
+        kernels[f"mxfp4_gemm_M{m}"] = {
+            "workload": v["workload"], "gemm_us": round(v["gemm_ms"] * 1e3, 3),
+            "linear_us": round(v["linear_ms"] * 1e3, 3), "gemm_TFLOP/s": round(v["gemm_tflops"], 2),
+            "mfma_frac": round(v["gemm_tflops"] / FP4_PEAK_TFLOPS, 4),
+            "gemm_GB/s": round(v["gemm_gbps"], 2), "hbm_frac": round(v["gemm_gbps"] / HBM_PEAK_GBS, 4)}
+    kernels["nvfp4_gemm_M4096_gate_up"] = {
+        "workload": nv["workload"], "gemm_us": round(nv["gemm_ms"] * 1e3, 3),
+        "gemm_TFLOP/s": round(nv["gemm_tflops"], 2),
+        "mfma_frac_of_f16_peak": round(nv["gemm_tflops"] / BF16_PEAK_TFLOPS, 4)}
     line = {
         "metric": METRIC,
-        "value": round(head["gbps"], 2),
-        "unit": "GB/s",
+        "value": round(head["linear_tflops"], 2),
+        "unit": "TFLOP/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
@@ -163,29 +280,37 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "fp4",
         "data": "synthetic",
-        "config": {"workload": head["workload"], "rotating_buffers": head["buffers"]},
+        "config": {"workload": head["workload"] + " (activation rotate+quantize then W4A4 GEMM)",
+                   "rotating_buffers": head["buffers"]},
         "roofline": {
+            "kernel": "MXFP4 W4A4 GEMM, M=2048 N=14336 K=4096",
+            "bound": "mfma",
+            "achieved": round(head["gemm_tflops"], 2),
+            "peak": FP4_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(head["gemm_tflops"] / FP4_PEAK_TFLOPS, 4),
+            "traffic": None,
+            "kernel_us": round(head["gemm_ms"] * 1e3, 3),
+            "algorithmic_flops_per_launch": int(head["flops"]),
+        },
+        "roofline_quantize": {
+            "kernel": "NVFP4 fused rotate+quantize, bf16 [8192, 4096], Hadamard 16",
             "bound": "hbm",
-            "achieved": round(head["gbps"], 2),
+            "achieved": round(quant["gbps"], 2),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(head["gbps"] / HBM_PEAK_GBS, 4),
+            "frac": round(quant["gbps"] / HBM_PEAK_GBS, 4),
             "traffic": None,
-            "kernel_us": round(head["kernel_ms"] * 1e3, 3),
-            "algorithmic_bytes_per_launch": int(head["algo_bytes"]),
+            "kernel_us": round(quant["kernel_ms"] * 1e3, 3),
+            "algorithmic_bytes_per_launch": int(quant["algo_bytes"]),
         },
-        "kernels": {
-            k: {"workload": v["workload"], "kernel_us": round(v["kernel_ms"] * 1e3, 3),
-                "GB/s": round(v["gbps"], 2), "hbm_frac": round(v["gbps"] / HBM_PEAK_GBS, 4)}
-            for k, v in results.items()
-        },
+        "kernels": kernels,
     }
     if not args.no_cpu_baseline:
-        fmt = "nvfp4" if args.workload.startswith("nvfp4") else "mxfp4"
-        shape = (8192, 4096, 16, 1) if fmt == "nvfp4" else (2048, 4096, 128, 0)
-        line["cpu_baseline"] = cpu_baseline_quantize(torch, fmt, shape[0], shape[1], shape[2], shape[3], 1024)
+        line["cpu_baseline"] = cpu_baseline_linear(torch, 64, 14336, 4096, 128, seed=2)
+        line["cpu_baseline_quantize"] = cpu_baseline_quantize(torch, "nvfp4", 8192, 4096, 16, 1, 1024)
     print(json.dumps(line))
 
 

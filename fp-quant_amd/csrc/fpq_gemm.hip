@@ -23,6 +23,7 @@ namespace fpq {
 
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
@@ -146,6 +147,264 @@ __global__ __launch_bounds__(256) void gemm_mxf4_direct_kernel(
   store_tile<TN, TM>(acc, y, bias, *alpha_p, n0, m0, M, N, r, kb);
 }
 
+// -------------------------------------------------------------------------------------------
+// LDS-tiled MXFP4 kernel for large M.  A block of 4 waves (2 x 2) owns a BN x BM output tile and
+// walks K in steps of 256 (one 128-byte line of codes per row).  Packed codes and scale bytes go
+// global -> LDS with direct 16-byte / 4-byte loads into a double buffer; the 16-byte chunks of a
+// row are XOR-swizzled by (row & 7) through the choice of the global chunk each lane fetches, so
+// that the 16-row x 64-byte MFMA operand reads are bank-conflict free.
+constexpr int kKS = 256;                    // K per stage
+constexpr int kRowBytes = kKS / 2;          // 128 bytes of codes per row per stage
+constexpr int kScaleBytes = kKS / 32;       // 8 scale bytes per row per stage
+
+typedef __attribute__((address_space(3))) void lds_void;
+typedef const __attribute__((address_space(1))) void global_void;
+
+template <int BN, int BM>
+struct MxLdsLayout {
+  static constexpr int kCodesW = 0;
+  static constexpr int kCodesX = BN * kRowBytes;
+  static constexpr int kScalesW = (BN + BM) * kRowBytes;
+  static constexpr int kScalesX = kScalesW + BN * kScaleBytes;
+  static constexpr int kStage = kScalesX + BM * kScaleBytes;
+};
+
+// Direct global -> LDS load of 16 (4) bytes per lane: LDS address = lds_base + lane * 16 (4).
+// Written as inline assembly so that the compiler does not serialise every later LDS read
+// behind these loads; completion is awaited explicitly with wait_vmem() before the barrier.
+// Nothing else in these kernels uses M0.
+__device__ __forceinline__ void lds_dma16(const uint8_t* gbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :: "s"(lds_base), "v"(voff), "s"(gbase) : "memory");
+}
+__device__ __forceinline__ void lds_dma4(const uint8_t* gbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2"
+               :: "s"(lds_base), "v"(voff), "s"(gbase) : "memory");
+}
+__device__ __forceinline__ void wait_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+}
+
+template <int BN, int BM>
+__global__ __launch_bounds__(256) void gemm_mxf4_lds_kernel(
+    const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, int xs_stride,
+    const uint8_t* __restrict__ wq, const uint8_t* __restrict__ ws, int ws_stride,
+    const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
+    int M, int N, int K, int tiles_m) {
+  using L = MxLdsLayout<BN, BM>;
+  constexpr int TN = BN / 64, TM = BM / 64;   // 32x32 MFMA tiles per wave along n and m
+  extern __shared__ __attribute__((aligned(128))) uint8_t smem[];
+  const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  // Consecutive workgroup ids land on different XCDs (8 of them, each with its own L2), so
+  // give every XCD a contiguous run of the tile list: its tiles then share weight row-panels.
+  int logical = blockIdx.x;
+  {
+    const int nb = gridDim.x, per = nb / 8;
+    if (blockIdx.x < (unsigned)(per * 8)) logical = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+  }
+  const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
+  const int n_blk = tile_n * BN, m_blk = tile_m * BM;
+  const int wn = wave & 1, wm = wave >> 1;
+  const int kbytes = K >> 1;
+
+  // ---- global -> LDS assignment.  Codes: one wave instruction moves 8 rows x 128 B.
+  constexpr int kInstrW = BN / 8 / 4, kInstrX = BM / 8 / 4;  // per wave
+  const int lrow = lane >> 3;                                // row within the 8-row slab
+  const int chunk = (lane & 7) ^ lrow;                       // swizzled 16-byte chunk this lane fetches
+  uint32_t w_off[kInstrW], x_off[kInstrX];
+#pragma unroll
+  for (int j = 0; j < kInstrW; ++j) {
+    const int row = min(n_blk + (wave * kInstrW + j) * 8 + lrow, N - 1);
+    w_off[j] = (uint32_t)row * (uint32_t)kbytes + chunk * 16;
+  }
+#pragma unroll
+  for (int j = 0; j < kInstrX; ++j) {
+    const int row = min(m_blk + (wave * kInstrX + j) * 8 + lrow, M - 1);
+    x_off[j] = (uint32_t)row * (uint32_t)kbytes + chunk * 16;
+  }
+  // Scales: one wave instruction moves 32 rows x 8 B (two dwords per row); wave w takes
+  // instructions j with j % 4 == w.
+  constexpr int kSInstrW = BN / 32, kSInstrX = BM / 32;
+  constexpr int kSW = (kSInstrW + 3) / 4, kSX = (kSInstrX + 3) / 4;
+  uint32_t ws_off[kSW], xs_off[kSX];
+#pragma unroll
+  for (int j = 0; j < kSW; ++j) {
+    const int row = min(n_blk + (j * 4 + wave) * 32 + (lane >> 1), N - 1);
+    ws_off[j] = (uint32_t)row * (uint32_t)ws_stride + (lane & 1) * 4;
+  }
+#pragma unroll
+  for (int j = 0; j < kSX; ++j) {
+    const int row = min(m_blk + (j * 4 + wave) * 32 + (lane >> 1), M - 1);
+    xs_off[j] = (uint32_t)row * (uint32_t)xs_stride + (lane & 1) * 4;
+  }
+
+  auto issue_loads = [&](int stage, int k0) {
+    const uint32_t base = smem_base + stage * L::kStage;
+    const uint8_t* wk = wq + (k0 >> 1);
+    const uint8_t* xk = xq + (k0 >> 1);
+    const uint8_t* wsk = ws + (k0 >> 5);
+    const uint8_t* xsk = xs + (k0 >> 5);
+#pragma unroll
+    for (int j = 0; j < kInstrW; ++j)
+      lds_dma16(wk, w_off[j], base + L::kCodesW + (wave * kInstrW + j) * 1024);
+#pragma unroll
+    for (int j = 0; j < kInstrX; ++j)
+      lds_dma16(xk, x_off[j], base + L::kCodesX + (wave * kInstrX + j) * 1024);
+#ifndef FPQ_EXP_NO_SCALE_DMA
+#pragma unroll
+    for (int j = 0; j < kSW; ++j)
+      if (j * 4 + wave < kSInstrW) lds_dma4(wsk, ws_off[j], base + L::kScalesW + (j * 4 + wave) * 256);
+#pragma unroll
+    for (int j = 0; j < kSX; ++j)
+      if (j * 4 + wave < kSInstrX) lds_dma4(xsk, xs_off[j], base + L::kScalesX + (j * 4 + wave) * 256);
+#endif
+  };
+
+  // 32x32x64 MFMA: lane = (row r32 = lane % 32, K half kh = lane / 32); one stage holds four
+  // K steps q of 64, the lane's 16-byte chunk in step q is c = 2q + kh, its scale byte is c too.
+  v16f acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int r32 = lane & 31, kh = lane >> 5;
+  const int rw = wn * (BN / 2) + r32, rx = wm * (BM / 2) + r32;
+  int slot[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) slot[q] = ((2 * q + kh) ^ (r32 & 7)) * 16;
+  const int cw0 = L::kCodesW + rw * kRowBytes, cx0 = L::kCodesX + rx * kRowBytes;
+  const int sw0 = L::kScalesW + rw * kScaleBytes, sx0 = L::kScalesX + rx * kScaleBytes;
+  // bytes kh, 2+kh, 4+kh, 6+kh of a row's 8 scale bytes -> one dword; op_sel q picks K step q
+  const uint32_t perm_sel = kh ? 0x07050301u : 0x06040200u;
+
+  const int nk = K / kKS;
+  issue_loads(0, 0);
+  for (int it = 0; it < nk; ++it) {
+    const int stage = it & 1;
+    wait_vmem();  // this wave's loads for `stage` have landed
+    __syncthreads();
+    const uint8_t* base = smem + stage * L::kStage;
+    // Operand stream of a stage: 4 K steps x TN weight tiles, each tile used by TM MFMAs.
+    // Weight tiles are read from LDS two steps ahead (ring of 3), the activation tiles of the
+    // next K step during the first steps of the current one; sched_barrier keeps that order.
+    uint4 bq[2][TM], aq[3];
+    int sa[TN], sb[TM];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) bq[0][j] = *(const uint4*)(base + cx0 + slot[0] + j * 32 * kRowBytes);
+    aq[0] = *(const uint4*)(base + cw0 + slot[0]);
+    aq[1] = *(const uint4*)(base + cw0 + slot[0] + 32 * kRowBytes);
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      const uint2 v = *(const uint2*)(base + sx0 + j * 32 * kScaleBytes);
+      sb[j] = (int)__builtin_amdgcn_perm(v.y, v.x, perm_sel);
+    }
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+      const uint2 v = *(const uint2*)(base + sw0 + i * 32 * kScaleBytes);
+      sa[i] = (int)__builtin_amdgcn_perm(v.y, v.x, perm_sel);
+    }
+#ifndef FPQ_EXP_NO_DMA
+    if (it + 1 < nk) issue_loads(stage ^ 1, (it + 1) * kKS);
+#endif
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < 4 * TN; ++t) {
+      const int q = t / TN, i = t % TN;
+      if (t + 2 < 4 * TN) {
+        const int q2 = (t + 2) / TN, i2 = (t + 2) % TN;
+        aq[(t + 2) % 3] = *(const uint4*)(base + cw0 + slot[q2] + i2 * 32 * kRowBytes);
+      }
+      if (q < 3 && i < (TM + 1) / 2) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int j = i * 2 + u;
+          if (j < TM) bq[(q + 1) & 1][j] = *(const uint4*)(base + cx0 + slot[q + 1] + j * 32 * kRowBytes);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      const uint4 av = aq[t % 3];
+      const v8i a = v8i{(int)av.x, (int)av.y, (int)av.z, (int)av.w, 0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < TM; ++j) {
+        const uint4 bv = bq[q & 1][j];
+        const v8i b = v8i{(int)bv.x, (int)bv.y, (int)bv.z, (int)bv.w, 0, 0, 0, 0};
+        if (q == 0) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], 4, 4, 0, sa[i], 0, sb[j]);
+        if (q == 1) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], 4, 4, 1, sa[i], 1, sb[j]);
+        if (q == 2) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], 4, 4, 2, sa[i], 2, sb[j]);
+        if (q == 3) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], 4, 4, 3, sa[i], 3, sb[j]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // ---- epilogue.  Accumulator register v of tile (i, j) is y[m][n] with m = j*32 + r32 and
+  // n = i*32 + 8*(v/4) + 4*kh + v%4 inside the wave's 128 x 128 quadrant.  The quadrant goes
+  // through this wave's share of the (now idle) LDS as bf16 [m][n] so that global stores are
+  // 256 contiguous bytes per row.
+  const float alpha = *alpha_p;
+#ifdef FPQ_EXP_NO_STORE
+  if (alpha != 12345.0f) return;
+#endif
+  constexpr int WT_N = BN / 2, WT_M = BM / 2;        // wave quadrant
+  constexpr int kStride = WT_N * 2 + 16;             // bytes per staged row (+16: spread banks)
+  static_assert(4 * WT_M * kStride <= 2 * L::kStage, "epilogue staging does not fit in LDS");
+  __syncthreads();                                   // every wave is done reading operands
+  uint8_t* stg = smem + wave * (WT_M * kStride);
+  const int n0 = n_blk + wn * WT_N, m0 = m_blk + wm * WT_M;
+#pragma unroll
+  for (int i = 0; i < TN; ++i) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int nl = i * 32 + 8 * g + 4 * kh;
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (bias) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (n0 + nl + u < N) bv[u] = __uint_as_float((uint32_t)bias[n0 + nl + u] << 16);
+      }
+#pragma unroll
+      for (int j = 0; j < TM; ++j) {
+        uint32_t lo = pack_bf16x2(acc[i][j][4 * g + 0] * alpha, acc[i][j][4 * g + 1] * alpha);
+        uint32_t hi = pack_bf16x2(acc[i][j][4 * g + 2] * alpha, acc[i][j][4 * g + 3] * alpha);
+        if (bias) {
+          lo = pack_bf16x2(__uint_as_float(lo << 16) + bv[0], __uint_as_float(lo & 0xffff0000u) + bv[1]);
+          hi = pack_bf16x2(__uint_as_float(hi << 16) + bv[2], __uint_as_float(hi & 0xffff0000u) + bv[3]);
+        }
+        *(uint2*)(stg + (j * 32 + r32) * kStride + nl * 2) = make_uint2(lo, hi);
+      }
+    }
+  }
+  // read back: 16 lanes x 16 B cover one 256-byte row, 4 rows per wave instruction
+  const int rr = lane >> 4, cc = lane & 15;
+  const bool vec_ok = (N & 7) == 0;
+#pragma unroll 4
+  for (int p = 0; p < WT_M / 4; ++p) {
+    const int ml = p * 4 + rr;
+    const uint4 v = *(const uint4*)(stg + ml * kStride + cc * 16);
+    const int m = m0 + ml, n = n0 + cc * 8;
+    if (m >= M || n >= N) continue;
+    uint16_t* dst = y + (size_t)m * N + n;
+    if (vec_ok && n + 7 < N) {
+      *(uint4*)dst = v;
+    } else {
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (n + u < N) dst[u] = (uint16_t)(w[u >> 1] >> (16 * (u & 1)));
+    }
+  }
+}
+
 // 8 E2M1 codes (one dword) times one E4M3 scale -> 8 exact fp16 values.
 __device__ __forceinline__ v8h dequant8_f16(uint32_t codes, uint32_t scale_byte) {
   const uint32_t h = ((scale_byte & 0x7fu) << 7) | ((scale_byte & 0x80u) << 8);
@@ -265,7 +524,7 @@ static int gemm_dispatch(const void* xq, const void* xs, int64_t xs_stride, cons
   if (K == 0 || K % GROUP != 0 || K % 32 != 0) return FPQ_E_SHAPE;
   if (xs_stride < K / GROUP || ws_stride < K / GROUP) return FPQ_E_SHAPE;
   if (M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return FPQ_E_SHAPE;
-  if (((uintptr_t)xq & 15u) || ((uintptr_t)wq & 15u) || ((uintptr_t)y & 7u)) return FPQ_E_ALIGN;
+  if (((uintptr_t)xq & 15u) || ((uintptr_t)wq & 15u) || ((uintptr_t)y & 15u)) return FPQ_E_ALIGN;
 
 #define FPQ_GEMM(TN, TM, WN, WM)                                                                   \
   do {                                                                                             \
@@ -284,6 +543,25 @@ static int gemm_dispatch(const void* xq, const void* xs, int64_t xs_stride, cons
     }                                                                                              \
   } while (0)
 
+  if (FMT == 0 && M > 64 && K % kKS == 0 && xs_stride % 4 == 0 && ws_stride % 4 == 0 &&
+      !((uintptr_t)xs & 3u) && !((uintptr_t)ws & 3u) && N * (K / 2) < ((int64_t)1 << 32) &&
+      M * (K / 2) < ((int64_t)1 << 32)) {
+    constexpr int BN = 256, BM = 256;
+    using L = MxLdsLayout<BN, BM>;
+    const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
+    static bool attr_set = false;
+    if (!attr_set) {
+      hipError_t e = hipFuncSetAttribute((const void*)gemm_mxf4_lds_kernel<BN, BM>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 2 * L::kStage);
+      if (e != hipSuccess) return (int)e;
+      attr_set = true;
+    }
+    hipLaunchKernelGGL((gemm_mxf4_lds_kernel<BN, BM>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256),
+                       2 * L::kStage, stream, (const uint8_t*)xq, (const uint8_t*)xs, (int)xs_stride,
+                       (const uint8_t*)wq, (const uint8_t*)ws, (int)ws_stride, alpha,
+                       (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K, tiles_m);
+    return (int)hipGetLastError();
+  }
   if (M <= 16) {
     FPQ_GEMM(1, 1, 4, 1);
   } else if (M <= 32) {

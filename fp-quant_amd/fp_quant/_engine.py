@@ -6,7 +6,9 @@ import ctypes
 import os
 import threading
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "libfpq_hip.so")
+# FPQ_LIBRARY_PATH lets a developer point the binding at another build of the same C ABI.
+_LIB_PATH = os.environ.get("FPQ_LIBRARY_PATH") or os.path.join(
+    os.path.dirname(os.path.abspath(__file__)), "_lib", "libfpq_hip.so")
 _lock = threading.Lock()
 _lib = None
 

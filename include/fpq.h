@@ -85,7 +85,7 @@ int fpq_quantize_nv(const void* x, int64_t rows, int64_t cols, int rot_kind, int
  * reference re-tiles them with to_blocked on every call; this engine needs no re-tiling).
  *   xq uint8 [M, K/2], wq uint8 [N, K/2] (16-byte aligned rows: K % 32 == 0)
  *   xs uint8 E8M0 [>=M, xs_stride], ws uint8 E8M0 [>=N, ws_stride], entry [row, k/32]
- *   alpha device pointer to one fp32; bias bf16 [N] or null; y bf16 [M, N]
+ *   alpha device pointer to one fp32; bias bf16 [N] or null; y bf16 [M, N], 16-byte aligned
  */
 int fpq_gemm_mxf4(const void* xq, const void* xs, int64_t xs_stride, const void* wq,
                   const void* ws, int64_t ws_stride, const float* alpha, const void* bias,
