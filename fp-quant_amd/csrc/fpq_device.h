@@ -153,4 +153,27 @@ __device__ __forceinline__ float scale_element(float x, const GroupScale& g) {
   return g.slow ? x / g.k1 : __builtin_fmaf(x, g.k1, x * g.k2);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Direct global -> LDS loads: 16 (4) bytes per lane land at lds_base + lane * 16 (4).  Written as
+// inline assembly so that the compiler does not serialise every later LDS read behind them;
+// completion is awaited explicitly with wait_vmem().  Nothing else in these kernels uses M0.
+__device__ __forceinline__ void lds_dma16(const uint8_t* gbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :: "s"(lds_base), "v"(voff), "s"(gbase) : "memory");
+}
+__device__ __forceinline__ void lds_dma4(const uint8_t* gbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2"
+               :: "s"(lds_base), "v"(voff), "s"(gbase) : "memory");
+}
+__device__ __forceinline__ void wait_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// a / 6 correctly rounded (the reference writes fl(fl(2a)/12), the same number): Markstein's
+// correction with RN(1/6), exact for every mantissa (checked exhaustively on the host).
+__device__ __forceinline__ float div6_rn(float a) {
+  const float c6 = 0.16666667163372039794921875f;
+  const float q = a * c6;
+  const float r = __builtin_fmaf(-q, 6.0f, a);
+  return __builtin_fmaf(r, c6, q);
+}
+
 }  // namespace fpq

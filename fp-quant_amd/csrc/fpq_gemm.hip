@@ -169,20 +169,6 @@ struct MxLdsLayout {
   static constexpr int kStage = kScalesX + BM * kScaleBytes;
 };
 
-// Direct global -> LDS load of 16 (4) bytes per lane: LDS address = lds_base + lane * 16 (4).
-// Written as inline assembly so that the compiler does not serialise every later LDS read
-// behind these loads; completion is awaited explicitly with wait_vmem() before the barrier.
-// Nothing else in these kernels uses M0.
-__device__ __forceinline__ void lds_dma16(const uint8_t* gbase, uint32_t voff, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :: "s"(lds_base), "v"(voff), "s"(gbase) : "memory");
-}
-__device__ __forceinline__ void lds_dma4(const uint8_t* gbase, uint32_t voff, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2"
-               :: "s"(lds_base), "v"(voff), "s"(gbase) : "memory");
-}
-__device__ __forceinline__ void wait_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 

@@ -12,6 +12,10 @@
 
 namespace fpq {
 
+#ifndef FPQ_EPL
+#define FPQ_EPL 64  // elements owned by one lane in the streaming kernel (64 or 128)
+#endif
+
 constexpr int kFmtMx = 0;
 constexpr int kFmtNv = 1;
 
@@ -19,16 +23,15 @@ constexpr int kFmtNv = 1;
 // Generic kernel: one lane owns 8 consecutive elements (one 16-byte load, 4 bytes of codes).
 // A rotation block of G elements spans G/8 neighbouring lanes; the butterflies with stride
 // >= 8 exchange registers between lanes.  Works for any cols % max(G, GROUP) == 0.
+// One lane quantizes 8 consecutive elements (chunk index `chunk`); the G/8 neighbouring lanes of
+// a rotation block exchange registers for the butterflies with stride >= 8.  Must be called by
+// all 64 lanes of a wave with consecutive chunk indices (inactive lanes pass active = false).
 template <int G, int FMT, int ROT, int ZERO>
-__global__ __launch_bounds__(256) void quantize_lane8_kernel(
-    const uint4* __restrict__ x, uint32_t* __restrict__ codes, uint8_t* __restrict__ scales,
-    uint32_t n_chunks, uint32_t chunks_per_row, uint32_t rows, uint32_t scale_rows,
-    uint32_t scale_stride, float norm, const float* __restrict__ global_scale) {
+__device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint32_t* __restrict__ codes,
+                                              uint8_t* __restrict__ scales, uint32_t chunk, bool active,
+                                              uint32_t lane, uint32_t chunks_per_row,
+                                              uint32_t scale_stride, float norm, float gscale, float rg) {
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
-  const uint32_t chunk = blockIdx.x * 256u + threadIdx.x;
-  const uint32_t lane = threadIdx.x & 63u;
-  const bool active = chunk < n_chunks;
-
   uint4 raw = make_uint4(0u, 0u, 0u, 0u);
   if (active) raw = x[chunk];
 
@@ -74,15 +77,14 @@ __global__ __launch_bounds__(256) void quantize_lane8_kernel(
   if (FMT == kFmtMx) {
     gs = mx_group_scale(a);
   } else {
-    const float g = *global_scale;
-    const float rg = g == 0.0f ? 0.0f : 1.0f / g;
-    gs = nv_group_scale(a, g, rg);
+    gs = nv_group_scale(a, gscale, rg);
   }
 
   uint32_t packed = 0u;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     float v = scale_element(p[i], gs);
+    if (ZERO == kZeroSigned) v = __builtin_copysignf(v, p[i]);  // x / s keeps the sign of x, also for -0
     if (FMT == kFmtNv) v = gs.zero ? 0.0f : v;
     packed |= e2m1_code<ZERO>(v) << (4 * i);
   }
@@ -95,17 +97,38 @@ __global__ __launch_bounds__(256) void quantize_lane8_kernel(
       scales[(size_t)row * scale_stride + col] = (uint8_t)gs.byte;
     }
   }
+}
 
-  // zero-fill the padded part of the scale tensor (rows >= rows, columns >= cols / GROUP)
-  const uint32_t valid_cols = chunks_per_row / (GROUP / 8);
+// zero-fill the padded part of a scale tensor (rows >= rows, columns >= valid_cols)
+__device__ __forceinline__ void fill_scale_padding(uint8_t* __restrict__ scales, uint32_t rows,
+                                                   uint32_t valid_cols, uint32_t scale_rows,
+                                                   uint32_t scale_stride) {
   if (scale_rows != rows || scale_stride != valid_cols) {
     const uint32_t total = scale_rows * scale_stride;
-    for (uint32_t i = chunk; i < total; i += gridDim.x * 256u) {
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
       const uint32_t r = i / scale_stride;
       const uint32_t c = i - r * scale_stride;
       if (r >= rows || c >= valid_cols) scales[i] = 0;
     }
   }
+}
+
+// Generic kernel: works for any cols % max(G, GROUP) == 0; one 8-element chunk per thread.
+template <int G, int FMT, int ROT, int ZERO>
+__global__ __launch_bounds__(256) void quantize_lane8_kernel(
+    const uint4* __restrict__ x, uint32_t* __restrict__ codes, uint8_t* __restrict__ scales,
+    uint32_t n_chunks, uint32_t chunks_per_row, uint32_t rows, uint32_t scale_rows,
+    uint32_t scale_stride, float norm, const float* __restrict__ global_scale) {
+  constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
+  const uint32_t chunk = blockIdx.x * 256u + threadIdx.x;
+  float g = 1.0f, rg = 1.0f;
+  if (FMT == kFmtNv) {
+    g = *global_scale;
+    rg = g == 0.0f ? 0.0f : 1.0f / g;
+  }
+  lane8_process<G, FMT, ROT, ZERO>(x, codes, scales, chunk, chunk < n_chunks, threadIdx.x & 63u,
+                                   chunks_per_row, scale_stride, norm, g, rg);
+  fill_scale_padding(scales, rows, chunks_per_row / (GROUP / 8), scale_rows, scale_stride);
 }
 
 template <int G, int FMT, int ROT>
@@ -123,6 +146,274 @@ static int launch_lane8(const void* x, int64_t rows, int64_t cols, float norm, c
     args(quantize_lane8_kernel<G, FMT, ROT, kZeroReference>);
   } else {
     args(quantize_lane8_kernel<G, FMT, ROT, kZeroSigned>);
+  }
+  return (int)hipGetLastError();
+}
+
+// -------------------------------------------------------------------------------------------
+// Streaming kernel for cols % EPL == 0 (EPL = 64 or 128): one lane owns EPL consecutive elements
+// (2*EPL bytes in, EPL/2 bytes of codes and EPL/32 or EPL/16 scale bytes out), so the butterfly
+// stages with stride < EPL, every group maximum and the packing stay inside the lane's registers;
+// a 128-wide rotation with EPL = 64 adds one exchange between neighbouring lanes.  A wave moves
+// 64 such chunks per tile: direct global -> LDS loads in full contiguous runs, then each lane
+// reads its own chunk back with 16-byte LDS reads.  The 16-byte pieces of a chunk are
+// XOR-swizzled by the lane number (through the choice of the piece each DMA lane fetches) so
+// those reads are bank-conflict free.  Codes return through the same LDS region so that global
+// stores are contiguous.
+constexpr float kKappa = -0x1.8p-26f;  // fma(x, 0.75, x * kKappa) rounds to the E2M1 code of x / fl(4/3)
+
+template <int ZERO>
+__device__ __forceinline__ uint32_t fix_zero_nibbles(uint32_t w) {
+  if (ZERO == kZeroReference) {
+    const uint32_t nz = ((w & 0x77777777u) + 0x77777777u) & 0x88888888u;  // bit 3 set where magnitude != 0
+    w |= nz ^ 0x88888888u;
+  }
+  return w;
+}
+
+template <int EPL, int G, int FMT, int ROT, int ZERO>
+__global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
+    const uint8_t* __restrict__ x, uint8_t* __restrict__ codes, uint8_t* __restrict__ scales,
+    uint32_t n_chunks, uint32_t chunks_per_row, uint32_t rows, uint32_t scale_rows,
+    uint32_t scale_stride, float norm, const float* __restrict__ global_scale) {
+  constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
+  constexpr int NG = EPL / GROUP;        // groups (= scale bytes) per chunk
+  constexpr int PIECES = EPL / 8;        // 16-byte input pieces per chunk
+  constexpr uint32_t CB = EPL * 2;       // input bytes per chunk
+  constexpr uint32_t TILE = 64 * CB;     // input bytes per wave tile
+  constexpr int CPI = 64 / PIECES;       // chunks filled by one DMA instruction
+  constexpr int CW = EPL / 8;            // code dwords per chunk
+  constexpr int CQ = CW / 4;             // 16-byte code pieces per chunk
+  __shared__ __attribute__((aligned(128))) uint8_t smem[4][TILE];
+  __shared__ float2 lut[128];
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t lane = threadIdx.x & 63u;
+  uint8_t* my = smem[wave];
+  const uint32_t my_base = (uint32_t)(uintptr_t)my;
+
+  float gs = 1.0f, rg = 1.0f;
+  bool nv_fast = true;
+  if (FMT == kFmtNv) {
+    gs = *global_scale;
+    rg = gs == 0.0f ? 0.0f : 1.0f / gs;
+    // with 2^-60 <= gs <= 2^60 no product of an E4M3 value with gs or 1/gs leaves the normal range
+    nv_fast = gs >= 8.673617379884035e-19f && gs <= 1.152921504606847e18f;
+    if (threadIdx.x < 128) {
+      const float s = e4m3_decode(threadIdx.x) * rg;
+      float2 e = make_float2(0.0f, 0.0f);
+      if (s != 0.0f && nv_fast) {
+        const float y = 1.0f / s;
+        e = make_float2(y, __builtin_fmaf(-s, y, 1.0f) / s);
+      }
+      lut[threadIdx.x] = e;
+    }
+    __syncthreads();
+  }
+
+  // DMA lane map: instruction i fills LDS pieces [64 i, 64 i + 64); piece p = PIECES * b + j
+  // belongs to chunk b and holds that chunk's 16-byte piece j ^ (b % PIECES).
+  const uint32_t b_lo = lane / PIECES, j_lo = lane % PIECES;
+  constexpr int NV_OFF = PIECES / CPI > 0 ? PIECES / CPI : 1;  // distinct swizzle phases over i
+  uint32_t voff[NV_OFF];
+#pragma unroll
+  for (int m = 0; m < NV_OFF; ++m)
+    voff[m] = b_lo * CB + ((j_lo ^ ((CPI * m + b_lo) % PIECES)) * 16u);
+  const uint32_t rd_base = lane * CB, l_sw = lane % PIECES;
+
+  const uint32_t n_tiles = (n_chunks + 63u) / 64u;
+  const uint32_t total_waves = gridDim.x * 4u;
+  for (uint32_t tile = blockIdx.x * 4u + wave; tile < n_tiles; tile += total_waves) {
+    const uint32_t valid = min(64u, n_chunks - tile * 64u);
+    const uint8_t* src = x + (size_t)tile * TILE;
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+      // The lane offset is an unsigned 32-bit addend to a scalar base, so it must never be
+      // negative.  Chunks past the end of the tensor re-read valid bytes instead: the first
+      // chunk of this instruction if that one is valid, else the first chunk of the tile.
+      uint32_t off = voff[i % NV_OFF];
+      const bool instr_valid = (uint32_t)(CPI * i) < valid;                // wave-uniform
+      const uint8_t* base_i = instr_valid ? src + i * 1024 : src;          // scalar address arithmetic
+      if (CPI * i + b_lo >= valid) off = j_lo * 16u;
+      lds_dma16(base_i, off, my_base + i * 1024u);
+    }
+    wait_vmem();
+
+    float v[EPL];
+#pragma unroll
+    for (int k = 0; k < PIECES; ++k) {
+      const uint4 raw = *(const uint4*)(my + rd_base + ((k ^ l_sw) * 16u));
+      v[8 * k + 0] = bf16_lo(raw.x); v[8 * k + 1] = bf16_hi(raw.x);
+      v[8 * k + 2] = bf16_lo(raw.y); v[8 * k + 3] = bf16_hi(raw.y);
+      v[8 * k + 4] = bf16_lo(raw.z); v[8 * k + 5] = bf16_hi(raw.z);
+      v[8 * k + 6] = bf16_lo(raw.w); v[8 * k + 7] = bf16_hi(raw.w);
+    }
+    if (ROT == FPQ_ROT_HADAMARD) {
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) v[i] *= norm;
+#pragma unroll
+      for (int s = 1; s < (G < EPL ? G : EPL); s *= 2) {
+        __builtin_amdgcn_sched_barrier(0);  // keep the stages in place: EPL live values, no more
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+          if ((i & s) == 0) {
+            const float a = v[i], b = v[i + s];
+            v[i] = a + b;
+            v[i + s] = a - b;
+          }
+        }
+      }
+      if (G > EPL) {
+        // stride EPL: the two halves of a rotation block sit in lanes 2u and 2u + 1.  The even
+        // lane needs a + b, the odd one a - b = (value of the even lane) + (-own value).
+        __builtin_amdgcn_sched_barrier(0);
+        const uint32_t flip = (lane & 1u) << 31;
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+          const float other = __uint_as_float((uint32_t)__builtin_amdgcn_mov_dpp(
+              (int)__float_as_uint(v[i]), 0xB1 /* quad_perm [1,0,3,2] */, 0xF, 0xF, true));
+          v[i] = other + __uint_as_float(__float_as_uint(v[i]) ^ flip);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    uint32_t cw[CW];
+    uint32_t sbytes = 0u, sb_lo = 0u;
+    bool need_slow = false;
+#pragma unroll
+    for (int gi = 0; gi < NG; ++gi) {
+      float a = 0.0f;
+#pragma unroll
+      for (int i = 0; i < GROUP; ++i) a = __builtin_fmaxf(a, __builtin_fabsf(v[gi * GROUP + i]));
+      uint32_t byte;
+      bool fast;
+      float k1, k2, cvt_scale;
+      if (FMT == kFmtMx) {
+        const uint32_t bits = __float_as_uint(a);
+        byte = bits >> 23;
+        fast = (byte - 29u) <= 198u || bits == 0u;                       // -98 <= e <= 100, or all zero
+        k1 = 0.75f;
+        k2 = kKappa;
+        cvt_scale = __uint_as_float((bits & 0x7f800000u) - (2u << 23));  // 2^(e-2)
+        if (bits == 0u) {  // a zero group stores 2^-126 and zero codes
+          byte = 1u;
+          cvt_scale = 1.0f;
+        }
+      } else {
+        float t = div6_rn(a) * gs;
+        t = t > 448.0f ? 448.0f : t;
+        byte = e4m3_encode(t);
+        fast = nv_fast;
+        const float2 e = lut[byte & 0x7fu];
+        k1 = e.x;
+        k2 = e.y;
+        cvt_scale = 1.0f;
+      }
+      need_slow |= !fast;
+#pragma unroll
+      for (int d = 0; d < GROUP / 8; ++d) {
+        uint32_t w = 0u;
+#pragma unroll
+        for (int h = 0; h < 4; ++h) {
+          const float x0 = v[gi * GROUP + d * 8 + 2 * h], x1 = v[gi * GROUP + d * 8 + 2 * h + 1];
+          float q0 = __builtin_fmaf(x0, k1, x0 * k2);
+          float q1 = __builtin_fmaf(x1, k1, x1 * k2);
+          if (ZERO == kZeroSigned) {  // x / s keeps the sign of x, also for -0
+            q0 = __builtin_copysignf(q0, x0);
+            q1 = __builtin_copysignf(q1, x1);
+          }
+          if (h == 0) w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, q0, q1, cvt_scale, 0);
+          if (h == 1) w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, q0, q1, cvt_scale, 1);
+          if (h == 2) w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, q0, q1, cvt_scale, 2);
+          if (h == 3) w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, q0, q1, cvt_scale, 3);
+        }
+        if (FMT == kFmtNv && ZERO == kZeroSigned) w = byte == 0u ? 0u : w;  // zero scale: +0 codes
+        cw[gi * (GROUP / 8) + d] = fix_zero_nibbles<ZERO>(w);
+      }
+      sbytes |= (byte & 0xffu) << (8 * (gi & 3));
+      if (NG == 8 && gi == 3) {  // eight scale bytes per chunk: park the first four
+        sb_lo = sbytes;
+        sbytes = 0u;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // codes: lane-major runs -> LDS (16-byte pieces swizzled so 8 neighbouring lanes hit 8
+    // different bank groups) -> contiguous rows
+#pragma unroll
+    for (int k4 = 0; k4 < CQ; ++k4) {
+      const uint32_t sw = CQ == 4 ? ((lane >> 1) & 3u) : ((lane >> 2) & 1u);
+      *(uint4*)(my + (lane * CQ + (k4 ^ sw)) * 16u) =
+          make_uint4(cw[4 * k4], cw[4 * k4 + 1], cw[4 * k4 + 2], cw[4 * k4 + 3]);
+    }
+    uint8_t* dst = codes + (size_t)tile * (64u * CW * 4u);
+#pragma unroll
+    for (int i = 0; i < CQ; ++i) {
+      const uint32_t g = 64u * i + lane, l = g / CQ, k4 = g % CQ;
+      const uint32_t sw = CQ == 4 ? ((l >> 1) & 3u) : ((l >> 2) & 1u);
+      const uint4 o = *(const uint4*)(my + (l * CQ + (k4 ^ sw)) * 16u);
+      if (l < valid) *(uint4*)(dst + g * 16u) = o;
+    }
+
+    if (lane < valid) {
+      const uint32_t chunk = tile * 64u + lane;
+      constexpr uint32_t SB = NG;  // scale bytes per chunk: 2, 4 or 8
+      size_t so;
+      if (scale_stride == chunks_per_row * SB) {
+        so = (size_t)chunk * SB;
+      } else {
+        const uint32_t row = chunk / chunks_per_row;
+        so = (size_t)row * scale_stride + (chunk - row * chunks_per_row) * SB;
+      }
+      if ((scale_stride & (SB - 1u)) == 0u) {
+        if (SB == 2) *(uint16_t*)(scales + so) = (uint16_t)sbytes;
+        else if (SB == 4) *(uint32_t*)(scales + so) = sbytes;
+        else *(uint2*)(scales + so) = make_uint2(sb_lo, sbytes);
+      } else {
+#pragma unroll
+        for (uint32_t u = 0; u < SB; ++u) {
+          const uint32_t word = (SB == 8 && u < 4) ? sb_lo : sbytes;
+          scales[so + u] = (uint8_t)(word >> (8 * (u & 3)));
+        }
+      }
+    }
+
+    // Scale exponents outside the fast range (tiny, huge, or an out-of-range global scale): redo
+    // the whole tile with the generic per-element arithmetic, after the stores above have landed.
+    if (__builtin_amdgcn_ballot_w64(need_slow) != 0ull) {
+      wait_vmem();
+#pragma unroll 1
+      for (uint32_t it = 0; it < (uint32_t)PIECES; ++it) {
+        const uint32_t c8 = tile * (64u * PIECES) + it * 64u + lane;
+        lane8_process<G, FMT, ROT, ZERO>((const uint4*)x, (uint32_t*)codes, scales, c8,
+                                         c8 < n_chunks * PIECES, lane, chunks_per_row * PIECES,
+                                         scale_stride, norm, gs, rg);
+      }
+    }
+    asm volatile("" ::: "memory");
+  }
+  fill_scale_padding(scales, rows, chunks_per_row * NG, scale_rows, scale_stride);
+}
+
+template <int EPL, int G, int FMT, int ROT>
+static int launch_stream(const void* x, int64_t rows, int64_t cols, float norm, const float* gsp,
+                         void* codes, void* scales, int64_t scale_rows, int64_t scale_stride,
+                         int zero_policy, hipStream_t stream) {
+  const int64_t n_chunks = rows * cols / EPL;
+  const int64_t n_tiles = (n_chunks + 63) / 64;
+  int64_t blocks = (n_tiles + 3) / 4;
+  if (blocks > 1024) blocks = 1024;  // resident workgroups on 256 CUs; waves stride over the tiles
+  const dim3 grid((unsigned)blocks), block(256);
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint8_t*)x, (uint8_t*)codes,
+                       (uint8_t*)scales, (uint32_t)n_chunks, (uint32_t)(cols / EPL), (uint32_t)rows,
+                       (uint32_t)scale_rows, (uint32_t)scale_stride, norm, gsp);
+  };
+  if (zero_policy == FPQ_ZERO_REFERENCE) {
+    go(quantize_stream_kernel<EPL, G, FMT, ROT, kZeroReference>);
+  } else {
+    go(quantize_stream_kernel<EPL, G, FMT, ROT, kZeroSigned>);
   }
   return (int)hipGetLastError();
 }
@@ -146,9 +437,14 @@ static int dispatch(const void* x, int64_t rows, int64_t cols, int rot_kind, int
   if (((uintptr_t)x & 15u) || ((uintptr_t)codes & 3u)) return FPQ_E_ALIGN;
   (void)h;
 
+  // cols % 128 == 0 and 16-byte aligned codes: the streaming kernel; otherwise the generic one
+  const bool stream_ok = cols % FPQ_EPL == 0 && rows * cols >= (int64_t)1 << 21 &&
+                         !((uintptr_t)codes & 15u) && !((uintptr_t)scales & 7u);
 #define FPQ_LAUNCH(GG, RR)                                                                       \
-  return launch_lane8<GG, FMT, RR>(x, rows, cols, norm, gsp, codes, scales, scale_rows,         \
-                                   scale_stride, zero_policy, stream)
+  return stream_ok ? launch_stream<FPQ_EPL, GG, FMT, RR>(x, rows, cols, norm, gsp, codes, scales,\
+                                                  scale_rows, scale_stride, zero_policy, stream) \
+                   : launch_lane8<GG, FMT, RR>(x, rows, cols, norm, gsp, codes, scales,          \
+                                               scale_rows, scale_stride, zero_policy, stream)
   if (rot_kind == FPQ_ROT_IDENTITY) {
     FPQ_LAUNCH(GROUP, FPQ_ROT_IDENTITY);
   } else if (rot_kind == FPQ_ROT_HADAMARD) {

@@ -116,6 +116,57 @@ def test_adversarial_values():
             _check(x[8:], "nvfp4", "hadamard", 64, zero, gs=gs)
 
 
+def _adversarial_rows(cols):
+    gen = torch.Generator().manual_seed(19)
+    base = torch.randn(cols, generator=gen)
+    rows = [torch.zeros(cols), base * 1e-30, base * 1e-38, base * 1e30, base * 3e37, base,
+            torch.full((cols,), 2.0), -torch.full((cols,), 0.0)]
+    r = torch.zeros(cols); r[5] = 1.0; rows.append(r)
+    r = base.clone(); r[: cols // 2] = 0; rows.append(r)
+    r = torch.zeros(cols); r[::2] = 1.0; r[1::2] = -1.0; rows.append(r)
+    rows.append(torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0] * (cols // 8)))
+    rows.append(-torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0] * (cols // 8)) * 8)
+    return torch.stack(rows)
+
+
+@pytest.mark.parametrize("cols", [128, 192, 4096])
+def test_streaming_kernel_adversarial_and_ragged(cols):
+    """Inputs of >= 2^21 elements take the streaming kernel: adversarial rows (zero groups, tiny,
+    huge, ties, negative zeros) scattered through random data, a row count that leaves a partial
+    last tile, padded scale strides, every block size and both zero policies."""
+    adv = _adversarial_rows(cols)
+    n_rows = (1 << 21) // cols + 37
+    x = make_outlier_normal(n_rows, cols, seed=cols).float()
+    pos = torch.randperm(n_rows, generator=torch.Generator().manual_seed(3))[: adv.shape[0] * 3]
+    for i, p in enumerate(pos.tolist()):
+        x[p] = adv[i % adv.shape[0]]
+    x[-1] = adv[2]
+    x = x.to(torch.bfloat16)
+    gs_mx = [g for g in (32, 64, 128) if cols % g == 0]
+    for zero in (0, 1):
+        for g in gs_mx:
+            _check(x, "mxfp4", "hadamard", g, zero, pad=(g == 32))
+        _check(x, "mxfp4", "identity", 32, zero)
+        for g in [16] + gs_mx:
+            _check(x, "nvfp4", "hadamard", g, zero, gs=10.0, pad=(g == 16))
+        _check(x, "nvfp4", "identity", 16, zero, gs=3.0)
+    _check(x, "nvfp4", "hadamard", 16, 0, gs=1e-25)   # global scale outside the fast range
+    _check(x, "nvfp4", "hadamard", 16, 0, gs=1e-3)
+    _check(x, "nvfp4", "hadamard", 16, 0, gs=2688.0 / 7.0)
+
+
+def test_negative_zero_inputs_keep_their_sign_under_signed_policy():
+    x = torch.zeros(64, 128)
+    x[::2] = -0.0
+    x[3, 5] = 1.0
+    x[4, 7] = -1.0
+    x = x.to(torch.bfloat16)
+    for zero in (0, 1):
+        _check(x, "mxfp4", "identity", 32, zero)
+        _check(x, "nvfp4", "identity", 16, zero, gs=3.0)
+        _check(x, "mxfp4", "hadamard", 32, zero)
+
+
 def test_mx_tie_inputs_after_division():
     """Inputs whose scaled value lands exactly on, or one ulp beside, an E2M1 midpoint:
     x = t * fl(4/3) * 2^k is not bf16-representable in general, so use identity rotation on
