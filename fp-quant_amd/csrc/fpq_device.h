@@ -161,6 +161,11 @@ __device__ __forceinline__ void lds_dma16(const uint8_t* gbase, uint32_t voff, u
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
                :: "s"(lds_base), "v"(voff), "s"(gbase) : "memory");
 }
+// Same, marked non-temporal: for data that is read exactly once (streaming kernels).
+__device__ __forceinline__ void lds_dma16_nt(const uint8_t* gbase, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+               :: "s"(lds_base), "v"(voff), "s"(gbase) : "memory");
+}
 __device__ __forceinline__ void lds_dma4(const uint8_t* gbase, uint32_t voff, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2"
                :: "s"(lds_base), "v"(voff), "s"(gbase) : "memory");

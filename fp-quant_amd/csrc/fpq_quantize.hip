@@ -30,7 +30,8 @@ template <int G, int FMT, int ROT, int ZERO>
 __device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint32_t* __restrict__ codes,
                                               uint8_t* __restrict__ scales, uint32_t chunk, bool active,
                                               uint32_t lane, uint32_t chunks_per_row,
-                                              uint32_t scale_stride, float norm, float gscale, float rg) {
+                                              uint32_t scale_stride, float norm, float gscale, float rg,
+                                              float* __restrict__ stage, const uint16_t* __restrict__ hmat) {
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
   uint4 raw = make_uint4(0u, 0u, 0u, 0u);
   if (active) raw = x[chunk];
@@ -41,7 +42,7 @@ __device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint3
   p[4] = bf16_lo(raw.z); p[5] = bf16_hi(raw.z);
   p[6] = bf16_lo(raw.w); p[7] = bf16_hi(raw.w);
 
-  if (ROT == FPQ_ROT_HADAMARD) {
+  if (ROT == FPQ_ROT_HADAMARD || ROT == FPQ_ROT_GSR) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) p[i] = p[i] * norm;
 #pragma unroll
@@ -65,6 +66,39 @@ __device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint3
         p[i] = upper ? other - p[i] : p[i] + other;
       }
     }
+  }
+  if (ROT == FPQ_ROT_GSR) {
+    // sequency order: output k of a block is Hadamard output bitreverse(k ^ (k >> 1))
+    // (inference_lib/src/fp_quant/module/linear.py:37-41); gathered through the wave's LDS stage
+    constexpr int LOG2G = G == 16 ? 4 : G == 32 ? 5 : G == 64 ? 6 : 7;
+    const uint32_t first = lane & ~(uint32_t)(G / 8 - 1);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) stage[lane * 8u + i] = p[i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t k = (lane - first) * 8u + i;
+      const uint32_t j = __brev(k ^ (k >> 1)) >> (32 - LOG2G);
+      p[i] = stage[first * 8u + j];
+    }
+  }
+  if (ROT == FPQ_ROT_GENERAL) {
+    // arbitrary matrix: y[j] = sum_i x[i] * H[i][j], fp32 fused multiply-adds in the order i = 0..G-1
+    const uint32_t first = lane & ~(uint32_t)(G / 8 - 1);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) stage[lane * 8u + i] = p[i];
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const uint16_t* hcol = hmat + (lane - first) * 8u;
+#pragma unroll 4
+    for (int ii = 0; ii < G; ++ii) {
+      const float xi = stage[first * 8u + ii];
+      const uint4 hv = *(const uint4*)(hcol + ii * G);
+      acc[0] = __builtin_fmaf(xi, bf16_lo(hv.x), acc[0]); acc[1] = __builtin_fmaf(xi, bf16_hi(hv.x), acc[1]);
+      acc[2] = __builtin_fmaf(xi, bf16_lo(hv.y), acc[2]); acc[3] = __builtin_fmaf(xi, bf16_hi(hv.y), acc[3]);
+      acc[4] = __builtin_fmaf(xi, bf16_lo(hv.z), acc[4]); acc[5] = __builtin_fmaf(xi, bf16_hi(hv.z), acc[5]);
+      acc[6] = __builtin_fmaf(xi, bf16_lo(hv.w), acc[6]); acc[7] = __builtin_fmaf(xi, bf16_hi(hv.w), acc[7]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) p[i] = acc[i];
   }
 
   float a = 0.0f;
@@ -118,8 +152,16 @@ template <int G, int FMT, int ROT, int ZERO>
 __global__ __launch_bounds__(256) void quantize_lane8_kernel(
     const uint4* __restrict__ x, uint32_t* __restrict__ codes, uint8_t* __restrict__ scales,
     uint32_t n_chunks, uint32_t chunks_per_row, uint32_t rows, uint32_t scale_rows,
-    uint32_t scale_stride, float norm, const float* __restrict__ global_scale) {
+    uint32_t scale_stride, float norm, const float* __restrict__ global_scale,
+    const uint16_t* __restrict__ h) {
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
+  constexpr bool kStage = ROT == FPQ_ROT_GSR || ROT == FPQ_ROT_GENERAL;
+  __shared__ float stage[kStage ? 4 : 1][kStage ? 512 : 1];
+  __shared__ __attribute__((aligned(16))) uint16_t hmat[ROT == FPQ_ROT_GENERAL ? G * G : 8];
+  if (ROT == FPQ_ROT_GENERAL) {
+    for (int i = threadIdx.x; i < G * G; i += 256) hmat[i] = h[i];
+    __syncthreads();
+  }
   const uint32_t chunk = blockIdx.x * 256u + threadIdx.x;
   float g = 1.0f, rg = 1.0f;
   if (FMT == kFmtNv) {
@@ -127,20 +169,21 @@ __global__ __launch_bounds__(256) void quantize_lane8_kernel(
     rg = g == 0.0f ? 0.0f : 1.0f / g;
   }
   lane8_process<G, FMT, ROT, ZERO>(x, codes, scales, chunk, chunk < n_chunks, threadIdx.x & 63u,
-                                   chunks_per_row, scale_stride, norm, g, rg);
+                                   chunks_per_row, scale_stride, norm, g, rg,
+                                   stage[kStage ? (threadIdx.x >> 6) : 0], hmat);
   fill_scale_padding(scales, rows, chunks_per_row / (GROUP / 8), scale_rows, scale_stride);
 }
 
 template <int G, int FMT, int ROT>
 static int launch_lane8(const void* x, int64_t rows, int64_t cols, float norm, const float* gsp,
                         void* codes, void* scales, int64_t scale_rows, int64_t scale_stride,
-                        int zero_policy, hipStream_t stream) {
+                        int zero_policy, hipStream_t stream, const void* h = nullptr) {
   const int64_t n_chunks = rows * cols / 8;
   const dim3 grid((unsigned)((n_chunks + 255) / 256)), block(256);
   auto args = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint4*)x, (uint32_t*)codes,
                        (uint8_t*)scales, (uint32_t)n_chunks, (uint32_t)(cols / 8), (uint32_t)rows,
-                       (uint32_t)scale_rows, (uint32_t)scale_stride, norm, gsp);
+                       (uint32_t)scale_rows, (uint32_t)scale_stride, norm, gsp, (const uint16_t*)h);
   };
   if (zero_policy == FPQ_ZERO_REFERENCE) {
     args(quantize_lane8_kernel<G, FMT, ROT, kZeroReference>);
@@ -161,6 +204,16 @@ static int launch_lane8(const void* x, int64_t rows, int64_t cols, float norm, c
 // those reads are bank-conflict free.  Codes return through the same LDS region so that global
 // stores are contiguous.
 constexpr float kKappa = -0x1.8p-26f;  // fma(x, 0.75, x * kKappa) rounds to the E2M1 code of x / fl(4/3)
+
+// Hadamard output index that sequency-ordered output k of a g-block takes: bitreverse(k ^ (k >> 1))
+__host__ __device__ constexpr int gsr_source(int k, int g) {
+  int gray = k ^ (k >> 1), r = 0;
+  for (int b = 1; b < g; b <<= 1) {
+    r = (r << 1) | (gray & 1);
+    gray >>= 1;
+  }
+  return r;
+}
 
 template <int ZERO>
 __device__ __forceinline__ uint32_t fix_zero_nibbles(uint32_t w) {
@@ -235,7 +288,7 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
       const bool instr_valid = (uint32_t)(CPI * i) < valid;                // wave-uniform
       const uint8_t* base_i = instr_valid ? src + i * 1024 : src;          // scalar address arithmetic
       if (CPI * i + b_lo >= valid) off = j_lo * 16u;
-      lds_dma16(base_i, off, my_base + i * 1024u);
+      lds_dma16_nt(base_i, off, my_base + i * 1024u);  // read once: keep it out of the caches
     }
     wait_vmem();
 
@@ -248,7 +301,7 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
       v[8 * k + 4] = bf16_lo(raw.z); v[8 * k + 5] = bf16_hi(raw.z);
       v[8 * k + 6] = bf16_lo(raw.w); v[8 * k + 7] = bf16_hi(raw.w);
     }
-    if (ROT == FPQ_ROT_HADAMARD) {
+    if (ROT == FPQ_ROT_HADAMARD || ROT == FPQ_ROT_GSR) {
 #pragma unroll
       for (int i = 0; i < EPL; ++i) v[i] *= norm;
 #pragma unroll
@@ -276,6 +329,15 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
         }
       }
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if (ROT == FPQ_ROT_GSR) {
+      // sequency order inside every G-block (G <= EPL here): a compile-time renaming of registers
+      static_assert(ROT != FPQ_ROT_GSR || G <= EPL, "GSR blocks must fit in one lane");
+      float w[EPL];
+#pragma unroll
+      for (int k = 0; k < EPL; ++k) w[k] = v[(k & ~(G - 1)) | gsr_source(k & (G - 1), G)];
+#pragma unroll
+      for (int k = 0; k < EPL; ++k) v[k] = w[k];
     }
 
     uint32_t cw[CW];
@@ -388,7 +450,7 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
         const uint32_t c8 = tile * (64u * PIECES) + it * 64u + lane;
         lane8_process<G, FMT, ROT, ZERO>((const uint4*)x, (uint32_t*)codes, scales, c8,
                                          c8 < n_chunks * PIECES, lane, chunks_per_row * PIECES,
-                                         scale_stride, norm, gs, rg);
+                                         scale_stride, norm, gs, rg, (float*)my, nullptr);
       }
     }
     asm volatile("" ::: "memory");
@@ -435,9 +497,8 @@ static int dispatch(const void* x, int64_t rows, int64_t cols, int rot_kind, int
   if (scale_rows < rows || scale_stride < cols / GROUP) return FPQ_E_SHAPE;
   if (rows * cols >= (int64_t)1 << 34 || scale_rows * scale_stride >= (int64_t)1 << 32) return FPQ_E_SHAPE;
   if (((uintptr_t)x & 15u) || ((uintptr_t)codes & 3u)) return FPQ_E_ALIGN;
-  (void)h;
 
-  // cols % 128 == 0 and 16-byte aligned codes: the streaming kernel; otherwise the generic one
+  // big inputs with cols % FPQ_EPL == 0 and aligned outputs: the streaming kernel; else the generic one
   const bool stream_ok = cols % FPQ_EPL == 0 && rows * cols >= (int64_t)1 << 21 &&
                          !((uintptr_t)codes & 15u) && !((uintptr_t)scales & 7u);
 #define FPQ_LAUNCH(GG, RR)                                                                       \
@@ -445,6 +506,9 @@ static int dispatch(const void* x, int64_t rows, int64_t cols, int rot_kind, int
                                                   scale_rows, scale_stride, zero_policy, stream) \
                    : launch_lane8<GG, FMT, RR>(x, rows, cols, norm, gsp, codes, scales,          \
                                                scale_rows, scale_stride, zero_policy, stream)
+#define FPQ_LAUNCH_GENERIC(GG, RR)                                                               \
+  return launch_lane8<GG, FMT, RR>(x, rows, cols, norm, gsp, codes, scales, scale_rows,         \
+                                   scale_stride, zero_policy, stream, h)
   if (rot_kind == FPQ_ROT_IDENTITY) {
     FPQ_LAUNCH(GROUP, FPQ_ROT_IDENTITY);
   } else if (rot_kind == FPQ_ROT_HADAMARD) {
@@ -454,9 +518,24 @@ static int dispatch(const void* x, int64_t rows, int64_t cols, int rot_kind, int
       case 64: FPQ_LAUNCH(64, FPQ_ROT_HADAMARD);
       case 128: FPQ_LAUNCH(128, FPQ_ROT_HADAMARD);
     }
-  } else if (rot_kind == FPQ_ROT_GSR || rot_kind == FPQ_ROT_GENERAL) {
-    return FPQ_E_UNSUPPORTED;
+  } else if (rot_kind == FPQ_ROT_GSR) {
+    switch (g) {
+      case 16: FPQ_LAUNCH(16, FPQ_ROT_GSR);
+      case 32: FPQ_LAUNCH(32, FPQ_ROT_GSR);
+      case 64: FPQ_LAUNCH(64, FPQ_ROT_GSR);
+      case 128: FPQ_LAUNCH_GENERIC(128, FPQ_ROT_GSR);  // a block spans two lanes of the streaming kernel
+    }
+  } else if (rot_kind == FPQ_ROT_GENERAL) {
+    if (!h) return FPQ_E_NULL;
+    if ((uintptr_t)h & 1u) return FPQ_E_ALIGN;
+    switch (g) {
+      case 16: FPQ_LAUNCH_GENERIC(16, FPQ_ROT_GENERAL);
+      case 32: FPQ_LAUNCH_GENERIC(32, FPQ_ROT_GENERAL);
+      case 64: FPQ_LAUNCH_GENERIC(64, FPQ_ROT_GENERAL);
+      case 128: FPQ_LAUNCH_GENERIC(128, FPQ_ROT_GENERAL);
+    }
   }
+#undef FPQ_LAUNCH_GENERIC
 #undef FPQ_LAUNCH
   return FPQ_E_ROTATION;
 }

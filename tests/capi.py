@@ -26,7 +26,8 @@ def quantize(x_bf16, fmt, rot="hadamard", g=128, norm=None, h=None, global_scale
     scales = torch.full((srow, scol), fill, dtype=torch.uint8, device="cuda")
     if norm is None:
         norm = float(torch.tensor(g ** -0.5, dtype=torch.bfloat16))
-    hp = h.to("cuda").contiguous().data_ptr() if h is not None else None
+    h_dev = h.to(device="cuda", dtype=torch.bfloat16).contiguous() if h is not None else None  # keep alive
+    hp = h_dev.data_ptr() if h_dev is not None else None
     stream = torch.cuda.current_stream().cuda_stream
     if fmt == "mxfp4":
         st = lib.fpq_quantize_mx(x.data_ptr(), rows, cols, ROT[rot], g, norm, hp, codes.data_ptr(),

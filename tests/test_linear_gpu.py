@@ -65,6 +65,41 @@ def test_linear_matches_oracle_pipeline(fmt, g, bias):
     assert rel < 0.25, rel
 
 
+@pytest.mark.parametrize("init", ["identity", "gsr"])
+def test_other_transform_inits(init):
+    """transform_init identity / gsr go through the same operators (matrix recognised on the host)."""
+    import fp_quant
+    from fp_quant.module import hip_ops
+    from fp_quant import _engine
+    gen = torch.Generator().manual_seed(5)
+    w = (torch.randn(64, 256, generator=gen) * 0.02).to(torch.bfloat16)
+    x = torch.randn(8, 256, generator=gen).to(torch.bfloat16)
+    lin = fp_quant.FPQuantLinear(256, 64, _cfg("mxfp4", 64, transform_init=init), bias=False, device="cuda",
+                                 dtype=torch.bfloat16)
+    lin.weight.data = w.cuda()
+    lin.pre_forward()
+    kind = {"identity": _engine.ROT_IDENTITY, "gsr": _engine.ROT_GSR}[init]
+    assert hip_ops.classify_rotation(lin.forward_hadamard_matrix)[0] == kind
+    okind = {"identity": O.ROT_IDENTITY, "gsr": O.ROT_GSR}[init]
+    wq, ws, _ = O.quantize_mx(w, okind, 64)
+    assert torch.equal(lin.qweight.cpu(), wq) and torch.equal(lin.scales.cpu(), ws)
+    xq, xs, _ = O.quantize_mx(x, okind, 64)
+    ref, mag = O.gemm_ref(xq, xs, wq, ws, 0.111328125, "mxfp4")
+    y = lin(x.cuda()).cpu()
+    assert ((y.double() - ref).abs() <= 2.0 ** -8 * ref.abs() + 1e-5 * mag).all()
+
+
+def test_general_matrix_through_the_operator():
+    from fp_quant.module import hip_ops
+    gen = torch.Generator().manual_seed(6)
+    q, _ = torch.linalg.qr(torch.randn(32, 32, generator=gen))
+    h = q.to(torch.bfloat16)
+    x = torch.randn(16, 128, generator=gen).to(torch.bfloat16)
+    codes, scales, _ = hip_ops.fused_quantize_mx_op(x.cuda(), h.cuda(), "abs_max", False)
+    wc, wsc, _ = O.quantize_mx(x, O.ROT_GENERAL, 32, h=h)
+    assert torch.equal(codes.cpu(), wc) and torch.equal(scales.view(torch.uint8).cpu()[:16, :4], wsc)
+
+
 def test_replace_quantize_and_skip_rule():
     import fp_quant
 

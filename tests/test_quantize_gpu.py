@@ -10,14 +10,15 @@ from oracle import fpq_oracle as O
 pytestmark = pytest.mark.gpu
 
 
-def _check(x, fmt, rot="hadamard", g=128, zero=0, pad=False, gs=None):
+def _check(x, fmt, rot="hadamard", g=128, zero=0, pad=False, gs=None, h=None):
     import capi
-    kind = {"hadamard": O.ROT_HADAMARD, "identity": O.ROT_IDENTITY, "gsr": O.ROT_GSR}[rot]
+    kind = {"hadamard": O.ROT_HADAMARD, "identity": O.ROT_IDENTITY, "gsr": O.ROT_GSR,
+            "general": O.ROT_GENERAL}[rot]
     if fmt == "mxfp4":
-        want_c, want_s, _ = O.quantize_mx(x, kind, g, zero_nibble=zero)
+        want_c, want_s, _ = O.quantize_mx(x, kind, g, h=h, zero_nibble=zero)
     else:
-        want_c, want_s, _ = O.quantize_nv(x, gs, kind, g, zero_nibble=zero)
-    got_c, got_s = capi.quantize(x, fmt, rot, g, global_scale=gs, zero_policy=zero, pad=pad)
+        want_c, want_s, _ = O.quantize_nv(x, gs, kind, g, h=h, zero_nibble=zero)
+    got_c, got_s = capi.quantize(x, fmt, rot, g, global_scale=gs, zero_policy=zero, pad=pad, h=h)
     r, c = want_s.shape
     bad_c = (got_c != want_c).sum().item()
     bad_s = (got_s[:r, :c] != want_s).sum().item()
@@ -79,6 +80,29 @@ def test_ragged_shapes_and_padding(rows, cols):
     _check(x, "mxfp4", "hadamard", g, pad=True)
     _check(x, "mxfp4", "hadamard", 32, pad=False)
     _check(x, "nvfp4", "hadamard", 16, pad=True, gs=10.0)
+
+
+@pytest.mark.parametrize("g", [16, 32, 64, 128])
+def test_gsr_rotation(g):
+    """Sequency-ordered Hadamard (transform_init="gsr"): small input (generic kernel) and an input
+    large enough for the streaming kernel."""
+    for rows in (40, (1 << 21) // 256 + 5):
+        x = make_outlier_normal(rows, 256, seed=300 + g)
+        if g >= 32:
+            _check(x, "mxfp4", "gsr", g, zero=0)
+        _check(x, "nvfp4", "gsr", g, zero=1, gs=3.0)
+
+
+@pytest.mark.parametrize("g", [16, 32, 64, 128])
+def test_general_rotation_matrix(g):
+    """An arbitrary (non-symmetric) bf16 matrix: sequential fp32 fma accumulation, bit-exact."""
+    gen = torch.Generator().manual_seed(400 + g)
+    q, _ = torch.linalg.qr(torch.randn(g, g, generator=gen))
+    h = q.to(torch.bfloat16)
+    x = make_outlier_normal(48, 256, seed=500 + g)
+    if g >= 32:
+        _check(x, "mxfp4", "general", g, h=h)
+    _check(x, "nvfp4", "general", g, gs=3.0, h=h, zero=1)
 
 
 def test_empty_input():
