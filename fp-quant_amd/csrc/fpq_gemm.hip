@@ -24,6 +24,11 @@ namespace fpq {
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+#ifndef FPQ_SPLITK_MAX_M
+#define FPQ_SPLITK_MAX_M 64  // largest M served by the weight-streaming split-K kernel
+#endif
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
@@ -145,6 +150,121 @@ __global__ __launch_bounds__(256) void gemm_mxf4_direct_kernel(
                                                                      sa[i], 0, sb[j]);
   }
   store_tile<TN, TM>(acc, y, bias, *alpha_p, n0, m0, M, N, r, kb);
+}
+
+// -------------------------------------------------------------------------------------------
+// Weight-streaming kernel for small M (the reference's disabled small-M entry, linear_fns.py:55).
+// The time is the 31 MB weight read, so the job is to keep many loads in flight: a workgroup owns
+// 16 weight rows, its four waves each take a quarter of K and issue all of their loads before the
+// first MFMA; the four partial 16 x (16 TM) tiles are then summed through LDS by wave 0.
+template <int TN, int TM>
+__global__ __launch_bounds__(256) void gemm_mxf4_splitk_kernel(
+    const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, int xs_stride,
+    const uint8_t* __restrict__ wq, const uint8_t* __restrict__ ws, int ws_stride,
+    const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
+    int M, int N, int K) {
+  __shared__ v4f part[3][TN][TM][64];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int r = lane & 15, kb = lane >> 4;
+  const int n0 = blockIdx.x * TN * 16, m0 = blockIdx.y * TM * 16;
+  const int kbytes = K >> 1;
+  const int kq = K >> 2;                       // K range of this wave: [wave * kq, wave * kq + kq)
+  const int steps = kq >> 7;                   // 128 per MFMA
+
+  const uint8_t* wp[TN];
+  const uint8_t* wsp[TN];
+#pragma unroll
+  for (int i = 0; i < TN; ++i) {
+    const int n = min(n0 + i * 16 + r, N - 1);
+    wp[i] = wq + (size_t)n * kbytes + ((wave * kq) >> 1) + kb * 16;
+    wsp[i] = ws + (size_t)n * ws_stride + ((wave * kq) >> 5);
+  }
+  const uint8_t* xp[TM];
+  const uint8_t* xsp[TM];
+#pragma unroll
+  for (int j = 0; j < TM; ++j) {
+    const int m = min(m0 + j * 16 + r, M - 1);
+    xp[j] = xq + (size_t)m * kbytes + ((wave * kq) >> 1) + kb * 16;
+    xsp[j] = xs + (size_t)m * xs_stride + ((wave * kq) >> 5);
+  }
+  v4f acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  // Loads are issued in batches of 4 * Q K steps: per row tile and group of 4 steps four 16-byte
+  // code loads and ONE 16-byte scale load (the row's 16 scale bytes of those steps; byte 4 u + kb
+  // is this lane's scale in step u), all before the first MFMA of the batch.
+  constexpr int Q = (TN + TM <= 4) ? 2 : 1;
+  for (int s0 = 0; s0 < steps; s0 += 4 * Q) {
+    uint4 a[Q][4][TN], b[Q][4][TM], sa4[Q][TN], sb4[Q][TM];
+#pragma unroll
+    for (int h = 0; h < Q; ++h) {
+      const bool on = s0 + 4 * h < steps;  // steps is a multiple of 4
+#pragma unroll
+      for (int i = 0; i < TN; ++i) {
+        sa4[h][i] = make_uint4(0x7f7f7f7fu, 0x7f7f7f7fu, 0x7f7f7f7fu, 0x7f7f7f7fu);
+        if (on) sa4[h][i] = *(const uint4*)(wsp[i] + (s0 + 4 * h) * 4);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          a[h][u][i] = make_uint4(0u, 0u, 0u, 0u);
+          if (on) {
+            const v4u ld = __builtin_nontemporal_load((const v4u*)(wp[i] + (s0 + 4 * h + u) * 64));
+            a[h][u][i] = make_uint4(ld.x, ld.y, ld.z, ld.w);
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < TM; ++j) {
+        sb4[h][j] = make_uint4(0x7f7f7f7fu, 0x7f7f7f7fu, 0x7f7f7f7fu, 0x7f7f7f7fu);
+        if (on) sb4[h][j] = *(const uint4*)(xsp[j] + (s0 + 4 * h) * 4);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          b[h][u][j] = make_uint4(0u, 0u, 0u, 0u);
+          if (on) b[h][u][j] = *(const uint4*)(xp[j] + (s0 + 4 * h + u) * 64);
+        }
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < Q; ++h) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+          const uint4 s4 = sb4[h][j];
+          const uint32_t sbw = u == 0 ? s4.x : u == 1 ? s4.y : u == 2 ? s4.z : s4.w;
+          const int sb = (int)((sbw >> (8 * kb)) & 0xffu);
+          const uint4 bq = b[h][u][j];
+          const v8i bv = v8i{(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w, 0, 0, 0, 0};
+#pragma unroll
+          for (int i = 0; i < TN; ++i) {
+            const uint4 t4 = sa4[h][i];
+            const uint32_t saw = u == 0 ? t4.x : u == 1 ? t4.y : u == 2 ? t4.z : t4.w;
+            const int sa = (int)((saw >> (8 * kb)) & 0xffu);
+            const uint4 aq = a[h][u][i];
+            const v8i av = v8i{(int)aq.x, (int)aq.y, (int)aq.z, (int)aq.w, 0, 0, 0, 0};
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[i][j], 4, 4, 0, sa, 0, sb);
+          }
+        }
+      }
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < TM; ++j) part[wave - 1][i][j][lane] = acc[i][j];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < TM; ++j)
+        acc[i][j] = ((acc[i][j] + part[0][i][j][lane]) + part[1][i][j][lane]) + part[2][i][j][lane];
+    store_tile<TN, TM>(acc, y, bias, *alpha_p, n0, m0, M, N, r, kb);
+  }
 }
 
 // -------------------------------------------------------------------------------------------
@@ -533,8 +653,8 @@ static int gemm_dispatch(const void* xq, const void* xs, int64_t xs_stride, cons
       !((uintptr_t)xs & 3u) && !((uintptr_t)ws & 3u) && N * (K / 2) < ((int64_t)1 << 32) &&
       M * (K / 2) < ((int64_t)1 << 32)) {
     constexpr int BN = 256, BM = 256;
-    using L = MxLdsLayout<BN, BM>;
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
+    using L = MxLdsLayout<BN, BM>;
     static bool attr_set = false;
     if (!attr_set) {
       hipError_t e = hipFuncSetAttribute((const void*)gemm_mxf4_lds_kernel<BN, BM>,
@@ -548,6 +668,28 @@ static int gemm_dispatch(const void* xq, const void* xs, int64_t xs_stride, cons
                        (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K, tiles_m);
     return (int)hipGetLastError();
   }
+#define FPQ_SPLITK(TNN, TMM)                                                                       \
+  do {                                                                                             \
+    const dim3 grid((unsigned)((N + TNN * 16 - 1) / (TNN * 16)),                                   \
+                    (unsigned)((M + TMM * 16 - 1) / (TMM * 16)));                                  \
+    hipLaunchKernelGGL((gemm_mxf4_splitk_kernel<TNN, TMM>), grid, dim3(256), 0, stream,            \
+                       (const uint8_t*)xq, (const uint8_t*)xs, (int)xs_stride, (const uint8_t*)wq, \
+                       (const uint8_t*)ws, (int)ws_stride, alpha, (const uint16_t*)bias,           \
+                       (uint16_t*)y, (int)M, (int)N, (int)K);                                      \
+    return (int)hipGetLastError();                                                                 \
+  } while (0)
+  // K % 2048 == 0: every wave's K quarter is a whole number of 4-step batches and every 16-byte
+  // scale load is aligned (scale strides and bases must be 16-byte multiples too)
+  if (FMT == 0 && K % 2048 == 0 && M <= FPQ_SPLITK_MAX_M && xs_stride % 16 == 0 && ws_stride % 16 == 0 &&
+      !((uintptr_t)xs & 15u) && !((uintptr_t)ws & 15u)) {
+    // 32 weight rows per workgroup once there is more than one activation row: halves the
+    // re-reading of the activations from L2 (measured best among 16 / 32 / 64 rows)
+    if (M == 1) FPQ_SPLITK(1, 1);
+    if (M <= 16) FPQ_SPLITK(2, 1);
+    if (M <= 32) FPQ_SPLITK(2, 2);
+    FPQ_SPLITK(2, 4);
+  }
+#undef FPQ_SPLITK
   if (M <= 16) {
     FPQ_GEMM(1, 1, 4, 1);
   } else if (M <= 32) {

@@ -6,7 +6,7 @@ reference's QuTLASS wrappers (inference_lib/src/fp_quant/module/qutlass_ops.py:3
 the boundary: scales are consumed row-major by the GEMMs (no per-call re-tiling), and the
 rotation matrix is recognised once (Hadamard / identity / GSR) and applied as butterflies.
 """
-from typing import Dict, Optional, Tuple
+from typing import Optional, Tuple
 
 import torch
 
@@ -18,9 +18,6 @@ HAS_HIP_ENGINE = _engine.available()
 # zero-nibble policy used by the operators (see include/fpq.h)
 ZERO_NIBBLE_POLICY = _engine.ZERO_REFERENCE
 
-_rotation_cache: Dict[Tuple, Tuple[int, float]] = {}
-
-
 def _sylvester(g: int) -> torch.Tensor:
     idx = torch.arange(g)
     anded = idx[:, None] & idx[None, :]
@@ -31,12 +28,12 @@ def _sylvester(g: int) -> torch.Tensor:
 
 
 def classify_rotation(h: torch.Tensor) -> Tuple[int, float]:
-    """(rotation kind, norm) of a [g, g] matrix; cached per storage/version so the one
-    device->host copy it needs happens once per matrix, not per call."""
-    key = (h.data_ptr(), h._version, tuple(h.shape), h.dtype, str(h.device))
-    hit = _rotation_cache.get(key)
-    if hit is not None:
-        return hit
+    """(rotation kind, norm) of a [g, g] matrix.  The result is remembered on the tensor object
+    itself (with its version counter), so the one device->host copy it needs happens once per
+    matrix and can never be confused with another tensor that later reuses the same memory."""
+    hit = getattr(h, "_fpq_rotation", None)
+    if hit is not None and hit[0] == h._version:
+        return hit[1], hit[2]
     g = h.shape[0]
     if h.dim() != 2 or h.shape[1] != g:
         raise ValueError(f"rotation matrix must be square, got {tuple(h.shape)}")
@@ -53,10 +50,27 @@ def classify_rotation(h: torch.Tensor) -> Tuple[int, float]:
             changes = torch.diff(signed, dim=0).ne(0).sum(dim=0)
             if torch.equal(hf, signed[:, torch.argsort(changes)]):
                 kind, norm = _engine.ROT_GSR, n
-    if len(_rotation_cache) > 4096:
-        _rotation_cache.clear()
-    _rotation_cache[key] = (kind, norm)
+    try:
+        h._fpq_rotation = (h._version, kind, norm)
+    except AttributeError:  # objects that refuse attributes: classify again next time
+        pass
     return kind, norm
+
+
+def as_bf16(h: torch.Tensor) -> torch.Tensor:
+    """`h` in bfloat16, contiguous; the converted copy is kept on the source tensor so that a
+    non-bf16 rotation buffer is converted (and later classified) once, not on every call."""
+    if h.dtype == torch.bfloat16 and h.is_contiguous():
+        return h
+    hit = getattr(h, "_fpq_bf16", None)
+    if hit is not None and hit[0] == h._version:
+        return hit[1]
+    conv = h.detach().to(torch.bfloat16).contiguous()
+    try:
+        h._fpq_bf16 = (h._version, conv)
+    except AttributeError:
+        pass
+    return conv
 
 
 def _stream(t: torch.Tensor) -> int:

@@ -11,6 +11,7 @@ from torch.autograd import Function
 
 from ..utils import FPQuantDtype
 from .hip_ops import (
+    as_bf16,
     fused_quantize_mx_op,
     fused_quantize_nv_op,
     matmul_mxf4_bf16_tn_bias_op,
@@ -30,13 +31,9 @@ def forward_quantize(
     """(packed codes, scales, clip mask or None) of x rotated by `hadamard_matrix`."""
     if dtype == FPQuantDtype.MXFP4:
         want_mask = forward_method == "quest" and x.requires_grad
-        return fused_quantize_mx_op(
-            x.to(torch.bfloat16), hadamard_matrix.to(torch.bfloat16), forward_method, want_mask
-        )
+        return fused_quantize_mx_op(x.to(torch.bfloat16), as_bf16(hadamard_matrix), forward_method, want_mask)
     if dtype == FPQuantDtype.NVFP4:
-        codes, scales = fused_quantize_nv_op(
-            x.to(torch.bfloat16), hadamard_matrix.to(torch.bfloat16), global_scale.float()
-        )
+        codes, scales = fused_quantize_nv_op(x.to(torch.bfloat16), as_bf16(hadamard_matrix), global_scale.float())
         return codes, scales, None
     raise ValueError(f"Unsupported forward dtype: {dtype}")
 
