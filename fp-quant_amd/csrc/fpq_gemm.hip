@@ -280,6 +280,79 @@ constexpr int kScaleBytes = kKS / 32;       // 8 scale bytes per row per stage
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void global_void;
 
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+}
+
+// Epilogue of the LDS-tiled kernels.  Accumulator register v of 32x32 tile (i, j) is y[m][n] with
+// m = j*32 + r32 and n = i*32 + 8*(v/4) + 4*kh + v%4 inside the wave's quadrant of the workgroup
+// tile.  The quadrant goes through this wave's share of the (now idle) LDS as bf16 [m][n] so that
+// global stores are 256 contiguous bytes per row.
+template <int BN, int BM, int LDS_BYTES>
+__device__ __forceinline__ void wave_quadrant_store(const v16f (&acc)[BN / 64][BM / 64], uint8_t* smem,
+                                                    uint16_t* __restrict__ y,
+                                                    const uint16_t* __restrict__ bias,
+                                                    const float* __restrict__ alpha_p, int n_blk, int m_blk,
+                                                    int wn, int wm, int wave, int lane, int M, int N) {
+  constexpr int TN = BN / 64, TM = BM / 64;
+  const int r32 = lane & 31, kh = lane >> 5;
+  const float alpha = *alpha_p;
+#ifdef FPQ_EXP_NO_STORE
+  if (alpha != 12345.0f) return;
+#endif
+  constexpr int WT_N = BN / 2, WT_M = BM / 2;        // wave quadrant
+  constexpr int kStride = WT_N * 2 + 16;             // bytes per staged row (+16: spread banks)
+  static_assert(4 * WT_M * kStride <= LDS_BYTES, "epilogue staging does not fit in LDS");
+  __syncthreads();                                   // every wave is done reading operands
+  uint8_t* stg = smem + wave * (WT_M * kStride);
+  const int n0 = n_blk + wn * WT_N, m0 = m_blk + wm * WT_M;
+#pragma unroll
+  for (int i = 0; i < TN; ++i) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int nl = i * 32 + 8 * g + 4 * kh;
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (bias) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (n0 + nl + u < N) bv[u] = __uint_as_float((uint32_t)bias[n0 + nl + u] << 16);
+      }
+#pragma unroll
+      for (int j = 0; j < TM; ++j) {
+        uint32_t lo = pack_bf16x2(acc[i][j][4 * g + 0] * alpha, acc[i][j][4 * g + 1] * alpha);
+        uint32_t hi = pack_bf16x2(acc[i][j][4 * g + 2] * alpha, acc[i][j][4 * g + 3] * alpha);
+        if (bias) {
+          lo = pack_bf16x2(__uint_as_float(lo << 16) + bv[0], __uint_as_float(lo & 0xffff0000u) + bv[1]);
+          hi = pack_bf16x2(__uint_as_float(hi << 16) + bv[2], __uint_as_float(hi & 0xffff0000u) + bv[3]);
+        }
+        *(uint2*)(stg + (j * 32 + r32) * kStride + nl * 2) = make_uint2(lo, hi);
+      }
+    }
+  }
+  // read back: 16 lanes x 16 B cover one 256-byte row, 4 rows per wave instruction
+  const int rr = lane >> 4, cc = lane & 15;
+  const bool vec_ok = (N & 7) == 0;
+#pragma unroll 4
+  for (int p = 0; p < WT_M / 4; ++p) {
+    const int ml = p * 4 + rr;
+    const uint4 v = *(const uint4*)(stg + ml * kStride + cc * 16);
+    const int m = m0 + ml, n = n0 + cc * 8;
+    if (m >= M || n >= N) continue;
+    uint16_t* dst = y + (size_t)m * N + n;
+    if (vec_ok && n + 7 < N) {
+      *(uint4*)dst = v;
+    } else {
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (n + u < N) dst[u] = (uint16_t)(w[u >> 1] >> (16 * (u & 1)));
+    }
+  }
+}
+
 template <int BN, int BM>
 struct MxLdsLayout {
   static constexpr int kCodesW = 0;
@@ -288,13 +361,6 @@ struct MxLdsLayout {
   static constexpr int kScalesX = kScalesW + BN * kScaleBytes;
   static constexpr int kStage = kScalesX + BM * kScaleBytes;
 };
-
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
-}
 
 template <int BN, int BM>
 __global__ __launch_bounds__(256) void gemm_mxf4_lds_kernel(
@@ -453,62 +519,7 @@ __global__ __launch_bounds__(256) void gemm_mxf4_lds_kernel(
     }
   }
 
-  // ---- epilogue.  Accumulator register v of tile (i, j) is y[m][n] with m = j*32 + r32 and
-  // n = i*32 + 8*(v/4) + 4*kh + v%4 inside the wave's 128 x 128 quadrant.  The quadrant goes
-  // through this wave's share of the (now idle) LDS as bf16 [m][n] so that global stores are
-  // 256 contiguous bytes per row.
-  const float alpha = *alpha_p;
-#ifdef FPQ_EXP_NO_STORE
-  if (alpha != 12345.0f) return;
-#endif
-  constexpr int WT_N = BN / 2, WT_M = BM / 2;        // wave quadrant
-  constexpr int kStride = WT_N * 2 + 16;             // bytes per staged row (+16: spread banks)
-  static_assert(4 * WT_M * kStride <= 2 * L::kStage, "epilogue staging does not fit in LDS");
-  __syncthreads();                                   // every wave is done reading operands
-  uint8_t* stg = smem + wave * (WT_M * kStride);
-  const int n0 = n_blk + wn * WT_N, m0 = m_blk + wm * WT_M;
-#pragma unroll
-  for (int i = 0; i < TN; ++i) {
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int nl = i * 32 + 8 * g + 4 * kh;
-      float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (bias) {
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-          if (n0 + nl + u < N) bv[u] = __uint_as_float((uint32_t)bias[n0 + nl + u] << 16);
-      }
-#pragma unroll
-      for (int j = 0; j < TM; ++j) {
-        uint32_t lo = pack_bf16x2(acc[i][j][4 * g + 0] * alpha, acc[i][j][4 * g + 1] * alpha);
-        uint32_t hi = pack_bf16x2(acc[i][j][4 * g + 2] * alpha, acc[i][j][4 * g + 3] * alpha);
-        if (bias) {
-          lo = pack_bf16x2(__uint_as_float(lo << 16) + bv[0], __uint_as_float(lo & 0xffff0000u) + bv[1]);
-          hi = pack_bf16x2(__uint_as_float(hi << 16) + bv[2], __uint_as_float(hi & 0xffff0000u) + bv[3]);
-        }
-        *(uint2*)(stg + (j * 32 + r32) * kStride + nl * 2) = make_uint2(lo, hi);
-      }
-    }
-  }
-  // read back: 16 lanes x 16 B cover one 256-byte row, 4 rows per wave instruction
-  const int rr = lane >> 4, cc = lane & 15;
-  const bool vec_ok = (N & 7) == 0;
-#pragma unroll 4
-  for (int p = 0; p < WT_M / 4; ++p) {
-    const int ml = p * 4 + rr;
-    const uint4 v = *(const uint4*)(stg + ml * kStride + cc * 16);
-    const int m = m0 + ml, n = n0 + cc * 8;
-    if (m >= M || n >= N) continue;
-    uint16_t* dst = y + (size_t)m * N + n;
-    if (vec_ok && n + 7 < N) {
-      *(uint4*)dst = v;
-    } else {
-      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (n + u < N) dst[u] = (uint16_t)(w[u >> 1] >> (16 * (u & 1)));
-    }
-  }
+  wave_quadrant_store<BN, BM, 2 * L::kStage>(acc, smem, y, bias, alpha_p, n_blk, m_blk, wn, wm, wave, lane, M, N);
 }
 
 // 8 E2M1 codes (one dword) times one E4M3 scale -> 8 exact fp16 values.
@@ -618,6 +629,168 @@ __global__ __launch_bounds__(256) void gemm_nvf4_direct_kernel(
   store_tile<TN, TM>(acc, y, bias, *alpha_p, n0, m0, M, N, r, kb);
 }
 
+// -------------------------------------------------------------------------------------------
+// LDS-tiled NVFP4 kernel for large M: the staging, swizzle, tile order and epilogue of the MXFP4
+// kernel, with the operands dequantized to exact fp16 in registers right before
+// v_mfma_f32_32x32x16_f16.  A lane's 16-byte chunk (32 codes, two E4M3 groups) feeds four MFMAs,
+// dword s of the chunk in MFMA s; both operands use that same K assignment.  Per K step of 64 a
+// wave dequantizes 8 tiles x 4 dwords (8 VALU ops each) for 64 MFMAs of 32 cycles, so the
+// conversion hides behind the matrix pipe.
+template <int BN, int BM>
+struct NvLdsLayout {
+  static constexpr int kScaleBytes = kKS / 16;  // 16 E4M3 bytes per row per stage
+  static constexpr int kCodesW = 0;
+  static constexpr int kCodesX = BN * kRowBytes;
+  static constexpr int kScalesW = (BN + BM) * kRowBytes;
+  static constexpr int kScalesX = kScalesW + BN * kScaleBytes;
+  static constexpr int kStage = kScalesX + BM * kScaleBytes;
+};
+
+// e4m3 byte (>= 0) -> the same value * 2^-8 as fp16, in both halves of a dword
+__device__ __forceinline__ v2h e4m3_pair_f16(uint32_t byte) {
+  const uint32_t h = (byte << 7) & 0x3f80u;
+  return __builtin_bit_cast(v2h, h | (h << 16));
+}
+
+__device__ __forceinline__ v8h dequant8_f16_s(uint32_t codes, v2h s2) {
+  const v2h p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 0) * s2;
+  const v2h p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 1) * s2;
+  const v2h p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 2) * s2;
+  const v2h p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 3) * s2;
+  return v8h{p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
+}
+
+template <int BN, int BM>
+__global__ __launch_bounds__(256) void gemm_nvf4_lds_kernel(
+    const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, int xs_stride,
+    const uint8_t* __restrict__ wq, const uint8_t* __restrict__ ws, int ws_stride,
+    const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
+    int M, int N, int K, int tiles_m) {
+  using L = NvLdsLayout<BN, BM>;
+  constexpr int TN = BN / 64, TM = BM / 64;
+  static_assert(BN == 256 && BM == 256, "scale DMA split assumes 64 rows per wave per operand");
+  extern __shared__ __attribute__((aligned(128))) uint8_t smem[];
+  const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  int logical = blockIdx.x;
+  {
+    const int nb = gridDim.x, per = nb / 8;
+    if (blockIdx.x < (unsigned)(per * 8)) logical = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+  }
+  const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
+  const int n_blk = tile_n * BN, m_blk = tile_m * BM;
+  const int wn = wave & 1, wm = wave >> 1;
+  const int kbytes = K >> 1;
+
+  constexpr int kInstrW = BN / 8 / 4, kInstrX = BM / 8 / 4;  // per wave: 8 rows x 128 B each
+  const int lrow = lane >> 3;
+  const int chunk = (lane & 7) ^ lrow;
+  uint32_t w_off[kInstrW], x_off[kInstrX];
+#pragma unroll
+  for (int j = 0; j < kInstrW; ++j) {
+    const int row = min(n_blk + (wave * kInstrW + j) * 8 + lrow, N - 1);
+    w_off[j] = (uint32_t)row * (uint32_t)kbytes + chunk * 16;
+  }
+#pragma unroll
+  for (int j = 0; j < kInstrX; ++j) {
+    const int row = min(m_blk + (wave * kInstrX + j) * 8 + lrow, M - 1);
+    x_off[j] = (uint32_t)row * (uint32_t)kbytes + chunk * 16;
+  }
+  // scales: one 16-byte load per row per stage; wave w moves rows [64 w, 64 w + 64) of both operands
+  const uint32_t ws_off = (uint32_t)min(n_blk + wave * 64 + lane, N - 1) * (uint32_t)ws_stride;
+  const uint32_t xs_off = (uint32_t)min(m_blk + wave * 64 + lane, M - 1) * (uint32_t)xs_stride;
+
+  auto issue_loads = [&](int stage, int k0) {
+    const uint32_t base = smem_base + stage * L::kStage;
+    const uint8_t* wk = wq + (k0 >> 1);
+    const uint8_t* xk = xq + (k0 >> 1);
+#pragma unroll
+    for (int j = 0; j < kInstrW; ++j)
+      lds_dma16(wk, w_off[j], base + L::kCodesW + (wave * kInstrW + j) * 1024);
+#pragma unroll
+    for (int j = 0; j < kInstrX; ++j)
+      lds_dma16(xk, x_off[j], base + L::kCodesX + (wave * kInstrX + j) * 1024);
+    lds_dma16(ws + (k0 >> 4), ws_off, base + L::kScalesW + wave * 1024);
+    lds_dma16(xs + (k0 >> 4), xs_off, base + L::kScalesX + wave * 1024);
+  };
+
+  v16f acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int r32 = lane & 31, kh = lane >> 5;
+  const int rw = wn * (BN / 2) + r32, rx = wm * (BM / 2) + r32;
+  int slot[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) slot[q] = ((2 * q + kh) ^ (r32 & 7)) * 16;
+  const int cw0 = L::kCodesW + rw * kRowBytes, cx0 = L::kCodesX + rx * kRowBytes;
+  // the lane's chunk in K step q covers E4M3 groups 4q + 2kh and 4q + 2kh + 1 of the stage
+  const int sw0 = L::kScalesW + rw * L::kScaleBytes + 2 * kh, sx0 = L::kScalesX + rx * L::kScaleBytes + 2 * kh;
+
+  const int nk = K / kKS;
+  issue_loads(0, 0);
+  for (int it = 0; it < nk; ++it) {
+    const int stage = it & 1;
+    wait_vmem();
+    __syncthreads();
+    const uint8_t* base = smem + stage * L::kStage;
+    uint4 aq[2][TN], bq[2][TM];
+    uint32_t sa[2][TN], sb[2][TM];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      bq[0][j] = *(const uint4*)(base + cx0 + slot[0] + j * 32 * kRowBytes);
+      sb[0][j] = *(const uint16_t*)(base + sx0 + j * 32 * L::kScaleBytes);
+    }
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+      aq[0][i] = *(const uint4*)(base + cw0 + slot[0] + i * 32 * kRowBytes);
+      sa[0][i] = *(const uint16_t*)(base + sw0 + i * 32 * L::kScaleBytes);
+    }
+    if (it + 1 < nk) issue_loads(stage ^ 1, (it + 1) * kKS);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (q < 3) {  // codes and scales of the next K step, read while this one computes
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+          bq[(q + 1) & 1][j] = *(const uint4*)(base + cx0 + slot[q + 1] + j * 32 * kRowBytes);
+          sb[(q + 1) & 1][j] = *(const uint16_t*)(base + sx0 + 4 * (q + 1) + j * 32 * L::kScaleBytes);
+        }
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+          aq[(q + 1) & 1][i] = *(const uint4*)(base + cw0 + slot[q + 1] + i * 32 * kRowBytes);
+          sa[(q + 1) & 1][i] = *(const uint16_t*)(base + sw0 + 4 * (q + 1) + i * 32 * L::kScaleBytes);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        v8h bh[TM];
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+          const uint4 c = bq[q & 1][j];
+          const uint32_t cd = s == 0 ? c.x : s == 1 ? c.y : s == 2 ? c.z : c.w;
+          bh[j] = dequant8_f16_s(cd, e4m3_pair_f16(sb[q & 1][j] >> (8 * (s >> 1))));
+        }
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+          const uint4 c = aq[q & 1][i];
+          const uint32_t cd = s == 0 ? c.x : s == 1 ? c.y : s == 2 ? c.z : c.w;
+          const v8h ah = dequant8_f16_s(cd, e4m3_pair_f16(sa[q & 1][i] >> (8 * (s >> 1))));
+#pragma unroll
+          for (int j = 0; j < TM; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[j], acc[i][j], 0, 0, 0);
+        }
+      }
+    }
+  }
+  wave_quadrant_store<BN, BM, 2 * L::kStage>(acc, smem, y, bias, alpha_p, n_blk, m_blk, wn, wm, wave, lane, M, N);
+}
+
 template <int FMT>
 static int gemm_dispatch(const void* xq, const void* xs, int64_t xs_stride, const void* wq,
                          const void* ws, int64_t ws_stride, const float* alpha, const void* bias,
@@ -649,6 +822,25 @@ static int gemm_dispatch(const void* xq, const void* xs, int64_t xs_stride, cons
     }                                                                                              \
   } while (0)
 
+  if (FMT == 1 && M > 64 && K % kKS == 0 && xs_stride % 16 == 0 && ws_stride % 16 == 0 &&
+      !((uintptr_t)xs & 15u) && !((uintptr_t)ws & 15u) && N * (K / 2) < ((int64_t)1 << 32) &&
+      M * (K / 2) < ((int64_t)1 << 32)) {
+    constexpr int BN = 256, BM = 256;
+    using L = NvLdsLayout<BN, BM>;
+    const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
+    static bool nv_attr_set = false;
+    if (!nv_attr_set) {
+      hipError_t e = hipFuncSetAttribute((const void*)gemm_nvf4_lds_kernel<BN, BM>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 2 * L::kStage);
+      if (e != hipSuccess) return (int)e;
+      nv_attr_set = true;
+    }
+    hipLaunchKernelGGL((gemm_nvf4_lds_kernel<BN, BM>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256),
+                       2 * L::kStage, stream, (const uint8_t*)xq, (const uint8_t*)xs, (int)xs_stride,
+                       (const uint8_t*)wq, (const uint8_t*)ws, (int)ws_stride, alpha,
+                       (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K, tiles_m);
+    return (int)hipGetLastError();
+  }
   if (FMT == 0 && M > 64 && K % kKS == 0 && xs_stride % 4 == 0 && ws_stride % 4 == 0 &&
       !((uintptr_t)xs & 3u) && !((uintptr_t)ws & 3u) && N * (K / 2) < ((int64_t)1 << 32) &&
       M * (K / 2) < ((int64_t)1 << 32)) {
