@@ -230,6 +230,11 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", default="", help="comma list of workloads to run (for profiling one kernel): "
+                    "nvfp4_quantize, mxfp4_quantize, mxfp4_linear_M2048, mxfp4_linear_M128, mxfp4_linear_M16, "
+                    "mxfp4_linear_M1, nvfp4_linear")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 256 MiB device copy (known traffic) to scale rocprofv3 byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path uses no collectives; run with --gpus 1", file=sys.stderr)
@@ -242,6 +247,29 @@ def main():
         print("bench.py needs a GPU (the HIP engine has no CPU path)", file=sys.stderr)
         sys.exit(2)
     _engine.lib()
+
+    only = [w for w in args.only.split(",") if w]
+    if args.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 256)
+        dst = torch.empty_like(src)
+        for _ in range(max(3, args.steps // 10)):
+            dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+    if only:
+        out = {}
+        if "nvfp4_quantize" in only:
+            out["nvfp4_quantize"] = bench_quantize(torch, "nvfp4", 8192, 4096, 16, args.steps, args.warmup, seed=1)
+        if "mxfp4_quantize" in only:
+            out["mxfp4_quantize"] = bench_quantize(torch, "mxfp4", 2048, 4096, 128, args.steps, args.warmup, seed=0)
+        for m in (2048, 128, 16, 1):
+            if f"mxfp4_linear_M{m}" in only:
+                out[f"mxfp4_linear_M{m}"] = bench_linear(torch, "mxfp4", m, 14336, 4096, 128, args.steps,
+                                                          args.warmup, seed=2)
+        if "nvfp4_linear" in only:
+            out["nvfp4_linear"] = bench_linear(torch, "nvfp4", 4096, 24576, 4096, 16, max(10, args.steps // 10),
+                                               max(2, args.warmup // 10), seed=3)
+        print(json.dumps({"only": only, "steps": args.steps, "results": out}))
+        return
 
     results = {}
     results["nvfp4_quantize"] = bench_quantize(torch, "nvfp4", 8192, 4096, 16, args.steps, args.warmup, seed=1)
@@ -269,6 +297,11 @@ def main():
         "workload": nv["workload"], "gemm_us": round(nv["gemm_ms"] * 1e3, 3),
         "gemm_TFLOP/s": round(nv["gemm_tflops"], 2),
         "mfma_frac_of_f16_peak": round(nv["gemm_tflops"] / BF16_PEAK_TFLOPS, 4)}
+    traffic = {}
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f)  # HBM bytes per launch measured with rocprofv3 --pmc (see profiles/)
     line = {
         "metric": METRIC,
         "value": round(head["linear_tflops"], 2),
@@ -291,7 +324,7 @@ def main():
             "peak": FP4_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(head["gemm_tflops"] / FP4_PEAK_TFLOPS, 4),
-            "traffic": None,
+            "traffic": traffic.get("mxfp4_gemm_M2048"),
             "kernel_us": round(head["gemm_ms"] * 1e3, 3),
             "algorithmic_flops_per_launch": int(head["flops"]),
         },
@@ -302,7 +335,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(quant["gbps"] / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": traffic.get("nvfp4_quantize"),
             "kernel_us": round(quant["kernel_ms"] * 1e3, 3),
             "algorithmic_bytes_per_launch": int(quant["algo_bytes"]),
         },
