@@ -26,6 +26,9 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
+#ifndef FPQ_GEMM_WM
+#define FPQ_GEMM_WM 2  // waves along m in the LDS-tiled MXFP4 kernel (2: 4 waves, 4: 8 waves)
+#endif
 #ifndef FPQ_SPLITK_MAX_M
 #define FPQ_SPLITK_MAX_M 64  // largest M served by the weight-streaming split-K kernel
 #endif
@@ -291,21 +294,21 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
 // m = j*32 + r32 and n = i*32 + 8*(v/4) + 4*kh + v%4 inside the wave's quadrant of the workgroup
 // tile.  The quadrant goes through this wave's share of the (now idle) LDS as bf16 [m][n] so that
 // global stores are 256 contiguous bytes per row.
-template <int BN, int BM, int LDS_BYTES>
-__device__ __forceinline__ void wave_quadrant_store(const v16f (&acc)[BN / 64][BM / 64], uint8_t* smem,
+template <int BN, int BM, int LDS_BYTES, int WM = 2>
+__device__ __forceinline__ void wave_quadrant_store(const v16f (&acc)[BN / 64][BM / (32 * WM)], uint8_t* smem,
                                                     uint16_t* __restrict__ y,
                                                     const uint16_t* __restrict__ bias,
                                                     const float* __restrict__ alpha_p, int n_blk, int m_blk,
                                                     int wn, int wm, int wave, int lane, int M, int N) {
-  constexpr int TN = BN / 64, TM = BM / 64;
+  constexpr int TN = BN / 64, TM = BM / (32 * WM);
   const int r32 = lane & 31, kh = lane >> 5;
   const float alpha = *alpha_p;
 #ifdef FPQ_EXP_NO_STORE
   if (alpha != 12345.0f) return;
 #endif
-  constexpr int WT_N = BN / 2, WT_M = BM / 2;        // wave quadrant
+  constexpr int WT_N = BN / 2, WT_M = BM / WM;       // this wave's part of the workgroup tile
   constexpr int kStride = WT_N * 2 + 16;             // bytes per staged row (+16: spread banks)
-  static_assert(4 * WT_M * kStride <= LDS_BYTES, "epilogue staging does not fit in LDS");
+  static_assert(2 * WM * WT_M * kStride <= LDS_BYTES, "epilogue staging does not fit in LDS");
   __syncthreads();                                   // every wave is done reading operands
   uint8_t* stg = smem + wave * (WT_M * kStride);
   const int n0 = n_blk + wn * WT_N, m0 = m_blk + wm * WT_M;
@@ -362,14 +365,15 @@ struct MxLdsLayout {
   static constexpr int kStage = kScalesX + BM * kScaleBytes;
 };
 
-template <int BN, int BM>
-__global__ __launch_bounds__(256) void gemm_mxf4_lds_kernel(
+template <int BN, int BM, int WM>
+__global__ __launch_bounds__(128 * WM) void gemm_mxf4_lds_kernel(
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, int xs_stride,
     const uint8_t* __restrict__ wq, const uint8_t* __restrict__ ws, int ws_stride,
     const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
     int M, int N, int K, int tiles_m) {
   using L = MxLdsLayout<BN, BM>;
-  constexpr int TN = BN / 64, TM = BM / 64;   // 32x32 MFMA tiles per wave along n and m
+  constexpr int NW = 2 * WM;                          // waves: 2 along n x WM along m
+  constexpr int TN = BN / 64, TM = BM / (32 * WM);    // 32x32 MFMA tiles per wave along n and m
   extern __shared__ __attribute__((aligned(128))) uint8_t smem[];
   const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
 
@@ -387,33 +391,38 @@ __global__ __launch_bounds__(256) void gemm_mxf4_lds_kernel(
   const int kbytes = K >> 1;
 
   // ---- global -> LDS assignment.  Codes: one wave instruction moves 8 rows x 128 B.
-  constexpr int kInstrW = BN / 8 / 4, kInstrX = BM / 8 / 4;  // per wave
+  constexpr int kInstrW = BN / 8 / NW, kInstrX = BM / 8 / NW;  // per wave
   const int lrow = lane >> 3;                                // row within the 8-row slab
-  const int chunk = (lane & 7) ^ lrow;                       // swizzled 16-byte chunk this lane fetches
+  // LDS holds chunk c of tile row r at 16-byte slot c ^ (r & 7) ^ ((r >> 3) & 1) of the row: with
+  // that swizzle the 32-row x 32-byte operand reads of the 32x32 MFMA layout hit every bank group
+  // exactly once per pass (checked with the bank-conflict counter); a lane of load instruction
+  // `idx` (8 rows) therefore fetches chunk (lane & 7) ^ lrow ^ (idx & 1)
   uint32_t w_off[kInstrW], x_off[kInstrX];
 #pragma unroll
   for (int j = 0; j < kInstrW; ++j) {
-    const int row = min(n_blk + (wave * kInstrW + j) * 8 + lrow, N - 1);
-    w_off[j] = (uint32_t)row * (uint32_t)kbytes + chunk * 16;
+    const int idx = wave * kInstrW + j;
+    const int row = min(n_blk + idx * 8 + lrow, N - 1);
+    w_off[j] = (uint32_t)row * (uint32_t)kbytes + (((lane & 7) ^ lrow ^ (idx & 1)) * 16);
   }
 #pragma unroll
   for (int j = 0; j < kInstrX; ++j) {
-    const int row = min(m_blk + (wave * kInstrX + j) * 8 + lrow, M - 1);
-    x_off[j] = (uint32_t)row * (uint32_t)kbytes + chunk * 16;
+    const int idx = wave * kInstrX + j;
+    const int row = min(m_blk + idx * 8 + lrow, M - 1);
+    x_off[j] = (uint32_t)row * (uint32_t)kbytes + (((lane & 7) ^ lrow ^ (idx & 1)) * 16);
   }
   // Scales: one wave instruction moves 32 rows x 8 B (two dwords per row); wave w takes
-  // instructions j with j % 4 == w.
+  // instructions j with j % NW == w.
   constexpr int kSInstrW = BN / 32, kSInstrX = BM / 32;
-  constexpr int kSW = (kSInstrW + 3) / 4, kSX = (kSInstrX + 3) / 4;
+  constexpr int kSW = (kSInstrW + NW - 1) / NW, kSX = (kSInstrX + NW - 1) / NW;
   uint32_t ws_off[kSW], xs_off[kSX];
 #pragma unroll
   for (int j = 0; j < kSW; ++j) {
-    const int row = min(n_blk + (j * 4 + wave) * 32 + (lane >> 1), N - 1);
+    const int row = min(n_blk + (j * NW + wave) * 32 + (lane >> 1), N - 1);
     ws_off[j] = (uint32_t)row * (uint32_t)ws_stride + (lane & 1) * 4;
   }
 #pragma unroll
   for (int j = 0; j < kSX; ++j) {
-    const int row = min(m_blk + (j * 4 + wave) * 32 + (lane >> 1), M - 1);
+    const int row = min(m_blk + (j * NW + wave) * 32 + (lane >> 1), M - 1);
     xs_off[j] = (uint32_t)row * (uint32_t)xs_stride + (lane & 1) * 4;
   }
 
@@ -432,10 +441,10 @@ __global__ __launch_bounds__(256) void gemm_mxf4_lds_kernel(
 #ifndef FPQ_EXP_NO_SCALE_DMA
 #pragma unroll
     for (int j = 0; j < kSW; ++j)
-      if (j * 4 + wave < kSInstrW) lds_dma4(wsk, ws_off[j], base + L::kScalesW + (j * 4 + wave) * 256);
+      if (j * NW + wave < kSInstrW) lds_dma4(wsk, ws_off[j], base + L::kScalesW + (j * NW + wave) * 256);
 #pragma unroll
     for (int j = 0; j < kSX; ++j)
-      if (j * 4 + wave < kSInstrX) lds_dma4(xsk, xs_off[j], base + L::kScalesX + (j * 4 + wave) * 256);
+      if (j * NW + wave < kSInstrX) lds_dma4(xsk, xs_off[j], base + L::kScalesX + (j * NW + wave) * 256);
 #endif
   };
 
@@ -450,10 +459,10 @@ __global__ __launch_bounds__(256) void gemm_mxf4_lds_kernel(
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   const int r32 = lane & 31, kh = lane >> 5;
-  const int rw = wn * (BN / 2) + r32, rx = wm * (BM / 2) + r32;
+  const int rw = wn * (BN / 2) + r32, rx = wm * (BM / WM) + r32;
   int slot[4];
 #pragma unroll
-  for (int q = 0; q < 4; ++q) slot[q] = ((2 * q + kh) ^ (r32 & 7)) * 16;
+  for (int q = 0; q < 4; ++q) slot[q] = ((2 * q + kh) ^ (r32 & 7) ^ ((r32 >> 3) & 1)) * 16;
   const int cw0 = L::kCodesW + rw * kRowBytes, cx0 = L::kCodesX + rx * kRowBytes;
   const int sw0 = L::kScalesW + rw * kScaleBytes, sx0 = L::kScalesX + rx * kScaleBytes;
   // bytes kh, 2+kh, 4+kh, 6+kh of a row's 8 scale bytes -> one dword; op_sel q picks K step q
@@ -464,7 +473,9 @@ __global__ __launch_bounds__(256) void gemm_mxf4_lds_kernel(
   for (int it = 0; it < nk; ++it) {
     const int stage = it & 1;
     wait_vmem();  // this wave's loads for `stage` have landed
+#ifndef FPQ_EXP_NO_BARRIER
     __syncthreads();
+#endif
     const uint8_t* base = smem + stage * L::kStage;
     // Operand stream of a stage: 4 K steps x TN weight tiles, each tile used by TM MFMAs.
     // Weight tiles are read from LDS two steps ahead (ring of 3), the activation tiles of the
@@ -519,7 +530,7 @@ __global__ __launch_bounds__(256) void gemm_mxf4_lds_kernel(
     }
   }
 
-  wave_quadrant_store<BN, BM, 2 * L::kStage>(acc, smem, y, bias, alpha_p, n_blk, m_blk, wn, wm, wave, lane, M, N);
+  wave_quadrant_store<BN, BM, 2 * L::kStage, WM>(acc, smem, y, bias, alpha_p, n_blk, m_blk, wn, wm, wave, lane, M, N);
 }
 
 // 8 E2M1 codes (one dword) times one E4M3 scale -> 8 exact fp16 values.
@@ -685,17 +696,18 @@ __global__ __launch_bounds__(256) void gemm_nvf4_lds_kernel(
 
   constexpr int kInstrW = BN / 8 / 4, kInstrX = BM / 8 / 4;  // per wave: 8 rows x 128 B each
   const int lrow = lane >> 3;
-  const int chunk = (lane & 7) ^ lrow;
-  uint32_t w_off[kInstrW], x_off[kInstrX];
+  uint32_t w_off[kInstrW], x_off[kInstrX];  // same chunk swizzle as the MXFP4 kernel
 #pragma unroll
   for (int j = 0; j < kInstrW; ++j) {
-    const int row = min(n_blk + (wave * kInstrW + j) * 8 + lrow, N - 1);
-    w_off[j] = (uint32_t)row * (uint32_t)kbytes + chunk * 16;
+    const int idx = wave * kInstrW + j;
+    const int row = min(n_blk + idx * 8 + lrow, N - 1);
+    w_off[j] = (uint32_t)row * (uint32_t)kbytes + (((lane & 7) ^ lrow ^ (idx & 1)) * 16);
   }
 #pragma unroll
   for (int j = 0; j < kInstrX; ++j) {
-    const int row = min(m_blk + (wave * kInstrX + j) * 8 + lrow, M - 1);
-    x_off[j] = (uint32_t)row * (uint32_t)kbytes + chunk * 16;
+    const int idx = wave * kInstrX + j;
+    const int row = min(m_blk + idx * 8 + lrow, M - 1);
+    x_off[j] = (uint32_t)row * (uint32_t)kbytes + (((lane & 7) ^ lrow ^ (idx & 1)) * 16);
   }
   // scales: one 16-byte load per row per stage; wave w moves rows [64 w, 64 w + 64) of both operands
   const uint32_t ws_off = (uint32_t)min(n_blk + wave * 64 + lane, N - 1) * (uint32_t)ws_stride;
@@ -727,7 +739,7 @@ __global__ __launch_bounds__(256) void gemm_nvf4_lds_kernel(
   const int rw = wn * (BN / 2) + r32, rx = wm * (BM / 2) + r32;
   int slot[4];
 #pragma unroll
-  for (int q = 0; q < 4; ++q) slot[q] = ((2 * q + kh) ^ (r32 & 7)) * 16;
+  for (int q = 0; q < 4; ++q) slot[q] = ((2 * q + kh) ^ (r32 & 7) ^ ((r32 >> 3) & 1)) * 16;
   const int cw0 = L::kCodesW + rw * kRowBytes, cx0 = L::kCodesX + rx * kRowBytes;
   // the lane's chunk in K step q covers E4M3 groups 4q + 2kh and 4q + 2kh + 1 of the stage
   const int sw0 = L::kScalesW + rw * L::kScaleBytes + 2 * kh, sx0 = L::kScalesX + rx * L::kScaleBytes + 2 * kh;
@@ -849,12 +861,13 @@ static int gemm_dispatch(const void* xq, const void* xs, int64_t xs_stride, cons
     using L = MxLdsLayout<BN, BM>;
     static bool attr_set = false;
     if (!attr_set) {
-      hipError_t e = hipFuncSetAttribute((const void*)gemm_mxf4_lds_kernel<BN, BM>,
+      hipError_t e = hipFuncSetAttribute((const void*)gemm_mxf4_lds_kernel<BN, BM, FPQ_GEMM_WM>,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, 2 * L::kStage);
       if (e != hipSuccess) return (int)e;
       attr_set = true;
     }
-    hipLaunchKernelGGL((gemm_mxf4_lds_kernel<BN, BM>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256),
+    hipLaunchKernelGGL((gemm_mxf4_lds_kernel<BN, BM, FPQ_GEMM_WM>), dim3((unsigned)(tiles_m * tiles_n)),
+                       dim3(128 * FPQ_GEMM_WM),
                        2 * L::kStage, stream, (const uint8_t*)xq, (const uint8_t*)xs, (int)xs_stride,
                        (const uint8_t*)wq, (const uint8_t*)ws, (int)ws_stride, alpha,
                        (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K, tiles_m);

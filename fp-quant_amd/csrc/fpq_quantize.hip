@@ -265,14 +265,17 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
   }
 
   // DMA lane map: instruction i fills LDS pieces [64 i, 64 i + 64); piece p = PIECES * b + j
-  // belongs to chunk b and holds that chunk's 16-byte piece j ^ (b % PIECES).
+  // belongs to chunk b and holds that chunk's 16-byte piece j ^ sw(b).  sw(b) is chosen so that
+  // the 16-byte reads "piece k of my own chunk" of all lanes hit every LDS bank group once per
+  // pass (checked with the bank-conflict counter): b % 16 for 256-byte chunks, and
+  // (b % 8) ^ ((b / 8) & 1) for 128-byte chunks.
+  auto sw = [](uint32_t b) -> uint32_t { return PIECES == 8 ? ((b & 7u) ^ ((b >> 3) & 1u)) : (b % PIECES); };
   const uint32_t b_lo = lane / PIECES, j_lo = lane % PIECES;
-  constexpr int NV_OFF = PIECES / CPI > 0 ? PIECES / CPI : 1;  // distinct swizzle phases over i
+  constexpr int NV_OFF = PIECES == 8 ? 2 : 4;  // distinct swizzle phases over the instruction index
   uint32_t voff[NV_OFF];
 #pragma unroll
-  for (int m = 0; m < NV_OFF; ++m)
-    voff[m] = b_lo * CB + ((j_lo ^ ((CPI * m + b_lo) % PIECES)) * 16u);
-  const uint32_t rd_base = lane * CB, l_sw = lane % PIECES;
+  for (int m = 0; m < NV_OFF; ++m) voff[m] = b_lo * CB + ((j_lo ^ sw(CPI * m + b_lo)) * 16u);
+  const uint32_t rd_base = lane * CB, l_sw = sw(lane);
 
   const uint32_t n_tiles = (n_chunks + 63u) / 64u;
   const uint32_t total_waves = gridDim.x * 4u;
