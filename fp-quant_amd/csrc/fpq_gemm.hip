@@ -18,12 +18,10 @@
 
 #include "../../include/fpq.h"
 #include "fpq_device.h"
+#include "fpq_gemm_epilogue.h"
 
 namespace fpq {
 
-typedef int v8i __attribute__((ext_vector_type(8)));
-typedef float v4f __attribute__((ext_vector_type(4)));
-typedef float v16f __attribute__((ext_vector_type(16)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
 #ifndef FPQ_GEMM_WM
@@ -280,82 +278,6 @@ constexpr int kKS = 256;                    // K per stage
 constexpr int kRowBytes = kKS / 2;          // 128 bytes of codes per row per stage
 constexpr int kScaleBytes = kKS / 32;       // 8 scale bytes per row per stage
 
-typedef __attribute__((address_space(3))) void lds_void;
-typedef const __attribute__((address_space(1))) void global_void;
-
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
-}
-
-// Epilogue of the LDS-tiled kernels.  Accumulator register v of 32x32 tile (i, j) is y[m][n] with
-// m = j*32 + r32 and n = i*32 + 8*(v/4) + 4*kh + v%4 inside the wave's quadrant of the workgroup
-// tile.  The quadrant goes through this wave's share of the (now idle) LDS as bf16 [m][n] so that
-// global stores are 256 contiguous bytes per row.
-template <int BN, int BM, int LDS_BYTES, int WM = 2>
-__device__ __forceinline__ void wave_quadrant_store(const v16f (&acc)[BN / 64][BM / (32 * WM)], uint8_t* smem,
-                                                    uint16_t* __restrict__ y,
-                                                    const uint16_t* __restrict__ bias,
-                                                    const float* __restrict__ alpha_p, int n_blk, int m_blk,
-                                                    int wn, int wm, int wave, int lane, int M, int N) {
-  constexpr int TN = BN / 64, TM = BM / (32 * WM);
-  const int r32 = lane & 31, kh = lane >> 5;
-  const float alpha = *alpha_p;
-#ifdef FPQ_EXP_NO_STORE
-  if (alpha != 12345.0f) return;
-#endif
-  constexpr int WT_N = BN / 2, WT_M = BM / WM;       // this wave's part of the workgroup tile
-  constexpr int kStride = WT_N * 2 + 16;             // bytes per staged row (+16: spread banks)
-  static_assert(2 * WM * WT_M * kStride <= LDS_BYTES, "epilogue staging does not fit in LDS");
-  __syncthreads();                                   // every wave is done reading operands
-  uint8_t* stg = smem + wave * (WT_M * kStride);
-  const int n0 = n_blk + wn * WT_N, m0 = m_blk + wm * WT_M;
-#pragma unroll
-  for (int i = 0; i < TN; ++i) {
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int nl = i * 32 + 8 * g + 4 * kh;
-      float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (bias) {
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-          if (n0 + nl + u < N) bv[u] = __uint_as_float((uint32_t)bias[n0 + nl + u] << 16);
-      }
-#pragma unroll
-      for (int j = 0; j < TM; ++j) {
-        uint32_t lo = pack_bf16x2(acc[i][j][4 * g + 0] * alpha, acc[i][j][4 * g + 1] * alpha);
-        uint32_t hi = pack_bf16x2(acc[i][j][4 * g + 2] * alpha, acc[i][j][4 * g + 3] * alpha);
-        if (bias) {
-          lo = pack_bf16x2(__uint_as_float(lo << 16) + bv[0], __uint_as_float(lo & 0xffff0000u) + bv[1]);
-          hi = pack_bf16x2(__uint_as_float(hi << 16) + bv[2], __uint_as_float(hi & 0xffff0000u) + bv[3]);
-        }
-        *(uint2*)(stg + (j * 32 + r32) * kStride + nl * 2) = make_uint2(lo, hi);
-      }
-    }
-  }
-  // read back: 16 lanes x 16 B cover one 256-byte row, 4 rows per wave instruction
-  const int rr = lane >> 4, cc = lane & 15;
-  const bool vec_ok = (N & 7) == 0;
-#pragma unroll 4
-  for (int p = 0; p < WT_M / 4; ++p) {
-    const int ml = p * 4 + rr;
-    const uint4 v = *(const uint4*)(stg + ml * kStride + cc * 16);
-    const int m = m0 + ml, n = n0 + cc * 8;
-    if (m >= M || n >= N) continue;
-    uint16_t* dst = y + (size_t)m * N + n;
-    if (vec_ok && n + 7 < N) {
-      *(uint4*)dst = v;
-    } else {
-      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (n + u < N) dst[u] = (uint16_t)(w[u >> 1] >> (16 * (u & 1)));
-    }
-  }
-}
-
 template <int BN, int BM>
 struct MxLdsLayout {
   static constexpr int kCodesW = 0;
@@ -402,13 +324,21 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_lds_kernel(
   for (int j = 0; j < kInstrW; ++j) {
     const int idx = wave * kInstrW + j;
     const int row = min(n_blk + idx * 8 + lrow, N - 1);
+#ifdef FPQ_EXP_LINEAR_CHUNKS
+    w_off[j] = (uint32_t)row * (uint32_t)kbytes + ((lane & 7) * 16);
+#else
     w_off[j] = (uint32_t)row * (uint32_t)kbytes + (((lane & 7) ^ lrow ^ (idx & 1)) * 16);
+#endif
   }
 #pragma unroll
   for (int j = 0; j < kInstrX; ++j) {
     const int idx = wave * kInstrX + j;
     const int row = min(m_blk + idx * 8 + lrow, M - 1);
+#ifdef FPQ_EXP_LINEAR_CHUNKS
+    x_off[j] = (uint32_t)row * (uint32_t)kbytes + ((lane & 7) * 16);
+#else
     x_off[j] = (uint32_t)row * (uint32_t)kbytes + (((lane & 7) ^ lrow ^ (idx & 1)) * 16);
+#endif
   }
   // Scales: one wave instruction moves 32 rows x 8 B (two dwords per row); wave w takes
   // instructions j with j % NW == w.
@@ -448,6 +378,42 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_lds_kernel(
 #endif
   };
 
+#ifdef FPQ_GEMM_STAGE_REGS
+  // Alternative operand path: global -> registers -> ds_write (same LDS image as the direct loads).
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  u32x4 w_reg[kInstrW], x_reg[kInstrX];
+  uint32_t ws_reg[kSW], xs_reg[kSX];
+#define FPQ_FETCH_REGS(k0_)                                                                     \
+  {                                                                                             \
+    const int k0__ = (k0_);                                                                     \
+    _Pragma("unroll") for (int j = 0; j < kInstrW; ++j)                                         \
+        w_reg[j] = *(const u32x4*)(wq + (k0__ >> 1) + w_off[j]);                                \
+    _Pragma("unroll") for (int j = 0; j < kInstrX; ++j)                                         \
+        x_reg[j] = *(const u32x4*)(xq + (k0__ >> 1) + x_off[j]);                                \
+    _Pragma("unroll") for (int j = 0; j < kSW; ++j)                                             \
+        ws_reg[j] = *(const uint32_t*)(ws + (k0__ >> 5) + ws_off[j]);                           \
+    _Pragma("unroll") for (int j = 0; j < kSX; ++j)                                             \
+        xs_reg[j] = *(const uint32_t*)(xs + (k0__ >> 5) + xs_off[j]);                           \
+  }
+#define FPQ_SPILL_REGS(stage_, part_, parts_)                                                   \
+  {                                                                                             \
+    uint8_t* sb__ = smem + (stage_) * L::kStage;                                                \
+    _Pragma("unroll") for (int j = 0; j < kInstrW; ++j)                                         \
+        if (j % (parts_) == (part_))                                                            \
+            *(u32x4*)(sb__ + L::kCodesW + (wave * kInstrW + j) * 1024 + lane * 16) = w_reg[j];  \
+    _Pragma("unroll") for (int j = 0; j < kInstrX; ++j)                                         \
+        if (j % (parts_) == (part_))                                                            \
+            *(u32x4*)(sb__ + L::kCodesX + (wave * kInstrX + j) * 1024 + lane * 16) = x_reg[j];  \
+    if ((part_) == (parts_) - 1) {                                                              \
+      _Pragma("unroll") for (int j = 0; j < kSW; ++j)                                           \
+          *(uint32_t*)(sb__ + L::kScalesW + (j * NW + wave) * 256 + lane * 4) = ws_reg[j];      \
+      _Pragma("unroll") for (int j = 0; j < kSX; ++j)                                           \
+          *(uint32_t*)(sb__ + L::kScalesX + (j * NW + wave) * 256 + lane * 4) = xs_reg[j];      \
+    }                                                                                           \
+  }
+  static_assert(kSInstrW % NW == 0 && kSInstrX % NW == 0, "scale loads must divide over the waves");
+#endif
+
   // 32x32x64 MFMA: lane = (row r32 = lane % 32, K half kh = lane / 32); one stage holds four
   // K steps q of 64, the lane's 16-byte chunk in step q is c = 2q + kh, its scale byte is c too.
   v16f acc[TN][TM];
@@ -469,68 +435,144 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_lds_kernel(
   const uint32_t perm_sel = kh ? 0x07050301u : 0x06040200u;
 
   const int nk = K / kKS;
-  issue_loads(0, 0);
-  for (int it = 0; it < nk; ++it) {
-    const int stage = it & 1;
-    wait_vmem();  // this wave's loads for `stage` have landed
-#ifndef FPQ_EXP_NO_BARRIER
-    __syncthreads();
+#ifdef FPQ_EXP_TIMING
+  const uint64_t tc0 = __builtin_readcyclecounter(), tr0 = __builtin_amdgcn_s_memrealtime();
 #endif
-    const uint8_t* base = smem + stage * L::kStage;
-    // Operand stream of a stage: 4 K steps x TN weight tiles, each tile used by TM MFMAs.
-    // Weight tiles are read from LDS two steps ahead (ring of 3), the activation tiles of the
-    // next K step during the first steps of the current one; sched_barrier keeps that order.
-    uint4 bq[2][TM], aq[3];
+  // Operand stream of a stage: 4 K steps x TN weight tiles (16 "steps"), each tile used by TM
+  // MFMAs.  Weight tiles are read from LDS three steps ahead (ring of 4), the activation tiles
+  // of the next K step during the first steps of the current one.  The one barrier of an
+  // iteration sits after step kSync: by then every wave has issued and completed all its reads
+  // of the current stage and its share of the next stage's loads has landed, so the steps after
+  // it already read the first tiles of the next stage (no bubble at the top of an iteration) and
+  // the current buffer is handed to the loads of the stage after next.
+  static_assert(TN == 4, "the step schedule below is written for four weight tiles per wave");
+  constexpr int kSteps = 4 * TN, kSync = kSteps - 4;
+  uint4 bq[2][TM], aq[4];
+  uint2 raw_sa[TN], raw_sb[TM];
+  auto read_w = [&](const uint8_t* b, int step) {
+    return *(const uint4*)(b + cw0 + slot[step / TN] + (step % TN) * 32 * kRowBytes);
+  };
+  auto read_x = [&](const uint8_t* b, int q, int j) {
+    return *(const uint4*)(b + cx0 + slot[q] + j * 32 * kRowBytes);
+  };
+
+#ifdef FPQ_GEMM_STAGE_REGS
+  FPQ_FETCH_REGS(0);
+  FPQ_SPILL_REGS(0, 0, 1);
+  if (nk > 1) FPQ_FETCH_REGS(kKS);
+  __syncthreads();
+#else
+  issue_loads(0, 0);
+#ifndef FPQ_EXP_NO_DMA
+  if (nk > 1) issue_loads(1, kKS);
+#endif
+  wait_vmem();
+  __syncthreads();
+#endif
+#pragma unroll
+  for (int j = 0; j < TM; ++j) bq[0][j] = read_x(smem, 0, j);
+#pragma unroll
+  for (int u = 0; u < 3; ++u) aq[u] = read_w(smem, u);
+#pragma unroll
+  for (int j = 0; j < TM; ++j) raw_sb[j] = *(const uint2*)(smem + sx0 + j * 32 * kScaleBytes);
+#pragma unroll
+  for (int i = 0; i < TN; ++i) raw_sa[i] = *(const uint2*)(smem + sw0 + i * 32 * kScaleBytes);
+
+  for (int it = 0; it < nk; ++it) {
+    const uint8_t* base = smem + (it & 1) * L::kStage;
+    const uint8_t* next = smem + ((it + 1) & 1) * L::kStage;  // stale bytes after the last stage: read, never used
     int sa[TN], sb[TM];
 #pragma unroll
-    for (int j = 0; j < TM; ++j) bq[0][j] = *(const uint4*)(base + cx0 + slot[0] + j * 32 * kRowBytes);
-    aq[0] = *(const uint4*)(base + cw0 + slot[0]);
-    aq[1] = *(const uint4*)(base + cw0 + slot[0] + 32 * kRowBytes);
+    for (int j = 0; j < TM; ++j) sb[j] = (int)__builtin_amdgcn_perm(raw_sb[j].y, raw_sb[j].x, perm_sel);
 #pragma unroll
-    for (int j = 0; j < TM; ++j) {
-      const uint2 v = *(const uint2*)(base + sx0 + j * 32 * kScaleBytes);
-      sb[j] = (int)__builtin_amdgcn_perm(v.y, v.x, perm_sel);
-    }
-#pragma unroll
-    for (int i = 0; i < TN; ++i) {
-      const uint2 v = *(const uint2*)(base + sw0 + i * 32 * kScaleBytes);
-      sa[i] = (int)__builtin_amdgcn_perm(v.y, v.x, perm_sel);
-    }
-#ifndef FPQ_EXP_NO_DMA
-    if (it + 1 < nk) issue_loads(stage ^ 1, (it + 1) * kKS);
-#endif
+    for (int i = 0; i < TN; ++i) sa[i] = (int)__builtin_amdgcn_perm(raw_sa[i].y, raw_sa[i].x, perm_sel);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int t = 0; t < 4 * TN; ++t) {
+    for (int t = 0; t < kSteps; ++t) {
       const int q = t / TN, i = t % TN;
-      if (t + 2 < 4 * TN) {
-        const int q2 = (t + 2) / TN, i2 = (t + 2) % TN;
-        aq[(t + 2) % 3] = *(const uint4*)(base + cw0 + slot[q2] + i2 * 32 * kRowBytes);
-      }
-      if (q < 3 && i < (TM + 1) / 2) {
+#ifdef FPQ_EXP_NO_MATH
+      if (alpha_p[0] == 12345.f)
+#endif
+      {
+      aq[(t + 3) % 4] = t + 3 < kSteps ? read_w(base, t + 3) : read_w(next, t + 3 - kSteps);
+      if (i < (TM + 1) / 2) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
           const int j = i * 2 + u;
-          if (j < TM) bq[(q + 1) & 1][j] = *(const uint4*)(base + cx0 + slot[q + 1] + j * 32 * kRowBytes);
+          if (j < TM && q < 3) bq[(q + 1) & 1][j] = read_x(base, q + 1, j);
         }
       }
+      if (t > kSync && i - 1 < (TM + 1) / 2) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int j = (i - 1) * 2 + u;
+          if (j < TM) bq[0][j] = read_x(next, 0, j);
+        }
+      }
+      if (t == kSteps - 1) {
+#pragma unroll
+        for (int j = 0; j < TM; ++j) raw_sb[j] = *(const uint2*)(next + sx0 + j * 32 * kScaleBytes);
+#pragma unroll
+        for (int i2 = 0; i2 < TN; ++i2) raw_sa[i2] = *(const uint2*)(next + sw0 + i2 * 32 * kScaleBytes);
+      }
       __builtin_amdgcn_sched_barrier(0);
-      const uint4 av = aq[t % 3];
+      const uint4 av = aq[t % 4];
       const v8i a = v8i{(int)av.x, (int)av.y, (int)av.z, (int)av.w, 0, 0, 0, 0};
 #pragma unroll
       for (int j = 0; j < TM; ++j) {
         const uint4 bv = bq[q & 1][j];
         const v8i b = v8i{(int)bv.x, (int)bv.y, (int)bv.z, (int)bv.w, 0, 0, 0, 0};
+#ifdef FPQ_EXP_NO_MFMA
+        if (j == i) acc[i][j][0] = __uint_as_float(__float_as_uint(acc[i][j][0]) ^ av.x ^ bv.w);
+#else
         if (q == 0) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], 4, 4, 0, sa[i], 0, sb[j]);
         if (q == 1) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], 4, 4, 1, sa[i], 1, sb[j]);
         if (q == 2) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], 4, 4, 2, sa[i], 2, sb[j]);
         if (q == 3) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], 4, 4, 3, sa[i], 3, sb[j]);
+#endif
+      }
       }
       __builtin_amdgcn_sched_barrier(0);
+#ifdef FPQ_GEMM_STAGE_REGS
+      // the next stage leaves the registers during the four steps before the barrier ...
+      if (t > kSync - 4 && t <= kSync && it + 1 < nk) {
+        FPQ_SPILL_REGS((it + 1) & 1, t - (kSync - 3), 4);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (t == kSync) {
+        __syncthreads();
+        if (it + 2 < nk) FPQ_FETCH_REGS((it + 2) * kKS);  // ... and the one after it enters them
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#else
+      if (t == kSync) {
+#ifdef FPQ_EXP_VMCNT
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(FPQ_EXP_VMCNT) : "memory");
+        __builtin_amdgcn_s_barrier();
+#else
+        wait_vmem();      // this wave's loads for the next stage have landed
+        __syncthreads();  // ... and everyone's; nobody reads the current stage any more
+#endif
+#ifndef FPQ_EXP_NO_DMA
+        if (it + 2 < nk) issue_loads(it & 1, (it + 2) * kKS);
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#endif
     }
   }
 
+#ifdef FPQ_EXP_TIMING
+  const uint64_t tc1 = __builtin_readcyclecounter(), tr1 = __builtin_amdgcn_s_memrealtime();
+#endif
   wave_quadrant_store<BN, BM, 2 * L::kStage, WM>(acc, smem, y, bias, alpha_p, n_blk, m_blk, wn, wm, wave, lane, M, N);
+#ifdef FPQ_EXP_TIMING
+  const uint64_t tc2 = __builtin_readcyclecounter(), tr2 = __builtin_amdgcn_s_memrealtime();
+  if (threadIdx.x == 0) {
+    uint64_t* d = (uint64_t*)y + (size_t)blockIdx.x * 8;
+    d[0] = tc0; d[1] = tc1; d[2] = tc2; d[3] = tr0; d[4] = tr1; d[5] = tr2;
+  }
+#endif
 }
 
 // 8 E2M1 codes (one dword) times one E4M3 scale -> 8 exact fp16 values.

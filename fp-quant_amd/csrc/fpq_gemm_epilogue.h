@@ -1,0 +1,89 @@
+// Pieces shared by the LDS-tiled GEMM kernels (gfx950 only): vector typedefs and the epilogue that
+// stages a wave's part of the output tile through LDS so that global stores are whole 256-byte rows.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fpq {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+typedef __attribute__((address_space(3))) void lds_void;
+typedef const __attribute__((address_space(1))) void global_void;
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+}
+
+// Epilogue of the LDS-tiled kernels.  Accumulator register v of 32x32 tile (i, j) is y[m][n] with
+// m = j*32 + r32 and n = i*32 + 8*(v/4) + 4*kh + v%4 inside the wave's quadrant of the workgroup
+// tile.  The quadrant goes through this wave's share of the (now idle) LDS as bf16 [m][n] so that
+// global stores are 256 contiguous bytes per row.
+template <int BN, int BM, int LDS_BYTES, int WM = 2>
+__device__ __forceinline__ void wave_quadrant_store(const v16f (&acc)[BN / 64][BM / (32 * WM)], uint8_t* smem,
+                                                    uint16_t* __restrict__ y,
+                                                    const uint16_t* __restrict__ bias,
+                                                    const float* __restrict__ alpha_p, int n_blk, int m_blk,
+                                                    int wn, int wm, int wave, int lane, int M, int N) {
+  constexpr int TN = BN / 64, TM = BM / (32 * WM);
+  const int r32 = lane & 31, kh = lane >> 5;
+  const float alpha = *alpha_p;
+#ifdef FPQ_EXP_NO_STORE
+  if (alpha != 12345.0f) return;
+#endif
+  constexpr int WT_N = BN / 2, WT_M = BM / WM;       // this wave's part of the workgroup tile
+  constexpr int kStride = WT_N * 2 + 16;             // bytes per staged row (+16: spread banks)
+  static_assert(2 * WM * WT_M * kStride <= LDS_BYTES, "epilogue staging does not fit in LDS");
+  __syncthreads();                                   // every wave is done reading operands
+  uint8_t* stg = smem + wave * (WT_M * kStride);
+  const int n0 = n_blk + wn * WT_N, m0 = m_blk + wm * WT_M;
+#pragma unroll
+  for (int i = 0; i < TN; ++i) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int nl = i * 32 + 8 * g + 4 * kh;
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (bias) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (n0 + nl + u < N) bv[u] = __uint_as_float((uint32_t)bias[n0 + nl + u] << 16);
+      }
+#pragma unroll
+      for (int j = 0; j < TM; ++j) {
+        uint32_t lo = pack_bf16x2(acc[i][j][4 * g + 0] * alpha, acc[i][j][4 * g + 1] * alpha);
+        uint32_t hi = pack_bf16x2(acc[i][j][4 * g + 2] * alpha, acc[i][j][4 * g + 3] * alpha);
+        if (bias) {
+          lo = pack_bf16x2(__uint_as_float(lo << 16) + bv[0], __uint_as_float(lo & 0xffff0000u) + bv[1]);
+          hi = pack_bf16x2(__uint_as_float(hi << 16) + bv[2], __uint_as_float(hi & 0xffff0000u) + bv[3]);
+        }
+        *(uint2*)(stg + (j * 32 + r32) * kStride + nl * 2) = make_uint2(lo, hi);
+      }
+    }
+  }
+  // read back: 16 lanes x 16 B cover one 256-byte row, 4 rows per wave instruction
+  const int rr = lane >> 4, cc = lane & 15;
+  const bool vec_ok = (N & 7) == 0;
+#pragma unroll 4
+  for (int p = 0; p < WT_M / 4; ++p) {
+    const int ml = p * 4 + rr;
+    const uint4 v = *(const uint4*)(stg + ml * kStride + cc * 16);
+    const int m = m0 + ml, n = n0 + cc * 8;
+    if (m >= M || n >= N) continue;
+    uint16_t* dst = y + (size_t)m * N + n;
+    if (vec_ok && n + 7 < N) {
+      *(uint4*)dst = v;
+    } else {
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (n + u < N) dst[u] = (uint16_t)(w[u >> 1] >> (16 * (u & 1)));
+    }
+  }
+}
+
+}  // namespace fpq

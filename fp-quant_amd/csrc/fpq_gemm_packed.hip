@@ -1,0 +1,340 @@
+// MXFP4 GEMM on operands re-tiled into the order the 32x32x64 block-scaled MFMA consumes them.
+//
+// Why a second layout.  With row-major codes a K slice of a 256x256 output tile is 512 separate
+// 128-byte row segments; the texture path of a CU moves such segments at about half the rate of
+// contiguous kilobytes, which makes operand fetch, not the matrix pipe, the limit of the
+// row-major kernel.  Here every 32-row x 64-K operand of one MFMA is one contiguous kilobyte in
+// memory, laid out lane by lane, so that
+//   * one direct global->LDS load instruction fetches exactly one operand (contiguous 1 KB),
+//   * the LDS image needs no swizzle: lane L reads its 16 bytes at block + 16 L (conflict-free),
+//   * any K granularity can be staged: the kernel keeps a ring of eight 64-K units in flight,
+//     enough to cover memory latency without stalling the matrix pipe.
+//
+// Packed codes   : block (rt, ks) = rows [32 rt, 32 rt + 32) x K [64 ks, 64 ks + 64) at byte
+//                  ((rt * K/64) + ks) * 1024; inside it lane L = 32 kh + r holds the 16 bytes
+//                  (32 codes) of row 32 rt + r, K [64 ks + 32 kh, +32)  -- one MX group.
+// Packed scales  : block (rt, kb) = the same rows x K [256 kb, 256 kb + 256) at byte
+//                  ((rt * K/256) + kb) * 256; lane L holds one dword whose byte q is the E8M0
+//                  scale of row 32 rt + r, group 8 kb + 2 q + kh  -- what MFMA number q of the
+//                  block takes through op_sel.
+// Rows are padded to a multiple of 32 with zero codes.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fpq.h"
+#include "fpq_device.h"
+#include "fpq_gemm_epilogue.h"
+
+namespace fpq {
+
+// ---------------------------------------------------------------------------------------------
+// Row-major -> packed.  One workgroup re-tiles 32 rows x 256 K: reads are 128-byte row segments,
+// writes cover 4 KB of codes and 256 B of scales contiguously.
+__global__ __launch_bounds__(256) void pack_mxf4_kernel(const uint8_t* __restrict__ codes,
+                                                        const uint8_t* __restrict__ scales,
+                                                        int64_t scale_stride, int rows, int K,
+                                                        uint8_t* __restrict__ pcodes,
+                                                        uint8_t* __restrict__ pscales) {
+  const int kb = blockIdx.x, rt = blockIdx.y;
+  const int t = threadIdx.x;
+  const int r = t >> 3, c = t & 7;  // row in the tile, 16-byte chunk of the 128-byte segment
+  const int row = rt * 32 + r;
+  uint4 v = make_uint4(0u, 0u, 0u, 0u);
+  if (row < rows) v = *(const uint4*)(codes + (size_t)row * (K >> 1) + kb * 128 + c * 16);
+  const int ks = kb * 4 + (c >> 1), kh = c & 1;
+  *(uint4*)(pcodes + (((size_t)rt * (K >> 6) + ks) * 64 + kh * 32 + r) * 16) = v;
+  if (t < 64) {
+    const int sr = t & 31, skh = t >> 5;
+    const int srow = rt * 32 + sr;
+    uint32_t out = 0u;
+    if (srow < rows) {
+      const uint8_t* sp = scales + (size_t)srow * scale_stride + kb * 8 + skh;
+      out = (uint32_t)sp[0] | ((uint32_t)sp[2] << 8) | ((uint32_t)sp[4] << 16) | ((uint32_t)sp[6] << 24);
+    }
+    *(uint32_t*)(pscales + (((size_t)rt * (K >> 8) + kb) * 64 + t) * 4) = out;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+constexpr int kRing = 8;                 // 64-K units resident or in flight
+constexpr int kUnitBytes = 16 * 1024;    // 8 weight + 8 activation operands of one unit
+constexpr int kScaleSlots = 4;           // 256-K scale blocks resident or in flight
+constexpr int kScaleSlotBytes = 16 * 256;
+constexpr int kPackedLds = kRing * kUnitBytes + kScaleSlots * kScaleSlotBytes;
+
+template <int N>
+__device__ __forceinline__ void wait_vmem_le() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// Workgroup barrier that orders LDS traffic only: this wave's LDS reads and writes are complete,
+// its outstanding global->LDS loads are NOT waited for (that is what wait_vmem_le is for).
+__device__ __forceinline__ void barrier_lds() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// 256 x 256 output tile per workgroup, WM = 2: four waves (2 x 2, 128 x 128 each), WM = 4: eight
+// waves (2 x 4, 128 x 64 each).
+template <int WM>
+__global__ __launch_bounds__(128 * WM) void gemm_mxf4_packed_kernel(
+    const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
+    const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p,
+    const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int tiles_m) {
+  constexpr int BN = 256, BM = 256;
+  constexpr int NW = 2 * WM;            // waves
+  constexpr int TN = 4, TM = 8 / WM;    // 32x32 MFMA tiles per wave along n and m
+  constexpr int kPer = 16 / NW;         // code loads per wave per unit
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
+  constexpr int kScaleBase = kRing * kUnitBytes;
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  // Consecutive workgroup ids land on different XCDs (8 of them, each with its own L2): give
+  // every XCD a contiguous run of the tile list so that its tiles share operand panels.
+  int logical = blockIdx.x;
+  {
+    const int nb = gridDim.x, per = nb / 8;
+    if (blockIdx.x < (unsigned)(per * 8)) logical = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+  }
+  const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
+  const int n_blk = tile_n * BN, m_blk = tile_m * BM;
+  const int wn = wave & 1, wm = wave >> 1;
+  const int nu = K >> 6, nkb = K >> 8;          // units, scale blocks
+  const int rt_n = (N + 31) >> 5, rt_m = (M + 31) >> 5;
+
+  // ---- loads.  Operand b of a unit: b < 8 weight row tile tile_n*8 + b, else activation row tile
+  // tile_m*8 + b - 8 (clamped at the edge: those rows are never stored).  Wave w loads operands
+  // w*kPer .. w*kPer + kPer - 1.
+  const uint8_t* op_base[kPer];
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int b = wave * kPer + j;
+    if (b < 8) {
+      const int rt = min(tile_n * 8 + b, rt_n - 1);
+      op_base[j] = wq + (size_t)rt * nu * 1024;
+    } else {
+      const int rt = min(tile_m * 8 + b - 8, rt_m - 1);
+      op_base[j] = xq + (size_t)rt * nu * 1024;
+    }
+  }
+  // Scale piece p (0..3) of a block: p < 2 weight row tiles 4p..4p+3, else activation row tiles
+  // 4(p-2)..; one load instruction, lane L fetches 16 bytes of row tile L / 16.
+  uint32_t sc_off_w[2], sc_off_x[2];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int rtw = min(tile_n * 8 + p * 4 + (lane >> 4), rt_n - 1);
+    const int rtx = min(tile_m * 8 + p * 4 + (lane >> 4), rt_m - 1);
+    sc_off_w[p] = (uint32_t)rtw * (uint32_t)nkb * 256u + (lane & 15) * 16;
+    sc_off_x[p] = (uint32_t)rtx * (uint32_t)nkb * 256u + (lane & 15) * 16;
+  }
+  const uint32_t lane16 = lane * 16;
+
+  static_assert(NW == 4, "one scale piece per wave");
+  const uint8_t* sc_base = wave < 2 ? ws : xs;
+  const uint32_t sc_off = wave < 2 ? sc_off_w[wave & 1] : sc_off_x[wave & 1];
+  // Unit u into its ring slot; with every fourth unit travel the scales of the block it opens
+  // (wave w brings piece w), issued first so that they have landed whenever the unit has.
+  auto issue_unit = [&](int u, bool with_scales) {
+    if (with_scales) {
+      const int blk = u >> 2;
+      lds_dma16(sc_base + (size_t)blk * 256, sc_off,
+                smem_base + kScaleBase + (blk % kScaleSlots) * kScaleSlotBytes + wave * 1024);
+    }
+    const uint32_t dst = smem_base + (u % kRing) * kUnitBytes + wave * kPer * 1024;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) lds_dma16(op_base[j] + (size_t)u * 1024, lane16, dst + j * 1024);
+  };
+
+  v16f acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  // operand registers of the current and the next unit; scales of the current block and, read
+  // ahead, of the next one
+  uint4 aq[2][TN], bq[2][TM];
+  int sa[TN], sb[TM], sa_next[TN], sb_next[TM];
+  const int a_off = (wn * 4) * 1024 + lane * 16, b_off = (8 + wm * TM) * 1024 + lane * 16;
+  const int sa_off = kScaleBase + (wn * 4) * 256 + lane * 4, sb_off = kScaleBase + (8 + wm * TM) * 256 + lane * 4;
+  auto read_unit = [&](int u, int set) {
+    const uint8_t* base = smem + (u % kRing) * kUnitBytes;
+#pragma unroll
+    for (int j = 0; j < TM; ++j) bq[set][j] = *(const uint4*)(base + b_off + j * 1024);
+#pragma unroll
+    for (int i = 0; i < TN; ++i) aq[set][i] = *(const uint4*)(base + a_off + i * 1024);
+  };
+  auto read_scales = [&](int blk) {
+    const uint8_t* base = smem + (blk % kScaleSlots) * kScaleSlotBytes;
+#pragma unroll
+    for (int j = 0; j < TM; ++j) sb_next[j] = *(const int*)(base + sb_off + j * 256);
+#pragma unroll
+    for (int i = 0; i < TN; ++i) sa_next[i] = *(const int*)(base + sa_off + i * 256);
+  };
+
+#ifdef FPQ_EXP_TIMING
+  const uint64_t tc0 = __builtin_readcyclecounter(), tr0 = __builtin_amdgcn_s_memrealtime();
+#endif
+  // ---- prologue: the first kRing units (scales of blocks 0 and 1 with units 0 and 4)
+  const int n_pro = min(nu, kRing);
+  for (int u = 0; u < n_pro; ++u) issue_unit(u, (u & 3) == 0);
+  // Loads complete in order: unit 0 and scale block 0 have landed once at most the loads of the
+  // younger units are outstanding (a wave issues kPer per unit, one more with scales).
+  if (n_pro == kRing) wait_vmem_le<(kRing - 1) * kPer>();
+  else wait_vmem();
+  barrier_lds();
+  read_unit(0, 0);
+  read_scales(0);
+
+  // One 64-K unit: 16 MFMAs per wave.  After the first row of MFMAs comes the hand-over: every
+  // wave holds unit u in registers, so its ring slot is free for unit u + kRing, and unit u + 1
+  // must have landed for everyone before it is read into the other register set.  The code
+  // between two hand-overs is branch-free (the compiler must not move MFMAs across them).
+#ifdef FPQ_EXP_NO_MATH
+#define FPQ_EXP_MATH_GUARD if (alpha_p[0] == 12345.f)
+#else
+#define FPQ_EXP_MATH_GUARD
+#endif
+#ifdef FPQ_EXP_NO_DMA
+#define FPQ_EXP_ISSUE false
+#else
+#define FPQ_EXP_ISSUE true
+#endif
+#define FPQ_MFMA_ROW(Q, I)                                                                          \
+  {                                                                                                 \
+    const uint4 av = aq[(Q) & 1][I];                                                                \
+    const v8i a = v8i{(int)av.x, (int)av.y, (int)av.z, (int)av.w, 0, 0, 0, 0};                      \
+    _Pragma("unroll") for (int j = 0; j < TM; ++j) {                                                \
+      const uint4 bv = bq[(Q) & 1][j];                                                              \
+      const v8i b = v8i{(int)bv.x, (int)bv.y, (int)bv.z, (int)bv.w, 0, 0, 0, 0};                    \
+      FPQ_EXP_MATH_GUARD                                                                            \
+      acc[I][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[I][j], 4, 4, Q, sa[I], \
+                                                                  Q, sb[j]);                        \
+    }                                                                                               \
+    __builtin_amdgcn_sched_barrier(0);                                                              \
+  }
+  // ALLOWED: loads of this wave that may still be outstanding while unit u + 1 is complete
+#define FPQ_UNIT(Q, U, ALLOWED, ISSUE, READ, READ_SCALES)                                           \
+  {                                                                                                 \
+    FPQ_MFMA_ROW(Q, 0)                                                                              \
+    wait_vmem_le<(ALLOWED)>();                                                                      \
+    barrier_lds();                                                                                  \
+    if (ISSUE) issue_unit((U) + kRing, (Q) == 0);                                                   \
+    if (READ) read_unit((U) + 1, ((Q) + 1) & 1);                                                    \
+    if (READ_SCALES) read_scales(((U) + 1) >> 2);                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                                              \
+    FPQ_MFMA_ROW(Q, 1)                                                                              \
+    FPQ_MFMA_ROW(Q, 2)                                                                              \
+    FPQ_MFMA_ROW(Q, 3)                                                                              \
+  }
+#define FPQ_TAKE_SCALES()                                                                           \
+  {                                                                                                 \
+    _Pragma("unroll") for (int i = 0; i < TN; ++i) sa[i] = sa_next[i];                              \
+    _Pragma("unroll") for (int j = 0; j < TM; ++j) sb[j] = sb_next[j];                              \
+  }
+
+  // steady state: every unit of these blocks still has a unit kRing ahead of it to issue
+  const int kb_tail = max(nkb - kRing / 4, 0);
+  for (int kb = 0; kb < kb_tail; ++kb) {
+    const int u0 = kb * 4;
+    FPQ_TAKE_SCALES()
+    FPQ_UNIT(0, u0 + 0, (kRing - 2) * kPer, FPQ_EXP_ISSUE, true, false)
+    FPQ_UNIT(1, u0 + 1, (kRing - 2) * kPer, FPQ_EXP_ISSUE, true, false)
+    FPQ_UNIT(2, u0 + 2, (kRing - 2) * kPer, FPQ_EXP_ISSUE, true, false)
+    FPQ_UNIT(3, u0 + 3, (kRing - 2) * kPer, FPQ_EXP_ISSUE, true, true)
+  }
+  // drain: the last kRing units (fewer if K is short); nothing is issued any more, and with t
+  // units to go after unit u + 1 exactly t * kPer loads may stay outstanding
+  if (nkb >= 2) {
+    const int u0 = (nkb - 2) * 4;
+    FPQ_TAKE_SCALES()
+    FPQ_UNIT(0, u0 + 0, 6 * kPer, false, true, false)
+    FPQ_UNIT(1, u0 + 1, 5 * kPer, false, true, false)
+    FPQ_UNIT(2, u0 + 2, 4 * kPer, false, true, false)
+    FPQ_UNIT(3, u0 + 3, 3 * kPer, false, true, true)
+  }
+  {
+    const int u0 = (nkb - 1) * 4;
+    FPQ_TAKE_SCALES()
+    FPQ_UNIT(0, u0 + 0, 2 * kPer, false, true, false)
+    FPQ_UNIT(1, u0 + 1, 1 * kPer, false, true, false)
+    FPQ_UNIT(2, u0 + 2, 0, false, true, false)
+    FPQ_UNIT(3, u0 + 3, 0, false, false, false)
+  }
+#undef FPQ_UNIT
+#undef FPQ_MFMA_ROW
+#undef FPQ_TAKE_SCALES
+
+#ifdef FPQ_EXP_TIMING
+  const uint64_t tc1 = __builtin_readcyclecounter(), tr1 = __builtin_amdgcn_s_memrealtime();
+#endif
+  wave_quadrant_store<BN, BM, kPackedLds, WM>(acc, smem, y, bias, alpha_p, n_blk, m_blk, wn, wm, wave, lane, M, N);
+#ifdef FPQ_EXP_TIMING
+  const uint64_t tc2 = __builtin_readcyclecounter(), tr2 = __builtin_amdgcn_s_memrealtime();
+  if (threadIdx.x == 0) {
+    uint64_t* d = (uint64_t*)y + (size_t)blockIdx.x * 8;
+    d[0] = tc0; d[1] = tc1; d[2] = tc2; d[3] = tr0; d[4] = tr1; d[5] = tr2;
+  }
+#endif
+}
+
+}  // namespace fpq
+
+extern "C" int64_t fpq_packed_codes_bytes(int64_t rows, int64_t K) {
+  return ((rows + 31) / 32) * 32 * (K / 2);
+}
+
+extern "C" int64_t fpq_packed_scales_bytes(int64_t rows, int64_t K) {
+  return ((rows + 31) / 32) * 32 * (K / 32);
+}
+
+extern "C" int fpq_pack_mxf4(const void* codes, const void* scales, int64_t scale_stride, int64_t rows,
+                             int64_t K, void* packed_codes, void* packed_scales, void* stream) {
+  if (rows < 0 || K < 0) return FPQ_E_SHAPE;
+  if (rows == 0) return FPQ_OK;
+  if (!codes || !scales || !packed_codes || !packed_scales) return FPQ_E_NULL;
+  if (K == 0 || K % 256 != 0 || scale_stride < K / 32) return FPQ_E_SHAPE;
+  if (rows > (1 << 24) || K > (1 << 24)) return FPQ_E_SHAPE;
+  if (((uintptr_t)codes & 15u) || ((uintptr_t)packed_codes & 15u) || ((uintptr_t)packed_scales & 3u))
+    return FPQ_E_ALIGN;
+  const dim3 grid((unsigned)(K / 256), (unsigned)((rows + 31) / 32));
+  hipLaunchKernelGGL(fpq::pack_mxf4_kernel, grid, dim3(256), 0, (hipStream_t)stream,
+                     (const uint8_t*)codes, (const uint8_t*)scales, scale_stride, (int)rows, (int)K,
+                     (uint8_t*)packed_codes, (uint8_t*)packed_scales);
+  return (int)hipGetLastError();
+}
+
+#ifndef FPQ_PACKED_WM
+#define FPQ_PACKED_WM 2
+#endif
+
+extern "C" int fpq_gemm_mxf4_packed(const void* xq, const void* xs, const void* wq, const void* ws,
+                                    const float* alpha, const void* bias, void* y, int64_t M,
+                                    int64_t N, int64_t K, void* stream) {
+  using namespace fpq;
+  if (M < 0 || N < 0 || K < 0) return FPQ_E_SHAPE;
+  if (M == 0 || N == 0) return FPQ_OK;
+  if (!xq || !xs || !wq || !ws || !alpha || !y) return FPQ_E_NULL;
+  if (K == 0 || K % 256 != 0) return FPQ_E_SHAPE;
+  if (M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return FPQ_E_SHAPE;
+  // scale offsets inside one operand are 32-bit
+  if (fpq_packed_scales_bytes(M, K) >= ((int64_t)1 << 32) || fpq_packed_scales_bytes(N, K) >= ((int64_t)1 << 32))
+    return FPQ_E_SHAPE;
+  if (((uintptr_t)xq & 15u) || ((uintptr_t)wq & 15u) || ((uintptr_t)xs & 15u) || ((uintptr_t)ws & 15u) ||
+      ((uintptr_t)y & 15u))
+    return FPQ_E_ALIGN;
+  const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mxf4_packed_kernel<FPQ_PACKED_WM>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kPackedLds);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((gemm_mxf4_packed_kernel<FPQ_PACKED_WM>), dim3((unsigned)(tiles_m * tiles_n)),
+                     dim3(128 * FPQ_PACKED_WM), kPackedLds, (hipStream_t)stream, (const uint8_t*)xq,
+                     (const uint8_t*)xs, (const uint8_t*)wq, (const uint8_t*)ws, alpha,
+                     (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K, tiles_m);
+  return (int)hipGetLastError();
+}
