@@ -8,6 +8,8 @@ rotation matrix is recognised once (Hadamard / identity / GSR) and applied as bu
 """
 from typing import Optional, Tuple
 
+import os
+
 import torch
 
 from .. import _engine
@@ -173,6 +175,43 @@ def _(x_flat, hadamard_matrix, global_scale):
 
 ### GEMMs
 
+# From this many activation rows on, the MXFP4 GEMM runs on operands re-tiled into the order the
+# matrix instructions consume them (bit-identical results, contiguous operand fetch).  The
+# re-tiled weights are made once per weight tensor and kept next to it, which doubles the memory
+# held by 4-bit weights; FPQ_PACKED_WEIGHTS=0 keeps every call on the row-major kernels.
+PACKED_MIN_M = 256
+
+
+def packed_weights_enabled() -> bool:
+    return os.environ.get("FPQ_PACKED_WEIGHTS", "1") != "0"
+
+
+def pack_mxf4(codes: torch.Tensor, scales: torch.Tensor, rows: int, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Row-major codes [rows, k/2] and E8M0 scales [>=rows, >=k/32] -> the packed layout of
+    fpq_gemm_mxf4_packed (rows padded to a multiple of 32)."""
+    lib = _engine.lib()
+    pc = torch.empty(lib.fpq_packed_codes_bytes(rows, k), dtype=torch.uint8, device=codes.device)
+    ps = torch.empty(lib.fpq_packed_scales_bytes(rows, k), dtype=torch.uint8, device=codes.device)
+    st = lib.fpq_pack_mxf4(codes.data_ptr(), scales.data_ptr(), scales.shape[1], rows, k,
+                           pc.data_ptr(), ps.data_ptr(), _stream(codes))
+    _engine.check(st, "fpq_pack_mxf4")
+    return pc, ps
+
+
+def packed_weight(wq: torch.Tensor, ws: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Packed copy of a weight, cached on the code tensor until either tensor is written to."""
+    key = (wq.data_ptr(), wq._version, ws.data_ptr(), ws._version, tuple(wq.shape))
+    hit = getattr(wq, "_fpq_packed", None)
+    if hit is not None and hit[0] == key:
+        return hit[1], hit[2]
+    pc, ps = pack_mxf4(wq, ws, wq.shape[0], wq.shape[1] * 2)
+    try:
+        wq._fpq_packed = (key, pc, ps)
+    except (AttributeError, RuntimeError):
+        pass
+    return pc, ps
+
+
 
 def _gemm(entry: str, x, w, xs, ws, alpha, bias: Optional[torch.Tensor], group: int) -> torch.Tensor:
     _require_cuda(x, w, xs, ws, alpha)
@@ -201,6 +240,15 @@ def _gemm(entry: str, x, w, xs, ws, alpha, bias: Optional[torch.Tensor], group: 
         bias = bias.contiguous()
         b_ptr = bias.data_ptr()
     a = alpha.contiguous()
+    if entry == "fpq_gemm_mxf4" and m >= PACKED_MIN_M and k % 256 == 0 and packed_weights_enabled():
+        with torch.cuda.device(x.device):
+            wp, wsp = packed_weight(wq, ws_b)
+            xp, xsp = pack_mxf4(xq, xs_b, m, k)
+            st = _engine.lib().fpq_gemm_mxf4_packed(
+                xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(), a.data_ptr(), b_ptr,
+                y.data_ptr(), m, n, k, _stream(x))
+        _engine.check(st, "fpq_gemm_mxf4_packed")
+        return y
     with torch.cuda.device(x.device):
         st = getattr(_engine.lib(), entry)(
             xq.data_ptr(), xs_b.data_ptr(), xs_b.shape[1], wq.data_ptr(), ws_b.data_ptr(),

@@ -100,6 +100,32 @@ int fpq_gemm_nvf4(const void* xq, const void* xs, int64_t xs_stride, const void*
                   void* y, int64_t M, int64_t N, int64_t K, void* stream);
 
 /*
+ * Packed MXFP4 operands: the codes and scales of a [rows, K] operand re-tiled into the order the
+ * 32x32x64 block-scaled matrix instruction consumes them, so that one operand of one instruction
+ * is one contiguous kilobyte (K % 256 == 0; rows padded to a multiple of 32 with zero codes):
+ *   codes   block (rt, ks) = rows [32 rt, +32) x K [64 ks, +64) at byte (rt * K/64 + ks) * 1024;
+ *           16 bytes at (32 kh + r) * 16 inside it = row 32 rt + r, K [64 ks + 32 kh, +32)
+ *   scales  block (rt, kb) = the same rows x K [256 kb, +256) at byte (rt * K/256 + kb) * 256;
+ *           byte q of the dword at (32 kh + r) * 4 = E8M0 scale of row 32 rt + r, group 8 kb + 2 q + kh
+ * This is the counterpart of the scale re-tiling the reference performs with to_blocked() before
+ * every CUTLASS GEMM (qutlass_ops.py:111-146), extended to the codes; it is done once per weight.
+ * fpq_packed_*_bytes return the buffer sizes; fpq_pack_mxf4 converts from the row-major layout of
+ * fpq_quantize_mx (codes 16-byte aligned; packed buffers 16-byte aligned).
+ */
+int64_t fpq_packed_codes_bytes(int64_t rows, int64_t K);
+int64_t fpq_packed_scales_bytes(int64_t rows, int64_t K);
+int fpq_pack_mxf4(const void* codes, const void* scales, int64_t scale_stride, int64_t rows,
+                  int64_t K, void* packed_codes, void* packed_scales, void* stream);
+
+/*
+ * fpq_gemm_mxf4 on packed operands (same arithmetic, bit-identical y): the kernel for large M.
+ * Stands in for qutlass.matmul_mxf4_bf16_tn (qutlass_ops.py:111-128) like fpq_gemm_mxf4.
+ */
+int fpq_gemm_mxf4_packed(const void* xq_packed, const void* xs_packed, const void* wq_packed,
+                         const void* ws_packed, const float* alpha, const void* bias, void* y,
+                         int64_t M, int64_t N, int64_t K, void* stream);
+
+/*
  * Test hook: E2M1 codes of n fp32 values exactly as the quantize kernels round them
  * (out[i] in 0..15, one byte per value).  Used to check the device rounding exhaustively.
  */
