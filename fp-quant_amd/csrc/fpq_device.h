@@ -158,18 +158,7 @@ __device__ __forceinline__ float scale_element(float x, const GroupScale& g) {
 // inline assembly so that the compiler does not serialise every later LDS read behind them;
 // completion is awaited explicitly with wait_vmem().  Nothing else in these kernels uses M0.
 __device__ __forceinline__ void lds_dma16(const uint8_t* gbase, uint32_t voff, uint32_t lds_base) {
-#if FPQ_EXP_DMA_SEL == 1
-#define FPQ_EXP_DMA_MOD " nt"
-#elif FPQ_EXP_DMA_SEL == 2
-#define FPQ_EXP_DMA_MOD " sc0"
-#elif FPQ_EXP_DMA_SEL == 3
-#define FPQ_EXP_DMA_MOD " sc1"
-#elif FPQ_EXP_DMA_SEL == 4
-#define FPQ_EXP_DMA_MOD " sc0 sc1"
-#else
-#define FPQ_EXP_DMA_MOD ""
-#endif
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" FPQ_EXP_DMA_MOD
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
                :: "s"(lds_base), "v"(voff), "s"(gbase) : "memory");
 }
 // Same, marked non-temporal: for data that is read exactly once (streaming kernels).

@@ -324,21 +324,13 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_lds_kernel(
   for (int j = 0; j < kInstrW; ++j) {
     const int idx = wave * kInstrW + j;
     const int row = min(n_blk + idx * 8 + lrow, N - 1);
-#ifdef FPQ_EXP_LINEAR_CHUNKS
-    w_off[j] = (uint32_t)row * (uint32_t)kbytes + ((lane & 7) * 16);
-#else
     w_off[j] = (uint32_t)row * (uint32_t)kbytes + (((lane & 7) ^ lrow ^ (idx & 1)) * 16);
-#endif
   }
 #pragma unroll
   for (int j = 0; j < kInstrX; ++j) {
     const int idx = wave * kInstrX + j;
     const int row = min(m_blk + idx * 8 + lrow, M - 1);
-#ifdef FPQ_EXP_LINEAR_CHUNKS
-    x_off[j] = (uint32_t)row * (uint32_t)kbytes + ((lane & 7) * 16);
-#else
     x_off[j] = (uint32_t)row * (uint32_t)kbytes + (((lane & 7) ^ lrow ^ (idx & 1)) * 16);
-#endif
   }
   // Scales: one wave instruction moves 32 rows x 8 B (two dwords per row); wave w takes
   // instructions j with j % NW == w.
@@ -368,51 +360,14 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_lds_kernel(
 #pragma unroll
     for (int j = 0; j < kInstrX; ++j)
       lds_dma16(xk, x_off[j], base + L::kCodesX + (wave * kInstrX + j) * 1024);
-#ifndef FPQ_EXP_NO_SCALE_DMA
 #pragma unroll
     for (int j = 0; j < kSW; ++j)
       if (j * NW + wave < kSInstrW) lds_dma4(wsk, ws_off[j], base + L::kScalesW + (j * NW + wave) * 256);
 #pragma unroll
     for (int j = 0; j < kSX; ++j)
       if (j * NW + wave < kSInstrX) lds_dma4(xsk, xs_off[j], base + L::kScalesX + (j * NW + wave) * 256);
-#endif
   };
 
-#ifdef FPQ_GEMM_STAGE_REGS
-  // Alternative operand path: global -> registers -> ds_write (same LDS image as the direct loads).
-  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-  u32x4 w_reg[kInstrW], x_reg[kInstrX];
-  uint32_t ws_reg[kSW], xs_reg[kSX];
-#define FPQ_FETCH_REGS(k0_)                                                                     \
-  {                                                                                             \
-    const int k0__ = (k0_);                                                                     \
-    _Pragma("unroll") for (int j = 0; j < kInstrW; ++j)                                         \
-        w_reg[j] = *(const u32x4*)(wq + (k0__ >> 1) + w_off[j]);                                \
-    _Pragma("unroll") for (int j = 0; j < kInstrX; ++j)                                         \
-        x_reg[j] = *(const u32x4*)(xq + (k0__ >> 1) + x_off[j]);                                \
-    _Pragma("unroll") for (int j = 0; j < kSW; ++j)                                             \
-        ws_reg[j] = *(const uint32_t*)(ws + (k0__ >> 5) + ws_off[j]);                           \
-    _Pragma("unroll") for (int j = 0; j < kSX; ++j)                                             \
-        xs_reg[j] = *(const uint32_t*)(xs + (k0__ >> 5) + xs_off[j]);                           \
-  }
-#define FPQ_SPILL_REGS(stage_, part_, parts_)                                                   \
-  {                                                                                             \
-    uint8_t* sb__ = smem + (stage_) * L::kStage;                                                \
-    _Pragma("unroll") for (int j = 0; j < kInstrW; ++j)                                         \
-        if (j % (parts_) == (part_))                                                            \
-            *(u32x4*)(sb__ + L::kCodesW + (wave * kInstrW + j) * 1024 + lane * 16) = w_reg[j];  \
-    _Pragma("unroll") for (int j = 0; j < kInstrX; ++j)                                         \
-        if (j % (parts_) == (part_))                                                            \
-            *(u32x4*)(sb__ + L::kCodesX + (wave * kInstrX + j) * 1024 + lane * 16) = x_reg[j];  \
-    if ((part_) == (parts_) - 1) {                                                              \
-      _Pragma("unroll") for (int j = 0; j < kSW; ++j)                                           \
-          *(uint32_t*)(sb__ + L::kScalesW + (j * NW + wave) * 256 + lane * 4) = ws_reg[j];      \
-      _Pragma("unroll") for (int j = 0; j < kSX; ++j)                                           \
-          *(uint32_t*)(sb__ + L::kScalesX + (j * NW + wave) * 256 + lane * 4) = xs_reg[j];      \
-    }                                                                                           \
-  }
-  static_assert(kSInstrW % NW == 0 && kSInstrX % NW == 0, "scale loads must divide over the waves");
-#endif
 
   // 32x32x64 MFMA: lane = (row r32 = lane % 32, K half kh = lane / 32); one stage holds four
   // K steps q of 64, the lane's 16-byte chunk in step q is c = 2q + kh, its scale byte is c too.
@@ -435,9 +390,6 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_lds_kernel(
   const uint32_t perm_sel = kh ? 0x07050301u : 0x06040200u;
 
   const int nk = K / kKS;
-#ifdef FPQ_EXP_TIMING
-  const uint64_t tc0 = __builtin_readcyclecounter(), tr0 = __builtin_amdgcn_s_memrealtime();
-#endif
   // Operand stream of a stage: 4 K steps x TN weight tiles (16 "steps"), each tile used by TM
   // MFMAs.  Weight tiles are read from LDS three steps ahead (ring of 4), the activation tiles
   // of the next K step during the first steps of the current one.  The one barrier of an
@@ -456,19 +408,10 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_lds_kernel(
     return *(const uint4*)(b + cx0 + slot[q] + j * 32 * kRowBytes);
   };
 
-#ifdef FPQ_GEMM_STAGE_REGS
-  FPQ_FETCH_REGS(0);
-  FPQ_SPILL_REGS(0, 0, 1);
-  if (nk > 1) FPQ_FETCH_REGS(kKS);
-  __syncthreads();
-#else
   issue_loads(0, 0);
-#ifndef FPQ_EXP_NO_DMA
   if (nk > 1) issue_loads(1, kKS);
-#endif
   wait_vmem();
   __syncthreads();
-#endif
 #pragma unroll
   for (int j = 0; j < TM; ++j) bq[0][j] = read_x(smem, 0, j);
 #pragma unroll
@@ -490,10 +433,6 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_lds_kernel(
 #pragma unroll
     for (int t = 0; t < kSteps; ++t) {
       const int q = t / TN, i = t % TN;
-#ifdef FPQ_EXP_NO_MATH
-      if (alpha_p[0] == 12345.f)
-#endif
-      {
       aq[(t + 3) % 4] = t + 3 < kSteps ? read_w(base, t + 3) : read_w(next, t + 3 - kSteps);
       if (i < (TM + 1) / 2) {
 #pragma unroll
@@ -522,57 +461,22 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_lds_kernel(
       for (int j = 0; j < TM; ++j) {
         const uint4 bv = bq[q & 1][j];
         const v8i b = v8i{(int)bv.x, (int)bv.y, (int)bv.z, (int)bv.w, 0, 0, 0, 0};
-#ifdef FPQ_EXP_NO_MFMA
-        if (j == i) acc[i][j][0] = __uint_as_float(__float_as_uint(acc[i][j][0]) ^ av.x ^ bv.w);
-#else
         if (q == 0) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], 4, 4, 0, sa[i], 0, sb[j]);
         if (q == 1) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], 4, 4, 1, sa[i], 1, sb[j]);
         if (q == 2) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], 4, 4, 2, sa[i], 2, sb[j]);
         if (q == 3) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[i][j], 4, 4, 3, sa[i], 3, sb[j]);
-#endif
-      }
       }
       __builtin_amdgcn_sched_barrier(0);
-#ifdef FPQ_GEMM_STAGE_REGS
-      // the next stage leaves the registers during the four steps before the barrier ...
-      if (t > kSync - 4 && t <= kSync && it + 1 < nk) {
-        FPQ_SPILL_REGS((it + 1) & 1, t - (kSync - 3), 4);
-        __builtin_amdgcn_sched_barrier(0);
-      }
       if (t == kSync) {
-        __syncthreads();
-        if (it + 2 < nk) FPQ_FETCH_REGS((it + 2) * kKS);  // ... and the one after it enters them
-        __builtin_amdgcn_sched_barrier(0);
-      }
-#else
-      if (t == kSync) {
-#ifdef FPQ_EXP_VMCNT
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(FPQ_EXP_VMCNT) : "memory");
-        __builtin_amdgcn_s_barrier();
-#else
         wait_vmem();      // this wave's loads for the next stage have landed
         __syncthreads();  // ... and everyone's; nobody reads the current stage any more
-#endif
-#ifndef FPQ_EXP_NO_DMA
         if (it + 2 < nk) issue_loads(it & 1, (it + 2) * kKS);
-#endif
         __builtin_amdgcn_sched_barrier(0);
       }
-#endif
     }
   }
 
-#ifdef FPQ_EXP_TIMING
-  const uint64_t tc1 = __builtin_readcyclecounter(), tr1 = __builtin_amdgcn_s_memrealtime();
-#endif
   wave_quadrant_store<BN, BM, 2 * L::kStage, WM>(acc, smem, y, bias, alpha_p, n_blk, m_blk, wn, wm, wave, lane, M, N);
-#ifdef FPQ_EXP_TIMING
-  const uint64_t tc2 = __builtin_readcyclecounter(), tr2 = __builtin_amdgcn_s_memrealtime();
-  if (threadIdx.x == 0) {
-    uint64_t* d = (uint64_t*)y + (size_t)blockIdx.x * 8;
-    d[0] = tc0; d[1] = tc1; d[2] = tc2; d[3] = tr0; d[4] = tr1; d[5] = tr2;
-  }
-#endif
 }
 
 // 8 E2M1 codes (one dword) times one E4M3 scale -> 8 exact fp16 values.

@@ -20,28 +20,24 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
 }
 
-// Epilogue of the LDS-tiled kernels.  Accumulator register v of 32x32 tile (i, j) is y[m][n] with
-// m = j*32 + r32 and n = i*32 + 8*(v/4) + 4*kh + v%4 inside the wave's quadrant of the workgroup
-// tile.  The quadrant goes through this wave's share of the (now idle) LDS as bf16 [m][n] so that
-// global stores are 256 contiguous bytes per row.
-template <int BN, int BM, int LDS_BYTES, int WM = 2>
-__device__ __forceinline__ void wave_quadrant_store(const v16f (&acc)[BN / 64][BM / (32 * WM)], uint8_t* smem,
-                                                    uint16_t* __restrict__ y,
-                                                    const uint16_t* __restrict__ bias,
-                                                    const float* __restrict__ alpha_p, int n_blk, int m_blk,
-                                                    int wn, int wm, int wave, int lane, int M, int N) {
-  constexpr int TN = BN / 64, TM = BM / (32 * WM);
+// Epilogue of the LDS-tiled kernels.  A wave owns TN x TM accumulator tiles of 32 x 32; register
+// v of tile (i, j) is y[m][n] with m = j*32 + r32 and n = i*32 + 8*(v/4) + 4*kh + v%4 relative to
+// the wave's origin (m0, n0).  The wave's part goes through its share of the (now idle) LDS as
+// bf16 [m][n] so that global stores are whole contiguous rows of TN*64 bytes.
+template <int TN, int TM, int LDS_BYTES, int NWAVES>
+__device__ __forceinline__ void wave_tile_store(const v16f (&acc)[TN][TM], uint8_t* smem,
+                                                uint16_t* __restrict__ y,
+                                                const uint16_t* __restrict__ bias,
+                                                const float* __restrict__ alpha_p, int n0, int m0,
+                                                int wave, int lane, int M, int N) {
   const int r32 = lane & 31, kh = lane >> 5;
   const float alpha = *alpha_p;
-#ifdef FPQ_EXP_NO_STORE
-  if (alpha != 12345.0f) return;
-#endif
-  constexpr int WT_N = BN / 2, WT_M = BM / WM;       // this wave's part of the workgroup tile
-  constexpr int kStride = WT_N * 2 + 16;             // bytes per staged row (+16: spread banks)
-  static_assert(2 * WM * WT_M * kStride <= LDS_BYTES, "epilogue staging does not fit in LDS");
+  constexpr int WT_N = TN * 32, WT_M = TM * 32;      // this wave's part of the workgroup tile
+  constexpr int kRowBytes = WT_N * 2;
+  constexpr int kStride = kRowBytes + 16;            // bytes per staged row (+16: spread banks)
+  static_assert(NWAVES * WT_M * kStride <= LDS_BYTES, "epilogue staging does not fit in LDS");
   __syncthreads();                                   // every wave is done reading operands
   uint8_t* stg = smem + wave * (WT_M * kStride);
-  const int n0 = n_blk + wn * WT_N, m0 = m_blk + wm * WT_M;
 #pragma unroll
   for (int i = 0; i < TN; ++i) {
 #pragma unroll
@@ -65,12 +61,16 @@ __device__ __forceinline__ void wave_quadrant_store(const v16f (&acc)[BN / 64][B
       }
     }
   }
-  // read back: 16 lanes x 16 B cover one 256-byte row, 4 rows per wave instruction
-  const int rr = lane >> 4, cc = lane & 15;
+  // read back: kLpr lanes x 16 B cover one row, 64 / kLpr rows per wave instruction
+  constexpr int kLpr = kRowBytes / 16 <= 16 ? 16 : 32;
+  constexpr int kRpi = 64 / kLpr;
+  static_assert(kRowBytes / 16 <= 32 && WT_M % kRpi == 0, "unsupported wave tile shape");
+  const int rr = lane / kLpr, cc = lane % kLpr;
   const bool vec_ok = (N & 7) == 0;
 #pragma unroll 4
-  for (int p = 0; p < WT_M / 4; ++p) {
-    const int ml = p * 4 + rr;
+  for (int p = 0; p < WT_M / kRpi; ++p) {
+    const int ml = p * kRpi + rr;
+    if (cc * 16 >= kRowBytes) continue;
     const uint4 v = *(const uint4*)(stg + ml * kStride + cc * 16);
     const int m = m0 + ml, n = n0 + cc * 8;
     if (m >= M || n >= N) continue;
@@ -84,6 +84,17 @@ __device__ __forceinline__ void wave_quadrant_store(const v16f (&acc)[BN / 64][B
         if (n + u < N) dst[u] = (uint16_t)(w[u >> 1] >> (16 * (u & 1)));
     }
   }
+}
+
+// The 2 x WM wave arrangement of the row-major kernels: wave (wn, wm) owns the BN/2 x BM/WM part.
+template <int BN, int BM, int LDS_BYTES, int WM = 2>
+__device__ __forceinline__ void wave_quadrant_store(const v16f (&acc)[BN / 64][BM / (32 * WM)], uint8_t* smem,
+                                                    uint16_t* __restrict__ y,
+                                                    const uint16_t* __restrict__ bias,
+                                                    const float* __restrict__ alpha_p, int n_blk, int m_blk,
+                                                    int wn, int wm, int wave, int lane, int M, int N) {
+  wave_tile_store<BN / 64, BM / (32 * WM), LDS_BYTES, 2 * WM>(acc, smem, y, bias, alpha_p, n_blk + wn * (BN / 2),
+                                                              m_blk + wm * (BM / WM), wave, lane, M, N);
 }
 
 }  // namespace fpq

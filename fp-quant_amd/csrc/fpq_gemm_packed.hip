@@ -72,16 +72,20 @@ __device__ __forceinline__ void barrier_lds() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-// 256 x 256 output tile per workgroup, WM = 2: four waves (2 x 2, 128 x 128 each), WM = 4: eight
-// waves (2 x 4, 128 x 64 each).
-template <int WM>
-__global__ __launch_bounds__(128 * WM) void gemm_mxf4_packed_kernel(
+// One workgroup of four waves (WN x WM) computes a tile of NT*32 weight rows (n) x 256 activation
+// rows (m); a wave owns TN x TM accumulator tiles of 32 x 32.  Built as <8, 2, 2>: a 256 x 256
+// tile, waves 128 x 128.  (<7, 1, 4>, 224 x 256 tiles that fill two whole rounds of 256 CUs at
+// N = 14336, works and measured the same time: the kernel runs at the matrix pipes' power
+// limit, not at their issue limit, so fuller rounds buy nothing.)
+template <int NT, int WN, int WM>
+__global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int tiles_m) {
-  constexpr int BN = 256, BM = 256;
-  constexpr int NW = 2 * WM;            // waves
-  constexpr int TN = 4, TM = 8 / WM;    // 32x32 MFMA tiles per wave along n and m
+  constexpr int BN = NT * 32, BM = 256;
+  constexpr int NW = WN * WM;           // waves
+  static_assert(NW == 4 && NT <= 8 && NT % WN == 0 && 8 % WM == 0, "unsupported wave arrangement");
+  constexpr int TN = NT / WN, TM = 8 / WM;  // 32x32 MFMA tiles per wave along n and m
   constexpr int kPer = 16 / NW;         // code loads per wave per unit
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
@@ -89,7 +93,9 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_packed_kernel(
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   // Consecutive workgroup ids land on different XCDs (8 of them, each with its own L2): give
-  // every XCD a contiguous run of the tile list so that its tiles share operand panels.
+  // every XCD a contiguous run of the tile list so that its tiles share operand panels.  (One
+  // workgroup per tile: a persistent variant that walked several tiles per CU measured slower,
+  // the hardware's own dispatch balances the XCDs better.)
   int logical = blockIdx.x;
   {
     const int nb = gridDim.x, per = nb / 8;
@@ -97,19 +103,20 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_packed_kernel(
   }
   const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
   const int n_blk = tile_n * BN, m_blk = tile_m * BM;
-  const int wn = wave & 1, wm = wave >> 1;
+  const int wn = wave % WN, wm = wave / WN;
   const int nu = K >> 6, nkb = K >> 8;          // units, scale blocks
   const int rt_n = (N + 31) >> 5, rt_m = (M + 31) >> 5;
 
-  // ---- loads.  Operand b of a unit: b < 8 weight row tile tile_n*8 + b, else activation row tile
-  // tile_m*8 + b - 8 (clamped at the edge: those rows are never stored).  Wave w loads operands
-  // w*kPer .. w*kPer + kPer - 1.
+  // ---- loads.  Operand b of a unit: b < 8 weight row tile tile_n*NT + b, else activation row tile
+  // tile_m*8 + b - 8 (clamped at the edge: those rows are never stored; with NT = 7 the eighth
+  // weight row tile is loaded and not used, which keeps every wave's load count the same).
+  // Wave w loads operands w*kPer .. w*kPer + kPer - 1.
   const uint8_t* op_base[kPer];
 #pragma unroll
   for (int j = 0; j < kPer; ++j) {
     const int b = wave * kPer + j;
     if (b < 8) {
-      const int rt = min(tile_n * 8 + b, rt_n - 1);
+      const int rt = min(tile_n * NT + b, rt_n - 1);
       op_base[j] = wq + (size_t)rt * nu * 1024;
     } else {
       const int rt = min(tile_m * 8 + b - 8, rt_m - 1);
@@ -121,7 +128,7 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_packed_kernel(
   uint32_t sc_off_w[2], sc_off_x[2];
 #pragma unroll
   for (int p = 0; p < 2; ++p) {
-    const int rtw = min(tile_n * 8 + p * 4 + (lane >> 4), rt_n - 1);
+    const int rtw = min(tile_n * NT + p * 4 + (lane >> 4), rt_n - 1);
     const int rtx = min(tile_m * 8 + p * 4 + (lane >> 4), rt_m - 1);
     sc_off_w[p] = (uint32_t)rtw * (uint32_t)nkb * 256u + (lane & 15) * 16;
     sc_off_x[p] = (uint32_t)rtx * (uint32_t)nkb * 256u + (lane & 15) * 16;
@@ -156,8 +163,8 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_packed_kernel(
   // ahead, of the next one
   uint4 aq[2][TN], bq[2][TM];
   int sa[TN], sb[TM], sa_next[TN], sb_next[TM];
-  const int a_off = (wn * 4) * 1024 + lane * 16, b_off = (8 + wm * TM) * 1024 + lane * 16;
-  const int sa_off = kScaleBase + (wn * 4) * 256 + lane * 4, sb_off = kScaleBase + (8 + wm * TM) * 256 + lane * 4;
+  const int a_off = (wn * TN) * 1024 + lane * 16, b_off = (8 + wm * TM) * 1024 + lane * 16;
+  const int sa_off = kScaleBase + (wn * TN) * 256 + lane * 4, sb_off = kScaleBase + (8 + wm * TM) * 256 + lane * 4;
   auto read_unit = [&](int u, int set) {
     const uint8_t* base = smem + (u % kRing) * kUnitBytes;
 #pragma unroll
@@ -173,9 +180,6 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_packed_kernel(
     for (int i = 0; i < TN; ++i) sa_next[i] = *(const int*)(base + sa_off + i * 256);
   };
 
-#ifdef FPQ_EXP_TIMING
-  const uint64_t tc0 = __builtin_readcyclecounter(), tr0 = __builtin_amdgcn_s_memrealtime();
-#endif
   // ---- prologue: the first kRing units (scales of blocks 0 and 1 with units 0 and 4)
   const int n_pro = min(nu, kRing);
   for (int u = 0; u < n_pro; ++u) issue_unit(u, (u & 3) == 0);
@@ -191,16 +195,6 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_packed_kernel(
   // wave holds unit u in registers, so its ring slot is free for unit u + kRing, and unit u + 1
   // must have landed for everyone before it is read into the other register set.  The code
   // between two hand-overs is branch-free (the compiler must not move MFMAs across them).
-#ifdef FPQ_EXP_NO_MATH
-#define FPQ_EXP_MATH_GUARD if (alpha_p[0] == 12345.f)
-#else
-#define FPQ_EXP_MATH_GUARD
-#endif
-#ifdef FPQ_EXP_NO_DMA
-#define FPQ_EXP_ISSUE false
-#else
-#define FPQ_EXP_ISSUE true
-#endif
 #define FPQ_MFMA_ROW(Q, I)                                                                          \
   {                                                                                                 \
     const uint4 av = aq[(Q) & 1][I];                                                                \
@@ -208,25 +202,23 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_packed_kernel(
     _Pragma("unroll") for (int j = 0; j < TM; ++j) {                                                \
       const uint4 bv = bq[(Q) & 1][j];                                                              \
       const v8i b = v8i{(int)bv.x, (int)bv.y, (int)bv.z, (int)bv.w, 0, 0, 0, 0};                    \
-      FPQ_EXP_MATH_GUARD                                                                            \
       acc[I][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[I][j], 4, 4, Q, sa[I], \
                                                                   Q, sb[j]);                        \
     }                                                                                               \
     __builtin_amdgcn_sched_barrier(0);                                                              \
   }
+  constexpr int kHand = TM >= 4 ? 1 : 2;  // rows of MFMAs (4 instructions) ahead of the hand-over
   // ALLOWED: loads of this wave that may still be outstanding while unit u + 1 is complete
 #define FPQ_UNIT(Q, U, ALLOWED, ISSUE, READ, READ_SCALES)                                           \
   {                                                                                                 \
-    FPQ_MFMA_ROW(Q, 0)                                                                              \
+    _Pragma("unroll") for (int i0 = 0; i0 < kHand; ++i0) FPQ_MFMA_ROW(Q, i0)                        \
     wait_vmem_le<(ALLOWED)>();                                                                      \
     barrier_lds();                                                                                  \
     if (ISSUE) issue_unit((U) + kRing, (Q) == 0);                                                   \
     if (READ) read_unit((U) + 1, ((Q) + 1) & 1);                                                    \
     if (READ_SCALES) read_scales(((U) + 1) >> 2);                                                   \
     __builtin_amdgcn_sched_barrier(0);                                                              \
-    FPQ_MFMA_ROW(Q, 1)                                                                              \
-    FPQ_MFMA_ROW(Q, 2)                                                                              \
-    FPQ_MFMA_ROW(Q, 3)                                                                              \
+    _Pragma("unroll") for (int i1 = kHand; i1 < TN; ++i1) FPQ_MFMA_ROW(Q, i1)                       \
   }
 #define FPQ_TAKE_SCALES()                                                                           \
   {                                                                                                 \
@@ -239,10 +231,10 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_packed_kernel(
   for (int kb = 0; kb < kb_tail; ++kb) {
     const int u0 = kb * 4;
     FPQ_TAKE_SCALES()
-    FPQ_UNIT(0, u0 + 0, (kRing - 2) * kPer, FPQ_EXP_ISSUE, true, false)
-    FPQ_UNIT(1, u0 + 1, (kRing - 2) * kPer, FPQ_EXP_ISSUE, true, false)
-    FPQ_UNIT(2, u0 + 2, (kRing - 2) * kPer, FPQ_EXP_ISSUE, true, false)
-    FPQ_UNIT(3, u0 + 3, (kRing - 2) * kPer, FPQ_EXP_ISSUE, true, true)
+    FPQ_UNIT(0, u0 + 0, (kRing - 2) * kPer, true, true, false)
+    FPQ_UNIT(1, u0 + 1, (kRing - 2) * kPer, true, true, false)
+    FPQ_UNIT(2, u0 + 2, (kRing - 2) * kPer, true, true, false)
+    FPQ_UNIT(3, u0 + 3, (kRing - 2) * kPer, true, true, true)
   }
   // drain: the last kRing units (fewer if K is short); nothing is issued any more, and with t
   // units to go after unit u + 1 exactly t * kPer loads may stay outstanding
@@ -266,17 +258,8 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_packed_kernel(
 #undef FPQ_MFMA_ROW
 #undef FPQ_TAKE_SCALES
 
-#ifdef FPQ_EXP_TIMING
-  const uint64_t tc1 = __builtin_readcyclecounter(), tr1 = __builtin_amdgcn_s_memrealtime();
-#endif
-  wave_quadrant_store<BN, BM, kPackedLds, WM>(acc, smem, y, bias, alpha_p, n_blk, m_blk, wn, wm, wave, lane, M, N);
-#ifdef FPQ_EXP_TIMING
-  const uint64_t tc2 = __builtin_readcyclecounter(), tr2 = __builtin_amdgcn_s_memrealtime();
-  if (threadIdx.x == 0) {
-    uint64_t* d = (uint64_t*)y + (size_t)blockIdx.x * 8;
-    d[0] = tc0; d[1] = tc1; d[2] = tc2; d[3] = tr0; d[4] = tr1; d[5] = tr2;
-  }
-#endif
+  wave_tile_store<TN, TM, kPackedLds, NW>(acc, smem, y, bias, alpha_p, n_blk + wn * TN * 32, m_blk + wm * TM * 32,
+                                          wave, lane, M, N);
 }
 
 }  // namespace fpq
@@ -305,9 +288,25 @@ extern "C" int fpq_pack_mxf4(const void* codes, const void* scales, int64_t scal
   return (int)hipGetLastError();
 }
 
-#ifndef FPQ_PACKED_WM
-#define FPQ_PACKED_WM 2
-#endif
+namespace fpq {
+template <int NT, int WN, int WM>
+static int launch_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
+                         const void* bias, void* y, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
+  const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + NT * 32 - 1) / (NT * 32));
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mxf4_packed_kernel<NT, WN, WM>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kPackedLds);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((gemm_mxf4_packed_kernel<NT, WN, WM>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256),
+                     kPackedLds, stream, (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq,
+                     (const uint8_t*)ws, alpha, (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K,
+                     tiles_m);
+  return (int)hipGetLastError();
+}
+}  // namespace fpq
 
 extern "C" int fpq_gemm_mxf4_packed(const void* xq, const void* xs, const void* wq, const void* ws,
                                     const float* alpha, const void* bias, void* y, int64_t M,
@@ -324,17 +323,5 @@ extern "C" int fpq_gemm_mxf4_packed(const void* xq, const void* xs, const void* 
   if (((uintptr_t)xq & 15u) || ((uintptr_t)wq & 15u) || ((uintptr_t)xs & 15u) || ((uintptr_t)ws & 15u) ||
       ((uintptr_t)y & 15u))
     return FPQ_E_ALIGN;
-  const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_mxf4_packed_kernel<FPQ_PACKED_WM>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kPackedLds);
-    if (e != hipSuccess) return (int)e;
-    attr_set = true;
-  }
-  hipLaunchKernelGGL((gemm_mxf4_packed_kernel<FPQ_PACKED_WM>), dim3((unsigned)(tiles_m * tiles_n)),
-                     dim3(128 * FPQ_PACKED_WM), kPackedLds, (hipStream_t)stream, (const uint8_t*)xq,
-                     (const uint8_t*)xs, (const uint8_t*)wq, (const uint8_t*)ws, alpha,
-                     (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K, tiles_m);
-  return (int)hipGetLastError();
+  return launch_packed<8, 2, 2>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
 }
