@@ -132,6 +132,32 @@ def bench_linear(torch, fmt, m, n, k, g, steps, warmup, seed):
     gemm = lib.fpq_gemm_mxf4 if fmt == "mxfp4" else lib.fpq_gemm_nvf4
     p = [(xs_[i].data_ptr(), xq[i].data_ptr(), xsc[i].data_ptr(), ys[i].data_ptr()) for i in range(n_buf)]
 
+    from fp_quant.module import hip_ops
+    if fmt == "mxfp4" and hip_ops.packed_linear_eligible(m, k, "abs_max"):
+        # what FPQuantLinear.forward runs for this many rows: activations quantized straight into the
+        # packed operand layout, weights re-tiled once (outside the timed region, like their quantization)
+        wp, wsp = hip_ops.pack_mxf4(wq, ws, n, k)
+        xp = [torch.empty(lib.fpq_packed_codes_bytes(m, k), dtype=torch.uint8, device=dev) for _ in range(n_buf)]
+        xsp = [torch.empty(lib.fpq_packed_scales_bytes(m, k), dtype=torch.uint8, device=dev) for _ in range(n_buf)]
+        pp = [(xs_[i].data_ptr(), xp[i].data_ptr(), xsp[i].data_ptr(), ys[i].data_ptr()) for i in range(n_buf)]
+
+        def run_linear(i):
+            a, b, c, d = pp[i]
+            st = lib.fpq_quantize_mx_packed(a, m, k, 0, g, norm, b, c, 0, stream)
+            st = st or lib.fpq_gemm_mxf4_packed(b, c, wp.data_ptr(), wsp.data_ptr(), alpha.data_ptr(), None,
+                                                d, m, n, k, stream)
+            if st != 0:
+                _engine.check(st, "bench packed linear")
+
+        def run_gemm(i):
+            a, b, c, d = pp[i]
+            st = lib.fpq_gemm_mxf4_packed(b, c, wp.data_ptr(), wsp.data_ptr(), alpha.data_ptr(), None,
+                                          d, m, n, k, stream)
+            if st != 0:
+                _engine.check(st, "bench packed gemm")
+
+        return _time_linear(torch, run_linear, run_gemm, fmt, m, n, k, g, group, n_buf, steps, warmup, "packed")
+
     def run_linear(i):
         a, b, c, d = p[i]
         st = quant(a, m, b, c)
@@ -147,6 +173,10 @@ def bench_linear(torch, fmt, m, n, k, g, steps, warmup, seed):
         if st != 0:
             _engine.check(st, "bench gemm")
 
+    return _time_linear(torch, run_linear, run_gemm, fmt, m, n, k, g, group, n_buf, steps, warmup, "row-major")
+
+
+def _time_linear(torch, run_linear, run_gemm, fmt, m, n, k, g, group, n_buf, steps, warmup, layout):
     wall, ev = time_kernel(torch, run_linear, n_buf, steps, warmup)
     _, ev_gemm = time_kernel(torch, run_gemm, n_buf, steps, warmup)
     flops = 2.0 * m * n * k
@@ -162,6 +192,7 @@ def bench_linear(torch, fmt, m, n, k, g, steps, warmup, seed):
         "gemm_tflops": flops / (ev_gemm * 1e-3) / 1e12,
         "gemm_gbps": gemm_bytes / (ev_gemm * 1e-3) / 1e9,
         "buffers": n_buf,
+        "operand_layout": layout,
     }
 
 

@@ -224,11 +224,18 @@ __device__ __forceinline__ uint32_t fix_zero_nibbles(uint32_t w) {
   return w;
 }
 
-template <int EPL, int G, int FMT, int ROT, int ZERO>
+//
+// PACKED (MXFP4, EPL = 64 only) writes the operand layout of fpq_gemm_mxf4_packed instead of
+// row-major codes and scales.  A wave tile is then 32 rows x two neighbouring chunks (lane =
+// 2 * row + chunk, so the lane pairing of a 128-wide rotation is unchanged): the loads are 256-byte
+// row segments, and every 16-byte half of a lane's codes is exactly one lane slot of a packed
+// kilobyte block, so codes are stored straight from registers in two 512-byte runs per store.
+template <int EPL, int G, int FMT, int ROT, int ZERO, bool PACKED = false>
 __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
     const uint8_t* __restrict__ x, uint8_t* __restrict__ codes, uint8_t* __restrict__ scales,
     uint32_t n_chunks, uint32_t chunks_per_row, uint32_t rows, uint32_t scale_rows,
     uint32_t scale_stride, float norm, const float* __restrict__ global_scale) {
+  static_assert(!PACKED || (FMT == kFmtMx && EPL == 64), "packed output: MXFP4 with 64-element chunks");
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
   constexpr int NG = EPL / GROUP;        // groups (= scale bytes) per chunk
   constexpr int PIECES = EPL / 8;        // 16-byte input pieces per chunk
@@ -272,30 +279,45 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
   auto sw = [](uint32_t b) -> uint32_t { return PIECES == 8 ? ((b & 7u) ^ ((b >> 3) & 1u)) : (b % PIECES); };
   const uint32_t b_lo = lane / PIECES, j_lo = lane % PIECES;
   constexpr int NV_OFF = PIECES == 8 ? 2 : 4;  // distinct swizzle phases over the instruction index
+  const uint32_t row_bytes = chunks_per_row * CB;
+  // PACKED: chunk b of the tile is row b / 2 of the row tile, chunk b % 2 of the pair
+  const uint32_t b_off = PACKED ? (b_lo >> 1) * row_bytes + (b_lo & 1u) * CB : b_lo * CB;
   uint32_t voff[NV_OFF];
 #pragma unroll
-  for (int m = 0; m < NV_OFF; ++m) voff[m] = b_lo * CB + ((j_lo ^ sw(CPI * m + b_lo)) * 16u);
+  for (int m = 0; m < NV_OFF; ++m) voff[m] = b_off + ((j_lo ^ sw(CPI * m + b_lo)) * 16u);
   const uint32_t rd_base = lane * CB, l_sw = sw(lane);
 
-  const uint32_t n_tiles = (n_chunks + 63u) / 64u;
+  const uint32_t pairs = chunks_per_row / 2u;  // PACKED: tiles per row tile
+  const uint32_t n_tiles = PACKED ? ((rows + 31u) / 32u) * pairs : (n_chunks + 63u) / 64u;
   const uint32_t total_waves = gridDim.x * 4u;
   for (uint32_t tile = blockIdx.x * 4u + wave; tile < n_tiles; tile += total_waves) {
-    const uint32_t valid = min(64u, n_chunks - tile * 64u);
-    const uint8_t* src = x + (size_t)tile * TILE;
+    const uint32_t rt = PACKED ? tile / pairs : 0u, pr = PACKED ? tile - rt * pairs : 0u;
+    // chunks (row-major) or rows (PACKED) of this tile that exist
+    const uint32_t valid = PACKED ? min(32u, rows - rt * 32u) : min(64u, n_chunks - tile * 64u);
+    const uint8_t* src = PACKED ? x + ((size_t)rt * 32u * chunks_per_row + 2u * pr) * CB
+                                : x + (size_t)tile * TILE;
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
       // The lane offset is an unsigned 32-bit addend to a scalar base, so it must never be
       // negative.  Chunks past the end of the tensor re-read valid bytes instead: the first
       // chunk of this instruction if that one is valid, else the first chunk of the tile.
       uint32_t off = voff[i % NV_OFF];
-      const bool instr_valid = (uint32_t)(CPI * i) < valid;                // wave-uniform
-      const uint8_t* base_i = instr_valid ? src + i * 1024 : src;          // scalar address arithmetic
-      if (CPI * i + b_lo >= valid) off = j_lo * 16u;
-      lds_dma16_nt(base_i, off, my_base + i * 1024u);  // read once: keep it out of the caches
+      if (PACKED) {
+        const bool instr_valid = (uint32_t)(CPI / 2 * i) < valid;          // wave-uniform
+        const uint8_t* base_i = instr_valid ? src + (size_t)(CPI / 2 * i) * row_bytes : src;
+        if (CPI / 2 * i + (b_lo >> 1) >= valid) off = (b_lo & 1u) * CB + j_lo * 16u;
+        lds_dma16_nt(base_i, off, my_base + i * 1024u);
+      } else {
+        const bool instr_valid = (uint32_t)(CPI * i) < valid;                // wave-uniform
+        const uint8_t* base_i = instr_valid ? src + i * 1024 : src;          // scalar address arithmetic
+        if (CPI * i + b_lo >= valid) off = j_lo * 16u;
+        lds_dma16_nt(base_i, off, my_base + i * 1024u);  // read once: keep it out of the caches
+      }
     }
     wait_vmem();
 
-    float v[EPL];
+    // this lane's chunk: out of LDS, rotated
+    auto load_rotate = [&](float (&v)[EPL]) {
 #pragma unroll
     for (int k = 0; k < PIECES; ++k) {
       const uint4 raw = *(const uint4*)(my + rd_base + ((k ^ l_sw) * 16u));
@@ -342,6 +364,9 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
 #pragma unroll
       for (int k = 0; k < EPL; ++k) v[k] = w[k];
     }
+    };
+    float v[EPL];
+    load_rotate(v);
 
     uint32_t cw[CW];
     uint32_t sbytes = 0u, sb_lo = 0u;
@@ -404,6 +429,57 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
       __builtin_amdgcn_sched_barrier(0);
     }
 
+    if constexpr (PACKED) {
+      // Scale exponents outside the fast range (tiny or huge values): redo the tile with the
+      // generic per-element arithmetic; the input is still in LDS.
+      if (__builtin_amdgcn_ballot_w64(need_slow) != 0ull) {
+        float u[EPL];
+        load_rotate(u);
+        sbytes = 0u;
+#pragma unroll 1
+        for (int gi = 0; gi < NG; ++gi) {
+          float a = 0.0f;
+#pragma unroll
+          for (int i = 0; i < GROUP; ++i) a = __builtin_fmaxf(a, __builtin_fabsf(u[gi * GROUP + i]));
+          const GroupScale g = mx_group_scale(a);
+#pragma unroll
+          for (int d = 0; d < GROUP / 8; ++d) {
+            uint32_t w = 0u;
+#pragma unroll
+            for (int h = 0; h < 8; ++h) {
+              const float xv = u[gi * GROUP + d * 8 + h];
+              float q = scale_element(xv, g);
+              if (ZERO == kZeroSigned) q = __builtin_copysignf(q, xv);
+              w |= e2m1_code<ZERO>(q) << (4 * h);
+            }
+            cw[gi * (GROUP / 8) + d] = w;
+          }
+          sbytes |= (g.byte & 0xffu) << (8 * gi);
+        }
+      }
+      const uint32_t r = lane >> 1, ksl = lane & 1u;
+      const bool row_ok = r < valid;
+      if (!row_ok) {  // padding rows of the last row tile: zero codes, zero scale bytes
+#pragma unroll
+        for (int k = 0; k < CW; ++k) cw[k] = 0u;
+        sbytes = 0u;
+      }
+      const uint32_t ks = 2u * pr + ksl;
+      uint8_t* blk = codes + (((size_t)rt * chunks_per_row + ks) * 64u + r) * 16u;
+      *(uint4*)blk = make_uint4(cw[0], cw[1], cw[2], cw[3]);                // K half 0
+      *(uint4*)(blk + 512) = make_uint4(cw[4], cw[5], cw[6], cw[7]);        // K half 1
+      // scale bytes: byte (ks % 4) of dword (kh, r) in block (rt, ks / 4).  The pair of lanes
+      // of a row holds bytes q and q + 1 of both dwords: the even lane stores the half-word of
+      // K half 0, the odd lane that of K half 1.
+      const uint32_t other = (uint32_t)__builtin_amdgcn_mov_dpp((int)sbytes, 0xB1, 0xF, 0xF, true);
+      const uint32_t hw = ksl == 0u ? ((sbytes & 0xffu) | ((other & 0xffu) << 8))
+                                    : (((other >> 8) & 0xffu) | (sbytes & 0xff00u));
+      uint8_t* sblk = scales + ((size_t)rt * (chunks_per_row / 4u) + (pr >> 1)) * 256u;
+      *(uint16_t*)(sblk + (ksl * 32u + r) * 4u + 2u * (pr & 1u)) = (uint16_t)hw;
+      asm volatile("" ::: "memory");
+      continue;
+    }
+
     // codes: lane-major runs -> LDS (16-byte pieces swizzled so 8 neighbouring lanes hit 8
     // different bank groups) -> contiguous rows
 #pragma unroll
@@ -458,7 +534,7 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
     }
     asm volatile("" ::: "memory");
   }
-  fill_scale_padding(scales, rows, chunks_per_row * NG, scale_rows, scale_stride);
+  if (!PACKED) fill_scale_padding(scales, rows, chunks_per_row * NG, scale_rows, scale_stride);
 }
 
 template <int EPL, int G, int FMT, int ROT>
@@ -481,6 +557,63 @@ static int launch_stream(const void* x, int64_t rows, int64_t cols, float norm, 
     go(quantize_stream_kernel<EPL, G, FMT, ROT, kZeroSigned>);
   }
   return (int)hipGetLastError();
+}
+
+template <int G, int ROT>
+static int launch_stream_packed(const void* x, int64_t rows, int64_t cols, float norm, void* codes,
+                                void* scales, int zero_policy, hipStream_t stream) {
+  const int64_t n_tiles = ((rows + 31) / 32) * (cols / 128);
+  int64_t blocks = (n_tiles + 3) / 4;
+  if (blocks > 1024) blocks = 1024;
+  const dim3 grid((unsigned)blocks), block(256);
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint8_t*)x, (uint8_t*)codes,
+                       (uint8_t*)scales, (uint32_t)(rows * cols / 64), (uint32_t)(cols / 64),
+                       (uint32_t)rows, 0u, 0u, norm, (const float*)nullptr);
+  };
+  if (zero_policy == FPQ_ZERO_REFERENCE) {
+    go(quantize_stream_kernel<64, G, kFmtMx, ROT, kZeroReference, true>);
+  } else {
+    go(quantize_stream_kernel<64, G, kFmtMx, ROT, kZeroSigned, true>);
+  }
+  return (int)hipGetLastError();
+}
+
+static int dispatch_packed(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                           void* codes, void* scales, int zero_policy, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (rows < 0 || cols < 0) return FPQ_E_SHAPE;
+  if (rows == 0 || cols == 0) return FPQ_OK;
+  if (!x || !codes || !scales) return FPQ_E_NULL;
+  if (zero_policy != FPQ_ZERO_REFERENCE && zero_policy != FPQ_ZERO_SIGNED) return FPQ_E_POLICY;
+  if (rot_kind == FPQ_ROT_IDENTITY) g = 32;
+  if (g != 16 && g != 32 && g != 64 && g != 128) return FPQ_E_ROTATION;
+  if (cols % 256 != 0) return FPQ_E_SHAPE;
+  if (rows * cols >= (int64_t)1 << 34) return FPQ_E_SHAPE;
+  if (((uintptr_t)x & 15u) || ((uintptr_t)codes & 15u) || ((uintptr_t)scales & 3u)) return FPQ_E_ALIGN;
+#define FPQ_LAUNCH_PACKED(GG, RR) \
+  return launch_stream_packed<GG, RR>(x, rows, cols, norm, codes, scales, zero_policy, stream)
+  if (rot_kind == FPQ_ROT_IDENTITY) {
+    FPQ_LAUNCH_PACKED(32, FPQ_ROT_IDENTITY);
+  } else if (rot_kind == FPQ_ROT_HADAMARD) {
+    switch (g) {
+      case 16: FPQ_LAUNCH_PACKED(16, FPQ_ROT_HADAMARD);
+      case 32: FPQ_LAUNCH_PACKED(32, FPQ_ROT_HADAMARD);
+      case 64: FPQ_LAUNCH_PACKED(64, FPQ_ROT_HADAMARD);
+      case 128: FPQ_LAUNCH_PACKED(128, FPQ_ROT_HADAMARD);
+    }
+  } else if (rot_kind == FPQ_ROT_GSR) {
+    switch (g) {
+      case 16: FPQ_LAUNCH_PACKED(16, FPQ_ROT_GSR);
+      case 32: FPQ_LAUNCH_PACKED(32, FPQ_ROT_GSR);
+      case 64: FPQ_LAUNCH_PACKED(64, FPQ_ROT_GSR);
+    }
+    return FPQ_E_UNSUPPORTED;  // a 128-wide sequency-ordered block spans two lanes
+  } else if (rot_kind == FPQ_ROT_GENERAL) {
+    return FPQ_E_UNSUPPORTED;    // arbitrary matrices: quantize row-major, then fpq_pack_mxf4
+  }
+#undef FPQ_LAUNCH_PACKED
+  return FPQ_E_ROTATION;
 }
 
 template <int FMT>
@@ -558,6 +691,13 @@ extern "C" int fpq_quantize_mx(const void* x, int64_t rows, int64_t cols, int ro
                                void* stream) {
   return fpq::dispatch<fpq::kFmtMx>(x, rows, cols, rot_kind, g, norm, h, nullptr, codes, scales,
                                     scale_rows, scale_stride, zero_policy, stream);
+}
+
+extern "C" int fpq_quantize_mx_packed(const void* x, int64_t rows, int64_t cols, int rot_kind, int g,
+                                      float norm, void* packed_codes, void* packed_scales,
+                                      int zero_policy, void* stream) {
+  return fpq::dispatch_packed(x, rows, cols, rot_kind, g, norm, packed_codes, packed_scales, zero_policy,
+                              stream);
 }
 
 extern "C" int fpq_quantize_nv(const void* x, int64_t rows, int64_t cols, int rot_kind, int g,

@@ -14,6 +14,7 @@ _lib = None
 
 ROT_HADAMARD, ROT_IDENTITY, ROT_GSR, ROT_GENERAL = 0, 1, 2, 3
 ZERO_REFERENCE, ZERO_SIGNED = 0, 1
+E_UNSUPPORTED = -6
 
 _P, _I64, _I, _F = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
 
@@ -29,6 +30,7 @@ _SIGNATURES = {
     "fpq_packed_codes_bytes": ([_I64, _I64], _I64),
     "fpq_packed_scales_bytes": ([_I64, _I64], _I64),
     "fpq_pack_mxf4": ([_P, _P, _I64, _I64, _I64, _P, _P, _P], _I),
+    "fpq_quantize_mx_packed": ([_P, _I64, _I64, _I, _I, _F, _P, _P, _I, _P], _I),
     "fpq_gemm_mxf4_packed": ([_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _I),
 }
 

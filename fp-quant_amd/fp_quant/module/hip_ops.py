@@ -92,6 +92,72 @@ def _padded(rows: int, groups: int) -> Tuple[int, int]:
 ### Forward quantization
 
 
+def quantize_mx_packed(x: torch.Tensor, hadamard_matrix: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """abs_max MXFP4 quantization of bf16 [rows, cols] straight into the packed GEMM layout
+    (cols % 256 == 0).  Rotations the packed quantizer has no kernel for go through the row-major
+    quantizer and the re-tiling kernel."""
+    lib = _engine.lib()
+    rows, cols = x.shape
+    kind, norm = classify_rotation(hadamard_matrix)
+    g = hadamard_matrix.shape[0]
+    pc = torch.empty(lib.fpq_packed_codes_bytes(rows, cols), dtype=torch.uint8, device=x.device)
+    ps = torch.empty(lib.fpq_packed_scales_bytes(rows, cols), dtype=torch.uint8, device=x.device)
+    st = lib.fpq_quantize_mx_packed(x.data_ptr(), rows, cols, kind, g, norm, pc.data_ptr(), ps.data_ptr(),
+                                    ZERO_NIBBLE_POLICY, _stream(x))
+    if st == _engine.E_UNSUPPORTED:
+        codes, scales, _ = fused_quantize_mx_op(x, hadamard_matrix, "abs_max", False)
+        return pack_mxf4(codes, scales.view(torch.uint8), rows, cols)
+    _engine.check(st, "fpq_quantize_mx_packed")
+    return pc, ps
+
+
+def packed_linear_eligible(rows: int, k: int, forward_method: str) -> bool:
+    return forward_method == "abs_max" and rows >= PACKED_LINEAR_MIN_M and k % 256 == 0 and packed_weights_enabled()
+
+
+@torch.library.custom_op("fp_quant::linear_mxf4_packed_op", mutates_args=())
+def linear_mxf4_packed_op(
+    x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, w: torch.Tensor, ws: torch.Tensor,
+    alpha: torch.Tensor, bias: Optional[torch.Tensor],
+) -> torch.Tensor:
+    """Activation rotate+quantize and W4A4 GEMM of one MXFP4 linear on packed operands: the same
+    codes, scales and output bits as fused_quantize_mx_op followed by matmul_mxf4_bf16_tn_op."""
+    _require_cuda(x_flat, hadamard_matrix, w, ws, alpha)
+    if x_flat.dtype != torch.bfloat16 or x_flat.dim() != 2:
+        raise ValueError("x_flat must be a 2-D bfloat16 tensor")
+    if alpha.dtype != torch.float32 or alpha.numel() != 1:
+        raise ValueError("alpha must be a one-element float32 tensor")
+    x = x_flat.contiguous()
+    m, k = x.shape
+    wq = w.contiguous()
+    n = wq.shape[0]
+    if wq.dtype != torch.uint8 or wq.shape[1] * 2 != k:
+        raise ValueError(f"inner dimensions differ: x has K={k}, w has K={wq.shape[1] * 2}")
+    ws_b = ws.contiguous().view(torch.uint8)
+    b_ptr = None
+    if bias is not None:
+        if bias.dtype != torch.bfloat16 or bias.numel() != n:
+            raise ValueError("bias must be a bfloat16 vector of length N")
+        bias = bias.contiguous()
+        b_ptr = bias.data_ptr()
+    y = torch.empty(m, n, dtype=torch.bfloat16, device=x.device)
+    a = alpha.contiguous()
+    with torch.cuda.device(x.device):
+        xp, xsp = quantize_mx_packed(x, hadamard_matrix)
+        wp, wsp = packed_weight(wq, ws_b)
+        st = _engine.lib().fpq_gemm_mxf4_packed(
+            xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(), a.data_ptr(), b_ptr,
+            y.data_ptr(), m, n, k, _stream(x))
+    _engine.check(st, "fpq_gemm_mxf4_packed")
+    return y
+
+
+@linear_mxf4_packed_op.register_fake
+def _(x_flat, hadamard_matrix, w, ws, alpha, bias):
+    return torch.empty(x_flat.size(0), w.size(0), dtype=torch.bfloat16, device=x_flat.device)
+
+
+
 @torch.library.custom_op("fp_quant::fused_quantize_mx_op", mutates_args=())
 def fused_quantize_mx_op(
     x_flat: torch.Tensor,
@@ -179,7 +245,8 @@ def _(x_flat, hadamard_matrix, global_scale):
 # matrix instructions consume them (bit-identical results, contiguous operand fetch).  The
 # re-tiled weights are made once per weight tensor and kept next to it, which doubles the memory
 # held by 4-bit weights; FPQ_PACKED_WEIGHTS=0 keeps every call on the row-major kernels.
-PACKED_MIN_M = 256
+PACKED_MIN_M = 256         # GEMM operator on row-major operands (pays for re-tiling the activations)
+PACKED_LINEAR_MIN_M = 65   # fused linear: activations are quantized straight into the packed layout
 
 
 def packed_weights_enabled() -> bool:

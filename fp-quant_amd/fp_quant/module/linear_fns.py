@@ -18,6 +18,8 @@ from .hip_ops import (
     matmul_mxf4_bf16_tn_op,
     matmul_nvf4_bf16_tn_bias_op,
     matmul_nvf4_bf16_tn_op,
+    linear_mxf4_packed_op,
+    packed_linear_eligible,
 )
 
 
@@ -69,6 +71,17 @@ class FPQuant4x16NoMasterFn(Function):
         forward_method: str,
     ):
         x_flat = x.contiguous().flatten(end_dim=-2)
+        if (dtype == FPQuantDtype.MXFP4 and x_flat.is_cuda
+                and packed_linear_eligible(x_flat.shape[0], x_flat.shape[1], forward_method)):
+            # large batches: quantize and multiply on operands in the matrix units' own order
+            alpha = 1.0 / (weight_global_scale * act_global_scale)
+            fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16) else None
+            y = linear_mxf4_packed_op(x_flat.to(torch.bfloat16), as_bf16(forward_hadamard_matrix), weight_q,
+                                      weight_scales, alpha.float(), fused_bias)
+            y = y.unflatten(dim=0, sizes=x.shape[:-1])
+            if bias is not None and fused_bias is None:
+                y += bias
+            return y
         x_q, x_scales, _ = forward_quantize(
             x_flat, forward_hadamard_matrix, act_global_scale, dtype, forward_method
         )

@@ -118,6 +118,16 @@ int fpq_pack_mxf4(const void* codes, const void* scales, int64_t scale_stride, i
                   int64_t K, void* packed_codes, void* packed_scales, void* stream);
 
 /*
+ * fpq_quantize_mx writing the packed layout directly (same codes and scale bytes; rows past
+ * `rows` in the last 32-row tile get zero codes and zero scale bytes).  cols % 256 == 0;
+ * Hadamard 16..128, identity and sequency-ordered Hadamard up to 64 wide; other rotations return
+ * FPQ_E_UNSUPPORTED (quantize row-major and call fpq_pack_mxf4).  Same reference counterpart as
+ * fpq_quantize_mx (qutlass_ops.py:36-71).
+ */
+int fpq_quantize_mx_packed(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                           void* packed_codes, void* packed_scales, int zero_policy, void* stream);
+
+/*
  * fpq_gemm_mxf4 on packed operands (same arithmetic, bit-identical y): the kernel for large M.
  * Stands in for qutlass.matmul_mxf4_bf16_tn (qutlass_ops.py:111-128) like fpq_gemm_mxf4.
  */

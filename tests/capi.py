@@ -57,3 +57,55 @@ def gemm(xq, xs, wq, ws, alpha, fmt, bias=None):
     _engine.check(st, "fpq_gemm")
     torch.cuda.synchronize()
     return y.cpu()
+
+
+def packed_sizes(rows, k):
+    lib = _engine.lib()
+    return lib.fpq_packed_codes_bytes(rows, k), lib.fpq_packed_scales_bytes(rows, k)
+
+
+def pack(codes, scales, fill=0xCD):
+    """fpq_pack_mxf4 on row-major codes [R, K/2] and E8M0 scales [>=R, >=K/32]; CPU uint8 results."""
+    lib = _engine.lib()
+    codes, scales = codes.to("cuda").contiguous(), scales.to("cuda").contiguous()
+    rows, k = codes.shape[0], codes.shape[1] * 2
+    nc, ns = packed_sizes(rows, k)
+    pc = torch.full((nc,), fill, dtype=torch.uint8, device="cuda")
+    ps = torch.full((ns,), fill, dtype=torch.uint8, device="cuda")
+    st = lib.fpq_pack_mxf4(codes.data_ptr(), scales.data_ptr(), scales.shape[1], rows, k, pc.data_ptr(),
+                           ps.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_pack_mxf4")
+    torch.cuda.synchronize()
+    return pc.cpu(), ps.cpu()
+
+
+def quantize_packed(x_bf16, rot="hadamard", g=128, norm=None, zero_policy=_engine.ZERO_REFERENCE, fill=0xCD):
+    """fpq_quantize_mx_packed; CPU uint8 (packed codes, packed scales)."""
+    lib = _engine.lib()
+    x = x_bf16.to("cuda").contiguous()
+    rows, cols = x.shape
+    nc, ns = packed_sizes(rows, cols)
+    pc = torch.full((nc,), fill, dtype=torch.uint8, device="cuda")
+    ps = torch.full((ns,), fill, dtype=torch.uint8, device="cuda")
+    if norm is None:
+        norm = float(torch.tensor(g ** -0.5, dtype=torch.bfloat16))
+    st = lib.fpq_quantize_mx_packed(x.data_ptr(), rows, cols, ROT[rot], g, norm, pc.data_ptr(), ps.data_ptr(),
+                                    zero_policy, torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_quantize_mx_packed")
+    torch.cuda.synchronize()
+    return pc.cpu(), ps.cpu()
+
+
+def gemm_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=None):
+    """fpq_gemm_mxf4_packed on packed operands; bf16 [M, N] on the CPU."""
+    lib = _engine.lib()
+    xp, xsp, wp, wsp = (t.to("cuda").contiguous() for t in (xp, xsp, wp, wsp))
+    y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    a = torch.tensor([alpha], dtype=torch.float32, device="cuda")
+    b = bias.to("cuda").contiguous() if bias is not None else None
+    st = lib.fpq_gemm_mxf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(), a.data_ptr(),
+                                  b.data_ptr() if b is not None else None, y.data_ptr(), m, n, k,
+                                  torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_gemm_mxf4_packed")
+    torch.cuda.synchronize()
+    return y.cpu()

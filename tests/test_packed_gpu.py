@@ -1,0 +1,138 @@
+"""Packed MXFP4 operand layout: the re-tiling kernel, the quantizer that writes it directly and
+the GEMM that reads it, each against an index-level restatement of the layout and the oracle."""
+import pytest
+import torch
+
+from oracle import fpq_oracle as O
+from fp_quant import _engine
+import capi
+from conftest import make_outlier_normal
+
+pytestmark = pytest.mark.gpu
+
+
+def pack_by_definition(codes, scales, k):
+    """The layout as include/fpq.h states it, written with reshapes (rows padded with zeros):
+    codes  [(rt, ks), (kh, r), 16 bytes] = row 32 rt + r, bytes 32 ks + 16 kh ...
+    scales [(rt, kb), (kh, r), q]        = row 32 rt + r, group 8 kb + 2 q + kh"""
+    rows = codes.shape[0]
+    rt = (rows + 31) // 32
+    c = torch.zeros(rt * 32, k // 2, dtype=torch.uint8)
+    c[:rows] = codes[:, : k // 2]
+    s = torch.zeros(rt * 32, k // 32, dtype=torch.uint8)
+    s[:rows] = scales[:rows, : k // 32]
+    pc = c.view(rt, 32, k // 64, 2, 16).permute(0, 2, 3, 1, 4).contiguous().view(-1)
+    ps = s.view(rt, 32, k // 256, 4, 2).permute(0, 2, 4, 1, 3).contiguous().view(-1)
+    return pc, ps
+
+
+@pytest.mark.parametrize("rows,k", [(32, 256), (64, 512), (33, 256), (100, 1024), (257, 768)])
+def test_pack_kernel_matches_definition(rows, k):
+    g = torch.Generator().manual_seed(rows + k)
+    codes = torch.randint(0, 256, (rows, k // 2), dtype=torch.uint8, generator=g)
+    scales = torch.randint(0, 256, (rows + 3, k // 32 + 4), dtype=torch.uint8, generator=g)  # padded tensor
+    pc, ps = capi.pack(codes, scales)
+    wc, ws = pack_by_definition(codes, scales, k)
+    assert torch.equal(pc, wc)
+    assert torch.equal(ps, ws)
+
+
+def test_pack_rejects():
+    codes = torch.zeros(32, 64, dtype=torch.uint8)
+    scales = torch.zeros(32, 4, dtype=torch.uint8)
+    with pytest.raises(ValueError):
+        capi.pack(codes, scales)  # K = 128 is not a multiple of 256
+
+
+CASES = [("hadamard", 128), ("hadamard", 64), ("hadamard", 32), ("hadamard", 16), ("identity", 32),
+         ("gsr", 64), ("gsr", 32), ("gsr", 16)]
+
+
+@pytest.mark.parametrize("rot,g", CASES)
+@pytest.mark.parametrize("policy", [_engine.ZERO_REFERENCE, _engine.ZERO_SIGNED])
+def test_quantize_packed_bit_exact(rot, g, policy):
+    rows, cols = 70, 512  # ragged last row tile
+    x = make_outlier_normal(rows, cols, 11 * g + len(rot))
+    x[3, 64:96] = 0.0            # a zero group
+    x[5, :32] = -0.0
+    x[7] *= 2.0 ** -110          # exponents outside the fast range
+    x[9] *= 2.0 ** 105
+    okind = {"hadamard": O.ROT_HADAMARD, "identity": O.ROT_IDENTITY, "gsr": O.ROT_GSR}[rot]
+    norm = float(O.hadamard_matrix(g)[0, 0])
+    wc, ws, _ = O.quantize_mx(x, okind, g, norm, zero_nibble=policy)
+    want_c, want_s = pack_by_definition(wc, ws, cols)
+    pc, ps = capi.quantize_packed(x, rot=rot, g=g, norm=norm, zero_policy=policy)
+    assert torch.equal(pc, want_c)
+    assert torch.equal(ps, want_s)
+
+
+def test_quantize_packed_large_matches_row_major_path():
+    """Full-size activation block: the packed quantizer equals re-tiling the row-major one."""
+    gen = torch.Generator().manual_seed(5)
+    x = (torch.randn(2048, 4096, generator=gen) * 3).to(torch.bfloat16)
+    rc, rs = capi.quantize(x, "mxfp4", g=128)
+    want_c, want_s = pack_by_definition(rc, rs, 4096)
+    pc, ps = capi.quantize_packed(x, g=128)
+    assert torch.equal(pc, want_c) and torch.equal(ps, want_s)
+
+
+def test_quantize_packed_rejects():
+    x = torch.zeros(32, 384, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        capi.quantize_packed(x, g=128)                       # cols % 256 != 0
+    with pytest.raises(ValueError):
+        capi.quantize_packed(torch.zeros(32, 512, dtype=torch.bfloat16), rot="gsr", g=128)
+
+
+@pytest.mark.parametrize("m,n,k", [(32, 32, 256), (65, 100, 256), (256, 256, 512), (300, 520, 768),
+                                   (256, 512, 2304), (512, 256, 4096)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_gemm_packed_matches_oracle_and_row_major_kernel(m, n, k, bias):
+    g = torch.Generator().manual_seed(m + n + k)
+    xq = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=g)
+    wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=g)
+    xs = torch.randint(118, 134, (m, k // 32), dtype=torch.uint8, generator=g)
+    ws = torch.randint(118, 134, (n, k // 32), dtype=torch.uint8, generator=g)
+    b = torch.randn(n, generator=g).to(torch.bfloat16) if bias else None
+    alpha = 0.111328125
+    xp, xsp = pack_by_definition(xq, xs, k)
+    wp, wsp = pack_by_definition(wq, ws, k)
+    y = capi.gemm_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=b)
+    assert not torch.isnan(y.float()).any()
+    ref, mag = O.gemm_ref(xq, xs, wq, ws, alpha, "mxfp4")
+    want = ref.to(torch.bfloat16)
+    if bias:
+        want = want + b
+    # fp32 accumulation in another order than the oracle's, then one bf16 rounding (two with bias)
+    tol = 2.0 ** -7 * want.double().abs() + 1e-5 * mag + 1e-6
+    assert ((y.double() - want.double()).abs() <= tol).all()
+    # the same MFMA sequence per output as the row-major kernel: identical bits
+    y_rm = capi.gemm(xq, xs, wq, ws, alpha, "mxfp4", bias=b)
+    assert torch.equal(y.view(torch.int16), y_rm.view(torch.int16))
+
+
+def test_gemm_packed_rejects():
+    z = torch.zeros(4096, dtype=torch.uint8)
+    with pytest.raises(ValueError):
+        capi.gemm_packed(z, z, z, z, 32, 32, 128, 1.0)       # K % 256 != 0
+
+
+def test_linear_uses_packed_path_and_matches_row_major(monkeypatch):
+    """FPQuantLinear above the row threshold runs quantize-to-packed + packed GEMM; the result is
+    bit-identical to the row-major kernels (FPQ_PACKED_WEIGHTS=0)."""
+    import fp_quant
+    from fp_quant.module import hip_ops
+    cfg = fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype.MXFP4, forward_method="abs_max",
+                                 backward_dtype=fp_quant.FPQuantDtype.BF16, hadamard_group_size=128)
+    torch.manual_seed(2)
+    lin = fp_quant.FPQuantLinear(512, 384, cfg, bias=True, device="cuda", dtype=torch.bfloat16)
+    lin.weight.data.normal_(0, 0.02)
+    lin.bias.data.normal_()
+    lin.pre_forward()
+    x = torch.randn(3, 100, 512, device="cuda", dtype=torch.bfloat16)
+    assert x.shape[0] * x.shape[1] >= hip_ops.PACKED_LINEAR_MIN_M
+    y_packed = lin(x)
+    assert getattr(lin.qweight, "_fpq_packed", None) is not None
+    monkeypatch.setenv("FPQ_PACKED_WEIGHTS", "0")
+    y_rm = lin(x)
+    assert torch.equal(y_packed, y_rm)
