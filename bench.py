@@ -196,6 +196,49 @@ def _time_linear(torch, run_linear, run_gemm, fmt, m, n, k, g, group, n_buf, ste
     }
 
 
+def bench_mfma_ceiling(torch, seed=4, iters=192):
+    """Register-resident FP4 MFMA loop (no memory system): the matrix throughput and clock the chip
+    sustains for all-zero operands and for operands with the bit statistics of quantized data, over
+    about the duration of the M=2048 GEMM.  The second number is the practical ceiling of that GEMM."""
+    from fp_quant import _engine
+    from fp_quant.module import hip_ops
+    lib = _engine.lib()
+    dev = torch.device("cuda:0")
+    blocks = torch.cuda.get_device_properties(0).multi_processor_count
+    n_words = blocks * 256 * 32
+    gen = torch.Generator().manual_seed(seed)
+    x = torch.randn(n_words * 4 * 2 // 4096, 4096, generator=gen).to(torch.bfloat16).to(dev)
+    from fp_quant.module.linear import get_hadamard_matrix
+    h = get_hadamard_matrix(128, torch.bfloat16, dev)
+    codes, _, _ = hip_ops.fused_quantize_mx_op(x, h, "abs_max", False)
+    words = {"zeros": torch.zeros(n_words, dtype=torch.int32, device=dev),
+             "quantized": codes.view(-1).view(torch.int32)[:n_words].contiguous()}
+    sink = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+    clocks = torch.empty(blocks * 2, dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    out = {"iters": iters, "workgroups": blocks}
+    for name, w in words.items():
+        best = None
+        for rep in range(6):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            st = lib.fpq_test_mfma_rate(w.data_ptr(), blocks, iters, sink.data_ptr(), clocks.data_ptr(), stream)
+            e1.record()
+            torch.cuda.synchronize()
+            if st != 0:
+                _engine.check(st, "fpq_test_mfma_rate")
+            c = clocks.view(blocks, 2).double().cpu()
+            us = float(c[:, 1].mean()) * 1e-2  # 100 MHz ticks -> us, inside the kernel (no launch overhead)
+            ghz = float(c[:, 0].sum() / (c[:, 1].sum() * 10.0))
+            if rep > 0 and (best is None or us < best[0]):
+                best = (us, ghz)
+        flops = blocks * 4 * iters * 16 * 131072.0
+        out[name] = {"TFLOP/s": round(flops / (best[0] * 1e-6) / 1e12, 1), "clock_GHz": round(best[1], 3),
+                     "loop_us": round(best[0], 1)}
+    return out
+
+
 def cpu_baseline_quantize(torch, fmt, rows, cols, g, seed, sample_rows):
     """The oracle (a torch-CPU restatement of the reference's PyTorch quantizer path) timed
     on a bounded row sample of the same workload."""
@@ -263,7 +306,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="comma list of workloads to run (for profiling one kernel): "
                     "nvfp4_quantize, mxfp4_quantize, mxfp4_linear_M2048, mxfp4_linear_M128, mxfp4_linear_M16, "
-                    "mxfp4_linear_M1, nvfp4_linear")
+                    "mxfp4_linear_M1, nvfp4_linear, mfma_ceiling")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB device copy (known traffic) to scale rocprofv3 byte counters")
     args = ap.parse_args()
@@ -299,6 +342,8 @@ def main():
         if "nvfp4_linear" in only:
             out["nvfp4_linear"] = bench_linear(torch, "nvfp4", 4096, 24576, 4096, 16, max(10, args.steps // 10),
                                                max(2, args.warmup // 10), seed=3)
+        if "mfma_ceiling" in only:
+            out["mfma_ceiling"] = bench_mfma_ceiling(torch)
         print(json.dumps({"only": only, "steps": args.steps, "results": out}))
         return
 
@@ -311,6 +356,7 @@ def main():
         linears[m] = bench_linear(torch, "mxfp4", m, 14336, 4096, 128, args.steps, args.warmup, seed=2)
     nv = bench_linear(torch, "nvfp4", 4096, 24576, 4096, 16, max(10, args.steps // 10), max(2, args.warmup // 10), seed=3)
 
+    ceiling = bench_mfma_ceiling(torch)
     quant = results["nvfp4_quantize"]
     head = linears[2048]
     kernels = {
@@ -358,6 +404,11 @@ def main():
             "traffic": traffic.get("mxfp4_gemm_M2048"),
             "kernel_us": round(head["gemm_ms"] * 1e3, 3),
             "algorithmic_flops_per_launch": int(head["flops"]),
+            "operand_layout": head["operand_layout"],
+            # what the matrix pipes alone sustain (register-resident operands): the clock drops with
+            # non-zero operand bits, so this, not `peak`, is what the kernel can approach
+            "sustained_mfma_only": ceiling,
+            "frac_of_sustained": round(head["gemm_tflops"] / ceiling["quantized"]["TFLOP/s"], 4),
         },
         "roofline_quantize": {
             "kernel": "NVFP4 fused rotate+quantize, bf16 [8192, 4096], Hadamard 16",

@@ -27,3 +27,56 @@ extern "C" int fpq_device_supported(int device) {
   if (err != hipSuccess) return (int)err;
   return strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 0;
 }
+
+// ---------------------------------------------------------------------------------------------
+// Measurement hook: the rate at which the matrix pipes execute the FP4 block-scaled MFMA on
+// operands that never leave registers -- no memory traffic, no LDS, no barriers -- so the only
+// limits left are the issue rate and the clock the chip sustains for the given operand bits.
+namespace fpq {
+typedef int probe_v8i __attribute__((ext_vector_type(8)));
+typedef float probe_v16f __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void mfma_rate_kernel(const int* __restrict__ words, int iters,
+                                                        float* __restrict__ sink,
+                                                        unsigned long long* __restrict__ clocks) {
+  const int t = threadIdx.x + blockIdx.x * 256;
+  probe_v8i a[4], b[4];
+  for (int i = 0; i < 4; ++i) {
+    const int* w = words + (size_t)t * 32 + i * 4;
+    a[i] = probe_v8i{w[0], w[1], w[2], w[3], 0, 0, 0, 0};
+    b[i] = probe_v8i{w[16], w[17], w[18], w[19], 0, 0, 0, 0};
+  }
+  const int sa = 0x7f7f7f7f, sb = 0x7f7f7f7f;  // scale 1.0 in every byte
+  probe_v16f acc[4][4];
+  for (int i = 0; i < 4; ++i)
+    for (int j = 0; j < 4; ++j)
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i], b[j], acc[i][j], 4, 4, 0, sa, 0, sb);
+  }
+  const unsigned long long c1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+  float s = 0.f;
+  for (int i = 0; i < 4; ++i)
+    for (int j = 0; j < 4; ++j)
+      for (int v = 0; v < 16; ++v) s += acc[i][j][v];
+  sink[t] = s;
+  if (threadIdx.x == 0) {
+    clocks[blockIdx.x * 2] = c1 - c0;       // shader clock cycles
+    clocks[blockIdx.x * 2 + 1] = r1 - r0;   // 100 MHz ticks
+  }
+}
+}  // namespace fpq
+
+extern "C" int fpq_test_mfma_rate(const int* words, int blocks, int iters, float* sink,
+                                  unsigned long long* clocks, void* stream) {
+  if (!words || !sink || !clocks) return FPQ_E_NULL;
+  if (blocks <= 0 || iters <= 0) return FPQ_E_SHAPE;
+  hipLaunchKernelGGL(fpq::mfma_rate_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, words,
+                     iters, sink, clocks);
+  return (int)hipGetLastError();
+}

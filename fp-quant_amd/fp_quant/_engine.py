@@ -27,6 +27,7 @@ _SIGNATURES = {
     "fpq_gemm_mxf4": ([_P, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _P], _I),
     "fpq_gemm_nvf4": ([_P, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _P], _I),
     "fpq_test_e2m1": ([_P, _P, _I64, _I, _P], _I),
+    "fpq_test_mfma_rate": ([_P, _I, _I, _P, _P, _P], _I),
     "fpq_packed_codes_bytes": ([_I64, _I64], _I64),
     "fpq_packed_scales_bytes": ([_I64, _I64], _I64),
     "fpq_pack_mxf4": ([_P, _P, _I64, _I64, _I64, _P, _P, _P], _I),

@@ -141,6 +141,17 @@ int fpq_gemm_mxf4_packed(const void* xq_packed, const void* xs_packed, const voi
  */
 int fpq_test_e2m1(const float* in, uint8_t* out, int64_t n, int zero_policy, void* stream);
 
+/*
+ * Measurement hook: `blocks` workgroups of four waves run `iters` x 16 FP4 32x32x64 block-scaled
+ * matrix instructions per wave on register-resident operands (words: blocks*256*32 ints of operand
+ * bits; sink: blocks*256 floats; clocks: per workgroup the elapsed shader-clock cycles and 100 MHz
+ * ticks).  It gives the matrix throughput and clock this chip sustains for given operand bits with
+ * no memory system involved: the practical ceiling a GEMM is compared with next to the nominal
+ * peak.  No counterpart in the reference.
+ */
+int fpq_test_mfma_rate(const int* words, int blocks, int iters, float* sink, unsigned long long* clocks,
+                       void* stream);
+
 #ifdef __cplusplus
 }
 #endif
