@@ -123,21 +123,15 @@ __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
       op_base[j] = xq + (size_t)rt * nu * 1024;
     }
   }
-  // Scale piece p (0..3) of a block: p < 2 weight row tiles 4p..4p+3, else activation row tiles
-  // 4(p-2)..; one load instruction, lane L fetches 16 bytes of row tile L / 16.
-  uint32_t sc_off_w[2], sc_off_x[2];
-#pragma unroll
-  for (int p = 0; p < 2; ++p) {
-    const int rtw = min(tile_n * NT + p * 4 + (lane >> 4), rt_n - 1);
-    const int rtx = min(tile_m * 8 + p * 4 + (lane >> 4), rt_m - 1);
-    sc_off_w[p] = (uint32_t)rtw * (uint32_t)nkb * 256u + (lane & 15) * 16;
-    sc_off_x[p] = (uint32_t)rtx * (uint32_t)nkb * 256u + (lane & 15) * 16;
-  }
+  // Scale piece w (0..3) of a block, loaded by wave w: w < 2 weight row tiles 4w..4w+3, else
+  // activation row tiles 4(w-2)..; one load instruction, lane L fetches 16 bytes of row tile L / 16.
+  const int sc_rt = min((wave < 2 ? tile_n * NT : tile_m * 8) + (wave & 1) * 4 + (lane >> 4),
+                        (wave < 2 ? rt_n : rt_m) - 1);
+  const uint32_t sc_off = (uint32_t)sc_rt * (uint32_t)nkb * 256u + (lane & 15) * 16;
   const uint32_t lane16 = lane * 16;
 
   static_assert(NW == 4, "one scale piece per wave");
   const uint8_t* sc_base = wave < 2 ? ws : xs;
-  const uint32_t sc_off = wave < 2 ? sc_off_w[wave & 1] : sc_off_x[wave & 1];
   // Unit u into its ring slot; with every fourth unit travel the scales of the block it opens
   // (wave w brings piece w), issued first so that they have landed whenever the unit has.
   auto issue_unit = [&](int u, bool with_scales) {
