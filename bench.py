@@ -239,6 +239,99 @@ def bench_mfma_ceiling(torch, seed=4, iters=192):
     return out
 
 
+def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=(1, 32, 64), decode_steps=8):
+    """Forward passes of a random-weight Llama-3.1-8B-architecture model (transformers' LlamaForCausalLM) whose
+    linears (all but lm_head) were replaced by MXFP4 FPQuantLinear with Hadamard-128: prefill tokens/s, decode
+    tokens/s against a `seq`-token bf16 KV cache, and the share of GPU time spent inside the quantized linears
+    (HIP events around every FPQuantLinear.forward)."""
+    import fp_quant
+    from transformers import LlamaConfig, LlamaForCausalLM
+    dev = torch.device("cuda:0")
+    cfg = LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=layers, num_attention_heads=32,
+                      num_key_value_heads=8, vocab_size=128256, max_position_embeddings=8192, rms_norm_eps=1e-5,
+                      rope_theta=500000.0, attn_implementation="sdpa")
+    old_dtype = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with dev:
+            model = LlamaForCausalLM(cfg)
+    finally:
+        torch.set_default_dtype(old_dtype)
+    model.eval()
+    qcfg = fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype.MXFP4, forward_method="abs_max",
+                                  backward_dtype=fp_quant.FPQuantDtype.BF16, hadamard_group_size=128)
+    fp_quant.replace_quantize_with_fp_quant_linear(model, qcfg)
+    qlinears = [m for m in model.modules() if isinstance(m, fp_quant.FPQuantLinear)]
+    spans = []
+
+    def pre(mod, args):
+        e = torch.cuda.Event(enable_timing=True)
+        e.record()
+        mod._bench_e0 = e
+
+    def post(mod, args, out):
+        e = torch.cuda.Event(enable_timing=True)
+        e.record()
+        spans.append((mod._bench_e0, e))
+
+    gen = torch.Generator().manual_seed(7)
+
+    def timed(fn, reps, with_hooks):
+        handles = []
+        if with_hooks:
+            for m in qlinears:
+                handles += [m.register_forward_pre_hook(pre), m.register_forward_hook(post)]
+        best, share = None, None
+        for _ in range(reps):
+            spans.clear()
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+            if best is None or ms < best:
+                best = ms
+                share = sum(a.elapsed_time(b) for a, b in spans) / ms if with_hooks else None
+        for h in handles:
+            h.remove()
+        return best, share
+
+    out = {"model": f"Llama-3.1-8B architecture, {layers} layers, random weights, MXFP4 W4A4 Hadamard-128",
+           "quantized_linears": len(qlinears)}
+    with torch.no_grad():
+        ids = torch.randint(0, cfg.vocab_size, (prefill_batch, seq), generator=gen).to(dev)
+        run = lambda: model(input_ids=ids, use_cache=False, logits_to_keep=1)
+        run()
+        ms, _ = timed(run, 3, False)
+        _, share = timed(run, 2, True)
+        out["prefill"] = {"batch": prefill_batch, "seq": seq, "ms": round(ms, 2),
+                          "tokens_per_s": round(prefill_batch * seq / (ms * 1e-3), 1),
+                          "linear_time_share": round(share, 3)}
+        out["decode"] = {}
+        for b in decode_batches:
+            ids = torch.randint(0, cfg.vocab_size, (b, seq), generator=gen).to(dev)
+            cache = model(input_ids=ids, use_cache=True, logits_to_keep=1).past_key_values
+            tok = torch.randint(0, cfg.vocab_size, (b, 1), generator=gen).to(dev)
+            state = {"cache": cache}
+
+            def step():
+                for _ in range(decode_steps):
+                    r = model(input_ids=tok, past_key_values=state["cache"], use_cache=True)
+                    state["cache"] = r.past_key_values
+
+            step()
+            ms, _ = timed(step, 2, False)
+            _, share = timed(step, 1, True)
+            out["decode"][f"batch{b}"] = {"kv_tokens": seq, "ms_per_step": round(ms / decode_steps, 3),
+                                          "tokens_per_s": round(b * decode_steps / (ms * 1e-3), 1),
+                                          "linear_time_share": round(share, 3)}
+            del cache, state
+            torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline_quantize(torch, fmt, rows, cols, g, seed, sample_rows):
     """The oracle (a torch-CPU restatement of the reference's PyTorch quantizer path) timed
     on a bounded row sample of the same workload."""
@@ -306,7 +399,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="comma list of workloads to run (for profiling one kernel): "
                     "nvfp4_quantize, mxfp4_quantize, mxfp4_linear_M2048, mxfp4_linear_M128, mxfp4_linear_M16, "
-                    "mxfp4_linear_M1, nvfp4_linear, mfma_ceiling")
+                    "mxfp4_linear_M1, nvfp4_linear, mfma_ceiling, e2e_llama (whole-model forward, not part of the default run)")
+    ap.add_argument("--e2e-layers", type=int, default=32, help="decoder layers of the --only e2e_llama model")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB device copy (known traffic) to scale rocprofv3 byte counters")
     args = ap.parse_args()
@@ -342,6 +436,8 @@ def main():
         if "nvfp4_linear" in only:
             out["nvfp4_linear"] = bench_linear(torch, "nvfp4", 4096, 24576, 4096, 16, max(10, args.steps // 10),
                                                max(2, args.warmup // 10), seed=3)
+        if "e2e_llama" in only:
+            out["e2e_llama"] = bench_e2e_llama(torch, layers=args.e2e_layers)
         if "mfma_ceiling" in only:
             out["mfma_ceiling"] = bench_mfma_ceiling(torch)
         print(json.dumps({"only": only, "steps": args.steps, "results": out}))

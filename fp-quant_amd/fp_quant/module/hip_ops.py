@@ -389,3 +389,93 @@ def matmul_nvf4_bf16_tn_bias_op(
 @matmul_nvf4_bf16_tn_bias_op.register_fake
 def _(x, w, xs, ws, alpha, bias):
     return x.new_empty(*x.shape[:-1], w.shape[0], dtype=torch.bfloat16)
+
+
+### Whole linear, eager fast path
+
+
+def cached_on(t: torch.Tensor, slot: str, key, make):
+    """`make()` remembered on tensor `t` under attribute `slot` while `key` stays the same."""
+    hit = getattr(t, slot, None)
+    if hit is not None and hit[0] == key:
+        return hit[1]
+    val = make()
+    try:
+        setattr(t, slot, (key, val))
+    except (AttributeError, RuntimeError):
+        pass
+    return val
+
+
+def linear_alpha(weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor) -> torch.Tensor:
+    """fp32 one-element `1 / (wgs * ags)` evaluated in the buffers' dtype as the reference does
+    (linear_fns.py:505; bf16 buffers round 1/9 to 0.111328125), cached until a buffer changes."""
+    key = (weight_global_scale._version, act_global_scale._version, act_global_scale.data_ptr(),
+           weight_global_scale.data_ptr())
+    return cached_on(weight_global_scale, "_fpq_alpha", key,
+                     lambda: (1.0 / (weight_global_scale * act_global_scale)).float().reshape(1).contiguous())
+
+
+def as_f32_scalar(t: torch.Tensor) -> torch.Tensor:
+    if t.dtype == torch.float32 and t.is_contiguous():
+        return t
+    return cached_on(t, "_fpq_f32", (t._version, t.data_ptr()), lambda: t.detach().float().contiguous())
+
+
+def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.Tensor, ws: torch.Tensor,
+                alpha: torch.Tensor, act_global_scale: torch.Tensor, bias: Optional[torch.Tensor],
+                nvfp4: bool) -> torch.Tensor:
+    """Activation rotate+quantize and W4A4 GEMM of one linear with as little host work as possible:
+    the eager (non-traced) body of FPQuantLinear.forward.  Same kernels and results as the
+    fused_quantize_* and matmul_* operators; `x_flat` bf16 [M, K] contiguous on the GPU, `alpha`
+    fp32 [1], `bias` bf16 [N] or None."""
+    if not x_flat.is_cuda:
+        raise ValueError("fp_quant HIP operators need tensors on a GPU; there is no CPU path")
+    lib = _engine.lib()
+    m, k = x_flat.shape
+    n = wq.shape[0]
+    if wq.shape[1] * 2 != k:
+        raise ValueError(f"inner dimensions differ: x has K={k}, w has K={wq.shape[1] * 2}")
+    dev = x_flat.device
+    if torch.cuda.current_device() != dev.index:
+        with torch.cuda.device(dev):
+            return linear_w4a4(x_flat, hadamard_matrix, wq, ws, alpha, act_global_scale, bias, nvfp4)
+    stream = torch.cuda.current_stream().cuda_stream
+    h = as_bf16(hadamard_matrix)
+    kind, norm = classify_rotation(h)
+    g = h.shape[0]
+    y = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    b_ptr = bias.data_ptr() if bias is not None else None
+    if not nvfp4 and packed_linear_eligible(m, k, "abs_max"):
+        pc = torch.empty(lib.fpq_packed_codes_bytes(m, k), dtype=torch.uint8, device=dev)
+        ps = torch.empty(lib.fpq_packed_scales_bytes(m, k), dtype=torch.uint8, device=dev)
+        st = lib.fpq_quantize_mx_packed(x_flat.data_ptr(), m, k, kind, g, norm, pc.data_ptr(), ps.data_ptr(),
+                                        ZERO_NIBBLE_POLICY, stream)
+        if st == _engine.E_UNSUPPORTED:
+            pc, ps = quantize_mx_packed(x_flat, h)
+        else:
+            _engine.check(st, "fpq_quantize_mx_packed")
+        wp, wsp = packed_weight(wq, ws)
+        st = lib.fpq_gemm_mxf4_packed(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(), alpha.data_ptr(),
+                                      b_ptr, y.data_ptr(), m, n, k, stream)
+        _engine.check(st, "fpq_gemm_mxf4_packed")
+        return y
+    group = 16 if nvfp4 else 32
+    codes = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
+    scales = torch.empty(m, k // group, dtype=torch.uint8, device=dev)
+    if nvfp4:
+        gs = as_f32_scalar(act_global_scale)
+        st = lib.fpq_quantize_nv(x_flat.data_ptr(), m, k, kind, g, norm, h.data_ptr(), gs.data_ptr(),
+                                 codes.data_ptr(), scales.data_ptr(), m, k // group, ZERO_NIBBLE_POLICY, stream)
+        _engine.check(st, "fpq_quantize_nv")
+        st = lib.fpq_gemm_nvf4(codes.data_ptr(), scales.data_ptr(), k // group, wq.data_ptr(), ws.data_ptr(),
+                               ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
+        _engine.check(st, "fpq_gemm_nvf4")
+    else:
+        st = lib.fpq_quantize_mx(x_flat.data_ptr(), m, k, kind, g, norm, h.data_ptr(), codes.data_ptr(),
+                                 scales.data_ptr(), m, k // group, ZERO_NIBBLE_POLICY, stream)
+        _engine.check(st, "fpq_quantize_mx")
+        st = lib.fpq_gemm_mxf4(codes.data_ptr(), scales.data_ptr(), k // group, wq.data_ptr(), ws.data_ptr(),
+                               ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
+        _engine.check(st, "fpq_gemm_mxf4")
+    return y

@@ -45,6 +45,10 @@ def get_gsr_matrix(group_size: int, dtype: torch.dtype, device: torch.device):
 _TRANSFORMS = {"hadamard": get_hadamard_matrix, "identity": get_identity_matrix, "gsr": get_gsr_matrix}
 
 
+def _no_master_forward(*args):
+    return FPQuant4x16NoMasterFn.forward(None, *args)
+
+
 class FPQuantLinear(nn.Module):
     def __init__(
         self,
@@ -144,7 +148,10 @@ class FPQuantLinear(nn.Module):
             and not cfg.store_master_weights
             and not cfg.pseudoquantization
         ):
-            return FPQuant4x16NoMasterFn.apply(
+            # no autograd graph to build (inference): call the forward directly
+            fn = (FPQuant4x16NoMasterFn.apply if (torch.is_grad_enabled() and x.requires_grad)
+                  else _no_master_forward)
+            return fn(
                 x,
                 self.qweight,
                 self.scales,

@@ -18,7 +18,9 @@ from .hip_ops import (
     matmul_mxf4_bf16_tn_op,
     matmul_nvf4_bf16_tn_bias_op,
     matmul_nvf4_bf16_tn_op,
+    linear_alpha,
     linear_mxf4_packed_op,
+    linear_w4a4,
     packed_linear_eligible,
 )
 
@@ -71,6 +73,19 @@ class FPQuant4x16NoMasterFn(Function):
         forward_method: str,
     ):
         x_flat = x.contiguous().flatten(end_dim=-2)
+        if (not torch.compiler.is_compiling() and forward_method == "abs_max"
+                and dtype in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4)
+                and weight_q.is_contiguous() and weight_scales.is_contiguous()):
+            # eager calls: the same kernels as the operators below without two operator dispatches,
+            # with alpha and the fp32 global scale computed once per layer instead of once per call
+            fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16 and bias.is_contiguous()) else None
+            y = linear_w4a4(x_flat.to(torch.bfloat16), forward_hadamard_matrix, weight_q, weight_scales,
+                            linear_alpha(weight_global_scale, act_global_scale), act_global_scale, fused_bias,
+                            dtype == FPQuantDtype.NVFP4)
+            y = y.unflatten(dim=0, sizes=x.shape[:-1])
+            if bias is not None and fused_bias is None:
+                y += bias
+            return y
         if (dtype == FPQuantDtype.MXFP4 and x_flat.is_cuda
                 and packed_linear_eligible(x_flat.shape[0], x_flat.shape[1], forward_method)):
             # large batches: quantize and multiply on operands in the matrix units' own order
