@@ -26,12 +26,23 @@ constexpr int kFmtNv = 1;
 // One lane quantizes 8 consecutive elements (chunk index `chunk`); the G/8 neighbouring lanes of
 // a rotation block exchange registers for the butterflies with stride >= 8.  Must be called by
 // all 64 lanes of a wave with consecutive chunk indices (inactive lanes pass active = false).
-template <int G, int FMT, int ROT, int ZERO>
+//
+// QUEST (MXFP4 only) replaces the abs-max scale by the reference's "quest" rule
+// (inference_lib/src/fp_quant/module/triton/mxfp4.py:51-59, constant from
+// pseudoquant_linear_fns.py:20-22): s = 2^floor(log2(fl(2.92247856/6) * std + 1e-8)) with the
+// population standard deviation of the 32 rotated values, values beyond +-6 s saturate, and the
+// optional mask gets bit (element % 8) of byte [row, element / 8] set where |x / s| < 6
+// (mxfp4.py:105-110, linear_fns.py:67-76).  fp32 evaluation order, fixed so that a CPU can
+// reproduce it: per octet of consecutive elements the sums of x and of fl(x*x) run left to right,
+// the four octet sums combine as (o0 + o1) + (o2 + o3); mean = sum/32, var = max(msq - fl(mean*mean), 0).
+template <int G, int FMT, int ROT, int ZERO, bool QUEST = false>
 __device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint32_t* __restrict__ codes,
                                               uint8_t* __restrict__ scales, uint32_t chunk, bool active,
                                               uint32_t lane, uint32_t chunks_per_row,
                                               uint32_t scale_stride, float norm, float gscale, float rg,
-                                              float* __restrict__ stage, const uint16_t* __restrict__ hmat) {
+                                              float* __restrict__ stage, const uint16_t* __restrict__ hmat,
+                                              uint8_t* __restrict__ mask = nullptr) {
+  static_assert(!QUEST || FMT == kFmtMx, "the quest rule exists for MXFP4 only");
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
   uint4 raw = make_uint4(0u, 0u, 0u, 0u);
   if (active) raw = x[chunk];
@@ -101,6 +112,43 @@ __device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint3
     for (int i = 0; i < 8; ++i) p[i] = acc[i];
   }
 
+  if (QUEST) {
+    float sum = p[0], sq = p[0] * p[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) {
+      sum = sum + p[i];
+      sq = sq + p[i] * p[i];
+    }
+#pragma unroll
+    for (int lm = 1; lm < 4; lm *= 2) {
+      sum = sum + __shfl_xor(sum, lm, 64);
+      sq = sq + __shfl_xor(sq, lm, 64);
+    }
+    const float mean = sum * 0.03125f, msq = sq * 0.03125f;
+    float var = msq - mean * mean;
+    var = var > 0.0f ? var : 0.0f;
+    const float sc = __builtin_sqrtf(var) * 0.48707976f + 1e-8f;   // fl32(2.92247856 / 6)
+    const uint32_t ex = (__float_as_uint(sc) >> 23) & 0xffu;        // sc >= 1e-8: a normal number
+    const float inv = __builtin_ldexpf(1.0f, 127 - (int)ex);        // 1 / s, exact
+    uint32_t packed = 0u, mbits = 0u;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float q = p[i] * inv;                                    // exact unless it underflows
+      packed |= e2m1_code<ZERO>(q) << (4 * i);
+      mbits |= (uint32_t)(__builtin_fabsf(q) < 6.0f) << i;
+    }
+    if (active) {
+      codes[chunk] = packed;
+      if (mask) mask[chunk] = (uint8_t)mbits;
+      if ((chunk & 3u) == 0u) {
+        const uint32_t row = chunk / chunks_per_row;
+        const uint32_t col = (chunk - row * chunks_per_row) / 4u;
+        scales[(size_t)row * scale_stride + col] = (uint8_t)ex;
+      }
+    }
+    return;
+  }
+
   float a = 0.0f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) a = __builtin_fmaxf(a, __builtin_fabsf(p[i]));
@@ -148,12 +196,12 @@ __device__ __forceinline__ void fill_scale_padding(uint8_t* __restrict__ scales,
 }
 
 // Generic kernel: works for any cols % max(G, GROUP) == 0; one 8-element chunk per thread.
-template <int G, int FMT, int ROT, int ZERO>
+template <int G, int FMT, int ROT, int ZERO, bool QUEST = false>
 __global__ __launch_bounds__(256) void quantize_lane8_kernel(
     const uint4* __restrict__ x, uint32_t* __restrict__ codes, uint8_t* __restrict__ scales,
     uint32_t n_chunks, uint32_t chunks_per_row, uint32_t rows, uint32_t scale_rows,
     uint32_t scale_stride, float norm, const float* __restrict__ global_scale,
-    const uint16_t* __restrict__ h) {
+    const uint16_t* __restrict__ h, uint8_t* __restrict__ mask = nullptr) {
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
   constexpr bool kStage = ROT == FPQ_ROT_GSR || ROT == FPQ_ROT_GENERAL;
   __shared__ float stage[kStage ? 4 : 1][kStage ? 512 : 1];
@@ -168,10 +216,82 @@ __global__ __launch_bounds__(256) void quantize_lane8_kernel(
     g = *global_scale;
     rg = g == 0.0f ? 0.0f : 1.0f / g;
   }
-  lane8_process<G, FMT, ROT, ZERO>(x, codes, scales, chunk, chunk < n_chunks, threadIdx.x & 63u,
-                                   chunks_per_row, scale_stride, norm, g, rg,
-                                   stage[kStage ? (threadIdx.x >> 6) : 0], hmat);
+  lane8_process<G, FMT, ROT, ZERO, QUEST>(x, codes, scales, chunk, chunk < n_chunks, threadIdx.x & 63u,
+                                          chunks_per_row, scale_stride, norm, g, rg,
+                                          stage[kStage ? (threadIdx.x >> 6) : 0], hmat, mask);
   fill_scale_padding(scales, rows, chunks_per_row / (GROUP / 8), scale_rows, scale_stride);
+}
+
+template <int G, int ROT>
+static int launch_lane8_quest(const void* x, int64_t rows, int64_t cols, float norm, void* codes, void* scales,
+                              int64_t scale_rows, int64_t scale_stride, void* mask, int zero_policy,
+                              hipStream_t stream, const void* h) {
+  const int64_t n_chunks = rows * cols / 8;
+  const dim3 grid((unsigned)((n_chunks + 255) / 256)), block(256);
+  auto args = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint4*)x, (uint32_t*)codes,
+                       (uint8_t*)scales, (uint32_t)n_chunks, (uint32_t)(cols / 8), (uint32_t)rows,
+                       (uint32_t)scale_rows, (uint32_t)scale_stride, norm, (const float*)nullptr,
+                       (const uint16_t*)h, (uint8_t*)mask);
+  };
+  if (zero_policy == FPQ_ZERO_REFERENCE) {
+    args(quantize_lane8_kernel<G, kFmtMx, ROT, kZeroReference, true>);
+  } else {
+    args(quantize_lane8_kernel<G, kFmtMx, ROT, kZeroSigned, true>);
+  }
+  return (int)hipGetLastError();
+}
+
+static int dispatch_quest(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                          const void* h, void* codes, void* scales, int64_t scale_rows, int64_t scale_stride,
+                          void* mask, int zero_policy, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (rows < 0 || cols < 0) return FPQ_E_SHAPE;
+  if (rows == 0 || cols == 0) return FPQ_OK;
+  if (!x || !codes || !scales) return FPQ_E_NULL;
+  if (zero_policy != FPQ_ZERO_REFERENCE && zero_policy != FPQ_ZERO_SIGNED) return FPQ_E_POLICY;
+  if (rot_kind == FPQ_ROT_IDENTITY) g = 32;
+  if (g != 16 && g != 32 && g != 64 && g != 128) return FPQ_E_ROTATION;
+  if (cols % g != 0 || cols % 32 != 0) return FPQ_E_SHAPE;
+  if (scale_rows < rows || scale_stride < cols / 32) return FPQ_E_SHAPE;
+  if (rows * cols >= (int64_t)1 << 34 || scale_rows * scale_stride >= (int64_t)1 << 32) return FPQ_E_SHAPE;
+  if (((uintptr_t)x & 15u) || ((uintptr_t)codes & 3u)) return FPQ_E_ALIGN;
+#define FPQ_LAUNCH_QUEST(GG, RR)                                                                   \
+  return launch_lane8_quest<GG, RR>(x, rows, cols, norm, codes, scales, scale_rows, scale_stride, \
+                                    mask, zero_policy, stream, h)
+  if (rot_kind == FPQ_ROT_GENERAL) {
+    if (!h) return FPQ_E_NULL;
+    if ((uintptr_t)h & 1u) return FPQ_E_ALIGN;
+  }
+  switch (rot_kind) {
+    case FPQ_ROT_IDENTITY: FPQ_LAUNCH_QUEST(32, FPQ_ROT_IDENTITY);
+    case FPQ_ROT_HADAMARD:
+      switch (g) {
+        case 16: FPQ_LAUNCH_QUEST(16, FPQ_ROT_HADAMARD);
+        case 32: FPQ_LAUNCH_QUEST(32, FPQ_ROT_HADAMARD);
+        case 64: FPQ_LAUNCH_QUEST(64, FPQ_ROT_HADAMARD);
+        case 128: FPQ_LAUNCH_QUEST(128, FPQ_ROT_HADAMARD);
+      }
+      break;
+    case FPQ_ROT_GSR:
+      switch (g) {
+        case 16: FPQ_LAUNCH_QUEST(16, FPQ_ROT_GSR);
+        case 32: FPQ_LAUNCH_QUEST(32, FPQ_ROT_GSR);
+        case 64: FPQ_LAUNCH_QUEST(64, FPQ_ROT_GSR);
+        case 128: FPQ_LAUNCH_QUEST(128, FPQ_ROT_GSR);
+      }
+      break;
+    case FPQ_ROT_GENERAL:
+      switch (g) {
+        case 16: FPQ_LAUNCH_QUEST(16, FPQ_ROT_GENERAL);
+        case 32: FPQ_LAUNCH_QUEST(32, FPQ_ROT_GENERAL);
+        case 64: FPQ_LAUNCH_QUEST(64, FPQ_ROT_GENERAL);
+        case 128: FPQ_LAUNCH_QUEST(128, FPQ_ROT_GENERAL);
+      }
+      break;
+  }
+#undef FPQ_LAUNCH_QUEST
+  return FPQ_E_ROTATION;
 }
 
 template <int G, int FMT, int ROT>
@@ -183,7 +303,8 @@ static int launch_lane8(const void* x, int64_t rows, int64_t cols, float norm, c
   auto args = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint4*)x, (uint32_t*)codes,
                        (uint8_t*)scales, (uint32_t)n_chunks, (uint32_t)(cols / 8), (uint32_t)rows,
-                       (uint32_t)scale_rows, (uint32_t)scale_stride, norm, gsp, (const uint16_t*)h);
+                       (uint32_t)scale_rows, (uint32_t)scale_stride, norm, gsp, (const uint16_t*)h,
+                       (uint8_t*)nullptr);
   };
   if (zero_policy == FPQ_ZERO_REFERENCE) {
     args(quantize_lane8_kernel<G, FMT, ROT, kZeroReference>);
@@ -691,6 +812,14 @@ extern "C" int fpq_quantize_mx(const void* x, int64_t rows, int64_t cols, int ro
                                void* stream) {
   return fpq::dispatch<fpq::kFmtMx>(x, rows, cols, rot_kind, g, norm, h, nullptr, codes, scales,
                                     scale_rows, scale_stride, zero_policy, stream);
+}
+
+extern "C" int fpq_quantize_mx_quest(const void* x, int64_t rows, int64_t cols, int rot_kind, int g,
+                                     float norm, const void* h, void* codes, void* scales,
+                                     int64_t scale_rows, int64_t scale_stride, void* mask, int zero_policy,
+                                     void* stream) {
+  return fpq::dispatch_quest(x, rows, cols, rot_kind, g, norm, h, codes, scales, scale_rows, scale_stride,
+                             mask, zero_policy, stream);
 }
 
 extern "C" int fpq_quantize_mx_packed(const void* x, int64_t rows, int64_t cols, int rot_kind, int g,

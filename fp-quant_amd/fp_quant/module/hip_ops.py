@@ -165,11 +165,9 @@ def fused_quantize_mx_op(
     forward_method: str,
     return_mask: bool,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    if forward_method != "abs_max":
-        raise NotImplementedError(
-            f"forward_method={forward_method!r}: this engine implements the abs_max MXFP4 quantizer only"
-        )
-    if return_mask:
+    if forward_method not in ("abs_max", "quest"):
+        raise ValueError(f"Unsupported forward method: {forward_method}")
+    if return_mask and forward_method != "quest":
         raise NotImplementedError("clip masks are only produced by the quest method")
     _require_cuda(x_flat, hadamard_matrix)
     if x_flat.dtype != torch.bfloat16 or x_flat.dim() != 2:
@@ -182,6 +180,14 @@ def fused_quantize_mx_op(
     codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=x.device)
     scales = torch.empty(prow, pcol, dtype=torch.uint8, device=x.device)
     h = hadamard_matrix.contiguous()
+    if forward_method == "quest":
+        mask = torch.empty(rows, cols // 8, dtype=torch.uint8, device=x.device) if return_mask else None
+        with torch.cuda.device(x.device):
+            st = _engine.lib().fpq_quantize_mx_quest(
+                x.data_ptr(), rows, cols, kind, g, norm, h.data_ptr(), codes.data_ptr(), scales.data_ptr(),
+                prow, pcol, mask.data_ptr() if mask is not None else None, ZERO_NIBBLE_POLICY, _stream(x))
+        _engine.check(st, "fused_quantize_mx_op")
+        return codes, scales.view(torch.float8_e8m0fnu), mask
     with torch.cuda.device(x.device):
         st = _engine.lib().fpq_quantize_mx(
             x.data_ptr(), rows, cols, kind, g, norm, h.data_ptr(), codes.data_ptr(),

@@ -68,6 +68,21 @@ int fpq_quantize_mx(const void* x, int64_t rows, int64_t cols, int rot_kind, int
                     int64_t scale_stride, int zero_policy, void* stream);
 
 /*
+ * fpq_quantize_mx with the reference's "quest" scale rule instead of abs-max
+ * (method="quest" of qutlass.fusedQuantizeMx, qutlass_ops.py:36-71; arithmetic as stated by
+ * module/triton/mxfp4.py:51-59 with the constant of pseudoquant_linear_fns.py:20-22):
+ *   s = 2^floor(log2(fl32(2.92247856/6) * std + 1e-8)),  std = population standard deviation of the
+ *   32 rotated values (fp32; sums per octet left to right, octets combined (o0+o1)+(o2+o3),
+ *   variance clamped at 0);  codes = E2M1 RNE of x/s saturated at +-6;  stored byte = e8m0(s).
+ *   mask  uint8 [rows, cols/8] or null: bit (c % 8) of byte [r, c/8] is 1 where |x/s| < 6
+ *         (mxfp4.py:105-110; bit order of linear_fns.py:67-76).
+ * Global scale for this method is 1.0 (linear.py:190-192).
+ */
+int fpq_quantize_mx_quest(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                          const void* h, void* codes, void* scales, int64_t scale_rows,
+                          int64_t scale_stride, void* mask, int zero_policy, void* stream);
+
+/*
  * Fused rotate + NVFP4 quantize (group 16, E4M3 scales, fp32 per-tensor multiplier).
  * Stands in for qutlass.fusedQuantizeNv behind fused_quantize_nv_op (qutlass_ops.py:74-105).
  *   global_scale  device pointer to one fp32 (the reference passes a 1-element tensor)

@@ -17,6 +17,9 @@ What it follows (all paths relative to the reference checkout):
 * nibble packing ............. src/quantization/quant_ops.py:15-16,31-40
 * stored scale bytes ......... src/quantization/rtn.py:187-188,
                                src/quantization/quant_ops.py:111-118
+* quest scale + clip mask .... inference_lib/src/fp_quant/module/triton/mxfp4.py:51-59,105-110,
+                               inference_lib/src/fp_quant/module/pseudoquant_linear_fns.py:20-22,
+                               inference_lib/src/fp_quant/module/linear_fns.py:67-76
 * linear ..................... inference_lib/src/fp_quant/module/linear_fns.py:496-514,
                                inference_lib/src/fp_quant/module/qutlass_ops.py:111-168
 
@@ -35,7 +38,8 @@ other (fp32 everywhere, bf16 only at the input and at the rotation matrix entrie
 
 Pin status (each function below is checked in tests/test_oracle_*.py against closed
 forms, exhaustive tables, library casts or brute force; none needed an import of the
-reference): rotation, E8M0 exponent, E2M1 RNE, packing, E4M3 cast, E8M0 cast, GEMM.
+reference): rotation, E8M0 exponent, E2M1 RNE, packing, E4M3 cast, E8M0 cast, GEMM, the quest
+scale (against numpy float64 statistics and a per-group Python loop) and clip mask.
 The third-party kernels the reference calls for this path (QuTLASS, un-vendored, version
 unpinned) have no fixtures in the reference: bit parity against QuTLASS itself is unpinned.
 """
@@ -313,6 +317,57 @@ def quantize_mx(x: torch.Tensor, kind: int = ROT_HADAMARD, g: int = 128,
     v = xg / s.unsqueeze(-1)
     codes = e2m1_codes(v, zero_nibble).view(r, c)
     return pack_nibbles(codes), stored, xr
+
+
+QUEST_GAUSSIAN_SCALE = 2.92247856 / 6.0  # pseudoquant_linear_fns.py:20-22
+
+
+def quest_scales(xg: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Working scale s = 2^floor(log2(fl32(2.92247856/6)*std + 1e-8)) and its E8M0 byte for
+    groups xg [..., 32] of rotated fp32 values (module/triton/mxfp4.py:51-59).
+
+    Triton leaves the order of its reductions open; the canonical order here (the one the HIP
+    kernel uses): per octet of consecutive elements the sums of x and of fl(x*x) run left to
+    right, the four octet sums combine as (o0 + o1) + (o2 + o3); mean = sum/32,
+    var = max(mean_sq - fl(mean*mean), 0) (the clamp keeps a constant group from producing
+    sqrt of a negative rounding residue; the reference would return NaN there)."""
+    f32 = torch.float32
+    assert xg.dtype == f32 and xg.shape[-1] == 32
+    oct_ = xg.reshape(*xg.shape[:-1], 4, 8)
+    sq8 = oct_ * oct_
+    s_sum, s_sq = oct_[..., 0].clone(), sq8[..., 0].clone()
+    for i in range(1, 8):
+        s_sum = s_sum + oct_[..., i]
+        s_sq = s_sq + sq8[..., i]
+    tot = (s_sum[..., 0] + s_sum[..., 1]) + (s_sum[..., 2] + s_sum[..., 3])
+    tot_sq = (s_sq[..., 0] + s_sq[..., 1]) + (s_sq[..., 2] + s_sq[..., 3])
+    mean = tot * torch.tensor(0.03125, dtype=f32)
+    msq = tot_sq * torch.tensor(0.03125, dtype=f32)
+    var = (msq - mean * mean).clamp_min(0.0)
+    sc = torch.sqrt(var) * torch.tensor(QUEST_GAUSSIAN_SCALE, dtype=f32) + torch.tensor(1e-8, dtype=f32)
+    e = floor_log2_exact(sc)
+    s = torch.ldexp(torch.ones_like(sc), e)
+    return s, (e + 127).to(torch.uint8)
+
+
+def quantize_mx_quest(x: torch.Tensor, kind: int = ROT_HADAMARD, g: int = 128,
+                      norm: Optional[float] = None, h: Optional[torch.Tensor] = None,
+                      zero_nibble: int = ZERO_NIBBLE_REFERENCE):
+    """MXFP4 "quest" rotate+quantize of a [R, C] bf16 tensor (mxfp4.py:51-59,105-110).
+
+    Returns (packed codes uint8 [R, C/2], E8M0 bytes uint8 [R, C/32], clip mask uint8 [R, C/8]
+    with bit (c % 8) of byte [r, c/8] set where |x/s| < 6 (linear_fns.py:67-76), rotated fp32)."""
+    if norm is None:
+        norm = float(hadamard_matrix(g)[0, 0])
+    xr = rotate(x, kind, g, norm, h)
+    r, c = xr.shape
+    xg = xr.view(r, c // MXFP_GROUPSIZE, MXFP_GROUPSIZE)
+    s, stored = quest_scales(xg)
+    v = xg / s.unsqueeze(-1)
+    codes = e2m1_codes(v, zero_nibble).view(r, c)  # magnitudes above 5 saturate at 6: the clip
+    inside = (v.abs() < 6.0).view(r, c // 8, 8).to(torch.int32)
+    mask = (inside << torch.arange(8, dtype=torch.int32)).sum(dim=-1).to(torch.uint8)
+    return pack_nibbles(codes), stored, mask, xr
 
 
 def nv_scales_from_absmax(a: torch.Tensor, global_scale: float):

@@ -109,3 +109,25 @@ def gemm_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=None):
     _engine.check(st, "fpq_gemm_mxf4_packed")
     torch.cuda.synchronize()
     return y.cpu()
+
+
+def quantize_quest(x_bf16, rot="hadamard", g=128, norm=None, h=None, zero_policy=_engine.ZERO_REFERENCE,
+                   want_mask=True, pad=False, fill=0xCD):
+    """fpq_quantize_mx_quest; CPU uint8 (codes [R, C/2], scales, mask [R, C/8] or None)."""
+    lib = _engine.lib()
+    x = x_bf16.to("cuda").contiguous()
+    rows, cols = x.shape
+    srow, scol = _padded(rows, cols // 32, pad)
+    codes = torch.full((rows, cols // 2), fill, dtype=torch.uint8, device="cuda")
+    scales = torch.full((srow, scol), fill, dtype=torch.uint8, device="cuda")
+    mask = torch.full((rows, cols // 8), fill, dtype=torch.uint8, device="cuda") if want_mask else None
+    if norm is None:
+        norm = float(torch.tensor(g ** -0.5, dtype=torch.bfloat16))
+    h_dev = h.to(device="cuda", dtype=torch.bfloat16).contiguous() if h is not None else None
+    st = lib.fpq_quantize_mx_quest(x.data_ptr(), rows, cols, ROT[rot], g, norm,
+                                   h_dev.data_ptr() if h_dev is not None else None, codes.data_ptr(),
+                                   scales.data_ptr(), srow, scol, mask.data_ptr() if want_mask else None,
+                                   zero_policy, torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_quantize_mx_quest")
+    torch.cuda.synchronize()
+    return codes.cpu(), scales.cpu(), (mask.cpu() if want_mask else None)

@@ -1,0 +1,84 @@
+"""MXFP4 "quest" quantizer on the GPU: codes, scale bytes and clip mask bit-exact against the oracle,
+and the operator / module surface for forward_method="quest"."""
+import pytest
+import torch
+
+from oracle import fpq_oracle as O
+from fp_quant import _engine
+import capi
+from conftest import make_outlier_normal, make_student_t
+
+pytestmark = pytest.mark.gpu
+
+OK = {"hadamard": O.ROT_HADAMARD, "identity": O.ROT_IDENTITY, "gsr": O.ROT_GSR}
+
+
+@pytest.mark.parametrize("rot,g", [("hadamard", 128), ("hadamard", 64), ("hadamard", 32), ("hadamard", 16),
+                                   ("identity", 32), ("gsr", 128), ("gsr", 32)])
+@pytest.mark.parametrize("policy", [_engine.ZERO_REFERENCE, _engine.ZERO_SIGNED])
+def test_quest_bit_exact(rot, g, policy):
+    rows, cols = 37, 384
+    x = make_outlier_normal(rows, cols, 5 * g + len(rot), frac=0.02, mult=40.0)
+    x[3, 64:96] = 0.0
+    x[4, 32:64] = 1.5            # a constant group: variance rounds to ~0
+    x[6] *= 2.0 ** -60
+    x[8] *= 2.0 ** 40           # (beyond about 2^60 the sum of squares overflows fp32, as in the reference)
+    norm = float(O.hadamard_matrix(g)[0, 0])
+    wc, ws, wm, _ = O.quantize_mx_quest(x, OK[rot], g, norm, zero_nibble=policy)
+    codes, scales, mask = capi.quantize_quest(x, rot=rot, g=g, norm=norm, zero_policy=policy)
+    assert torch.equal(scales, ws)
+    assert torch.equal(mask, wm)
+    assert torch.equal(codes, wc)
+    assert (wm != 0xff).any()    # something clipped, so the mask is not trivially all ones
+
+
+def test_quest_general_matrix_and_padded_scales():
+    gen = torch.Generator().manual_seed(12)
+    q, _ = torch.linalg.qr(torch.randn(32, 32, generator=gen))
+    h = q.to(torch.bfloat16)
+    x = make_student_t(20, 256, 3)
+    wc, ws, wm, _ = O.quantize_mx_quest(x, O.ROT_GENERAL, 32, h=h)
+    codes, scales, mask = capi.quantize_quest(x, rot="general", g=32, h=h, pad=True)
+    assert torch.equal(codes, wc) and torch.equal(mask, wm)
+    assert torch.equal(scales[:20, :8], ws)
+    assert (scales[20:] == 0).all() and (scales[:, 8:] == 0).all()
+    c2, s2, none = capi.quantize_quest(x, rot="general", g=32, h=h, want_mask=False)
+    assert none is None and torch.equal(c2, wc) and torch.equal(s2, ws)
+
+
+def test_quest_full_size_block():
+    x = make_outlier_normal(2048, 4096, 0)
+    wc, ws, wm, _ = O.quantize_mx_quest(x, O.ROT_HADAMARD, 128)
+    codes, scales, mask = capi.quantize_quest(x, g=128)
+    assert torch.equal(codes, wc) and torch.equal(scales, ws) and torch.equal(mask, wm)
+
+
+def test_quest_operator_and_linear():
+    import fp_quant
+    from fp_quant.module import hip_ops
+    x = make_outlier_normal(40, 256, 4).cuda()
+    h = O.hadamard_matrix(64).cuda()
+    codes, scales, mask = hip_ops.fused_quantize_mx_op(x, h, "quest", True)
+    wc, ws, wm, _ = O.quantize_mx_quest(x.cpu(), O.ROT_HADAMARD, 64)
+    assert mask.shape == (40, 32) and mask.dtype == torch.uint8
+    assert scales.shape == (128, 8) and scales.dtype == torch.float8_e8m0fnu
+    assert torch.equal(codes.cpu(), wc) and torch.equal(mask.cpu(), wm)
+    assert torch.equal(scales.view(torch.uint8).cpu()[:40], ws)
+    _, _, none = hip_ops.fused_quantize_mx_op(x, h, "quest", False)
+    assert none is None
+
+    cfg = fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype.MXFP4, forward_method="quest",
+                                 backward_dtype=fp_quant.FPQuantDtype.BF16, hadamard_group_size=64)
+    gen = torch.Generator().manual_seed(8)
+    w = (torch.randn(96, 256, generator=gen) * 0.02).to(torch.bfloat16)
+    lin = fp_quant.FPQuantLinear(256, 96, cfg, bias=False, device="cuda", dtype=torch.bfloat16)
+    lin.weight.data = w.cuda()
+    lin.pre_forward()
+    assert float(lin.weight_global_scale) == 1.0 and float(lin.act_global_scale) == 1.0   # linear.py:190-192
+    wq, wsc, _, _ = O.quantize_mx_quest(w, O.ROT_HADAMARD, 64)
+    assert torch.equal(lin.qweight.cpu(), wq) and torch.equal(lin.scales.cpu(), wsc)
+    y = lin(x).cpu()
+    ref, mag = O.gemm_ref(wc, ws, wq, wsc, 1.0, "mxfp4")
+    assert ((y.double() - ref).abs() <= 2.0 ** -8 * ref.abs() + 1e-5 * mag).all()
+    dense = x.cpu().double() @ w.double().T
+    assert (y.double() - dense).norm() / dense.norm() < 0.3
