@@ -170,3 +170,51 @@ def test_unsupported_branches_raise():
         lin(torch.zeros(1, 64, device="cuda", dtype=torch.bfloat16))
     with pytest.raises(ValueError):
         fp_quant.FPQuantLinear(64, 32, fp_quant.FPQuantConfig(pseudoquantization=True), device="cuda")
+
+
+def test_meta_replacement_then_realquant_checkpoint(tmp_path):
+    """The loader route (replace.py:7-71): every nn.Linear becomes an empty meta-device FPQuantLinear,
+    then the tensors of a realquant checkpoint (qweight / scales / *_global_scale / *_hadamard_matrix,
+    rtn.py:185-193) are loaded from a safetensors file and the model runs without pre_forward."""
+    import fp_quant
+    from safetensors.torch import load_file, save_file
+
+    class Tiny(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up = nn.Linear(256, 512, bias=False)
+            self.down = nn.Linear(512, 256, bias=True)
+            self.lm_head = nn.Linear(256, 32, bias=False)
+
+        def forward(self, x):
+            return self.lm_head(self.down(torch.relu(self.up(x))))
+
+    cfg = _cfg("mxfp4", 128)
+    torch.manual_seed(4)
+    src = Tiny().to(device="cuda", dtype=torch.bfloat16)
+    fp_quant.replace_quantize_with_fp_quant_linear(src, cfg)
+    x = torch.randn(70, 256, device="cuda", dtype=torch.bfloat16)
+    want = src(x)
+    path = str(tmp_path / "realquant.safetensors")
+    save_file({k: v.contiguous().cpu() for k, v in src.state_dict().items()}, path)
+
+    # loaders build the model under the checkpoint's default dtype, so the new modules' buffers get it
+    # (alpha = 1 / (wgs * ags) is evaluated in the buffers' dtype, linear_fns.py:505)
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device("meta"):
+            dst = Tiny()
+        dst, replaced = fp_quant.replace_with_fp_quant_linear(dst, cfg)
+    finally:
+        torch.set_default_dtype(torch.float32)
+    assert replaced
+    assert isinstance(dst.up, fp_quant.FPQuantLinear) and dst.up.qweight.is_meta and type(dst.lm_head) is nn.Linear
+    assert dst.up.source_cls is nn.Linear and not any(p.requires_grad for p in dst.up.parameters())
+    for m in dst.modules():
+        if isinstance(m, fp_quant.FPQuantLinear):
+            m.weight = None       # a realquant checkpoint holds no dense weights
+            m.dqweight = None
+    dst.to_empty(device="cuda")
+    missing, unexpected = dst.load_state_dict(load_file(path, device="cuda"), strict=True)
+    assert not missing and not unexpected
+    assert torch.equal(dst(x), want)
