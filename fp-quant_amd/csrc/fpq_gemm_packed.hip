@@ -57,10 +57,10 @@ __global__ __launch_bounds__(256) void pack_mxf4_kernel(const uint8_t* __restric
 
 // ---------------------------------------------------------------------------------------------
 constexpr int kRing = 8;                 // 64-K units resident or in flight
-constexpr int kUnitBytes = 16 * 1024;    // 8 weight + 8 activation operands of one unit
 constexpr int kScaleSlots = 4;           // 256-K scale blocks resident or in flight
 constexpr int kScaleSlotBytes = 16 * 256;
-constexpr int kPackedLds = kRing * kUnitBytes + kScaleSlots * kScaleSlotBytes;
+// LDS of a workgroup whose unit holds `blocks` operand kilobytes (weight + activation row tiles)
+constexpr int packed_lds_bytes(int blocks) { return kRing * blocks * 1024 + kScaleSlots * kScaleSlotBytes; }
 
 template <int N>
 __device__ __forceinline__ void wait_vmem_le() {
@@ -72,21 +72,30 @@ __device__ __forceinline__ void barrier_lds() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-// One workgroup of four waves (WN x WM) computes a tile of NT*32 weight rows (n) x 256 activation
-// rows (m); a wave owns TN x TM accumulator tiles of 32 x 32.  Built as <8, 2, 2>: a 256 x 256
-// tile, waves 128 x 128.  (<7, 1, 4>, 224 x 256 tiles that fill two whole rounds of 256 CUs at
-// N = 14336, works and measured the same time: the kernel runs at the matrix pipes' power
-// limit, not at their issue limit, so fuller rounds buy nothing.)
-template <int NT, int WN, int WM>
+// One workgroup of four waves (WN x WM) computes a tile of NT*32 weight rows (n) x MT*32 activation
+// rows (m); a wave owns TN x TM accumulator tiles of 32 x 32.  A unit holds KW >= NT weight and MT
+// activation operand blocks (KW, MT multiples of 4 so that loads and scale pieces split evenly).
+//   <8, 8, 8, 2, 2>  256 x 256 tile, waves 128 x 128: large M, one workgroup per CU
+//   <4, 4, 4, 2, 2>  128 x 128 tile, waves 64 x 64, 80 KB of LDS: two workgroups per CU; used when
+//                    the big tiles would leave most CUs idle (M of a few hundred rows)
+// (<7, 8, 8, 1, 4>, 224 x 256 tiles that fill two whole rounds of 256 CUs at N = 14336, works and
+// measured the same time as 256 x 256: the kernel runs at the matrix pipes' power limit, not at
+// their issue limit, so fuller rounds buy nothing.)
+template <int NT, int KW, int MT, int WN, int WM>
 __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int tiles_m) {
-  constexpr int BN = NT * 32, BM = 256;
+  constexpr int BN = NT * 32, BM = MT * 32;
   constexpr int NW = WN * WM;           // waves
-  static_assert(NW == 4 && NT <= 8 && NT % WN == 0 && 8 % WM == 0, "unsupported wave arrangement");
-  constexpr int TN = NT / WN, TM = 8 / WM;  // 32x32 MFMA tiles per wave along n and m
-  constexpr int kPer = 16 / NW;         // code loads per wave per unit
+  static_assert(NW == 4 && NT <= KW && KW % 4 == 0 && MT % 4 == 0 && NT % WN == 0 && MT % WM == 0,
+                "unsupported tile / wave arrangement");
+  constexpr int TN = NT / WN, TM = MT / WM;  // 32x32 MFMA tiles per wave along n and m
+  constexpr int kBlocks = KW + MT;      // operand kilobytes per unit
+  constexpr int kPer = kBlocks / NW;    // code loads per wave per unit
+  constexpr int kPieces = kBlocks / 4;  // 1 KB scale pieces (4 row tiles each) per 256-K block
+  constexpr int kUnitBytes = kBlocks * 1024;
+  constexpr int kPackedLds = packed_lds_bytes(kBlocks);
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
   constexpr int kScaleBase = kRing * kUnitBytes;
@@ -107,31 +116,34 @@ __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
   const int nu = K >> 6, nkb = K >> 8;          // units, scale blocks
   const int rt_n = (N + 31) >> 5, rt_m = (M + 31) >> 5;
 
-  // ---- loads.  Operand b of a unit: b < 8 weight row tile tile_n*NT + b, else activation row tile
-  // tile_m*8 + b - 8 (clamped at the edge: those rows are never stored; with NT = 7 the eighth
-  // weight row tile is loaded and not used, which keeps every wave's load count the same).
+  // ---- loads.  Operand b of a unit: b < KW weight row tile tile_n*NT + b, else activation row tile
+  // tile_m*MT + b - KW (clamped at the edge: those rows are never stored; weight row tiles past NT
+  // are loaded and not used, which keeps every wave's load count the same).
   // Wave w loads operands w*kPer .. w*kPer + kPer - 1.
   const uint8_t* op_base[kPer];
 #pragma unroll
   for (int j = 0; j < kPer; ++j) {
     const int b = wave * kPer + j;
-    if (b < 8) {
+    if (b < KW) {
       const int rt = min(tile_n * NT + b, rt_n - 1);
       op_base[j] = wq + (size_t)rt * nu * 1024;
     } else {
-      const int rt = min(tile_m * 8 + b - 8, rt_m - 1);
+      const int rt = min(tile_m * MT + b - KW, rt_m - 1);
       op_base[j] = xq + (size_t)rt * nu * 1024;
     }
   }
-  // Scale piece w (0..3) of a block, loaded by wave w: w < 2 weight row tiles 4w..4w+3, else
-  // activation row tiles 4(w-2)..; one load instruction, lane L fetches 16 bytes of row tile L / 16.
-  const int sc_rt = min((wave < 2 ? tile_n * NT : tile_m * 8) + (wave & 1) * 4 + (lane >> 4),
-                        (wave < 2 ? rt_n : rt_m) - 1);
+  // Scale piece p of a block (4 row tiles, one load instruction, lane L fetches 16 bytes of row tile
+  // L / 16): p < KW/4 weight row tiles 4p.., else activation row tiles 4(p - KW/4)...  Wave w
+  // loads piece w % kPieces into kilobyte w of the slot (with fewer pieces than waves the copies in
+  // the upper kilobytes are never read: every wave issues the same instructions, no branch).
+  const int sc_piece = wave % kPieces;
+  const bool sc_w = sc_piece < KW / 4;
+  const int sc_rt = min(sc_w ? tile_n * NT + sc_piece * 4 + (lane >> 4) : tile_m * MT + (sc_piece - KW / 4) * 4 + (lane >> 4),
+                        (sc_w ? rt_n : rt_m) - 1);
   const uint32_t sc_off = (uint32_t)sc_rt * (uint32_t)nkb * 256u + (lane & 15) * 16;
   const uint32_t lane16 = lane * 16;
 
-  static_assert(NW == 4, "one scale piece per wave");
-  const uint8_t* sc_base = wave < 2 ? ws : xs;
+  const uint8_t* sc_base = sc_w ? ws : xs;
   // Unit u into its ring slot; with every fourth unit travel the scales of the block it opens
   // (wave w brings piece w), issued first so that they have landed whenever the unit has.
   auto issue_unit = [&](int u, bool with_scales) {
@@ -157,8 +169,8 @@ __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
   // ahead, of the next one
   uint4 aq[2][TN], bq[2][TM];
   int sa[TN], sb[TM], sa_next[TN], sb_next[TM];
-  const int a_off = (wn * TN) * 1024 + lane * 16, b_off = (8 + wm * TM) * 1024 + lane * 16;
-  const int sa_off = kScaleBase + (wn * TN) * 256 + lane * 4, sb_off = kScaleBase + (8 + wm * TM) * 256 + lane * 4;
+  const int a_off = (wn * TN) * 1024 + lane * 16, b_off = (KW + wm * TM) * 1024 + lane * 16;
+  const int sa_off = kScaleBase + (wn * TN) * 256 + lane * 4, sb_off = kScaleBase + (KW + wm * TM) * 256 + lane * 4;
   auto read_unit = [&](int u, int set) {
     const uint8_t* base = smem + (u % kRing) * kUnitBytes;
 #pragma unroll
@@ -201,7 +213,7 @@ __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
     }                                                                                               \
     __builtin_amdgcn_sched_barrier(0);                                                              \
   }
-  constexpr int kHand = TM >= 4 ? 1 : 2;  // rows of MFMAs (4 instructions) ahead of the hand-over
+  constexpr int kHand = (TM >= 4 || TN <= 2) ? 1 : 2;  // rows of MFMAs ahead of the hand-over
   // ALLOWED: loads of this wave that may still be outstanding while unit u + 1 is complete
 #define FPQ_UNIT(Q, U, ALLOWED, ISSUE, READ, READ_SCALES)                                           \
   {                                                                                                 \
@@ -283,24 +295,29 @@ extern "C" int fpq_pack_mxf4(const void* codes, const void* scales, int64_t scal
 }
 
 namespace fpq {
-template <int NT, int WN, int WM>
+template <int NT, int KW, int MT, int WN, int WM>
 static int launch_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                          const void* bias, void* y, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
-  const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + NT * 32 - 1) / (NT * 32));
+  constexpr int kLds = packed_lds_bytes(KW + MT);
+  const int tiles_m = (int)((M + MT * 32 - 1) / (MT * 32)), tiles_n = (int)((N + NT * 32 - 1) / (NT * 32));
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_mxf4_packed_kernel<NT, WN, WM>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kPackedLds);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mxf4_packed_kernel<NT, KW, MT, WN, WM>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  hipLaunchKernelGGL((gemm_mxf4_packed_kernel<NT, WN, WM>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256),
-                     kPackedLds, stream, (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq,
+  hipLaunchKernelGGL((gemm_mxf4_packed_kernel<NT, KW, MT, WN, WM>), dim3((unsigned)(tiles_m * tiles_n)),
+                     dim3(256), kLds, stream, (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq,
                      (const uint8_t*)ws, alpha, (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K,
                      tiles_m);
   return (int)hipGetLastError();
 }
 }  // namespace fpq
+
+#ifndef FPQ_PACKED_SMALL_BELOW
+#define FPQ_PACKED_SMALL_BELOW 192  // 256x256 tiles from this many of them on, else 128x128 tiles
+#endif
 
 extern "C" int fpq_gemm_mxf4_packed(const void* xq, const void* xs, const void* wq, const void* ws,
                                     const float* alpha, const void* bias, void* y, int64_t M,
@@ -317,5 +334,8 @@ extern "C" int fpq_gemm_mxf4_packed(const void* xq, const void* xs, const void* 
   if (((uintptr_t)xq & 15u) || ((uintptr_t)wq & 15u) || ((uintptr_t)xs & 15u) || ((uintptr_t)ws & 15u) ||
       ((uintptr_t)y & 15u))
     return FPQ_E_ALIGN;
-  return launch_packed<8, 2, 2>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
+  const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  if (big_tiles < FPQ_PACKED_SMALL_BELOW)
+    return launch_packed<4, 4, 4, 2, 2>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
+  return launch_packed<8, 8, 8, 2, 2>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
 }
