@@ -30,8 +30,6 @@ typedef unsigned v4u __attribute__((ext_vector_type(4)));
 #ifndef FPQ_SPLITK_MAX_M
 #define FPQ_SPLITK_MAX_M 64  // largest M served by the weight-streaming split-K kernel
 #endif
-typedef _Float16 v2h __attribute__((ext_vector_type(2)));
-typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 __device__ __forceinline__ uint16_t bf16_bits_rne(float f) {
   uint32_t b = __float_as_uint(f);
@@ -602,20 +600,6 @@ struct NvLdsLayout {
   static constexpr int kScalesX = kScalesW + BN * kScaleBytes;
   static constexpr int kStage = kScalesX + BM * kScaleBytes;
 };
-
-// e4m3 byte (>= 0) -> the same value * 2^-8 as fp16, in both halves of a dword
-__device__ __forceinline__ v2h e4m3_pair_f16(uint32_t byte) {
-  const uint32_t h = (byte << 7) & 0x3f80u;
-  return __builtin_bit_cast(v2h, h | (h << 16));
-}
-
-__device__ __forceinline__ v8h dequant8_f16_s(uint32_t codes, v2h s2) {
-  const v2h p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 0) * s2;
-  const v2h p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 1) * s2;
-  const v2h p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 2) * s2;
-  const v2h p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 3) * s2;
-  return v8h{p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
-}
 
 template <int BN, int BM>
 __global__ __launch_bounds__(256) void gemm_nvf4_lds_kernel(

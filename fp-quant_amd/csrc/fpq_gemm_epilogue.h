@@ -13,6 +13,24 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void global_void;
 
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+// NVFP4 operands for the fp16 MFMA.  e4m3 byte (>= 0) -> the same value * 2^-8 as fp16, in both
+// halves of a dword (bits above the byte are ignored) ...
+__device__ __forceinline__ v2h e4m3_pair_f16(uint32_t byte) {
+  const uint32_t h = (byte << 7) & 0x3f80u;
+  return __builtin_bit_cast(v2h, h | (h << 16));
+}
+// ... and 8 E2M1 codes (one dword) times that scale -> 8 exact fp16 values (code * 2^8 * scale * 2^-8)
+__device__ __forceinline__ v8h dequant8_f16_s(uint32_t codes, v2h s2) {
+  const v2h p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 0) * s2;
+  const v2h p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 1) * s2;
+  const v2h p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 2) * s2;
+  const v2h p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 3) * s2;
+  return v8h{p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
+}
+
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 

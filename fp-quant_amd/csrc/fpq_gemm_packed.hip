@@ -30,7 +30,8 @@ namespace fpq {
 // ---------------------------------------------------------------------------------------------
 // Row-major -> packed.  One workgroup re-tiles 32 rows x 256 K: reads are 128-byte row segments,
 // writes cover 4 KB of codes and 256 B of scales contiguously.
-__global__ __launch_bounds__(256) void pack_mxf4_kernel(const uint8_t* __restrict__ codes,
+template <bool NV>
+__global__ __launch_bounds__(256) void pack_fp4_kernel(const uint8_t* __restrict__ codes,
                                                         const uint8_t* __restrict__ scales,
                                                         int64_t scale_stride, int rows, int K,
                                                         uint8_t* __restrict__ pcodes,
@@ -46,21 +47,42 @@ __global__ __launch_bounds__(256) void pack_mxf4_kernel(const uint8_t* __restric
   if (t < 64) {
     const int sr = t & 31, skh = t >> 5;
     const int srow = rt * 32 + sr;
-    uint32_t out = 0u;
-    if (srow < rows) {
-      const uint8_t* sp = scales + (size_t)srow * scale_stride + kb * 8 + skh;
-      out = (uint32_t)sp[0] | ((uint32_t)sp[2] << 8) | ((uint32_t)sp[4] << 16) | ((uint32_t)sp[6] << 24);
+    if (NV) {
+      // 16 E4M3 bytes per row and 256 K; K step q, half kh uses bytes 4q + 2kh and 4q + 2kh + 1
+      uint32_t lo = 0u, hi = 0u;
+      if (srow < rows) {
+        const uint8_t* sp = scales + (size_t)srow * scale_stride + kb * 16 + 2 * skh;
+        lo = (uint32_t)sp[0] | ((uint32_t)sp[1] << 8) | ((uint32_t)sp[4] << 16) | ((uint32_t)sp[5] << 24);
+        hi = (uint32_t)sp[8] | ((uint32_t)sp[9] << 8) | ((uint32_t)sp[12] << 16) | ((uint32_t)sp[13] << 24);
+      }
+      *(uint2*)(pscales + (((size_t)rt * (K >> 8) + kb) * 64 + t) * 8) = make_uint2(lo, hi);
+    } else {
+      uint32_t out = 0u;
+      if (srow < rows) {
+        const uint8_t* sp = scales + (size_t)srow * scale_stride + kb * 8 + skh;
+        out = (uint32_t)sp[0] | ((uint32_t)sp[2] << 8) | ((uint32_t)sp[4] << 16) | ((uint32_t)sp[6] << 24);
+      }
+      *(uint32_t*)(pscales + (((size_t)rt * (K >> 8) + kb) * 64 + t) * 4) = out;
     }
-    *(uint32_t*)(pscales + (((size_t)rt * (K >> 8) + kb) * 64 + t) * 4) = out;
   }
 }
 
 // ---------------------------------------------------------------------------------------------
 constexpr int kRing = 8;                 // 64-K units resident or in flight
-constexpr int kScaleSlots = 4;           // 256-K scale blocks resident or in flight
-constexpr int kScaleSlotBytes = 16 * 256;
+// Scales of a 256-K block: 256 bytes per row tile for MXFP4 (one E8M0 byte per lane and K step), 512
+// for NVFP4 (two E4M3 bytes per lane and K step).  They travel with the first unit of their block,
+// issued eight units ahead, and are read into registers one unit before the block starts, so the
+// slot a block lands in was last read several hand-overs (barriers) earlier: 2 slots would do.
+constexpr int kScaleSlots = 4;
+constexpr int scale_block_bytes(bool nv) { return nv ? 512 : 256; }
+constexpr int scale_slot_bytes(int blocks, bool nv) {
+  return (blocks * scale_block_bytes(nv) > 4096 ? blocks * scale_block_bytes(nv) : 4096);
+}
+constexpr int scale_slots(bool nv) { return nv ? 2 : kScaleSlots; }
 // LDS of a workgroup whose unit holds `blocks` operand kilobytes (weight + activation row tiles)
-constexpr int packed_lds_bytes(int blocks) { return kRing * blocks * 1024 + kScaleSlots * kScaleSlotBytes; }
+constexpr int packed_lds_bytes(int blocks, bool nv = false) {
+  return kRing * blocks * 1024 + scale_slots(nv) * scale_slot_bytes(blocks, nv);
+}
 
 template <int N>
 __device__ __forceinline__ void wait_vmem_le() {
@@ -81,7 +103,11 @@ __device__ __forceinline__ void barrier_lds() {
 // (<7, 8, 8, 1, 4>, 224 x 256 tiles that fill two whole rounds of 256 CUs at N = 14336, works and
 // measured the same time as 256 x 256: the kernel runs at the matrix pipes' power limit, not at
 // their issue limit, so fuller rounds buy nothing.)
-template <int NT, int KW, int MT, int WN, int WM>
+// NV = true: NVFP4 operands (same packed codes; E4M3 scales, two bytes per lane and K step, 512-byte
+// scale blocks): codes are dequantized in registers to exact fp16 and fed to the fp16 MFMA; a lane's
+// dword s of a block goes to MFMA s of the unit on both operands, so the K order is permuted
+// consistently and the sum is complete.
+template <int NT, int KW, int MT, int WN, int WM, bool NV = false>
 __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p,
@@ -93,9 +119,13 @@ __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
   constexpr int TN = NT / WN, TM = MT / WM;  // 32x32 MFMA tiles per wave along n and m
   constexpr int kBlocks = KW + MT;      // operand kilobytes per unit
   constexpr int kPer = kBlocks / NW;    // code loads per wave per unit
-  constexpr int kPieces = kBlocks / 4;  // 1 KB scale pieces (4 row tiles each) per 256-K block
+  constexpr int kSB = scale_block_bytes(NV);            // scale bytes per row tile and 256-K block
+  constexpr int kRpp = 1024 / kSB;                      // row tiles per 1 KB scale piece
+  constexpr int kPieces = kBlocks / kRpp;               // scale pieces per 256-K block
+  constexpr int kScLoads = kPieces >= NW ? kPieces / NW : 1;  // scale loads per wave per block
+  constexpr int kSlots = scale_slots(NV), kSlotBytes = scale_slot_bytes(kBlocks, NV);
   constexpr int kUnitBytes = kBlocks * 1024;
-  constexpr int kPackedLds = packed_lds_bytes(kBlocks);
+  constexpr int kPackedLds = packed_lds_bytes(kBlocks, NV);
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
   constexpr int kScaleBase = kRing * kUnitBytes;
@@ -132,25 +162,33 @@ __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
       op_base[j] = xq + (size_t)rt * nu * 1024;
     }
   }
-  // Scale piece p of a block (4 row tiles, one load instruction, lane L fetches 16 bytes of row tile
-  // L / 16): p < KW/4 weight row tiles 4p.., else activation row tiles 4(p - KW/4)...  Wave w
-  // loads piece w % kPieces into kilobyte w of the slot (with fewer pieces than waves the copies in
-  // the upper kilobytes are never read: every wave issues the same instructions, no branch).
-  const int sc_piece = wave % kPieces;
-  const bool sc_w = sc_piece < KW / 4;
-  const int sc_rt = min(sc_w ? tile_n * NT + sc_piece * 4 + (lane >> 4) : tile_m * MT + (sc_piece - KW / 4) * 4 + (lane >> 4),
-                        (sc_w ? rt_n : rt_m) - 1);
-  const uint32_t sc_off = (uint32_t)sc_rt * (uint32_t)nkb * 256u + (lane & 15) * 16;
+  // Scale piece p of a block: one load instruction for kRpp row tiles (unit operand order), lane L
+  // fetches 16 bytes of row tile L / (64 / kRpp).  Wave w loads pieces (w*kScLoads + j) % kPieces
+  // into kilobyte w*kScLoads + j of the slot (with fewer pieces than waves the copies in the upper
+  // kilobytes are never read: every wave issues the same instructions, no branch).
+  const uint8_t* sc_base[kScLoads];
+  uint32_t sc_off[kScLoads];
+#pragma unroll
+  for (int j = 0; j < kScLoads; ++j) {
+    const int fb = ((wave * kScLoads + j) % kPieces) * kRpp;   // first operand block of the piece
+    const bool is_w = fb < KW;
+    constexpr int kLpr = 64 / kRpp;                            // lanes per row tile
+    const int rt = min((is_w ? tile_n * NT + fb : tile_m * MT + fb - KW) + (int)(lane / kLpr),
+                       (is_w ? rt_n : rt_m) - 1);
+    sc_base[j] = is_w ? ws : xs;
+    sc_off[j] = (uint32_t)rt * (uint32_t)nkb * (uint32_t)kSB + (lane % kLpr) * 16;
+  }
   const uint32_t lane16 = lane * 16;
 
-  const uint8_t* sc_base = sc_w ? ws : xs;
-  // Unit u into its ring slot; with every fourth unit travel the scales of the block it opens
-  // (wave w brings piece w), issued first so that they have landed whenever the unit has.
+  // Unit u into its ring slot; with every fourth unit travel the scales of the block it opens,
+  // issued first so that they have landed whenever the unit has.
   auto issue_unit = [&](int u, bool with_scales) {
     if (with_scales) {
       const int blk = u >> 2;
-      lds_dma16(sc_base + (size_t)blk * 256, sc_off,
-                smem_base + kScaleBase + (blk % kScaleSlots) * kScaleSlotBytes + wave * 1024);
+#pragma unroll
+      for (int j = 0; j < kScLoads; ++j)
+        lds_dma16(sc_base[j] + (size_t)blk * kSB, sc_off[j],
+                  smem_base + kScaleBase + (blk % kSlots) * kSlotBytes + (wave * kScLoads + j) * 1024);
     }
     const uint32_t dst = smem_base + (u % kRing) * kUnitBytes + wave * kPer * 1024;
 #pragma unroll
@@ -168,9 +206,10 @@ __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
   // operand registers of the current and the next unit; scales of the current block and, read
   // ahead, of the next one
   uint4 aq[2][TN], bq[2][TM];
-  int sa[TN], sb[TM], sa_next[TN], sb_next[TM];
+  uint2 sa[TN], sb[TM], sa_next[TN], sb_next[TM];   // MXFP4 uses .x only
   const int a_off = (wn * TN) * 1024 + lane * 16, b_off = (KW + wm * TM) * 1024 + lane * 16;
-  const int sa_off = kScaleBase + (wn * TN) * 256 + lane * 4, sb_off = kScaleBase + (KW + wm * TM) * 256 + lane * 4;
+  const int sa_off = kScaleBase + (wn * TN) * kSB + lane * (kSB / 64);
+  const int sb_off = kScaleBase + (KW + wm * TM) * kSB + lane * (kSB / 64);
   auto read_unit = [&](int u, int set) {
     const uint8_t* base = smem + (u % kRing) * kUnitBytes;
 #pragma unroll
@@ -179,11 +218,18 @@ __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
     for (int i = 0; i < TN; ++i) aq[set][i] = *(const uint4*)(base + a_off + i * 1024);
   };
   auto read_scales = [&](int blk) {
-    const uint8_t* base = smem + (blk % kScaleSlots) * kScaleSlotBytes;
+    const uint8_t* base = smem + (blk % kSlots) * kSlotBytes;
+    if (NV) {
 #pragma unroll
-    for (int j = 0; j < TM; ++j) sb_next[j] = *(const int*)(base + sb_off + j * 256);
+      for (int j = 0; j < TM; ++j) sb_next[j] = *(const uint2*)(base + sb_off + j * kSB);
 #pragma unroll
-    for (int i = 0; i < TN; ++i) sa_next[i] = *(const int*)(base + sa_off + i * 256);
+      for (int i = 0; i < TN; ++i) sa_next[i] = *(const uint2*)(base + sa_off + i * kSB);
+    } else {
+#pragma unroll
+      for (int j = 0; j < TM; ++j) sb_next[j].x = *(const uint32_t*)(base + sb_off + j * kSB);
+#pragma unroll
+      for (int i = 0; i < TN; ++i) sa_next[i].x = *(const uint32_t*)(base + sa_off + i * kSB);
+    }
   };
 
   // ---- prologue: the first kRing units (scales of blocks 0 and 1 with units 0 and 4)
@@ -202,21 +248,44 @@ __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
   // must have landed for everyone before it is read into the other register set.  The code
   // between two hand-overs is branch-free (the compiler must not move MFMAs across them).
 #define FPQ_MFMA_ROW(Q, I)                                                                          \
-  {                                                                                                 \
+  if constexpr (NV) {                                                                               \
+    const uint4 av = aq[(Q) & 1][I];                                                                \
+    const uint32_t aw[4] = {av.x, av.y, av.z, av.w};                                                \
+    const uint32_t asc = ((Q) < 2 ? sa[I].x : sa[I].y) >> (16 * ((Q) & 1));                         \
+    _Pragma("unroll") for (int s4 = 0; s4 < 4; ++s4) {                                              \
+      const v8h ah = dequant8_f16_s(aw[s4], e4m3_pair_f16(asc >> (8 * (s4 >> 1))));                 \
+      _Pragma("unroll") for (int j = 0; j < TM; ++j)                                                \
+        acc[I][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[j][s4], acc[I][j], 0, 0, 0);      \
+    }                                                                                               \
+    __builtin_amdgcn_sched_barrier(0);                                                              \
+  } else {                                                                                          \
     const uint4 av = aq[(Q) & 1][I];                                                                \
     const v8i a = v8i{(int)av.x, (int)av.y, (int)av.z, (int)av.w, 0, 0, 0, 0};                      \
     _Pragma("unroll") for (int j = 0; j < TM; ++j) {                                                \
       const uint4 bv = bq[(Q) & 1][j];                                                              \
       const v8i b = v8i{(int)bv.x, (int)bv.y, (int)bv.z, (int)bv.w, 0, 0, 0, 0};                    \
-      acc[I][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[I][j], 4, 4, Q, sa[I], \
-                                                                  Q, sb[j]);                        \
+      acc[I][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[I][j], 4, 4, Q,        \
+                                                                  (int)sa[I].x, Q, (int)sb[j].x);   \
     }                                                                                               \
     __builtin_amdgcn_sched_barrier(0);                                                              \
+  }
+  // NVFP4: the activation operands of the unit, dequantized once for all rows of MFMAs
+  v8h bh[NV ? TM : 1][4];
+#define FPQ_PREP_B(Q)                                                                               \
+  if constexpr (NV) {                                                                               \
+    _Pragma("unroll") for (int j = 0; j < TM; ++j) {                                                \
+      const uint4 bv = bq[(Q) & 1][j];                                                              \
+      const uint32_t bw[4] = {bv.x, bv.y, bv.z, bv.w};                                              \
+      const uint32_t bsc = ((Q) < 2 ? sb[j].x : sb[j].y) >> (16 * ((Q) & 1));                       \
+      _Pragma("unroll") for (int s4 = 0; s4 < 4; ++s4)                                              \
+        bh[j][s4] = dequant8_f16_s(bw[s4], e4m3_pair_f16(bsc >> (8 * (s4 >> 1))));                  \
+    }                                                                                               \
   }
   constexpr int kHand = (TM >= 4 || TN <= 2) ? 1 : 2;  // rows of MFMAs ahead of the hand-over
   // ALLOWED: loads of this wave that may still be outstanding while unit u + 1 is complete
 #define FPQ_UNIT(Q, U, ALLOWED, ISSUE, READ, READ_SCALES)                                           \
   {                                                                                                 \
+    FPQ_PREP_B(Q)                                                                                   \
     _Pragma("unroll") for (int i0 = 0; i0 < kHand; ++i0) FPQ_MFMA_ROW(Q, i0)                        \
     wait_vmem_le<(ALLOWED)>();                                                                      \
     barrier_lds();                                                                                  \
@@ -261,6 +330,7 @@ __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
     FPQ_UNIT(3, u0 + 3, 0, false, false, false)
   }
 #undef FPQ_UNIT
+#undef FPQ_PREP_B
 #undef FPQ_MFMA_ROW
 #undef FPQ_TAKE_SCALES
 
@@ -268,6 +338,76 @@ __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
                                           wave, lane, M, N);
 }
 
+}  // namespace fpq
+
+namespace fpq {
+template <int NT, int KW, int MT, int WN, int WM, bool NV>
+static int launch_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
+                         const void* bias, void* y, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
+  constexpr int kLds = packed_lds_bytes(KW + MT, NV);
+  const int tiles_m = (int)((M + MT * 32 - 1) / (MT * 32)), tiles_n = (int)((N + NT * 32 - 1) / (NT * 32));
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_mxf4_packed_kernel<NT, KW, MT, WN, WM, NV>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((gemm_mxf4_packed_kernel<NT, KW, MT, WN, WM, NV>), dim3((unsigned)(tiles_m * tiles_n)),
+                     dim3(256), kLds, stream, (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq,
+                     (const uint8_t*)ws, alpha, (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K,
+                     tiles_m);
+  return (int)hipGetLastError();
+}
+
+template <bool NV>
+static int gemm_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
+                       const void* bias, void* y, int64_t M, int64_t N, int64_t K, void* stream);
+
+template <bool NV>
+static int pack_operand(const void* codes, const void* scales, int64_t scale_stride, int64_t rows, int64_t K,
+                        void* packed_codes, void* packed_scales, void* stream) {
+  constexpr int GROUP = NV ? 16 : 32;
+  if (rows < 0 || K < 0) return FPQ_E_SHAPE;
+  if (rows == 0) return FPQ_OK;
+  if (!codes || !scales || !packed_codes || !packed_scales) return FPQ_E_NULL;
+  if (K == 0 || K % 256 != 0 || scale_stride < K / GROUP) return FPQ_E_SHAPE;
+  if (rows > (1 << 24) || K > (1 << 24)) return FPQ_E_SHAPE;
+  if (((uintptr_t)codes & 15u) || ((uintptr_t)packed_codes & 15u) || ((uintptr_t)packed_scales & 7u))
+    return FPQ_E_ALIGN;
+  const dim3 grid((unsigned)(K / 256), (unsigned)((rows + 31) / 32));
+  hipLaunchKernelGGL(pack_fp4_kernel<NV>, grid, dim3(256), 0, (hipStream_t)stream, (const uint8_t*)codes,
+                     (const uint8_t*)scales, scale_stride, (int)rows, (int)K, (uint8_t*)packed_codes,
+                     (uint8_t*)packed_scales);
+  return (int)hipGetLastError();
+}
+}  // namespace fpq
+
+#ifndef FPQ_PACKED_SMALL_BELOW
+#define FPQ_PACKED_SMALL_BELOW 192  // 256x256 tiles from this many of them on, else 128x128 tiles
+#endif
+
+namespace fpq {
+template <bool NV>
+static int gemm_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
+                       const void* bias, void* y, int64_t M, int64_t N, int64_t K, void* stream) {
+  if (M < 0 || N < 0 || K < 0) return FPQ_E_SHAPE;
+  if (M == 0 || N == 0) return FPQ_OK;
+  if (!xq || !xs || !wq || !ws || !alpha || !y) return FPQ_E_NULL;
+  if (K == 0 || K % 256 != 0) return FPQ_E_SHAPE;
+  if (M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return FPQ_E_SHAPE;
+  // scale offsets inside one operand are 32-bit
+  const int64_t sdiv = NV ? 16 : 32;
+  if (((M + 31) / 32) * 32 * (K / sdiv) >= ((int64_t)1 << 32) || ((N + 31) / 32) * 32 * (K / sdiv) >= ((int64_t)1 << 32))
+    return FPQ_E_SHAPE;
+  if (((uintptr_t)xq & 15u) || ((uintptr_t)wq & 15u) || ((uintptr_t)xs & 15u) || ((uintptr_t)ws & 15u) ||
+      ((uintptr_t)y & 15u))
+    return FPQ_E_ALIGN;
+  const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  if (big_tiles < FPQ_PACKED_SMALL_BELOW)
+    return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
+  return launch_packed<8, 8, 8, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
+}
 }  // namespace fpq
 
 extern "C" int64_t fpq_packed_codes_bytes(int64_t rows, int64_t K) {
@@ -278,64 +418,28 @@ extern "C" int64_t fpq_packed_scales_bytes(int64_t rows, int64_t K) {
   return ((rows + 31) / 32) * 32 * (K / 32);
 }
 
+extern "C" int64_t fpq_packed_scales_bytes_nv(int64_t rows, int64_t K) {
+  return ((rows + 31) / 32) * 32 * (K / 16);
+}
+
 extern "C" int fpq_pack_mxf4(const void* codes, const void* scales, int64_t scale_stride, int64_t rows,
                              int64_t K, void* packed_codes, void* packed_scales, void* stream) {
-  if (rows < 0 || K < 0) return FPQ_E_SHAPE;
-  if (rows == 0) return FPQ_OK;
-  if (!codes || !scales || !packed_codes || !packed_scales) return FPQ_E_NULL;
-  if (K == 0 || K % 256 != 0 || scale_stride < K / 32) return FPQ_E_SHAPE;
-  if (rows > (1 << 24) || K > (1 << 24)) return FPQ_E_SHAPE;
-  if (((uintptr_t)codes & 15u) || ((uintptr_t)packed_codes & 15u) || ((uintptr_t)packed_scales & 3u))
-    return FPQ_E_ALIGN;
-  const dim3 grid((unsigned)(K / 256), (unsigned)((rows + 31) / 32));
-  hipLaunchKernelGGL(fpq::pack_mxf4_kernel, grid, dim3(256), 0, (hipStream_t)stream,
-                     (const uint8_t*)codes, (const uint8_t*)scales, scale_stride, (int)rows, (int)K,
-                     (uint8_t*)packed_codes, (uint8_t*)packed_scales);
-  return (int)hipGetLastError();
+  return fpq::pack_operand<false>(codes, scales, scale_stride, rows, K, packed_codes, packed_scales, stream);
 }
 
-namespace fpq {
-template <int NT, int KW, int MT, int WN, int WM>
-static int launch_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
-                         const void* bias, void* y, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
-  constexpr int kLds = packed_lds_bytes(KW + MT);
-  const int tiles_m = (int)((M + MT * 32 - 1) / (MT * 32)), tiles_n = (int)((N + NT * 32 - 1) / (NT * 32));
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_mxf4_packed_kernel<NT, KW, MT, WN, WM>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e != hipSuccess) return (int)e;
-    attr_set = true;
-  }
-  hipLaunchKernelGGL((gemm_mxf4_packed_kernel<NT, KW, MT, WN, WM>), dim3((unsigned)(tiles_m * tiles_n)),
-                     dim3(256), kLds, stream, (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq,
-                     (const uint8_t*)ws, alpha, (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K,
-                     tiles_m);
-  return (int)hipGetLastError();
+extern "C" int fpq_pack_nvf4(const void* codes, const void* scales, int64_t scale_stride, int64_t rows,
+                             int64_t K, void* packed_codes, void* packed_scales, void* stream) {
+  return fpq::pack_operand<true>(codes, scales, scale_stride, rows, K, packed_codes, packed_scales, stream);
 }
-}  // namespace fpq
-
-#ifndef FPQ_PACKED_SMALL_BELOW
-#define FPQ_PACKED_SMALL_BELOW 192  // 256x256 tiles from this many of them on, else 128x128 tiles
-#endif
 
 extern "C" int fpq_gemm_mxf4_packed(const void* xq, const void* xs, const void* wq, const void* ws,
                                     const float* alpha, const void* bias, void* y, int64_t M,
                                     int64_t N, int64_t K, void* stream) {
-  using namespace fpq;
-  if (M < 0 || N < 0 || K < 0) return FPQ_E_SHAPE;
-  if (M == 0 || N == 0) return FPQ_OK;
-  if (!xq || !xs || !wq || !ws || !alpha || !y) return FPQ_E_NULL;
-  if (K == 0 || K % 256 != 0) return FPQ_E_SHAPE;
-  if (M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return FPQ_E_SHAPE;
-  // scale offsets inside one operand are 32-bit
-  if (fpq_packed_scales_bytes(M, K) >= ((int64_t)1 << 32) || fpq_packed_scales_bytes(N, K) >= ((int64_t)1 << 32))
-    return FPQ_E_SHAPE;
-  if (((uintptr_t)xq & 15u) || ((uintptr_t)wq & 15u) || ((uintptr_t)xs & 15u) || ((uintptr_t)ws & 15u) ||
-      ((uintptr_t)y & 15u))
-    return FPQ_E_ALIGN;
-  const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  if (big_tiles < FPQ_PACKED_SMALL_BELOW)
-    return launch_packed<4, 4, 4, 2, 2>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
-  return launch_packed<8, 8, 8, 2, 2>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
+  return fpq::gemm_packed<false>(xq, xs, wq, ws, alpha, bias, y, M, N, K, stream);
+}
+
+extern "C" int fpq_gemm_nvf4_packed(const void* xq, const void* xs, const void* wq, const void* ws,
+                                    const float* alpha, const void* bias, void* y, int64_t M,
+                                    int64_t N, int64_t K, void* stream) {
+  return fpq::gemm_packed<true>(xq, xs, wq, ws, alpha, bias, y, M, N, K, stream);
 }

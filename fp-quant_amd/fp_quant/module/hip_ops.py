@@ -252,7 +252,9 @@ def _(x_flat, hadamard_matrix, global_scale):
 # re-tiled weights are made once per weight tensor and kept next to it, which doubles the memory
 # held by 4-bit weights; FPQ_PACKED_WEIGHTS=0 keeps every call on the row-major kernels.
 PACKED_MIN_M = 256         # GEMM operator on row-major operands (pays for re-tiling the activations)
-PACKED_LINEAR_MIN_M = 65   # fused linear: activations are quantized straight into the packed layout
+NV_PACKED_MIN_M = 32       # NVFP4 fused linear: from here on (and while the 128x128 tiles apply) packed
+PACKED_LINEAR_MIN_M = 25   # fused linear: activations are quantized straight into the packed layout
+#                            (below, the weight-streaming split-K kernel on row-major operands is faster)
 
 
 def packed_weights_enabled() -> bool:
@@ -271,13 +273,32 @@ def pack_mxf4(codes: torch.Tensor, scales: torch.Tensor, rows: int, k: int) -> T
     return pc, ps
 
 
-def packed_weight(wq: torch.Tensor, ws: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+def pack_nvf4(codes: torch.Tensor, scales: torch.Tensor, rows: int, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Row-major codes [rows, k/2] and E4M3 scales [>=rows, >=k/16] -> the packed layout of
+    fpq_gemm_nvf4_packed."""
+    lib = _engine.lib()
+    pc = torch.empty(lib.fpq_packed_codes_bytes(rows, k), dtype=torch.uint8, device=codes.device)
+    ps = torch.empty(lib.fpq_packed_scales_bytes_nv(rows, k), dtype=torch.uint8, device=codes.device)
+    st = lib.fpq_pack_nvf4(codes.data_ptr(), scales.data_ptr(), scales.shape[1], rows, k,
+                           pc.data_ptr(), ps.data_ptr(), _stream(codes))
+    _engine.check(st, "fpq_pack_nvf4")
+    return pc, ps
+
+
+def nv_packed_eligible(m: int, n: int, k: int) -> bool:
+    """NVFP4: the packed kernel wins where its 128x128 tiles apply (mid-sized M); large M runs at
+    the same speed on row-major operands, tiny M is faster on the direct kernel."""
+    return (NV_PACKED_MIN_M <= m and k % 256 == 0 and packed_weights_enabled()
+            and ((m + 255) // 256) * ((n + 255) // 256) < 192)
+
+
+def packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """Packed copy of a weight, cached on the code tensor until either tensor is written to."""
-    key = (wq.data_ptr(), wq._version, ws.data_ptr(), ws._version, tuple(wq.shape))
+    key = (wq.data_ptr(), wq._version, ws.data_ptr(), ws._version, tuple(wq.shape), nvfp4)
     hit = getattr(wq, "_fpq_packed", None)
     if hit is not None and hit[0] == key:
         return hit[1], hit[2]
-    pc, ps = pack_mxf4(wq, ws, wq.shape[0], wq.shape[1] * 2)
+    pc, ps = (pack_nvf4 if nvfp4 else pack_mxf4)(wq, ws, wq.shape[0], wq.shape[1] * 2)
     try:
         wq._fpq_packed = (key, pc, ps)
     except (AttributeError, RuntimeError):
@@ -474,6 +495,13 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
         st = lib.fpq_quantize_nv(x_flat.data_ptr(), m, k, kind, g, norm, h.data_ptr(), gs.data_ptr(),
                                  codes.data_ptr(), scales.data_ptr(), m, k // group, ZERO_NIBBLE_POLICY, stream)
         _engine.check(st, "fpq_quantize_nv")
+        if nv_packed_eligible(m, n, k):
+            xp, xsp = pack_nvf4(codes, scales, m, k)
+            wp, wsp = packed_weight(wq, ws, True)
+            st = lib.fpq_gemm_nvf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
+                                          alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
+            _engine.check(st, "fpq_gemm_nvf4_packed")
+            return y
         st = lib.fpq_gemm_nvf4(codes.data_ptr(), scales.data_ptr(), k // group, wq.data_ptr(), ws.data_ptr(),
                                ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
         _engine.check(st, "fpq_gemm_nvf4")

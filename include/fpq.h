@@ -157,6 +157,21 @@ int fpq_gemm_mxf4_packed(const void* xq_packed, const void* xs_packed, const voi
 int fpq_test_e2m1(const float* in, uint8_t* out, int64_t n, int zero_policy, void* stream);
 
 /*
+ * NVFP4 on the packed layout: codes exactly as for MXFP4; scales in blocks (rt, kb) of 512 bytes at
+ * byte (rt * K/256 + kb) * 512, the 8 bytes at (32 kh + r) * 8 being, for K step q = 0..3 of the
+ * block, the two E4M3 bytes of row 32 rt + r, groups 16 kb + 4 q + 2 kh and + 1 (bytes 2q, 2q + 1).
+ * fpq_pack_nvf4 converts from the row-major layout of fpq_quantize_nv; fpq_gemm_nvf4_packed is
+ * fpq_gemm_nvf4 on packed operands (same arithmetic: exact fp16 dequantization, fp32 accumulation in
+ * another K order).  Stands in for qutlass.matmul_nvf4_bf16_tn (qutlass_ops.py:149-168).
+ */
+int64_t fpq_packed_scales_bytes_nv(int64_t rows, int64_t K);
+int fpq_pack_nvf4(const void* codes, const void* scales, int64_t scale_stride, int64_t rows,
+                  int64_t K, void* packed_codes, void* packed_scales, void* stream);
+int fpq_gemm_nvf4_packed(const void* xq_packed, const void* xs_packed, const void* wq_packed,
+                         const void* ws_packed, const float* alpha, const void* bias, void* y,
+                         int64_t M, int64_t N, int64_t K, void* stream);
+
+/*
  * Measurement hook: `blocks` workgroups of four waves run `iters` x 16 FP4 32x32x64 block-scaled
  * matrix instructions per wave on register-resident operands (words: blocks*256*32 ints of operand
  * bits; sink: blocks*256 floats; clocks: per workgroup the elapsed shader-clock cycles and 100 MHz

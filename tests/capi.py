@@ -131,3 +131,32 @@ def quantize_quest(x_bf16, rot="hadamard", g=128, norm=None, h=None, zero_policy
     _engine.check(st, "fpq_quantize_mx_quest")
     torch.cuda.synchronize()
     return codes.cpu(), scales.cpu(), (mask.cpu() if want_mask else None)
+
+
+def pack_nv(codes, scales, fill=0xCD):
+    """fpq_pack_nvf4 on row-major codes [R, K/2] and E4M3 scales [>=R, >=K/16]; CPU uint8 results."""
+    lib = _engine.lib()
+    codes, scales = codes.to("cuda").contiguous(), scales.to("cuda").contiguous()
+    rows, k = codes.shape[0], codes.shape[1] * 2
+    pc = torch.full((lib.fpq_packed_codes_bytes(rows, k),), fill, dtype=torch.uint8, device="cuda")
+    ps = torch.full((lib.fpq_packed_scales_bytes_nv(rows, k),), fill, dtype=torch.uint8, device="cuda")
+    st = lib.fpq_pack_nvf4(codes.data_ptr(), scales.data_ptr(), scales.shape[1], rows, k, pc.data_ptr(),
+                           ps.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_pack_nvf4")
+    torch.cuda.synchronize()
+    return pc.cpu(), ps.cpu()
+
+
+def gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=None):
+    """fpq_gemm_nvf4_packed on packed operands; bf16 [M, N] on the CPU."""
+    lib = _engine.lib()
+    xp, xsp, wp, wsp = (t.to("cuda").contiguous() for t in (xp, xsp, wp, wsp))
+    y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    a = torch.tensor([alpha], dtype=torch.float32, device="cuda")
+    b = bias.to("cuda").contiguous() if bias is not None else None
+    st = lib.fpq_gemm_nvf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(), a.data_ptr(),
+                                  b.data_ptr() if b is not None else None, y.data_ptr(), m, n, k,
+                                  torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_gemm_nvf4_packed")
+    torch.cuda.synchronize()
+    return y.cpu()

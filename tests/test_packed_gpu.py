@@ -136,3 +136,79 @@ def test_linear_uses_packed_path_and_matches_row_major(monkeypatch):
     monkeypatch.setenv("FPQ_PACKED_WEIGHTS", "0")
     y_rm = lin(x)
     assert torch.equal(y_packed, y_rm)
+
+
+def pack_nv_by_definition(codes, scales, k):
+    """NVFP4 packed scales as include/fpq.h states them: [(rt, kb), (kh, r), q, 2 bytes] = row 32 rt + r,
+    groups 16 kb + 4 q + 2 kh (+1); codes as for MXFP4."""
+    rows = codes.shape[0]
+    rt = (rows + 31) // 32
+    pc, _ = pack_by_definition(codes, torch.zeros(rows, k // 32, dtype=torch.uint8), k)
+    s = torch.zeros(rt * 32, k // 16, dtype=torch.uint8)
+    s[:rows] = scales[:rows, : k // 16]
+    ps = s.view(rt, 32, k // 256, 4, 2, 2).permute(0, 2, 4, 1, 3, 5).contiguous().view(-1)
+    return pc, ps
+
+
+@pytest.mark.parametrize("rows,k", [(32, 256), (70, 512), (257, 768)])
+def test_pack_nv_kernel_matches_definition(rows, k):
+    g = torch.Generator().manual_seed(rows * 3 + k)
+    codes = torch.randint(0, 256, (rows, k // 2), dtype=torch.uint8, generator=g)
+    scales = torch.randint(0, 127, (rows + 5, k // 16 + 16), dtype=torch.uint8, generator=g)
+    pc, ps = capi.pack_nv(codes, scales)
+    wc, ws = pack_nv_by_definition(codes, scales, k)
+    assert torch.equal(pc, wc)
+    assert torch.equal(ps, ws)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 64, 256), (32, 32, 256), (65, 100, 512), (256, 256, 768), (300, 520, 1024),
+                                   (512, 256, 4096)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_gemm_nv_packed_matches_oracle(m, n, k, bias):
+    g = torch.Generator().manual_seed(m + 2 * n + k)
+    xq = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=g)
+    wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=g)
+    xs = torch.randint(1, 0x7f, (m, k // 16), dtype=torch.uint8, generator=g)    # every positive E4M3 value
+    ws = torch.randint(24, 72, (n, k // 16), dtype=torch.uint8, generator=g)
+    b = torch.randn(n, generator=g).to(torch.bfloat16) if bias else None
+    alpha = 2.0 ** -6
+    xp, xsp = pack_nv_by_definition(xq, xs, k)
+    wp, wsp = pack_nv_by_definition(wq, ws, k)
+    y = capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=b)
+    assert not torch.isnan(y.float()).any()
+    ref, mag = O.gemm_ref(xq, xs, wq, ws, alpha, "nvfp4")
+    want = ref.to(torch.bfloat16)
+    if bias:
+        want = want + b
+    # one bf16 rounding of a sum accumulated in another order; with bias a second rounding on top
+    tol = (2.0 if bias else 1.0) * 2.0 ** -7 * torch.maximum(want.double().abs(), ref.abs()) + 1e-5 * mag + 1e-6
+    assert ((y.double() - want.double()).abs() <= tol).all()
+    exact = (y.view(torch.int16) == want.view(torch.int16)).double().mean()
+    assert exact > 0.97
+
+
+def test_nvfp4_linear_mid_m_runs_packed_and_matches_oracle(monkeypatch):
+    import fp_quant
+    from fp_quant.module import hip_ops
+    cfg = fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype.NVFP4, forward_method="abs_max",
+                                 backward_dtype=fp_quant.FPQuantDtype.BF16, hadamard_group_size=16)
+    gen = torch.Generator().manual_seed(21)
+    k, n, m = 512, 384, 100
+    w = (torch.randn(n, k, generator=gen) * 0.02).to(torch.bfloat16)
+    x = torch.randn(m, k, generator=gen).to(torch.bfloat16)
+    lin = fp_quant.FPQuantLinear(k, n, cfg, bias=False, device="cuda", dtype=torch.bfloat16)
+    lin.weight.data = w.cuda()
+    lin.pre_forward()
+    assert hip_ops.nv_packed_eligible(m, n, k)
+    y = lin(x.cuda()).cpu()
+    assert getattr(lin.qweight, "_fpq_packed", None) is not None
+    gs = float(lin.act_global_scale)
+    norm = float(O.hadamard_matrix(16)[0, 0])
+    wq, ws, _ = O.quantize_nv(w, gs, O.ROT_HADAMARD, 16, norm)
+    xq, xs, _ = O.quantize_nv(x, gs, O.ROT_HADAMARD, 16, norm)
+    alpha = O.alpha_from_global_scales(lin.weight_global_scale.cpu(), lin.act_global_scale.cpu())
+    ref, mag = O.gemm_ref(xq, xs, wq, ws, alpha, "nvfp4")
+    assert ((y.double() - ref).abs() <= 2.0 ** -8 * ref.abs() + 1e-5 * mag + 1e-6).all()
+    monkeypatch.setenv("FPQ_PACKED_WEIGHTS", "0")
+    y_rm = lin(x.cuda()).cpu()
+    assert ((y.double() - y_rm.double()).abs() <= 2.0 ** -7 * ref.abs() + 1e-5 * mag + 1e-6).all()
