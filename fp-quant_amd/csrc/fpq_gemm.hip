@@ -266,6 +266,114 @@ __global__ __launch_bounds__(256) void gemm_mxf4_splitk_kernel(
   }
 }
 
+// The same weight-streaming scheme for NVFP4: a lane's 16 bytes of codes (32 K values) carry two
+// E4M3 scales; per batch of four 128-K steps a row's 32 scale bytes arrive as two 16-byte loads.
+// Dword s of every code load feeds fp16 MFMA s of the step on both operands (K order permuted
+// consistently), after exact in-register dequantization to fp16.
+template <int TN, int TM>
+__global__ __launch_bounds__(256) void gemm_nvf4_splitk_kernel(
+    const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, int xs_stride,
+    const uint8_t* __restrict__ wq, const uint8_t* __restrict__ ws, int ws_stride,
+    const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias, uint16_t* __restrict__ y,
+    int M, int N, int K) {
+  __shared__ v4f part[3][TN][TM][64];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int r = lane & 15, kb = lane >> 4;
+  const int n0 = blockIdx.x * TN * 16, m0 = blockIdx.y * TM * 16;
+  const int kbytes = K >> 1;
+  const int kq = K >> 2;                       // K range of this wave: [wave * kq, wave * kq + kq)
+  const int steps = kq >> 7;                   // 128 K per step (four fp16 MFMAs)
+
+  const uint8_t* wp[TN];
+  const uint8_t* wsp[TN];
+#pragma unroll
+  for (int i = 0; i < TN; ++i) {
+    const int n = min(n0 + i * 16 + r, N - 1);
+    wp[i] = wq + (size_t)n * kbytes + ((wave * kq) >> 1) + kb * 16;
+    wsp[i] = ws + (size_t)n * ws_stride + ((wave * kq) >> 4);
+  }
+  const uint8_t* xp[TM];
+  const uint8_t* xsp[TM];
+#pragma unroll
+  for (int j = 0; j < TM; ++j) {
+    const int m = min(m0 + j * 16 + r, M - 1);
+    xp[j] = xq + (size_t)m * kbytes + ((wave * kq) >> 1) + kb * 16;
+    xsp[j] = xs + (size_t)m * xs_stride + ((wave * kq) >> 4);
+  }
+  v4f acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  for (int s0 = 0; s0 < steps; s0 += 4) {  // steps is a multiple of 4
+    uint4 a[4][TN], b[4][TM], sa8[2][TN], sb8[2][TM];
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+      sa8[0][i] = *(const uint4*)(wsp[i] + s0 * 8);
+      sa8[1][i] = *(const uint4*)(wsp[i] + s0 * 8 + 16);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const v4u ld = __builtin_nontemporal_load((const v4u*)(wp[i] + (s0 + u) * 64));
+        a[u][i] = make_uint4(ld.x, ld.y, ld.z, ld.w);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      sb8[0][j] = *(const uint4*)(xsp[j] + s0 * 8);
+      sb8[1][j] = *(const uint4*)(xsp[j] + s0 * 8 + 16);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) b[u][j] = *(const uint4*)(xp[j] + (s0 + u) * 64);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      // step u: scale bytes 8 (u % 2) + 2 kb and + 1 of 16-byte load u / 2
+      v8h bh[TM][4];
+#pragma unroll
+      for (int j = 0; j < TM; ++j) {
+        const uint4 s4 = sb8[u >> 1][j];
+        const uint32_t lo = (u & 1) ? s4.z : s4.x, hi = (u & 1) ? s4.w : s4.y;
+        const uint32_t two = ((kb & 2) ? hi : lo) >> (16 * (kb & 1));
+        const uint4 c = b[u][j];
+        bh[j][0] = dequant8_f16_s(c.x, e4m3_pair_f16(two));
+        bh[j][1] = dequant8_f16_s(c.y, e4m3_pair_f16(two));
+        bh[j][2] = dequant8_f16_s(c.z, e4m3_pair_f16(two >> 8));
+        bh[j][3] = dequant8_f16_s(c.w, e4m3_pair_f16(two >> 8));
+      }
+#pragma unroll
+      for (int i = 0; i < TN; ++i) {
+        const uint4 s4 = sa8[u >> 1][i];
+        const uint32_t lo = (u & 1) ? s4.z : s4.x, hi = (u & 1) ? s4.w : s4.y;
+        const uint32_t two = ((kb & 2) ? hi : lo) >> (16 * (kb & 1));
+        const uint4 c = a[u][i];
+        const uint32_t cw[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const v8h ah = dequant8_f16_s(cw[s], e4m3_pair_f16(two >> (8 * (s >> 1))));
+#pragma unroll
+          for (int j = 0; j < TM; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, bh[j][s], acc[i][j], 0, 0, 0);
+        }
+      }
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < TM; ++j) part[wave - 1][i][j][lane] = acc[i][j];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < TM; ++j)
+        acc[i][j] = ((acc[i][j] + part[0][i][j][lane]) + part[1][i][j][lane]) + part[2][i][j][lane];
+    store_tile<TN, TM>(acc, y, bias, *alpha_p, n0, m0, M, N, r, kb);
+  }
+}
+
 // -------------------------------------------------------------------------------------------
 // LDS-tiled MXFP4 kernel for large M.  A block of 4 waves (2 x 2) owns a BN x BM output tile and
 // walks K in steps of 256 (one 128-byte line of codes per row).  Packed codes and scale bytes go
@@ -815,6 +923,24 @@ static int gemm_dispatch(const void* xq, const void* xs, int64_t xs_stride, cons
   } while (0)
   // K % 2048 == 0: every wave's K quarter is a whole number of 4-step batches and every 16-byte
   // scale load is aligned (scale strides and bases must be 16-byte multiples too)
+#define FPQ_SPLITK_NV(TNN, TMM)                                                                    \
+  do {                                                                                             \
+    const dim3 grid((unsigned)((N + TNN * 16 - 1) / (TNN * 16)),                                   \
+                    (unsigned)((M + TMM * 16 - 1) / (TMM * 16)));                                  \
+    hipLaunchKernelGGL((gemm_nvf4_splitk_kernel<TNN, TMM>), grid, dim3(256), 0, stream,            \
+                       (const uint8_t*)xq, (const uint8_t*)xs, (int)xs_stride, (const uint8_t*)wq, \
+                       (const uint8_t*)ws, (int)ws_stride, alpha, (const uint16_t*)bias,           \
+                       (uint16_t*)y, (int)M, (int)N, (int)K);                                      \
+    return (int)hipGetLastError();                                                                 \
+  } while (0)
+  if (FMT == 1 && K % 2048 == 0 && M <= 64 && xs_stride % 16 == 0 && ws_stride % 16 == 0 &&
+      !((uintptr_t)xs & 15u) && !((uintptr_t)ws & 15u)) {
+    if (M == 1) FPQ_SPLITK_NV(1, 1);
+    if (M <= 16) FPQ_SPLITK_NV(2, 1);
+    if (M <= 32) FPQ_SPLITK_NV(2, 2);
+    FPQ_SPLITK_NV(2, 4);
+  }
+#undef FPQ_SPLITK_NV
   if (FMT == 0 && K % 2048 == 0 && M <= FPQ_SPLITK_MAX_M && xs_stride % 16 == 0 && ws_stride % 16 == 0 &&
       !((uintptr_t)xs & 15u) && !((uintptr_t)ws & 15u)) {
     // 32 weight rows per workgroup once there is more than one activation row: halves the

@@ -252,7 +252,8 @@ def _(x_flat, hadamard_matrix, global_scale):
 # re-tiled weights are made once per weight tensor and kept next to it, which doubles the memory
 # held by 4-bit weights; FPQ_PACKED_WEIGHTS=0 keeps every call on the row-major kernels.
 PACKED_MIN_M = 256         # GEMM operator on row-major operands (pays for re-tiling the activations)
-NV_PACKED_MIN_M = 32       # NVFP4 fused linear: from here on (and while the 128x128 tiles apply) packed
+NV_PACKED_MIN_M = 65       # NVFP4 fused linear: from here on (and while the 128x128 tiles apply) packed;
+#                            below, the split-K weight-streaming kernel on row-major operands is faster
 PACKED_LINEAR_MIN_M = 25   # fused linear: activations are quantized straight into the packed layout
 #                            (below, the weight-streaming split-K kernel on row-major operands is faster)
 
