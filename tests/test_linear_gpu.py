@@ -218,3 +218,35 @@ def test_meta_replacement_then_realquant_checkpoint(tmp_path):
     missing, unexpected = dst.load_state_dict(load_file(path, device="cuda"), strict=True)
     assert not missing and not unexpected
     assert torch.equal(dst(x), want)
+
+
+@pytest.mark.parametrize("fmt,g,m", [("mxfp4", 128, 1), ("mxfp4", 128, 200), ("nvfp4", 16, 8), ("nvfp4", 16, 100)])
+def test_forward_is_graph_capturable(fmt, g, m):
+    """After one eager warm-up call (rotation classified, alpha and packed weights cached) a forward
+    records into a HIP graph: no host synchronisation, no allocation outside torch's capture pool.
+    Replays, interleaved with eager work, must equal eager results on the new input contents."""
+    import fp_quant
+    torch.manual_seed(11)
+    lin = fp_quant.FPQuantLinear(512, 256, _cfg(fmt, g), bias=True, device="cuda", dtype=torch.bfloat16)
+    lin.weight.data.normal_(0, 0.02)
+    lin.bias.data.normal_()
+    lin.pre_forward()
+    static_x = torch.randn(m, 512, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        lin(static_x)                                  # warm-up outside the capture
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            lin(static_x)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_y = lin(static_x)
+        for rep in range(3):
+            fresh = torch.randn(m, 512, device="cuda", dtype=torch.bfloat16)
+            want = lin(fresh)                          # eager work between replays
+            torch.cuda.synchronize()
+            static_x.copy_(fresh)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_y, want), rep
