@@ -99,7 +99,9 @@ __device__ __forceinline__ void barrier_lds() {
 // activation operand blocks (KW, MT multiples of 4 so that loads and scale pieces split evenly).
 //   <8, 8, 8, 2, 2>  256 x 256 tile, waves 128 x 128: large M, one workgroup per CU
 //   <4, 4, 4, 2, 2>  128 x 128 tile, waves 64 x 64, 80 KB of LDS: two workgroups per CU; used when
-//                    the big tiles would leave most CUs idle (M of a few hundred rows)
+//                    the big tiles would leave most CUs idle (M of a few hundred rows).  Its time
+//                    has a floor of about 12 us at K = 4096; two K steps per hand-over and a ring
+//                    twice as deep were both built and measured the same, so neither is kept.
 // (<7, 8, 8, 1, 4>, 224 x 256 tiles that fill two whole rounds of 256 CUs at N = 14336, works and
 // measured the same time as 256 x 256: the kernel runs at the matrix pipes' power limit, not at
 // their issue limit, so fuller rounds buy nothing.)
@@ -129,6 +131,7 @@ __global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
   constexpr int kScaleBase = kRing * kUnitBytes;
+  static_assert(kScaleBase + kSlots * kSlotBytes == kPackedLds, "LDS map does not match the allocation");
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   // Consecutive workgroup ids land on different XCDs (8 of them, each with its own L2): give
