@@ -56,8 +56,9 @@ def time_kernel(torch, fn, n_variants, steps, warmup):
     return wall, e0.elapsed_time(e1) / steps
 
 
-def bench_quantize(torch, fmt, rows, cols, g, steps, warmup, seed):
-    """Fused rotate+quantize on rotating input buffers through the C ABI."""
+def bench_quantize(torch, fmt, rows, cols, g, steps, warmup, seed, packed=False):
+    """Fused rotate+quantize on rotating input buffers through the C ABI (packed: MXFP4 written in the
+    packed GEMM operand layout, same bytes in another order)."""
     from fp_quant import _engine
     lib = _engine.lib()
     dev = torch.device("cuda:0")
@@ -79,7 +80,9 @@ def bench_quantize(torch, fmt, rows, cols, g, steps, warmup, seed):
 
     def run(i):
         xp, cp, sp = ptrs[i]
-        if fmt == "mxfp4":
+        if fmt == "mxfp4" and packed:
+            st = lib.fpq_quantize_mx_packed(xp, rows, cols, 0, g, norm, cp, sp, 0, stream)
+        elif fmt == "mxfp4":
             st = lib.fpq_quantize_mx(xp, rows, cols, 0, g, norm, None, cp, sp, rows, cols // group, 0, stream)
         else:
             st = lib.fpq_quantize_nv(xp, rows, cols, 0, g, norm, None, gs.data_ptr(), cp, sp, rows,
@@ -90,7 +93,7 @@ def bench_quantize(torch, fmt, rows, cols, g, steps, warmup, seed):
     wall, ev = time_kernel(torch, run, n_buf, steps, warmup)
     algo_bytes = rows * cols * (2 + 0.5 + 1.0 / group)
     return {
-        "workload": f"{fmt}_quantize_{rows}x{cols}_had{g}",
+        "workload": f"{fmt}_quantize_{rows}x{cols}_had{g}" + ("_packed" if packed else ""),
         "ms_per_step": wall,
         "kernel_ms": ev,
         "algo_bytes": algo_bytes,
@@ -429,6 +432,8 @@ def main():
             out["nvfp4_quantize"] = bench_quantize(torch, "nvfp4", 8192, 4096, 16, args.steps, args.warmup, seed=1)
         if "mxfp4_quantize" in only:
             out["mxfp4_quantize"] = bench_quantize(torch, "mxfp4", 2048, 4096, 128, args.steps, args.warmup, seed=0)
+            out["mxfp4_quantize_packed"] = bench_quantize(torch, "mxfp4", 2048, 4096, 128, args.steps, args.warmup,
+                                                          seed=0, packed=True)
         for m in (2048, 128, 16, 1):
             if f"mxfp4_linear_M{m}" in only:
                 out[f"mxfp4_linear_M{m}"] = bench_linear(torch, "mxfp4", m, 14336, 4096, 128, args.steps,
@@ -446,6 +451,8 @@ def main():
     results = {}
     results["nvfp4_quantize"] = bench_quantize(torch, "nvfp4", 8192, 4096, 16, args.steps, args.warmup, seed=1)
     results["mxfp4_quantize"] = bench_quantize(torch, "mxfp4", 2048, 4096, 128, args.steps, args.warmup, seed=0)
+    results["mxfp4_quantize_packed"] = bench_quantize(torch, "mxfp4", 2048, 4096, 128, args.steps, args.warmup,
+                                                      seed=0, packed=True)
 
     linears = {}
     for m in (2048, 128, 16, 1):
