@@ -878,13 +878,8 @@ static int gemm_dispatch(const void* xq, const void* xs, int64_t xs_stride, cons
     constexpr int BN = 256, BM = 256;
     using L = NvLdsLayout<BN, BM>;
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
-    static bool nv_attr_set = false;
-    if (!nv_attr_set) {
-      hipError_t e = hipFuncSetAttribute((const void*)gemm_nvf4_lds_kernel<BN, BM>,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 2 * L::kStage);
-      if (e != hipSuccess) return (int)e;
-      nv_attr_set = true;
-    }
+    static LdsLimitOnce nv_lds_limit;
+    if (const int st = nv_lds_limit.ensure((const void*)gemm_nvf4_lds_kernel<BN, BM>, 2 * L::kStage)) return st;
     hipLaunchKernelGGL((gemm_nvf4_lds_kernel<BN, BM>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256),
                        2 * L::kStage, stream, (const uint8_t*)xq, (const uint8_t*)xs, (int)xs_stride,
                        (const uint8_t*)wq, (const uint8_t*)ws, (int)ws_stride, alpha,
@@ -897,13 +892,8 @@ static int gemm_dispatch(const void* xq, const void* xs, int64_t xs_stride, cons
     constexpr int BN = 256, BM = 256;
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
     using L = MxLdsLayout<BN, BM>;
-    static bool attr_set = false;
-    if (!attr_set) {
-      hipError_t e = hipFuncSetAttribute((const void*)gemm_mxf4_lds_kernel<BN, BM, FPQ_GEMM_WM>,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 2 * L::kStage);
-      if (e != hipSuccess) return (int)e;
-      attr_set = true;
-    }
+    static LdsLimitOnce mx_lds_limit;
+    if (const int st = mx_lds_limit.ensure((const void*)gemm_mxf4_lds_kernel<BN, BM, FPQ_GEMM_WM>, 2 * L::kStage)) return st;
     hipLaunchKernelGGL((gemm_mxf4_lds_kernel<BN, BM, FPQ_GEMM_WM>), dim3((unsigned)(tiles_m * tiles_n)),
                        dim3(128 * FPQ_GEMM_WM),
                        2 * L::kStage, stream, (const uint8_t*)xq, (const uint8_t*)xs, (int)xs_stride,

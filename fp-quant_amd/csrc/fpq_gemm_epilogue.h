@@ -4,7 +4,27 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace fpq {
+
+// Raises a kernel's dynamic-LDS limit once per device (the attribute is per device; one
+// function-local static instance per kernel lives in the launcher).  Safe from any host thread: a
+// race only repeats the idempotent call.
+struct LdsLimitOnce {
+  std::atomic<uint64_t> done{0};  // bit d: set for device d (devices >= 64 set it on every call)
+  int ensure(const void* kernel, int bytes) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    const uint64_t bit = dev < 64 ? (uint64_t)1 << dev : 0;
+    if (bit && (done.load(std::memory_order_acquire) & bit)) return 0;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return (int)e;
+    if (bit) done.fetch_or(bit, std::memory_order_release);
+    return 0;
+  }
+};
 
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));

@@ -110,7 +110,7 @@ __device__ __forceinline__ void barrier_lds() {
 // dword s of a block goes to MFMA s of the unit on both operands, so the K order is permuted
 // consistently and the sum is complete.
 template <int NT, int KW, int MT, int WN, int WM, bool NV = false>
-__global__ __launch_bounds__(256) void gemm_mxf4_packed_kernel(
+__global__ __launch_bounds__(256) void gemm_fp4_packed_kernel(
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int tiles_m) {
@@ -349,14 +349,9 @@ static int launch_packed(const void* xq, const void* xs, const void* wq, const v
                          const void* bias, void* y, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
   constexpr int kLds = packed_lds_bytes(KW + MT, NV);
   const int tiles_m = (int)((M + MT * 32 - 1) / (MT * 32)), tiles_n = (int)((N + NT * 32 - 1) / (NT * 32));
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_mxf4_packed_kernel<NT, KW, MT, WN, WM, NV>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e != hipSuccess) return (int)e;
-    attr_set = true;
-  }
-  hipLaunchKernelGGL((gemm_mxf4_packed_kernel<NT, KW, MT, WN, WM, NV>), dim3((unsigned)(tiles_m * tiles_n)),
+  static LdsLimitOnce lds_limit;
+  if (const int st = lds_limit.ensure((const void*)gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV>, kLds)) return st;
+  hipLaunchKernelGGL((gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV>), dim3((unsigned)(tiles_m * tiles_n)),
                      dim3(256), kLds, stream, (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq,
                      (const uint8_t*)ws, alpha, (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K,
                      tiles_m);
