@@ -247,11 +247,11 @@ def _(x_flat, hadamard_matrix, global_scale):
 
 ### GEMMs
 
-# From this many activation rows on, the MXFP4 GEMM runs on operands re-tiled into the order the
+# From these many activation rows on, the MXFP4 GEMM runs on operands re-tiled into the order the
 # matrix instructions consume them (bit-identical results, contiguous operand fetch).  The
 # re-tiled weights are made once per weight tensor and kept next to it, which doubles the memory
 # held by 4-bit weights; FPQ_PACKED_WEIGHTS=0 keeps every call on the row-major kernels.
-PACKED_MIN_M = 256         # GEMM operator on row-major operands (pays for re-tiling the activations)
+PACKED_MIN_M = 48          # GEMM operator on row-major operands (pays for re-tiling the activations)
 NV_PACKED_MIN_M = 65       # NVFP4 fused linear: from here on (and while the 128x128 tiles apply) packed;
 #                            below, the split-K weight-streaming kernel on row-major operands is faster
 PACKED_LINEAR_MIN_M = 25   # fused linear: activations are quantized straight into the packed layout
@@ -343,6 +343,15 @@ def _gemm(entry: str, x, w, xs, ws, alpha, bias: Optional[torch.Tensor], group: 
                 xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(), a.data_ptr(), b_ptr,
                 y.data_ptr(), m, n, k, _stream(x))
         _engine.check(st, "fpq_gemm_mxf4_packed")
+        return y
+    if entry == "fpq_gemm_nvf4" and nv_packed_eligible(m, n, k):
+        with torch.cuda.device(x.device):
+            wp, wsp = packed_weight(wq, ws_b, True)
+            xp, xsp = pack_nvf4(xq, xs_b, m, k)
+            st = _engine.lib().fpq_gemm_nvf4_packed(
+                xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(), a.data_ptr(), b_ptr,
+                y.data_ptr(), m, n, k, _stream(x))
+        _engine.check(st, "fpq_gemm_nvf4_packed")
         return y
     with torch.cuda.device(x.device):
         st = getattr(_engine.lib(), entry)(
