@@ -80,8 +80,14 @@ constexpr int scale_slot_bytes(int blocks, bool nv) {
 }
 constexpr int scale_slots(bool nv) { return nv ? 2 : kScaleSlots; }
 // LDS of a workgroup whose unit holds `blocks` operand kilobytes (weight + activation row tiles)
-constexpr int packed_lds_bytes(int blocks, bool nv = false) {
-  return kRing * blocks * 1024 + scale_slots(nv) * scale_slot_bytes(blocks, nv);
+constexpr int packed_lds_bytes(int blocks, bool nv = false, int ring = kRing) {
+  return ring * blocks * 1024 + scale_slots(nv) * scale_slot_bytes(blocks, nv);
+}
+// ... and what is allocated: at least the epilogue's staging area (four waves, each WT_M rows of
+// WT_N bf16 + 16 bytes)
+constexpr int packed_lds_alloc(int blocks, bool nv, int ring, int wt_n, int wt_m) {
+  return packed_lds_bytes(blocks, nv, ring) > 4 * wt_m * (wt_n * 2 + 16) ? packed_lds_bytes(blocks, nv, ring)
+                                                                         : 4 * wt_m * (wt_n * 2 + 16);
 }
 
 template <int N>
@@ -97,7 +103,12 @@ __device__ __forceinline__ void barrier_lds() {
 // One workgroup of four waves (WN x WM) computes a tile of NT*32 weight rows (n) x MT*32 activation
 // rows (m); a wave owns TN x TM accumulator tiles of 32 x 32.  A unit holds KW >= NT weight and MT
 // activation operand blocks (KW, MT multiples of 4 so that loads and scale pieces split evenly).
-//   <8, 8, 8, 2, 2>  256 x 256 tile, waves 128 x 128: large M, one workgroup per CU
+//   <8, 8, 4, 2, 2>  256 x 128 tile, waves 128 x 64, ring of 4 units, 68 KB of LDS and 193 registers:
+//                    two workgroups per CU.  Large M, MXFP4: while one workgroup stores its tile
+//                    the other keeps the matrix pipes busy, which is worth more than the 1.5x
+//                    operand traffic costs (62.4 us against 66.1 us at M = 2048, N = 14336)
+//   <8, 8, 8, 2, 2>  256 x 256 tile, waves 128 x 128, one workgroup per CU: large M, NVFP4 (whose
+//                    limit is the register dequantization; half tiles measured mixed there)
 //   <4, 4, 4, 2, 2>  128 x 128 tile, waves 64 x 64, 80 KB of LDS: two workgroups per CU; used when
 //                    the big tiles would leave most CUs idle (M of a few hundred rows).  Its time
 //                    has a floor of about 12 us at K = 4096; two K steps per hand-over and a ring
@@ -109,8 +120,8 @@ __device__ __forceinline__ void barrier_lds() {
 // scale blocks): codes are dequantized in registers to exact fp16 and fed to the fp16 MFMA; a lane's
 // dword s of a block goes to MFMA s of the unit on both operands, so the K order is permuted
 // consistently and the sum is complete.
-template <int NT, int KW, int MT, int WN, int WM, bool NV = false>
-__global__ __launch_bounds__(256) void gemm_fp4_packed_kernel(
+template <int NT, int KW, int MT, int WN, int WM, bool NV = false, int RING = kRing>
+__global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_kernel(
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int tiles_m) {
@@ -127,10 +138,11 @@ __global__ __launch_bounds__(256) void gemm_fp4_packed_kernel(
   constexpr int kScLoads = kPieces >= NW ? kPieces / NW : 1;  // scale loads per wave per block
   constexpr int kSlots = scale_slots(NV), kSlotBytes = scale_slot_bytes(kBlocks, NV);
   constexpr int kUnitBytes = kBlocks * 1024;
-  constexpr int kPackedLds = packed_lds_bytes(kBlocks, NV);
+  static_assert(RING == 4 || RING == 8, "the ring holds one or two 256-K blocks");
+  constexpr int kPackedLds = packed_lds_bytes(kBlocks, NV, RING);
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
-  constexpr int kScaleBase = kRing * kUnitBytes;
+  constexpr int kScaleBase = RING * kUnitBytes;
   static_assert(kScaleBase + kSlots * kSlotBytes == kPackedLds, "LDS map does not match the allocation");
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -193,7 +205,7 @@ __global__ __launch_bounds__(256) void gemm_fp4_packed_kernel(
         lds_dma16(sc_base[j] + (size_t)blk * kSB, sc_off[j],
                   smem_base + kScaleBase + (blk % kSlots) * kSlotBytes + (wave * kScLoads + j) * 1024);
     }
-    const uint32_t dst = smem_base + (u % kRing) * kUnitBytes + wave * kPer * 1024;
+    const uint32_t dst = smem_base + (u % RING) * kUnitBytes + wave * kPer * 1024;
 #pragma unroll
     for (int j = 0; j < kPer; ++j) lds_dma16(op_base[j] + (size_t)u * 1024, lane16, dst + j * 1024);
   };
@@ -214,7 +226,7 @@ __global__ __launch_bounds__(256) void gemm_fp4_packed_kernel(
   const int sa_off = kScaleBase + (wn * TN) * kSB + lane * (kSB / 64);
   const int sb_off = kScaleBase + (KW + wm * TM) * kSB + lane * (kSB / 64);
   auto read_unit = [&](int u, int set) {
-    const uint8_t* base = smem + (u % kRing) * kUnitBytes;
+    const uint8_t* base = smem + (u % RING) * kUnitBytes;
 #pragma unroll
     for (int j = 0; j < TM; ++j) bq[set][j] = *(const uint4*)(base + b_off + j * 1024);
 #pragma unroll
@@ -235,19 +247,19 @@ __global__ __launch_bounds__(256) void gemm_fp4_packed_kernel(
     }
   };
 
-  // ---- prologue: the first kRing units (scales of blocks 0 and 1 with units 0 and 4)
-  const int n_pro = min(nu, kRing);
+  // ---- prologue: the first RING units (scales of blocks 0 and 1 with units 0 and 4)
+  const int n_pro = min(nu, RING);
   for (int u = 0; u < n_pro; ++u) issue_unit(u, (u & 3) == 0);
   // Loads complete in order: unit 0 and scale block 0 have landed once at most the loads of the
   // younger units are outstanding (a wave issues kPer per unit, one more with scales).
-  if (n_pro == kRing) wait_vmem_le<(kRing - 1) * kPer>();
+  if (n_pro == RING) wait_vmem_le<(RING - 1) * kPer>();
   else wait_vmem();
   barrier_lds();
   read_unit(0, 0);
   read_scales(0);
 
   // One 64-K unit: 16 MFMAs per wave.  After the first row of MFMAs comes the hand-over: every
-  // wave holds unit u in registers, so its ring slot is free for unit u + kRing, and unit u + 1
+  // wave holds unit u in registers, so its ring slot is free for unit u + RING, and unit u + 1
   // must have landed for everyone before it is read into the other register set.  The code
   // between two hand-overs is branch-free (the compiler must not move MFMAs across them).
 #define FPQ_MFMA_ROW(Q, I)                                                                          \
@@ -292,7 +304,7 @@ __global__ __launch_bounds__(256) void gemm_fp4_packed_kernel(
     _Pragma("unroll") for (int i0 = 0; i0 < kHand; ++i0) FPQ_MFMA_ROW(Q, i0)                        \
     wait_vmem_le<(ALLOWED)>();                                                                      \
     barrier_lds();                                                                                  \
-    if (ISSUE) issue_unit((U) + kRing, (Q) == 0);                                                   \
+    if (ISSUE) issue_unit((U) + RING, (Q) == 0);                                                   \
     if (READ) read_unit((U) + 1, ((Q) + 1) & 1);                                                    \
     if (READ_SCALES) read_scales(((U) + 1) >> 2);                                                   \
     __builtin_amdgcn_sched_barrier(0);                                                              \
@@ -304,25 +316,28 @@ __global__ __launch_bounds__(256) void gemm_fp4_packed_kernel(
     _Pragma("unroll") for (int j = 0; j < TM; ++j) sb[j] = sb_next[j];                              \
   }
 
-  // steady state: every unit of these blocks still has a unit kRing ahead of it to issue
-  const int kb_tail = max(nkb - kRing / 4, 0);
+  // steady state: every unit of these blocks still has a unit RING ahead of it to issue
+  constexpr int kDrain = RING / 4;   // blocks in the last ring of units
+  const int kb_tail = max(nkb - kDrain, 0);
   for (int kb = 0; kb < kb_tail; ++kb) {
     const int u0 = kb * 4;
     FPQ_TAKE_SCALES()
-    FPQ_UNIT(0, u0 + 0, (kRing - 2) * kPer, true, true, false)
-    FPQ_UNIT(1, u0 + 1, (kRing - 2) * kPer, true, true, false)
-    FPQ_UNIT(2, u0 + 2, (kRing - 2) * kPer, true, true, false)
-    FPQ_UNIT(3, u0 + 3, (kRing - 2) * kPer, true, true, true)
+    FPQ_UNIT(0, u0 + 0, (RING - 2) * kPer, true, true, false)
+    FPQ_UNIT(1, u0 + 1, (RING - 2) * kPer, true, true, false)
+    FPQ_UNIT(2, u0 + 2, (RING - 2) * kPer, true, true, false)
+    FPQ_UNIT(3, u0 + 3, (RING - 2) * kPer, true, true, true)
   }
-  // drain: the last kRing units (fewer if K is short); nothing is issued any more, and with t
+  // drain: the last ring of units (fewer if K is short); nothing is issued any more, and with t
   // units to go after unit u + 1 exactly t * kPer loads may stay outstanding
-  if (nkb >= 2) {
-    const int u0 = (nkb - 2) * 4;
-    FPQ_TAKE_SCALES()
-    FPQ_UNIT(0, u0 + 0, 6 * kPer, false, true, false)
-    FPQ_UNIT(1, u0 + 1, 5 * kPer, false, true, false)
-    FPQ_UNIT(2, u0 + 2, 4 * kPer, false, true, false)
-    FPQ_UNIT(3, u0 + 3, 3 * kPer, false, true, true)
+  if constexpr (RING == 8) {
+    if (nkb >= 2) {
+      const int u0 = (nkb - 2) * 4;
+      FPQ_TAKE_SCALES()
+      FPQ_UNIT(0, u0 + 0, 6 * kPer, false, true, false)
+      FPQ_UNIT(1, u0 + 1, 5 * kPer, false, true, false)
+      FPQ_UNIT(2, u0 + 2, 4 * kPer, false, true, false)
+      FPQ_UNIT(3, u0 + 3, 3 * kPer, false, true, true)
+    }
   }
   {
     const int u0 = (nkb - 1) * 4;
@@ -337,21 +352,21 @@ __global__ __launch_bounds__(256) void gemm_fp4_packed_kernel(
 #undef FPQ_MFMA_ROW
 #undef FPQ_TAKE_SCALES
 
-  wave_tile_store<TN, TM, kPackedLds, NW>(acc, smem, y, bias, alpha_p, n_blk + wn * TN * 32, m_blk + wm * TM * 32,
+  wave_tile_store<TN, TM, packed_lds_alloc(kBlocks, NV, RING, TN * 32, TM * 32), NW>(acc, smem, y, bias, alpha_p, n_blk + wn * TN * 32, m_blk + wm * TM * 32,
                                           wave, lane, M, N);
 }
 
 }  // namespace fpq
 
 namespace fpq {
-template <int NT, int KW, int MT, int WN, int WM, bool NV>
+template <int NT, int KW, int MT, int WN, int WM, bool NV, int RING = kRing>
 static int launch_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                          const void* bias, void* y, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
-  constexpr int kLds = packed_lds_bytes(KW + MT, NV);
+  constexpr int kLds = packed_lds_alloc(KW + MT, NV, RING, NT / WN * 32, MT / WM * 32);
   const int tiles_m = (int)((M + MT * 32 - 1) / (MT * 32)), tiles_n = (int)((N + NT * 32 - 1) / (NT * 32));
   static LdsLimitOnce lds_limit;
-  if (const int st = lds_limit.ensure((const void*)gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV>, kLds)) return st;
-  hipLaunchKernelGGL((gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV>), dim3((unsigned)(tiles_m * tiles_n)),
+  if (const int st = lds_limit.ensure((const void*)gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV, RING>, kLds)) return st;
+  hipLaunchKernelGGL((gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV, RING>), dim3((unsigned)(tiles_m * tiles_n)),
                      dim3(256), kLds, stream, (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq,
                      (const uint8_t*)ws, alpha, (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K,
                      tiles_m);
@@ -381,6 +396,9 @@ static int pack_operand(const void* codes, const void* scales, int64_t scale_str
 }
 }  // namespace fpq
 
+#ifndef FPQ_PACKED_HALF_TILES
+#define FPQ_PACKED_HALF_TILES 1  // large M: 1 = 256x128 tiles for MXFP4, 2 = for NVFP4 too, 0 = 256x256
+#endif
 #ifndef FPQ_PACKED_SMALL_BELOW
 #define FPQ_PACKED_SMALL_BELOW 192  // 256x256 tiles from this many of them on, else 128x128 tiles
 #endif
@@ -404,6 +422,10 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
   if (big_tiles < FPQ_PACKED_SMALL_BELOW)
     return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
+#if FPQ_PACKED_HALF_TILES
+  if (!NV || FPQ_PACKED_HALF_TILES > 1)
+    return launch_packed<8, 8, 4, 2, 2, NV, 4>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
+#endif
   return launch_packed<8, 8, 8, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
 }
 }  // namespace fpq
