@@ -400,7 +400,7 @@ static int pack_operand(const void* codes, const void* scales, int64_t scale_str
 #define FPQ_PACKED_HALF_TILES 1  // large M: 1 = 256x128 tiles for MXFP4, 2 = for NVFP4 too, 0 = 256x256
 #endif
 #ifndef FPQ_PACKED_SMALL_BELOW
-#define FPQ_PACKED_SMALL_BELOW 192  // 256x256 tiles from this many of them on, else 128x128 tiles
+#define FPQ_PACKED_SMALL_BELOW 100  // fewer 256x256 tiles than this (under about 200 of 256x128): 128x128 tiles
 #endif
 
 namespace fpq {

@@ -290,7 +290,7 @@ def nv_packed_eligible(m: int, n: int, k: int) -> bool:
     """NVFP4: the packed kernel wins where its 128x128 tiles apply (mid-sized M); large M runs at
     the same speed on row-major operands, tiny M is faster on the direct kernel."""
     return (NV_PACKED_MIN_M <= m and k % 256 == 0 and packed_weights_enabled()
-            and ((m + 255) // 256) * ((n + 255) // 256) < 192)
+            and ((m + 255) // 256) * ((n + 255) // 256) < 100)
 
 
 def packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
