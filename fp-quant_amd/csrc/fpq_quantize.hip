@@ -23,31 +23,17 @@ constexpr int kFmtNv = 1;
 // Generic kernel: one lane owns 8 consecutive elements (one 16-byte load, 4 bytes of codes).
 // A rotation block of G elements spans G/8 neighbouring lanes; the butterflies with stride
 // >= 8 exchange registers between lanes.  Works for any cols % max(G, GROUP) == 0.
-// One lane quantizes 8 consecutive elements (chunk index `chunk`); the G/8 neighbouring lanes of
-// a rotation block exchange registers for the butterflies with stride >= 8.  Must be called by
-// all 64 lanes of a wave with consecutive chunk indices (inactive lanes pass active = false).
 //
-// QUEST (MXFP4 only) replaces the abs-max scale by the reference's "quest" rule
-// (inference_lib/src/fp_quant/module/triton/mxfp4.py:51-59, constant from
-// pseudoquant_linear_fns.py:20-22): s = 2^floor(log2(fl(2.92247856/6) * std + 1e-8)) with the
-// population standard deviation of the 32 rotated values, values beyond +-6 s saturate, and the
-// optional mask gets bit (element % 8) of byte [row, element / 8] set where |x / s| < 6
-// (mxfp4.py:105-110, linear_fns.py:67-76).  fp32 evaluation order, fixed so that a CPU can
-// reproduce it: per octet of consecutive elements the sums of x and of fl(x*x) run left to right,
-// the four octet sums combine as (o0 + o1) + (o2 + o3); mean = sum/32, var = max(msq - fl(mean*mean), 0).
-template <int G, int FMT, int ROT, int ZERO, bool QUEST = false>
-__device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint32_t* __restrict__ codes,
-                                              uint8_t* __restrict__ scales, uint32_t chunk, bool active,
-                                              uint32_t lane, uint32_t chunks_per_row,
-                                              uint32_t scale_stride, float norm, float gscale, float rg,
-                                              float* __restrict__ stage, const uint16_t* __restrict__ hmat,
-                                              uint8_t* __restrict__ mask = nullptr) {
-  static_assert(!QUEST || FMT == kFmtMx, "the quest rule exists for MXFP4 only");
-  constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
+// lane8_load_rotate leaves the lane's 8 rotated values of chunk `chunk` in p (zeros for an
+// inactive lane).  Must be called by all 64 lanes of a wave with consecutive chunk indices
+// (inactive lanes pass active = false).
+template <int G, int ROT>
+__device__ __forceinline__ void lane8_load_rotate(const uint4* __restrict__ x, uint32_t chunk, bool active,
+                                                  uint32_t lane, float norm, float* __restrict__ stage,
+                                                  const uint16_t* __restrict__ hmat, float (&p)[8]) {
   uint4 raw = make_uint4(0u, 0u, 0u, 0u);
   if (active) raw = x[chunk];
 
-  float p[8];
   p[0] = bf16_lo(raw.x); p[1] = bf16_hi(raw.x);
   p[2] = bf16_lo(raw.y); p[3] = bf16_hi(raw.y);
   p[4] = bf16_lo(raw.z); p[5] = bf16_hi(raw.z);
@@ -111,6 +97,27 @@ __device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint3
 #pragma unroll
     for (int i = 0; i < 8; ++i) p[i] = acc[i];
   }
+}
+
+// Rotates and quantizes the lane's 8 elements: abs-max scales, or with QUEST (MXFP4 only) the
+// reference's "quest" rule (inference_lib/src/fp_quant/module/triton/mxfp4.py:51-59, constant from
+// pseudoquant_linear_fns.py:20-22): s = 2^floor(log2(fl(2.92247856/6) * std + 1e-8)) with the
+// population standard deviation of the 32 rotated values, values beyond +-6 s saturate, and the
+// optional mask gets bit (element % 8) of byte [row, element / 8] set where |x / s| < 6
+// (mxfp4.py:105-110, linear_fns.py:67-76).  fp32 evaluation order, fixed so that a CPU can
+// reproduce it: per octet of consecutive elements the sums of x and of fl(x*x) run left to right,
+// the four octet sums combine as (o0 + o1) + (o2 + o3); mean = sum/32, var = max(msq - fl(mean*mean), 0).
+template <int G, int FMT, int ROT, int ZERO, bool QUEST = false>
+__device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint32_t* __restrict__ codes,
+                                              uint8_t* __restrict__ scales, uint32_t chunk, bool active,
+                                              uint32_t lane, uint32_t chunks_per_row,
+                                              uint32_t scale_stride, float norm, float gscale, float rg,
+                                              float* __restrict__ stage, const uint16_t* __restrict__ hmat,
+                                              uint8_t* __restrict__ mask = nullptr) {
+  static_assert(!QUEST || FMT == kFmtMx, "the quest rule exists for MXFP4 only");
+  constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
+  float p[8];
+  lane8_load_rotate<G, ROT>(x, chunk, active, lane, norm, stage, hmat, p);
 
   if (QUEST) {
     float sum = p[0], sq = p[0] * p[0];
@@ -798,6 +805,81 @@ static int dispatch(const void* x, int64_t rows, int64_t cols, int rot_kind, int
 }
 
 // ------------------------------------------------------------------------------------------
+// max |rotate(x)| over a whole tensor, folded into *amax with an atomic maximum on the bit
+// pattern (non-negative floats order like unsigned integers).  The rotation is the quantizers'
+// own, so the value is the one their group maxima are taken from.
+template <int G, int ROT>
+__global__ __launch_bounds__(256) void rotated_absmax_kernel(const uint4* __restrict__ x, uint32_t n_chunks,
+                                                             float norm, const uint16_t* __restrict__ h,
+                                                             uint32_t* __restrict__ amax) {
+  constexpr bool kStage = ROT == FPQ_ROT_GSR || ROT == FPQ_ROT_GENERAL;
+  __shared__ float stage[kStage ? 4 : 1][kStage ? 512 : 1];
+  __shared__ __attribute__((aligned(16))) uint16_t hmat[ROT == FPQ_ROT_GENERAL ? G * G : 8];
+  if (ROT == FPQ_ROT_GENERAL) {
+    for (int i = threadIdx.x; i < G * G; i += 256) hmat[i] = h[i];
+    __syncthreads();
+  }
+  float a = 0.0f;
+  for (uint32_t base = blockIdx.x * 256u; base < n_chunks; base += gridDim.x * 256u) {
+    const uint32_t chunk = base + threadIdx.x;
+    float p[8];
+    lane8_load_rotate<G, ROT>(x, chunk, chunk < n_chunks, threadIdx.x & 63u, norm,
+                              stage[kStage ? (threadIdx.x >> 6) : 0], hmat, p);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a = __builtin_fmaxf(a, __builtin_fabsf(p[i]));
+  }
+#pragma unroll
+  for (int lm = 1; lm < 64; lm *= 2) a = __builtin_fmaxf(a, __shfl_xor(a, lm, 64));
+  if ((threadIdx.x & 63u) == 0u) atomicMax(amax, __float_as_uint(a));
+}
+
+template <int G, int ROT>
+static int launch_absmax(const void* x, int64_t rows, int64_t cols, float norm, const void* h, float* amax,
+                         hipStream_t stream) {
+  const int64_t n_chunks = rows * cols / 8;
+  const int64_t blocks = (n_chunks + 255) / 256;
+  hipLaunchKernelGGL((rotated_absmax_kernel<G, ROT>), dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256),
+                     0, stream, (const uint4*)x, (uint32_t)n_chunks, norm, (const uint16_t*)h, (uint32_t*)amax);
+  return (int)hipGetLastError();
+}
+
+static int dispatch_absmax(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                           const void* h, float* amax, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (rows < 0 || cols < 0) return FPQ_E_SHAPE;
+  if (!amax) return FPQ_E_NULL;
+  if (rows == 0 || cols == 0) return FPQ_OK;
+  if (!x) return FPQ_E_NULL;
+  if (rot_kind == FPQ_ROT_IDENTITY) g = 16;
+  if (g != 16 && g != 32 && g != 64 && g != 128) return FPQ_E_ROTATION;
+  if (cols % g != 0) return FPQ_E_SHAPE;
+  if (rows * cols >= (int64_t)1 << 34) return FPQ_E_SHAPE;
+  if (((uintptr_t)x & 15u) || ((uintptr_t)amax & 3u)) return FPQ_E_ALIGN;
+  if (rot_kind == FPQ_ROT_GENERAL) {
+    if (!h) return FPQ_E_NULL;
+    if ((uintptr_t)h & 1u) return FPQ_E_ALIGN;
+  }
+#define FPQ_LAUNCH_ABSMAX(GG, RR) return launch_absmax<GG, RR>(x, rows, cols, norm, h, amax, stream)
+#define FPQ_ABSMAX_BY_G(RR)                       \
+  switch (g) {                                    \
+    case 16: FPQ_LAUNCH_ABSMAX(16, RR);           \
+    case 32: FPQ_LAUNCH_ABSMAX(32, RR);           \
+    case 64: FPQ_LAUNCH_ABSMAX(64, RR);           \
+    case 128: FPQ_LAUNCH_ABSMAX(128, RR);         \
+  }                                               \
+  break
+  switch (rot_kind) {
+    case FPQ_ROT_IDENTITY: FPQ_LAUNCH_ABSMAX(16, FPQ_ROT_IDENTITY);
+    case FPQ_ROT_HADAMARD: FPQ_ABSMAX_BY_G(FPQ_ROT_HADAMARD);
+    case FPQ_ROT_GSR: FPQ_ABSMAX_BY_G(FPQ_ROT_GSR);
+    case FPQ_ROT_GENERAL: FPQ_ABSMAX_BY_G(FPQ_ROT_GENERAL);
+  }
+#undef FPQ_ABSMAX_BY_G
+#undef FPQ_LAUNCH_ABSMAX
+  return FPQ_E_ROTATION;
+}
+
+// ------------------------------------------------------------------------------------------
 template <int ZERO>
 __global__ void e2m1_test_kernel(const float* in, uint8_t* out, int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -835,6 +917,11 @@ extern "C" int fpq_quantize_nv(const void* x, int64_t rows, int64_t cols, int ro
                                int zero_policy, void* stream) {
   return fpq::dispatch<fpq::kFmtNv>(x, rows, cols, rot_kind, g, norm, h, global_scale, codes,
                                     scales, scale_rows, scale_stride, zero_policy, stream);
+}
+
+extern "C" int fpq_rotated_absmax(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                                  const void* h, float* amax, void* stream) {
+  return fpq::dispatch_absmax(x, rows, cols, rot_kind, g, norm, h, amax, stream);
 }
 
 extern "C" int fpq_test_e2m1(const float* in, uint8_t* out, int64_t n, int zero_policy,

@@ -245,6 +245,28 @@ def _(x_flat, hadamard_matrix, global_scale):
     return codes, scales
 
 
+def rotated_absmax(x: torch.Tensor, hadamard_matrix: torch.Tensor, amax: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """max |x @ blockdiag(H)| as a one-element fp32 tensor, folded into `amax` when one is given
+    (running maximum over calls).  Same rotation arithmetic as the quantize operators."""
+    _require_cuda(x, hadamard_matrix)
+    if x.dtype != torch.bfloat16:
+        raise ValueError("x must be a bfloat16 tensor")
+    x = x.contiguous()
+    cols = x.shape[-1]
+    rows = x.numel() // cols if cols else 0
+    if amax is None:
+        amax = torch.zeros(1, dtype=torch.float32, device=x.device)
+    elif amax.dtype != torch.float32 or amax.numel() != 1 or amax.device != x.device:
+        raise ValueError("amax must be a one-element float32 tensor on the device of x")
+    kind, norm = classify_rotation(hadamard_matrix)
+    h = as_bf16(hadamard_matrix)
+    with torch.cuda.device(x.device):
+        st = _engine.lib().fpq_rotated_absmax(x.data_ptr(), rows, cols, kind, hadamard_matrix.shape[0], norm,
+                                              h.data_ptr(), amax.data_ptr(), _stream(x))
+    _engine.check(st, "fpq_rotated_absmax")
+    return amax
+
+
 ### GEMMs
 
 # From these many activation rows on, the MXFP4 GEMM runs on operands re-tiled into the order the

@@ -151,6 +151,16 @@ int fpq_gemm_mxf4_packed(const void* xq_packed, const void* xs_packed, const voi
                          int64_t M, int64_t N, int64_t K, void* stream);
 
 /*
+ * *amax = max(*amax, max |rotate(x)|) as fp32, with the rotation of the quantize entry points
+ * (rot_kind, g, norm, h as there; cols % g == 0).  The NVFP4 per-tensor multiplier the reference's
+ * exporter tracks is 448 * 6 / this maximum, minimised over calls
+ * (src/quantization/quantizer.py:145-150); the caller zeroes *amax before the first call and may
+ * keep folding further tensors (calibration batches, fused q/k/v weights) into it.
+ */
+int fpq_rotated_absmax(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                       const void* h, float* amax, void* stream);
+
+/*
  * Test hook: E2M1 codes of n fp32 values exactly as the quantize kernels round them
  * (out[i] in 0..15, one byte per value).  Used to check the device rounding exhaustively.
  */

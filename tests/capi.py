@@ -160,3 +160,20 @@ def gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=None):
     _engine.check(st, "fpq_gemm_nvf4_packed")
     torch.cuda.synchronize()
     return y.cpu()
+
+
+def rotated_absmax(x_bf16, rot="hadamard", g=128, norm=None, h=None, start=0.0):
+    """Run fpq_rotated_absmax on `x_bf16` with *amax preset to `start`; returns the fp32 value."""
+    lib = _engine.lib()
+    x = x_bf16.to("cuda").contiguous()
+    rows, cols = x.shape
+    if norm is None:
+        norm = float(torch.tensor(g ** -0.5, dtype=torch.bfloat16))
+    h_dev = h.to(device="cuda", dtype=torch.bfloat16).contiguous() if h is not None else None  # keep alive
+    amax = torch.tensor([start], dtype=torch.float32, device="cuda")
+    st = lib.fpq_rotated_absmax(x.data_ptr(), rows, cols, ROT[rot], g, norm,
+                                h_dev.data_ptr() if h_dev is not None else None, amax.data_ptr(),
+                                torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_rotated_absmax")
+    torch.cuda.synchronize()
+    return float(amax.cpu())
