@@ -9,6 +9,7 @@ rotation matrix is recognised once (Hadamard / identity / GSR) and applied as bu
 from typing import Optional, Tuple
 
 import os
+import weakref
 
 import torch
 
@@ -481,13 +482,61 @@ def as_f32_scalar(t: torch.Tensor) -> torch.Tensor:
     return cached_on(t, "_fpq_f32", (t._version, t.data_ptr()), lambda: t.detach().float().contiguous())
 
 
+# Several layers that consume one tensor (q/k/v projections, gate/up projections) would rotate and
+# quantize it once each.  The quantized activations of the latest call are kept per device and reused
+# while the next call passes the very same tensor object, unmodified (its version counter), with the
+# same rotation, global scale and stream.  The source is held weakly, so a freed tensor whose address
+# is reused can never match.  Nothing is shared while a stream is being captured: a captured
+# quantization has not run yet, so its output cannot serve a later eager call.  FPQ_SHARE_ACT_QUANT=0
+# turns the sharing off.
+SHARE_ACT_QUANT = os.environ.get("FPQ_SHARE_ACT_QUANT", "1") != "0"
+
+
+class _SharedActivations:
+    __slots__ = ("ref", "version", "key", "keep", "mx_packed", "row_major", "nv_packed")
+
+    def __init__(self, src, key, keep):
+        self.ref = weakref.ref(src)
+        self.version = src._version
+        self.key = key
+        self.keep = keep   # objects whose id() is part of the key stay alive with the entry
+        self.mx_packed = self.row_major = self.nv_packed = None
+
+    def matches(self, src, key) -> bool:
+        return self.ref() is src and self.version == src._version and self.key == key
+
+
+_shared_activations = {}   # device index -> _SharedActivations of the latest call
+
+
+def _shared_entry(src, x_flat, h, kind: int, norm: float, act_global_scale, stream: int):
+    """The sharing slot for this call (fresh unless the previous call quantized the same thing), or
+    None when nothing may be shared.  Layers own separate but equal rotation and global-scale
+    buffers, so those are compared by value: (kind, norm, size) of a recognised rotation, the host
+    copy of the scale (read once per buffer); an unrecognised rotation matrix only matches itself."""
+    if src is None or not SHARE_ACT_QUANT or torch.cuda.is_current_stream_capturing():
+        return None
+    rot = (kind, norm, h.shape[0]) if kind != _engine.ROT_GENERAL else (kind, id(h), h._version)
+    gs = None
+    if act_global_scale is not None:
+        gs = cached_on(act_global_scale, "_fpq_host", (act_global_scale._version, act_global_scale.data_ptr()),
+                       lambda: float(act_global_scale))
+    key = (rot, gs, stream, tuple(x_flat.shape))
+    dev = x_flat.device.index
+    entry = _shared_activations.get(dev)
+    if entry is None or not entry.matches(src, key):
+        entry = _shared_activations[dev] = _SharedActivations(src, key, h)
+    return entry
+
+
 def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.Tensor, ws: torch.Tensor,
                 alpha: torch.Tensor, act_global_scale: torch.Tensor, bias: Optional[torch.Tensor],
-                nvfp4: bool) -> torch.Tensor:
+                nvfp4: bool, shared_source: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Activation rotate+quantize and W4A4 GEMM of one linear with as little host work as possible:
     the eager (non-traced) body of FPQuantLinear.forward.  Same kernels and results as the
     fused_quantize_* and matmul_* operators; `x_flat` bf16 [M, K] contiguous on the GPU, `alpha`
-    fp32 [1], `bias` bf16 [N] or None."""
+    fp32 [1], `bias` bf16 [N] or None.  `shared_source` is the tensor object `x_flat` was derived
+    from: consecutive calls with the same, unmodified object reuse its quantized form."""
     if not x_flat.is_cuda:
         raise ValueError("fp_quant HIP operators need tensors on a GPU; there is no CPU path")
     lib = _engine.lib()
@@ -498,37 +547,58 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
     dev = x_flat.device
     if torch.cuda.current_device() != dev.index:
         with torch.cuda.device(dev):
-            return linear_w4a4(x_flat, hadamard_matrix, wq, ws, alpha, act_global_scale, bias, nvfp4)
+            return linear_w4a4(x_flat, hadamard_matrix, wq, ws, alpha, act_global_scale, bias, nvfp4, shared_source)
     stream = torch.cuda.current_stream().cuda_stream
     h = as_bf16(hadamard_matrix)
     kind, norm = classify_rotation(h)
     g = h.shape[0]
     y = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
     b_ptr = bias.data_ptr() if bias is not None else None
+    shared = _shared_entry(shared_source, x_flat, h, kind, norm, act_global_scale if nvfp4 else None, stream)
     if not nvfp4 and packed_linear_eligible(m, k, "abs_max"):
-        pc = torch.empty(lib.fpq_packed_codes_bytes(m, k), dtype=torch.uint8, device=dev)
-        ps = torch.empty(lib.fpq_packed_scales_bytes(m, k), dtype=torch.uint8, device=dev)
-        st = lib.fpq_quantize_mx_packed(x_flat.data_ptr(), m, k, kind, g, norm, pc.data_ptr(), ps.data_ptr(),
-                                        ZERO_NIBBLE_POLICY, stream)
-        if st == _engine.E_UNSUPPORTED:
-            pc, ps = quantize_mx_packed(x_flat, h)
+        if shared is not None and shared.mx_packed is not None:
+            pc, ps = shared.mx_packed
         else:
-            _engine.check(st, "fpq_quantize_mx_packed")
+            pc = torch.empty(lib.fpq_packed_codes_bytes(m, k), dtype=torch.uint8, device=dev)
+            ps = torch.empty(lib.fpq_packed_scales_bytes(m, k), dtype=torch.uint8, device=dev)
+            st = lib.fpq_quantize_mx_packed(x_flat.data_ptr(), m, k, kind, g, norm, pc.data_ptr(), ps.data_ptr(),
+                                            ZERO_NIBBLE_POLICY, stream)
+            if st == _engine.E_UNSUPPORTED:
+                pc, ps = quantize_mx_packed(x_flat, h)
+            else:
+                _engine.check(st, "fpq_quantize_mx_packed")
+            if shared is not None:
+                shared.mx_packed = (pc, ps)
         wp, wsp = packed_weight(wq, ws)
         st = lib.fpq_gemm_mxf4_packed(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(), alpha.data_ptr(),
                                       b_ptr, y.data_ptr(), m, n, k, stream)
         _engine.check(st, "fpq_gemm_mxf4_packed")
         return y
     group = 16 if nvfp4 else 32
-    codes = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
-    scales = torch.empty(m, k // group, dtype=torch.uint8, device=dev)
+    if shared is not None and shared.row_major is not None:
+        codes, scales = shared.row_major
+    else:
+        codes = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
+        scales = torch.empty(m, k // group, dtype=torch.uint8, device=dev)
+        if nvfp4:
+            gs = as_f32_scalar(act_global_scale)
+            st = lib.fpq_quantize_nv(x_flat.data_ptr(), m, k, kind, g, norm, h.data_ptr(), gs.data_ptr(),
+                                     codes.data_ptr(), scales.data_ptr(), m, k // group, ZERO_NIBBLE_POLICY, stream)
+            _engine.check(st, "fpq_quantize_nv")
+        else:
+            st = lib.fpq_quantize_mx(x_flat.data_ptr(), m, k, kind, g, norm, h.data_ptr(), codes.data_ptr(),
+                                     scales.data_ptr(), m, k // group, ZERO_NIBBLE_POLICY, stream)
+            _engine.check(st, "fpq_quantize_mx")
+        if shared is not None:
+            shared.row_major = (codes, scales)
     if nvfp4:
-        gs = as_f32_scalar(act_global_scale)
-        st = lib.fpq_quantize_nv(x_flat.data_ptr(), m, k, kind, g, norm, h.data_ptr(), gs.data_ptr(),
-                                 codes.data_ptr(), scales.data_ptr(), m, k // group, ZERO_NIBBLE_POLICY, stream)
-        _engine.check(st, "fpq_quantize_nv")
         if nv_packed_eligible(m, n, k):
-            xp, xsp = pack_nvf4(codes, scales, m, k)
+            if shared is not None and shared.nv_packed is not None:
+                xp, xsp = shared.nv_packed
+            else:
+                xp, xsp = pack_nvf4(codes, scales, m, k)
+                if shared is not None:
+                    shared.nv_packed = (xp, xsp)
             wp, wsp = packed_weight(wq, ws, True)
             st = lib.fpq_gemm_nvf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
                                           alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
@@ -538,9 +608,6 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
                                ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
         _engine.check(st, "fpq_gemm_nvf4")
     else:
-        st = lib.fpq_quantize_mx(x_flat.data_ptr(), m, k, kind, g, norm, h.data_ptr(), codes.data_ptr(),
-                                 scales.data_ptr(), m, k // group, ZERO_NIBBLE_POLICY, stream)
-        _engine.check(st, "fpq_quantize_mx")
         st = lib.fpq_gemm_mxf4(codes.data_ptr(), scales.data_ptr(), k // group, wq.data_ptr(), ws.data_ptr(),
                                ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
         _engine.check(st, "fpq_gemm_mxf4")

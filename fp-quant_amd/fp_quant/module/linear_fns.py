@@ -81,7 +81,7 @@ class FPQuant4x16NoMasterFn(Function):
             fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16 and bias.is_contiguous()) else None
             y = linear_w4a4(x_flat.to(torch.bfloat16), forward_hadamard_matrix, weight_q, weight_scales,
                             linear_alpha(weight_global_scale, act_global_scale), act_global_scale, fused_bias,
-                            dtype == FPQuantDtype.NVFP4)
+                            dtype == FPQuantDtype.NVFP4, shared_source=x)
             y = y.unflatten(dim=0, sizes=x.shape[:-1])
             if bias is not None and fused_bias is None:
                 y += bias

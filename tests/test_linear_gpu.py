@@ -250,3 +250,73 @@ def test_forward_is_graph_capturable(fmt, g, m):
             graph.replay()
             torch.cuda.synchronize()
             assert torch.equal(static_y, want), rep
+
+
+def _quantized_linear(fmt, g, k, n, seed, bias=False):
+    import fp_quant
+    torch.manual_seed(seed)
+    lin = fp_quant.FPQuantLinear(k, n, _cfg(fmt, g), bias=bias, device="cuda", dtype=torch.bfloat16)
+    lin.weight.data.normal_(0, 0.02)
+    if bias:
+        lin.bias.data.normal_()
+    lin.pre_forward()
+    return lin
+
+
+@pytest.mark.parametrize("fmt,g,m", [("mxfp4", 128, 1), ("mxfp4", 32, 200), ("nvfp4", 16, 8), ("nvfp4", 16, 100),
+                                     ("nvfp4", 64, 700)])
+def test_layers_sharing_an_input_share_its_quantization(fmt, g, m):
+    """q/k/v-style layers called with the same tensor object reuse the quantized activations of the
+    first call; outputs are bit-identical to unshared calls, and any change of the input (in-place
+    write, another tensor, another rotation or global scale) quantizes again."""
+    from fp_quant.module import hip_ops
+    k = 512
+    layers = [_quantized_linear(fmt, g, k, n, seed) for seed, n in enumerate((256, 128, 384))]
+    x = torch.randn(2, m, k, device="cuda", dtype=torch.bfloat16)
+
+    def unshared(inp, lins):
+        hip_ops.SHARE_ACT_QUANT = False
+        try:
+            return [lin(inp) for lin in lins]
+        finally:
+            hip_ops.SHARE_ACT_QUANT = True
+
+    want = unshared(x, layers)
+    hip_ops._shared_activations.clear()
+    got0 = layers[0](x)
+    slot = hip_ops._shared_activations[0]
+    filled = [f for f in ("mx_packed", "row_major", "nv_packed") if getattr(slot, f) is not None]
+    assert filled
+    got = [got0] + [lin(x) for lin in layers[1:]]
+    assert hip_ops._shared_activations[0] is slot          # the later calls found the first call's entry
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+
+    # in-place write: same object, new version -> quantized again
+    x.mul_(-1.5)
+    want2 = unshared(x, layers[:2])
+    assert torch.equal(layers[0](x), want2[0]) and hip_ops._shared_activations[0] is not slot
+    assert torch.equal(layers[1](x), want2[1])
+
+    # a new tensor (very likely at the freed address) never matches the dead one
+    shape = x.shape
+    del x, want, got, got0, want2
+    x2 = torch.randn(shape, device="cuda", dtype=torch.bfloat16)
+    want3 = unshared(x2, layers[:1])[0]
+    assert torch.equal(layers[0](x2), want3)
+
+    # same tensor into a layer with another rotation size: not shared, still right
+    other_g = 64 if g != 64 else 32
+    other = _quantized_linear(fmt, other_g, k, 256, 7)
+    want4 = unshared(x2, [other])[0]
+    layers[0](x2)
+    assert torch.equal(other(x2), want4)
+
+    if fmt == "nvfp4":
+        # another activation global scale quantizes differently and must not reuse the entry
+        scaled = _quantized_linear(fmt, g, k, 256, 8)
+        scaled.act_global_scale.fill_(5.0)
+        want5 = unshared(x2, [scaled])[0]
+        layers[0](x2)
+        got5 = scaled(x2)
+        assert torch.equal(got5, want5) and not torch.equal(got5, unshared(x2, [_quantized_linear(fmt, g, k, 256, 8)])[0])
