@@ -27,17 +27,102 @@ constexpr int kFmtNv = 1;
 // lane8_load_rotate leaves the lane's 8 rotated values of chunk `chunk` in p (zeros for an
 // inactive lane).  Must be called by all 64 lanes of a wave with consecutive chunk indices
 // (inactive lanes pass active = false).
-template <int G, int ROT>
-__device__ __forceinline__ void lane8_load_rotate(const uint4* __restrict__ x, uint32_t chunk, bool active,
-                                                  uint32_t lane, float norm, float* __restrict__ stage,
-                                                  const uint16_t* __restrict__ hmat, float (&p)[8]) {
-  uint4 raw = make_uint4(0u, 0u, 0u, 0u);
-  if (active) raw = x[chunk];
+//
+// A prologue computes the tensor that is quantized from its producer's inputs, so that the bf16
+// intermediate never travels through memory (src/utils/llama_utils.py:60-71: act_fn(gate) * up
+// feeds down_proj's quantizer, the RMSNorm output feeds those of q/k/v and gate/up).  Each
+// PyTorch operator of the unfused sequence rounds to bf16 once, and so do these:
+//   kProRmsNorm  bf16(gamma[c] * bf16(x[r, c] * inv_rms[r]))
+//   kProSiluMul  bf16(bf16(silu(x[r, c])) * second[r, c]),  silu(g) = g / (1 + exp_det(-g))
+// with plain fp32 multiplies, adds and divisions in a fixed order (this file is built without
+// contraction), so a CPU reproduces every bit.
+constexpr int kProNone = 0;
+constexpr int kProRmsNorm = 1;
+constexpr int kProSiluMul = 2;
 
+struct Prologue {
+  const float* row_scale;   // kProRmsNorm: 1 / rms per row
+  const uint4* col_scale;   // kProRmsNorm: bf16 weight per column
+  const uint4* second;      // kProSiluMul: the multiplier ("up") tensor
+  uint4* out;               // optional: the prologue's bf16 result, row-major [rows, cols]
+  uint32_t chunks_per_row;  // cols / 8
+  uint32_t ld_first;        // row stride of x in 8-element chunks
+  uint32_t ld_second;       // row stride of `second` in 8-element chunks
+};
+
+__device__ __forceinline__ float bf16_rne(float v) {
+  uint32_t b = __float_as_uint(v);
+  b += 0x7fffu + ((b >> 16) & 1u);
+  return __uint_as_float(b & 0xffff0000u);
+}
+
+// exp(t): clamp to +-200, n = rint(t * log2e), r = (t - n*ln2_hi) - n*ln2_lo (n*ln2_hi is exact),
+// degree-5 Horner polynomial with separate multiplies and adds, ldexp by n (overflows to inf,
+// underflows gradually).  Within 1e-7 of exp over the whole range.
+__device__ __forceinline__ float exp_det(float t) {
+  t = t < -200.0f ? -200.0f : t;
+  t = t > 200.0f ? 200.0f : t;
+  const float n = __builtin_rintf(t * 1.44269504088896341f);
+  const float r = (t - n * 0.693359375f) - n * -2.12194440e-4f;
+  float p = 1.9875691500e-4f;
+  p = p * r + 1.3981999507e-3f;
+  p = p * r + 8.3334519073e-3f;
+  p = p * r + 4.1665795894e-2f;
+  p = p * r + 1.6666665459e-1f;
+  p = p * r + 5.0000001201e-1f;
+  const float y = (p * (r * r) + r) + 1.0f;
+  return __builtin_ldexpf(y, (int)n);
+}
+
+__device__ __forceinline__ void unpack8(const uint4& raw, float (&p)[8]) {
   p[0] = bf16_lo(raw.x); p[1] = bf16_hi(raw.x);
   p[2] = bf16_lo(raw.y); p[3] = bf16_hi(raw.y);
   p[4] = bf16_lo(raw.z); p[5] = bf16_hi(raw.z);
   p[6] = bf16_lo(raw.w); p[7] = bf16_hi(raw.w);
+}
+
+template <int G, int ROT, int PRO = kProNone>
+__device__ __forceinline__ void lane8_load_rotate(const uint4* __restrict__ x, uint32_t chunk, bool active,
+                                                  uint32_t lane, float norm, float* __restrict__ stage,
+                                                  const uint16_t* __restrict__ hmat, float (&p)[8],
+                                                  const Prologue& pro = Prologue{}) {
+  uint4 raw = make_uint4(0u, 0u, 0u, 0u);
+  if (PRO == kProNone) {
+    if (active) raw = x[chunk];
+    unpack8(raw, p);
+  } else {
+    uint4 aux = make_uint4(0u, 0u, 0u, 0u);
+    float rs = 0.0f;
+    if (active) {
+      const uint32_t row = chunk / pro.chunks_per_row, cc = chunk - row * pro.chunks_per_row;
+      raw = x[(size_t)row * pro.ld_first + cc];
+      if (PRO == kProRmsNorm) {
+        aux = pro.col_scale[cc];
+        rs = pro.row_scale[row];
+      } else {
+        aux = pro.second[(size_t)row * pro.ld_second + cc];
+      }
+    }
+    float q[8];
+    unpack8(raw, p);
+    unpack8(aux, q);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float t;
+      if (PRO == kProRmsNorm) {
+        t = bf16_rne(p[i] * rs);
+      } else {
+        t = bf16_rne(p[i] / (1.0f + exp_det(-p[i])));
+      }
+      p[i] = bf16_rne(t * q[i]);
+    }
+    if (active && pro.out) {
+      pro.out[chunk] = make_uint4((__float_as_uint(p[0]) >> 16) | (__float_as_uint(p[1]) & 0xffff0000u),
+                                  (__float_as_uint(p[2]) >> 16) | (__float_as_uint(p[3]) & 0xffff0000u),
+                                  (__float_as_uint(p[4]) >> 16) | (__float_as_uint(p[5]) & 0xffff0000u),
+                                  (__float_as_uint(p[6]) >> 16) | (__float_as_uint(p[7]) & 0xffff0000u));
+    }
+  }
 
   if (ROT == FPQ_ROT_HADAMARD || ROT == FPQ_ROT_GSR) {
 #pragma unroll
@@ -107,17 +192,18 @@ __device__ __forceinline__ void lane8_load_rotate(const uint4* __restrict__ x, u
 // (mxfp4.py:105-110, linear_fns.py:67-76).  fp32 evaluation order, fixed so that a CPU can
 // reproduce it: per octet of consecutive elements the sums of x and of fl(x*x) run left to right,
 // the four octet sums combine as (o0 + o1) + (o2 + o3); mean = sum/32, var = max(msq - fl(mean*mean), 0).
-template <int G, int FMT, int ROT, int ZERO, bool QUEST = false>
+template <int G, int FMT, int ROT, int ZERO, bool QUEST = false, int PRO = kProNone>
 __device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint32_t* __restrict__ codes,
                                               uint8_t* __restrict__ scales, uint32_t chunk, bool active,
                                               uint32_t lane, uint32_t chunks_per_row,
                                               uint32_t scale_stride, float norm, float gscale, float rg,
                                               float* __restrict__ stage, const uint16_t* __restrict__ hmat,
-                                              uint8_t* __restrict__ mask = nullptr) {
+                                              uint8_t* __restrict__ mask = nullptr,
+                                              const Prologue& pro = Prologue{}) {
   static_assert(!QUEST || FMT == kFmtMx, "the quest rule exists for MXFP4 only");
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
   float p[8];
-  lane8_load_rotate<G, ROT>(x, chunk, active, lane, norm, stage, hmat, p);
+  lane8_load_rotate<G, ROT, PRO>(x, chunk, active, lane, norm, stage, hmat, p, pro);
 
   if (QUEST) {
     float sum = p[0], sq = p[0] * p[0];
@@ -203,12 +289,12 @@ __device__ __forceinline__ void fill_scale_padding(uint8_t* __restrict__ scales,
 }
 
 // Generic kernel: works for any cols % max(G, GROUP) == 0; one 8-element chunk per thread.
-template <int G, int FMT, int ROT, int ZERO, bool QUEST = false>
+template <int G, int FMT, int ROT, int ZERO, bool QUEST = false, int PRO = kProNone>
 __global__ __launch_bounds__(256) void quantize_lane8_kernel(
     const uint4* __restrict__ x, uint32_t* __restrict__ codes, uint8_t* __restrict__ scales,
     uint32_t n_chunks, uint32_t chunks_per_row, uint32_t rows, uint32_t scale_rows,
     uint32_t scale_stride, float norm, const float* __restrict__ global_scale,
-    const uint16_t* __restrict__ h, uint8_t* __restrict__ mask = nullptr) {
+    const uint16_t* __restrict__ h, uint8_t* __restrict__ mask = nullptr, Prologue pro = Prologue{}) {
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
   constexpr bool kStage = ROT == FPQ_ROT_GSR || ROT == FPQ_ROT_GENERAL;
   __shared__ float stage[kStage ? 4 : 1][kStage ? 512 : 1];
@@ -223,9 +309,9 @@ __global__ __launch_bounds__(256) void quantize_lane8_kernel(
     g = *global_scale;
     rg = g == 0.0f ? 0.0f : 1.0f / g;
   }
-  lane8_process<G, FMT, ROT, ZERO, QUEST>(x, codes, scales, chunk, chunk < n_chunks, threadIdx.x & 63u,
-                                          chunks_per_row, scale_stride, norm, g, rg,
-                                          stage[kStage ? (threadIdx.x >> 6) : 0], hmat, mask);
+  lane8_process<G, FMT, ROT, ZERO, QUEST, PRO>(x, codes, scales, chunk, chunk < n_chunks, threadIdx.x & 63u,
+                                               chunks_per_row, scale_stride, norm, g, rg,
+                                               stage[kStage ? (threadIdx.x >> 6) : 0], hmat, mask, pro);
   fill_scale_padding(scales, rows, chunks_per_row / (GROUP / 8), scale_rows, scale_stride);
 }
 
@@ -239,7 +325,7 @@ static int launch_lane8_quest(const void* x, int64_t rows, int64_t cols, float n
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint4*)x, (uint32_t*)codes,
                        (uint8_t*)scales, (uint32_t)n_chunks, (uint32_t)(cols / 8), (uint32_t)rows,
                        (uint32_t)scale_rows, (uint32_t)scale_stride, norm, (const float*)nullptr,
-                       (const uint16_t*)h, (uint8_t*)mask);
+                       (const uint16_t*)h, (uint8_t*)mask, Prologue{});
   };
   if (zero_policy == FPQ_ZERO_REFERENCE) {
     args(quantize_lane8_kernel<G, kFmtMx, ROT, kZeroReference, true>);
@@ -311,7 +397,7 @@ static int launch_lane8(const void* x, int64_t rows, int64_t cols, float norm, c
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint4*)x, (uint32_t*)codes,
                        (uint8_t*)scales, (uint32_t)n_chunks, (uint32_t)(cols / 8), (uint32_t)rows,
                        (uint32_t)scale_rows, (uint32_t)scale_stride, norm, gsp, (const uint16_t*)h,
-                       (uint8_t*)nullptr);
+                       (uint8_t*)nullptr, Prologue{});
   };
   if (zero_policy == FPQ_ZERO_REFERENCE) {
     args(quantize_lane8_kernel<G, FMT, ROT, kZeroReference>);
@@ -805,6 +891,107 @@ static int dispatch(const void* x, int64_t rows, int64_t cols, int rot_kind, int
 }
 
 // ------------------------------------------------------------------------------------------
+// Quantizers with a prologue (generic kernel).
+template <int G, int FMT, int ROT, int PRO>
+static int launch_lane8_prologue(const void* x, int64_t rows, int64_t cols, float norm, const float* gsp,
+                                 void* codes, void* scales, int64_t scale_rows, int64_t scale_stride,
+                                 int zero_policy, hipStream_t stream, const Prologue& pro) {
+  const int64_t n_chunks = rows * cols / 8;
+  const dim3 grid((unsigned)((n_chunks + 255) / 256)), block(256);
+  auto args = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint4*)x, (uint32_t*)codes,
+                       (uint8_t*)scales, (uint32_t)n_chunks, (uint32_t)(cols / 8), (uint32_t)rows,
+                       (uint32_t)scale_rows, (uint32_t)scale_stride, norm, gsp, (const uint16_t*)nullptr,
+                       (uint8_t*)nullptr, pro);
+  };
+  if (zero_policy == FPQ_ZERO_REFERENCE) {
+    args(quantize_lane8_kernel<G, FMT, ROT, kZeroReference, false, PRO>);
+  } else {
+    args(quantize_lane8_kernel<G, FMT, ROT, kZeroSigned, false, PRO>);
+  }
+  return (int)hipGetLastError();
+}
+
+// x: the prologue's first input with row stride ld_first elements (kProSiluMul: `second` with
+// ld_second); Hadamard rotations of 16..128 and the identity only.
+template <int FMT, int PRO>
+static int dispatch_prologue(const void* x, int64_t ld_first, const void* second, int64_t ld_second,
+                             const float* row_scale, const void* col_scale, void* out, int64_t rows,
+                             int64_t cols, int rot_kind, int g, float norm, const float* gsp, void* codes,
+                             void* scales, int64_t scale_rows, int64_t scale_stride, int zero_policy,
+                             void* stream_) {
+  constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
+  hipStream_t stream = (hipStream_t)stream_;
+  if (rows < 0 || cols < 0) return FPQ_E_SHAPE;
+  if (rows == 0 || cols == 0) return FPQ_OK;
+  if (!x || !codes || !scales) return FPQ_E_NULL;
+  if (PRO == kProRmsNorm && (!row_scale || !col_scale)) return FPQ_E_NULL;
+  if (PRO == kProSiluMul && !second) return FPQ_E_NULL;
+  if (FMT == kFmtNv && !gsp) return FPQ_E_NULL;
+  if (zero_policy != FPQ_ZERO_REFERENCE && zero_policy != FPQ_ZERO_SIGNED) return FPQ_E_POLICY;
+  if (rot_kind == FPQ_ROT_IDENTITY) g = GROUP;
+  if (rot_kind != FPQ_ROT_IDENTITY && rot_kind != FPQ_ROT_HADAMARD) {
+    return (rot_kind == FPQ_ROT_GSR || rot_kind == FPQ_ROT_GENERAL) ? FPQ_E_UNSUPPORTED : FPQ_E_ROTATION;
+  }
+  if (g != 16 && g != 32 && g != 64 && g != 128) return FPQ_E_ROTATION;
+  if (cols % g != 0 || cols % GROUP != 0) return FPQ_E_SHAPE;
+  if (ld_first < cols || ld_first % 8 != 0) return FPQ_E_SHAPE;
+  if (PRO == kProSiluMul && (ld_second < cols || ld_second % 8 != 0)) return FPQ_E_SHAPE;
+  if (scale_rows < rows || scale_stride < cols / GROUP) return FPQ_E_SHAPE;
+  if (rows * ld_first >= (int64_t)1 << 34 || rows * ld_second >= (int64_t)1 << 34 ||
+      scale_rows * scale_stride >= (int64_t)1 << 32) {
+    return FPQ_E_SHAPE;
+  }
+  if (((uintptr_t)x & 15u) || ((uintptr_t)second & 15u) || ((uintptr_t)col_scale & 15u) ||
+      ((uintptr_t)out & 15u) || ((uintptr_t)row_scale & 3u) || ((uintptr_t)codes & 3u)) {
+    return FPQ_E_ALIGN;
+  }
+  Prologue pro;
+  pro.row_scale = row_scale;
+  pro.col_scale = (const uint4*)col_scale;
+  pro.second = (const uint4*)second;
+  pro.out = (uint4*)out;
+  pro.chunks_per_row = (uint32_t)(cols / 8);
+  pro.ld_first = (uint32_t)(ld_first / 8);
+  pro.ld_second = (uint32_t)(ld_second / 8);
+#define FPQ_LAUNCH_PRO(GG, RR)                                                                            \
+  return launch_lane8_prologue<GG, FMT, RR, PRO>(x, rows, cols, norm, gsp, codes, scales, scale_rows,    \
+                                                 scale_stride, zero_policy, stream, pro)
+  if (rot_kind == FPQ_ROT_IDENTITY) FPQ_LAUNCH_PRO(GROUP, FPQ_ROT_IDENTITY);
+  switch (g) {
+    case 16: FPQ_LAUNCH_PRO(16, FPQ_ROT_HADAMARD);
+    case 32: FPQ_LAUNCH_PRO(32, FPQ_ROT_HADAMARD);
+    case 64: FPQ_LAUNCH_PRO(64, FPQ_ROT_HADAMARD);
+    case 128: FPQ_LAUNCH_PRO(128, FPQ_ROT_HADAMARD);
+  }
+#undef FPQ_LAUNCH_PRO
+  return FPQ_E_ROTATION;
+}
+
+// 1 / sqrt(mean(x^2) + eps) of every row, one wave per row.  Fixed summation order: squares of 8
+// consecutive elements left to right; lane l accumulates the octets l, l + 64, ... in that order;
+// the 64 lane sums combine by the butterfly a += a[lane ^ m], m = 1, 2, ..., 32.
+__global__ __launch_bounds__(256) void row_inv_rms_kernel(const uint4* __restrict__ x, uint32_t rows,
+                                                          uint32_t chunks_per_row, uint32_t ld, float cols_f,
+                                                          float eps, float* __restrict__ out) {
+  const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
+  if (row >= rows) return;
+  const uint4* src = x + (size_t)row * ld;
+  float a = 0.0f;
+  for (uint32_t c = lane; c < chunks_per_row; c += 64u) {
+    float p[8];
+    unpack8(src[c], p);
+    float s = p[0] * p[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) s = s + p[i] * p[i];
+    a = a + s;
+  }
+#pragma unroll
+  for (int lm = 1; lm < 64; lm *= 2) a = a + __shfl_xor(a, lm, 64);
+  if (lane == 0u) out[row] = 1.0f / __builtin_sqrtf(a / cols_f + eps);
+}
+
+// ------------------------------------------------------------------------------------------
 // max |rotate(x)| over a whole tensor, folded into *amax with an atomic maximum on the bit
 // pattern (non-negative floats order like unsigned integers).  The rotation is the quantizers'
 // own, so the value is the one their group maxima are taken from.
@@ -917,6 +1104,59 @@ extern "C" int fpq_quantize_nv(const void* x, int64_t rows, int64_t cols, int ro
                                int zero_policy, void* stream) {
   return fpq::dispatch<fpq::kFmtNv>(x, rows, cols, rot_kind, g, norm, h, global_scale, codes,
                                     scales, scale_rows, scale_stride, zero_policy, stream);
+}
+
+extern "C" int fpq_row_inv_rms(const void* x, int64_t ld, int64_t rows, int64_t cols, float eps, float* inv_rms,
+                               void* stream) {
+  if (rows < 0 || cols < 0) return FPQ_E_SHAPE;
+  if (rows == 0) return FPQ_OK;
+  if (!x || !inv_rms) return FPQ_E_NULL;
+  if (cols == 0 || cols % 8 != 0 || ld < cols || ld % 8 != 0 || rows * ld >= (int64_t)1 << 34) return FPQ_E_SHAPE;
+  if (((uintptr_t)x & 15u) || ((uintptr_t)inv_rms & 3u)) return FPQ_E_ALIGN;
+  hipLaunchKernelGGL(fpq::row_inv_rms_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+                     (const uint4*)x, (uint32_t)rows, (uint32_t)(cols / 8), (uint32_t)(ld / 8), (float)cols, eps,
+                     inv_rms);
+  return (int)hipGetLastError();
+}
+
+extern "C" int fpq_rmsnorm_quantize_mx(const void* x, int64_t ld, const float* inv_rms, const void* weight,
+                                       int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                                       void* normed, void* codes, void* scales, int64_t scale_rows,
+                                       int64_t scale_stride, int zero_policy, void* stream) {
+  return fpq::dispatch_prologue<fpq::kFmtMx, fpq::kProRmsNorm>(x, ld, nullptr, 0, inv_rms, weight, normed, rows,
+                                                               cols, rot_kind, g, norm, nullptr, codes, scales,
+                                                               scale_rows, scale_stride, zero_policy, stream);
+}
+
+extern "C" int fpq_rmsnorm_quantize_nv(const void* x, int64_t ld, const float* inv_rms, const void* weight,
+                                       int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                                       const float* global_scale, void* normed, void* codes, void* scales,
+                                       int64_t scale_rows, int64_t scale_stride, int zero_policy, void* stream) {
+  return fpq::dispatch_prologue<fpq::kFmtNv, fpq::kProRmsNorm>(x, ld, nullptr, 0, inv_rms, weight, normed, rows,
+                                                               cols, rot_kind, g, norm, global_scale, codes,
+                                                               scales, scale_rows, scale_stride, zero_policy,
+                                                               stream);
+}
+
+extern "C" int fpq_silu_mul_quantize_mx(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                                        int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                                        void* product, void* codes, void* scales, int64_t scale_rows,
+                                        int64_t scale_stride, int zero_policy, void* stream) {
+  return fpq::dispatch_prologue<fpq::kFmtMx, fpq::kProSiluMul>(gate, ld_gate, up, ld_up, nullptr, nullptr, product,
+                                                               rows, cols, rot_kind, g, norm, nullptr, codes,
+                                                               scales, scale_rows, scale_stride, zero_policy,
+                                                               stream);
+}
+
+extern "C" int fpq_silu_mul_quantize_nv(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                                        int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                                        const float* global_scale, void* product, void* codes, void* scales,
+                                        int64_t scale_rows, int64_t scale_stride, int zero_policy,
+                                        void* stream) {
+  return fpq::dispatch_prologue<fpq::kFmtNv, fpq::kProSiluMul>(gate, ld_gate, up, ld_up, nullptr, nullptr, product,
+                                                               rows, cols, rot_kind, g, norm, global_scale, codes,
+                                                               scales, scale_rows, scale_stride, zero_policy,
+                                                               stream);
 }
 
 extern "C" int fpq_rotated_absmax(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,

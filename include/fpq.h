@@ -151,6 +151,45 @@ int fpq_gemm_mxf4_packed(const void* xq_packed, const void* xs_packed, const voi
                          int64_t M, int64_t N, int64_t K, void* stream);
 
 /*
+ * Quantizers fused with the elementwise producer of their input, so that the bf16 tensor between
+ * the two never travels through memory.  The reference's Llama blocks quantize exactly these
+ * tensors: act_fn(gate) * up before down_proj (src/utils/llama_utils.py:60-71) and the RMSNorm
+ * output before q/k/v and gate/up; each stands in for that elementwise sequence followed by
+ * qutlass.fusedQuantizeMx / fusedQuantizeNv (qutlass_ops.py:36-105).  Every PyTorch operator of
+ * the unfused sequence rounds to bf16 once, and so do these, in IEEE fp32 with a fixed operation
+ * order (no fused multiply-add, exp as a fixed polynomial), so codes and scales are bit-identical
+ * to quantizing the bf16 tensor the stated formula gives:
+ *   rmsnorm   v[r, c] = bf16(weight[c] * bf16(x[r, c] * inv_rms[r]))
+ *   silu_mul  v[r, c] = bf16(bf16(g / (1 + exp(-g))) * up[r, c]),  g = gate[r, c]
+ * x / gate / up are bf16 with row strides ld* (elements, multiples of 8, >= cols); `normed` /
+ * `product` is null or a bf16 [rows, cols] buffer that receives v; codes, scales, rot_kind, g,
+ * norm, zero_policy and global_scale as for fpq_quantize_mx / fpq_quantize_nv.  Hadamard
+ * (16..128) and identity rotations; others return FPQ_E_UNSUPPORTED.
+ *
+ * fpq_row_inv_rms: inv_rms[r] = 1 / sqrt(sum_c x[r, c]^2 / cols + eps), fp32, with the summation
+ * order: squares of 8 consecutive elements left to right, octet k into accumulator k % 64 in
+ * increasing k, accumulators combined by the butterfly a[i] += a[i ^ m], m = 1, 2, ..., 32.
+ */
+int fpq_row_inv_rms(const void* x, int64_t ld, int64_t rows, int64_t cols, float eps, float* inv_rms,
+                    void* stream);
+int fpq_rmsnorm_quantize_mx(const void* x, int64_t ld, const float* inv_rms, const void* weight,
+                            int64_t rows, int64_t cols, int rot_kind, int g, float norm, void* normed,
+                            void* codes, void* scales, int64_t scale_rows, int64_t scale_stride,
+                            int zero_policy, void* stream);
+int fpq_rmsnorm_quantize_nv(const void* x, int64_t ld, const float* inv_rms, const void* weight,
+                            int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                            const float* global_scale, void* normed, void* codes, void* scales,
+                            int64_t scale_rows, int64_t scale_stride, int zero_policy, void* stream);
+int fpq_silu_mul_quantize_mx(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                             int64_t rows, int64_t cols, int rot_kind, int g, float norm, void* product,
+                             void* codes, void* scales, int64_t scale_rows, int64_t scale_stride,
+                             int zero_policy, void* stream);
+int fpq_silu_mul_quantize_nv(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                             int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                             const float* global_scale, void* product, void* codes, void* scales,
+                             int64_t scale_rows, int64_t scale_stride, int zero_policy, void* stream);
+
+/*
  * *amax = max(*amax, max |rotate(x)|) as fp32, with the rotation of the quantize entry points
  * (rot_kind, g, norm, h as there; cols % g == 0).  The NVFP4 per-tensor multiplier the reference's
  * exporter tracks is 448 * 6 / this maximum, minimised over calls

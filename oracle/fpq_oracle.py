@@ -20,6 +20,8 @@ What it follows (all paths relative to the reference checkout):
 * quest scale + clip mask .... inference_lib/src/fp_quant/module/triton/mxfp4.py:51-59,105-110,
                                inference_lib/src/fp_quant/module/pseudoquant_linear_fns.py:20-22,
                                inference_lib/src/fp_quant/module/linear_fns.py:67-76
+* producers of x ............. src/utils/llama_utils.py:60-71 (act_fn(gate) * up before down_proj;
+                               RMSNorm before the q/k/v and gate/up quantizers)
 * linear ..................... inference_lib/src/fp_quant/module/linear_fns.py:496-514,
                                inference_lib/src/fp_quant/module/qutlass_ops.py:111-168
 
@@ -39,7 +41,8 @@ other (fp32 everywhere, bf16 only at the input and at the rotation matrix entrie
 Pin status (each function below is checked in tests/test_oracle_*.py against closed
 forms, exhaustive tables, library casts or brute force; none needed an import of the
 reference): rotation, E8M0 exponent, E2M1 RNE, packing, E4M3 cast, E8M0 cast, GEMM, the quest
-scale (against numpy float64 statistics and a per-group Python loop) and clip mask.
+scale (against numpy float64 statistics and a per-group Python loop) and clip mask; the two
+producers (silu_mul, rmsnorm) against float64 evaluations and torch's own operators.
 The third-party kernels the reference calls for this path (QuTLASS, un-vendored, version
 unpinned) have no fixtures in the reference: bit parity against QuTLASS itself is unpinned.
 """
@@ -344,7 +347,9 @@ def quest_scales(xg: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     mean = tot * torch.tensor(0.03125, dtype=f32)
     msq = tot_sq * torch.tensor(0.03125, dtype=f32)
     var = (msq - mean * mean).clamp_min(0.0)
-    sc = torch.sqrt(var) * torch.tensor(QUEST_GAUSSIAN_SCALE, dtype=f32) + torch.tensor(1e-8, dtype=f32)
+    # numpy's sqrt is the correctly rounded one on every machine (torch's vectorised CPU sqrt is not)
+    std = torch.from_numpy(np.sqrt(var.contiguous().numpy()))
+    sc = std * torch.tensor(QUEST_GAUSSIAN_SCALE, dtype=f32) + torch.tensor(1e-8, dtype=f32)
     e = floor_log2_exact(sc)
     s = torch.ldexp(torch.ones_like(sc), e)
     return s, (e + 127).to(torch.uint8)
@@ -414,6 +419,86 @@ def nv_tracked_global_scale(xr: torch.Tensor) -> float:
     amax = xr.abs().max().to(f32)
     rec = torch.where(amax == 0, torch.zeros_like(amax), torch.tensor(1.0, dtype=f32) / amax)
     return float(torch.tensor(FP8_E4M3_MAX * FP4_E2M1_MAX, dtype=f32) * rec)
+
+
+# ----------------------------------------------------------------------------- producers of x
+# The two elementwise producers whose output the quantizer consumes in a Llama block
+# (src/utils/llama_utils.py:60-71: act_fn(gate) * up feeds down_proj's quantizer; the block's
+# RMSNorm output feeds the q/k/v and gate/up quantizers), stated so that fusing them into the
+# quantize kernel is checkable bit for bit: bf16 in, bf16 out, every intermediate an IEEE fp32
+# operation in a fixed order (no fused multiply-add, no library exp).
+EXP_LOG2E = np.float32(1.44269504088896341)
+EXP_LN2_HI = np.float32(0.693359375)           # 9 significant bits: n * hi is exact
+EXP_LN2_LO = np.float32(-2.12194440e-4)
+EXP_POLY = tuple(np.float32(c) for c in (1.9875691500e-4, 1.3981999507e-3, 8.3334519073e-3,
+                                         4.1665795894e-2, 1.6666665459e-1, 5.0000001201e-1))
+
+
+def bf16_round(t: torch.Tensor) -> torch.Tensor:
+    """fp32 -> nearest-even bf16 -> fp32."""
+    return t.to(torch.float32).to(torch.bfloat16).to(torch.float32)
+
+
+def exp_det(t: torch.Tensor) -> torch.Tensor:
+    """exp(t) in fp32 by a fixed operation sequence: clamp to +-200, n = rint(t * log2e),
+    r = (t - n*ln2_hi) - n*ln2_lo, degree-5 polynomial in Horner form with separate multiply and
+    add, y = (p*r*r + r) + 1, result = ldexp(y, n) (overflows to inf, underflows gradually)."""
+    a = t.to(torch.float32).clamp(-200.0, 200.0).numpy()
+    n = np.rint(a * EXP_LOG2E).astype(np.float32)
+    r = (a - n * EXP_LN2_HI) - n * EXP_LN2_LO
+    p = np.full_like(r, EXP_POLY[0])
+    for c in EXP_POLY[1:]:
+        p = p * r + c
+    y = (p * (r * r) + r) + np.float32(1.0)
+    with np.errstate(over="ignore", under="ignore"):
+        out = np.ldexp(y, n.astype(np.int32)).astype(np.float32)
+    return torch.from_numpy(out)
+
+
+def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """bf16(bf16(silu(gate)) * up) with silu(g) = g / (1 + exp_det(-g)) in fp32: the bf16 tensor
+    `act_fn(gate) * up` of a Llama MLP (one rounding per PyTorch operator)."""
+    g = gate.to(torch.float32)
+    with np.errstate(over="ignore"):
+        d = torch.from_numpy(np.float32(1.0) + exp_det(-g).numpy())
+    s = bf16_round(g / d)
+    return (s * up.to(torch.float32)).to(torch.bfloat16)
+
+
+def row_inv_rms(x: torch.Tensor, eps: float) -> torch.Tensor:
+    """1 / sqrt(mean(x^2) + eps) per row in fp32.  Summation order: squares of 8 consecutive elements
+    left to right; those octet sums are dealt to 64 accumulators (octet c to accumulator c % 64, in
+    increasing c); the accumulators combine by the butterfly a[i] += a[i ^ m], m = 1, 2, ..., 32."""
+    xf = x.to(torch.float32)
+    rows, cols = xf.shape
+    sq = (xf * xf).view(rows, cols // 8, 8)
+    octet = sq[..., 0].clone()
+    for i in range(1, 8):
+        octet = octet + sq[..., i]
+    n_oct = cols // 8
+    pad = (-n_oct) % 64
+    if pad:
+        octet = torch.cat((octet, torch.zeros(rows, pad)), dim=1)
+    acc = torch.zeros(rows, 64)
+    for it in range(octet.shape[1] // 64):
+        acc = acc + octet[:, 64 * it: 64 * it + 64]
+    idx = torch.arange(64)
+    for m in (1, 2, 4, 8, 16, 32):
+        acc = acc + acc[:, idx ^ m]
+    # numpy for the correctly rounded division and square root (torch's CPU sqrt is vectorised
+    # differently from machine to machine and is not always the correctly rounded one)
+    total = acc[:, 0].contiguous().numpy()
+    mean = total / np.float32(cols)
+    inv = np.float32(1.0) / np.sqrt(mean + np.float32(eps))
+    return torch.from_numpy(inv.astype(np.float32))
+
+
+def rmsnorm(x: torch.Tensor, gamma: torch.Tensor, eps: float) -> torch.Tensor:
+    """bf16(gamma * bf16(x * inv_rms)): RMSNorm as a Llama block applies it to bf16 activations
+    (normalised value rounded to bf16, then the bf16 product with the weight)."""
+    r = row_inv_rms(x, eps)
+    n1 = bf16_round(x.to(torch.float32) * r.unsqueeze(-1))
+    return (n1 * gamma.to(torch.float32)).to(torch.bfloat16)
 
 
 # ----------------------------------------------------------------------------- dequantize / linear

@@ -177,3 +177,64 @@ def rotated_absmax(x_bf16, rot="hadamard", g=128, norm=None, h=None, start=0.0):
     _engine.check(st, "fpq_rotated_absmax")
     torch.cuda.synchronize()
     return float(amax.cpu())
+
+
+def row_inv_rms(x_bf16, eps, ld=None):
+    """Run fpq_row_inv_rms; `ld` > cols places the rows in a wider buffer.  Returns CPU fp32 [rows]."""
+    lib = _engine.lib()
+    rows, cols = x_bf16.shape
+    ld = cols if ld is None else ld
+    buf = torch.full((rows, ld), 7.0, dtype=torch.bfloat16, device="cuda")
+    buf[:, :cols] = x_bf16.to("cuda")
+    out = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda")
+    st = lib.fpq_row_inv_rms(buf.data_ptr(), ld, rows, cols, eps, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_row_inv_rms")
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+def _strided(t_bf16, ld):
+    rows, cols = t_bf16.shape
+    buf = torch.full((rows, ld), -3.0, dtype=torch.bfloat16, device="cuda")
+    buf[:, :cols] = t_bf16.to("cuda")
+    return buf
+
+
+def fused_quantize(kind, fmt, a, b, g=128, rot="hadamard", norm=None, global_scale=None, eps=1e-5,
+                   want_out=True, ld_a=None, ld_b=None, zero_policy=_engine.ZERO_REFERENCE, fill=0xCD):
+    """Run fpq_rmsnorm_quantize_* (kind "rmsnorm": a = x [R, C], b = weight [C]) or
+    fpq_silu_mul_quantize_* (kind "silu_mul": a = gate, b = up).  Returns CPU (codes, scales, out or None)."""
+    lib = _engine.lib()
+    rows, cols = a.shape
+    ld_a = cols if ld_a is None else ld_a
+    ld_b = cols if ld_b is None else ld_b
+    group = 32 if fmt == "mxfp4" else 16
+    a_dev = _strided(a, ld_a)
+    codes = torch.full((rows, cols // 2), fill, dtype=torch.uint8, device="cuda")
+    scales = torch.full((rows, cols // group), fill, dtype=torch.uint8, device="cuda")
+    out = torch.full((rows, cols), float("nan"), dtype=torch.bfloat16, device="cuda") if want_out else None
+    optr = out.data_ptr() if out is not None else None
+    if norm is None:
+        norm = float(torch.tensor(g ** -0.5, dtype=torch.bfloat16))
+    stream = torch.cuda.current_stream().cuda_stream
+    gs = torch.tensor([global_scale if global_scale is not None else 1.0], dtype=torch.float32, device="cuda")
+    tail = (codes.data_ptr(), scales.data_ptr(), rows, cols // group, zero_policy, stream)
+    if kind == "rmsnorm":
+        w = b.to("cuda").contiguous()
+        inv = torch.empty(rows, dtype=torch.float32, device="cuda")
+        _engine.check(lib.fpq_row_inv_rms(a_dev.data_ptr(), ld_a, rows, cols, eps, inv.data_ptr(), stream), "fpq_row_inv_rms")
+        head = (a_dev.data_ptr(), ld_a, inv.data_ptr(), w.data_ptr(), rows, cols, ROT[rot], g, norm)
+        if fmt == "mxfp4":
+            st = lib.fpq_rmsnorm_quantize_mx(*head, optr, *tail)
+        else:
+            st = lib.fpq_rmsnorm_quantize_nv(*head, gs.data_ptr(), optr, *tail)
+    else:
+        b_dev = _strided(b, ld_b)
+        head = (a_dev.data_ptr(), ld_a, b_dev.data_ptr(), ld_b, rows, cols, ROT[rot], g, norm)
+        if fmt == "mxfp4":
+            st = lib.fpq_silu_mul_quantize_mx(*head, optr, *tail)
+        else:
+            st = lib.fpq_silu_mul_quantize_nv(*head, gs.data_ptr(), optr, *tail)
+    _engine.check(st, f"fpq_{kind}_quantize")
+    torch.cuda.synchronize()
+    return codes.cpu(), scales.cpu(), (out.cpu() if out is not None else None)
