@@ -303,35 +303,45 @@ def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=
 
     out = {"model": f"Llama-3.1-8B architecture, {layers} layers, random weights, MXFP4 W4A4 Hadamard-128",
            "quantized_linears": len(qlinears)}
-    with torch.no_grad():
-        ids = torch.randint(0, cfg.vocab_size, (prefill_batch, seq), generator=gen).to(dev)
-        run = lambda: model(input_ids=ids, use_cache=False, logits_to_keep=1)
-        run()
-        ms, _ = timed(run, 3, False)
-        _, share = timed(run, 2, True)
-        out["prefill"] = {"batch": prefill_batch, "seq": seq, "ms": round(ms, 2),
-                          "tokens_per_s": round(prefill_batch * seq / (ms * 1e-3), 1),
-                          "linear_time_share": round(share, 3)}
-        out["decode"] = {}
-        for b in decode_batches:
-            ids = torch.randint(0, cfg.vocab_size, (b, seq), generator=gen).to(dev)
-            cache = model(input_ids=ids, use_cache=True, logits_to_keep=1).past_key_values
-            tok = torch.randint(0, cfg.vocab_size, (b, 1), generator=gen).to(dev)
-            state = {"cache": cache}
 
-            def step():
-                for _ in range(decode_steps):
-                    r = model(input_ids=tok, past_key_values=state["cache"], use_cache=True)
-                    state["cache"] = r.past_key_values
+    def measure(out, with_share):
+        with torch.no_grad():
+            ids = torch.randint(0, cfg.vocab_size, (prefill_batch, seq), generator=gen).to(dev)
+            run = lambda: model(input_ids=ids, use_cache=False, logits_to_keep=1)
+            run()
+            ms, _ = timed(run, 3, False)
+            _, share = timed(run, 2, True) if with_share else (None, None)
+            out["prefill"] = {"batch": prefill_batch, "seq": seq, "ms": round(ms, 2),
+                              "tokens_per_s": round(prefill_batch * seq / (ms * 1e-3), 1),
+                              "linear_time_share": round(share, 3) if share is not None else None}
+            out["decode"] = {}
+            for b in decode_batches:
+                ids = torch.randint(0, cfg.vocab_size, (b, seq), generator=gen).to(dev)
+                cache = model(input_ids=ids, use_cache=True, logits_to_keep=1).past_key_values
+                tok = torch.randint(0, cfg.vocab_size, (b, 1), generator=gen).to(dev)
+                state = {"cache": cache}
 
-            step()
-            ms, _ = timed(step, 2, False)
-            _, share = timed(step, 1, True)
-            out["decode"][f"batch{b}"] = {"kv_tokens": seq, "ms_per_step": round(ms / decode_steps, 3),
-                                          "tokens_per_s": round(b * decode_steps / (ms * 1e-3), 1),
-                                          "linear_time_share": round(share, 3)}
-            del cache, state
-            torch.cuda.empty_cache()
+                def step():
+                    for _ in range(decode_steps):
+                        r = model(input_ids=tok, past_key_values=state["cache"], use_cache=True)
+                        state["cache"] = r.past_key_values
+
+                step()
+                ms, _ = timed(step, 2, False)
+                _, share = timed(step, 1, True) if with_share else (None, None)
+                out["decode"][f"batch{b}"] = {"kv_tokens": seq, "ms_per_step": round(ms / decode_steps, 3),
+                                              "tokens_per_s": round(b * decode_steps / (ms * 1e-3), 1),
+                                              "linear_time_share": round(share, 3) if share is not None else None}
+                del cache, state
+                torch.cuda.empty_cache()
+
+    measure(out, True)
+    # the same model with the RMSNorms and the SiLU*up of every block fused into the quantizers that consume
+    # them (one fused kernel instead of PyTorch's elementwise operators followed by a quantizer)
+    from fp_quant.utils import fuse_producers
+    fused = {"patched_modules": fuse_producers(model)}
+    measure(fused, False)
+    out["fused_producers"] = fused
     return out
 
 

@@ -28,6 +28,16 @@ extern "C" int fpq_device_supported(int device) {
   return strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 0;
 }
 
+extern "C" int fpq_stream_capture_id(void* stream, unsigned long long* id) {
+  if (!id) return FPQ_E_NULL;
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  unsigned long long cid = 0;
+  const hipError_t err = hipStreamGetCaptureInfo((hipStream_t)stream, &status, &cid);
+  if (err != hipSuccess) return (int)err;
+  *id = status == hipStreamCaptureStatusNone ? 0ull : (cid ? cid : ~0ull);
+  return FPQ_OK;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Measurement hook: the rate at which the matrix pipes execute the FP4 block-scaled MFMA on
 // operands that never leave registers -- no memory traffic, no LDS, no barriers -- so the only

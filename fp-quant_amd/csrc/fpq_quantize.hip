@@ -7,6 +7,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/fpq.h"
 #include "fpq_device.h"
 
@@ -74,6 +76,21 @@ __device__ __forceinline__ float exp_det(float t) {
   return __builtin_ldexpf(y, (int)n);
 }
 
+// bf16(silu(g)) for every bf16 bit pattern g, filled once per device by silu_table_kernel: the
+// activation costs one 2-byte lookup per element (the hot part of the table stays in the L1)
+// instead of ~50 VALU operations, which would make the fused kernel compute-bound.
+__device__ uint16_t g_silu_table[65536];
+
+__global__ __launch_bounds__(256) void silu_table_kernel() {
+  const uint32_t bits = blockIdx.x * 256u + threadIdx.x;
+  const float g = __uint_as_float(bits << 16);
+  g_silu_table[bits] = (uint16_t)(__float_as_uint(bf16_rne(g / (1.0f + exp_det(-g)))) >> 16);
+}
+
+__device__ __forceinline__ float silu_bf16(uint32_t bits) {
+  return __uint_as_float((uint32_t)g_silu_table[bits] << 16);
+}
+
 __device__ __forceinline__ void unpack8(const uint4& raw, float (&p)[8]) {
   p[0] = bf16_lo(raw.x); p[1] = bf16_hi(raw.x);
   p[2] = bf16_lo(raw.y); p[3] = bf16_hi(raw.y);
@@ -106,14 +123,17 @@ __device__ __forceinline__ void lane8_load_rotate(const uint4* __restrict__ x, u
     float q[8];
     unpack8(raw, p);
     unpack8(aux, q);
+    if (PRO == kProSiluMul) {
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        p[2 * i] = silu_bf16(w[i] & 0xffffu);
+        p[2 * i + 1] = silu_bf16(w[i] >> 16);
+      }
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      float t;
-      if (PRO == kProRmsNorm) {
-        t = bf16_rne(p[i] * rs);
-      } else {
-        t = bf16_rne(p[i] / (1.0f + exp_det(-p[i])));
-      }
+      const float t = PRO == kProRmsNorm ? bf16_rne(p[i] * rs) : p[i];
       p[i] = bf16_rne(t * q[i]);
     }
     if (active && pro.out) {
@@ -912,6 +932,29 @@ static int launch_lane8_prologue(const void* x, int64_t rows, int64_t cols, floa
   return (int)hipGetLastError();
 }
 
+// Fills g_silu_table once per device.  The first call on a device builds the table on the caller's
+// stream and waits for it, so that calls on other streams can rely on it afterwards; while a stream
+// is being captured the build is recorded into the capture instead and nothing is remembered.
+static int ensure_silu_table(hipStream_t stream) {
+  static std::atomic<uint64_t> built{0};  // bit d: device d holds the table (devices >= 64 rebuild every call)
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  const uint64_t bit = dev < 64 ? (uint64_t)1 << dev : 0;
+  if (bit && (built.load(std::memory_order_acquire) & bit)) return 0;
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  e = hipStreamIsCapturing(stream, &cap);
+  if (e != hipSuccess) return (int)e;
+  hipLaunchKernelGGL(silu_table_kernel, dim3(256), dim3(256), 0, stream);
+  e = hipGetLastError();
+  if (e != hipSuccess) return (int)e;
+  if (cap != hipStreamCaptureStatusNone) return 0;
+  e = hipStreamSynchronize(stream);
+  if (e != hipSuccess) return (int)e;
+  if (bit) built.fetch_or(bit, std::memory_order_release);
+  return 0;
+}
+
 // x: the prologue's first input with row stride ld_first elements (kProSiluMul: `second` with
 // ld_second); Hadamard rotations of 16..128 and the identity only.
 template <int FMT, int PRO>
@@ -945,6 +988,9 @@ static int dispatch_prologue(const void* x, int64_t ld_first, const void* second
   if (((uintptr_t)x & 15u) || ((uintptr_t)second & 15u) || ((uintptr_t)col_scale & 15u) ||
       ((uintptr_t)out & 15u) || ((uintptr_t)row_scale & 3u) || ((uintptr_t)codes & 3u)) {
     return FPQ_E_ALIGN;
+  }
+  if (PRO == kProSiluMul) {
+    if (const int st = ensure_silu_table(stream)) return st;
   }
   Prologue pro;
   pro.row_scale = row_scale;

@@ -22,6 +22,7 @@ _SIGNATURES = {
     "fpq_version": ([], _I),
     "fpq_status_string": ([_I], ctypes.c_char_p),
     "fpq_device_supported": ([_I], _I),
+    "fpq_stream_capture_id": ([_P, ctypes.POINTER(ctypes.c_ulonglong)], _I),
     "fpq_quantize_mx": ([_P, _I64, _I64, _I, _I, _F, _P, _P, _P, _I64, _I64, _I, _P], _I),
     "fpq_quantize_nv": ([_P, _I64, _I64, _I, _I, _F, _P, _P, _P, _P, _I64, _I64, _I, _P], _I),
     "fpq_gemm_mxf4": ([_P, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _P], _I),

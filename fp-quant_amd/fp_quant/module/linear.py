@@ -167,3 +167,17 @@ class FPQuantLinear(nn.Module):
             f"store_master_weights: {cfg.store_master_weights}, pseudoquantization: "
             f"{cfg.pseudoquantization} isn't supported yet."
         )
+
+    def forward_quantized(self, activations, leading_shape) -> torch.Tensor:
+        """The GEMM (+ bias) of `forward` on activations that a fused producer has already rotated and
+        quantized for this layer (`hip_ops.QuantizedActivations`); returns [*leading_shape, out]."""
+        alpha = hip_ops.linear_alpha(self.weight_global_scale, self.act_global_scale)
+        bias = self.bias
+        fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16 and bias.is_contiguous()) else None
+        with torch.cuda.device(self.qweight.device):
+            y = hip_ops.linear_on(activations, self.qweight, self.scales, alpha, fused_bias,
+                                  torch.cuda.current_stream().cuda_stream)
+        y = y.unflatten(dim=0, sizes=tuple(leading_shape))
+        if bias is not None and fused_bias is None:
+            y += bias
+        return y

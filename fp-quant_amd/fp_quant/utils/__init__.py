@@ -4,3 +4,4 @@ from .replace import (
     replace_quantize_with_fp_quant_linear,
     replace_with_fp_quant_linear,
 )
+from .fuse import fuse_producers, unfuse_producers

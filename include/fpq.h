@@ -50,6 +50,14 @@ const char* fpq_status_string(int status);
 int fpq_device_supported(int device);
 
 /*
+ * *id = 0 if `stream` is not being captured into a graph, else a value unique to the capture in
+ * progress.  Host code that keeps results of one call for the next (activations quantized once for
+ * several layers) uses it to reuse them only within the same capture, or only outside any: work
+ * recorded during a capture has not run when the capture ends.
+ */
+int fpq_stream_capture_id(void* stream, unsigned long long* id);
+
+/*
  * Fused rotate + MXFP4 abs-max quantize.
  * Stands in for qutlass.fusedQuantizeMx behind fused_quantize_mx_op (qutlass_ops.py:36-71,
  * called from forward_quantize, linear_fns.py:34-41) with method "abs_max".

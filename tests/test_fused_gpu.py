@@ -100,3 +100,122 @@ def test_fused_quantize_argument_checks():
                                         c.data_ptr(), s.data_ptr(), 4, 4, 0, st) == -1
     assert lib.fpq_row_inv_rms(x.data_ptr(), 128, 4, 100, 1e-5, inv.data_ptr(), st) == -2
     torch.cuda.synchronize()
+
+
+# ---------------------------------------------------------------------------------------------
+# Module level: fuse_producers on Llama-style blocks
+
+
+def _cfg(fmt, g):
+    import fp_quant
+    return fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype(fmt), forward_method="abs_max",
+                                  backward_dtype=fp_quant.FPQuantDtype.BF16, hadamard_group_size=g)
+
+
+def _tiny_llama(fmt, g, seed=0):
+    import fp_quant
+    from transformers import LlamaConfig, LlamaForCausalLM
+    torch.manual_seed(seed)
+    cfg = LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                      num_key_value_heads=2, vocab_size=128, max_position_embeddings=256, rms_norm_eps=1e-5)
+    model = LlamaForCausalLM(cfg).to(device="cuda", dtype=torch.bfloat16).eval()
+    for p in model.parameters():        # norm weights away from 1 so that the weight product matters
+        if p.dim() == 1:
+            p.data.add_(0.1 * torch.randn_like(p))
+    return fp_quant.replace_quantize_with_fp_quant_linear(model, _cfg(fmt, g))
+
+
+@pytest.mark.parametrize("fmt,g", [("mxfp4", 32), ("mxfp4", 128), ("nvfp4", 16)])
+@pytest.mark.parametrize("tokens", [3, 40])
+def test_fused_norm_and_mlp_match_the_oracle_composition(fmt, g, tokens):
+    """A fused RMSNorm returns the oracle's bf16 tensor and its consumers give what they give when
+    handed that tensor unfused; the fused MLP equals down_proj on the oracle's silu*up."""
+    from fp_quant.module import hip_ops
+    from fp_quant.utils import fuse_producers, unfuse_producers
+    model = _tiny_llama(fmt, g)
+    block = model.model.layers[1]
+    x = (torch.randn(2, tokens, 256, device="cuda") * 1.5).to(torch.bfloat16)
+    with torch.no_grad():
+        want_y = O.rmsnorm(x.cpu().view(-1, 256), block.input_layernorm.weight.cpu(), 1e-5).view(x.shape).cuda()
+        want_q = block.self_attn.q_proj(want_y)
+        want_k = block.self_attn.k_proj(want_y.clone())
+        gate, up = block.mlp.gate_proj(x), block.mlp.up_proj(x)
+        h = O.silu_mul(gate.cpu().view(-1, 512), up.cpu().view(-1, 512)).view(gate.shape).cuda()
+        want_mlp = block.mlp.down_proj(h)
+
+        assert fuse_producers(model) == 6                     # two norms and one MLP per block
+        assert sorted(model.state_dict()) == sorted(_tiny_llama(fmt, g).state_dict())
+        hip_ops._shared_activations.clear()
+        y = block.input_layernorm(x)
+        assert torch.equal(y, want_y)
+        slot = hip_ops._shared_activations[0]
+        assert slot.ref() is y and slot.row_major is not None
+        assert torch.equal(block.self_attn.q_proj(y), want_q)
+        assert torch.equal(block.self_attn.k_proj(y), want_k)
+        assert hip_ops._shared_activations[0] is slot         # both projections used the norm's quantization
+        assert torch.equal(block.mlp(x), want_mlp)
+
+        # a consumer that does not match (other tensor) still computes its own quantization
+        assert torch.equal(block.self_attn.q_proj(want_y.clone()), want_q)
+
+        unfuse_producers(model)
+        hip_ops._shared_activations.clear()
+        block.input_layernorm(x)
+        assert 0 not in hip_ops._shared_activations
+
+
+@pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])
+def test_fused_llama_matches_unfused(fmt, g):
+    """Whole model: fused and unfused logits agree up to the rare bf16 flips between this library's
+    RMSNorm / SiLU arithmetic and PyTorch's, for prefill-sized and decode-sized batches."""
+    from fp_quant.utils import fuse_producers
+    model = _tiny_llama(fmt, g, seed=1)
+    ids = torch.randint(0, 128, (2, 48), generator=torch.Generator().manual_seed(2)).cuda()
+    with torch.no_grad():
+        want = model(ids).logits.float()
+        want1 = model(ids[:, :1]).logits.float()
+        assert fuse_producers(model) == 6
+        got = model(ids).logits.float()
+        got1 = model(ids[:, :1]).logits.float()
+    for a, b in ((got, want), (got1, want1)):
+        err = (a - b).norm() / b.norm()
+        assert float(err) < 0.02, float(err)
+    # generation through the fused model runs (KV cache, single-token steps)
+    out = model.generate(ids[:, :8], max_new_tokens=4, do_sample=False)
+    assert out.shape == (2, 12)
+
+
+@pytest.mark.parametrize("fmt,g,m", [("mxfp4", 128, 4), ("mxfp4", 128, 64), ("nvfp4", 16, 4)])
+def test_fused_block_is_graph_capturable(fmt, g, m):
+    """Inside a capture the norm's quantization is shared with the projections recorded after it;
+    replays follow new input contents, and eager calls afterwards never use captured results."""
+    from fp_quant.utils import fuse_producers
+    model = _tiny_llama(fmt, g, seed=3)
+    fuse_producers(model)
+    block = model.model.layers[0]
+
+    def step(x):
+        y = block.input_layernorm(x)
+        return block.self_attn.q_proj(y) + block.self_attn.o_proj(y), block.mlp(x)
+
+    static_x = torch.randn(m, 256, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        step(static_x)                                   # warm-up: tables, caches, packed weights
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_out = step(static_x)
+        for seed in range(3):
+            fresh = torch.randn(m, 256, device="cuda", generator=torch.Generator("cuda").manual_seed(seed)).to(torch.bfloat16)
+            eager = step(fresh.clone())                  # eager work between replays
+            static_x.copy_(fresh)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_out[0], eager[0]) and torch.equal(static_out[1], eager[1])
+        # an eager call on the captured input object right after a capture must quantize for itself
+        graph2 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph2):
+            step(static_x)
+        eager = step(static_x)
+        again = step(static_x.clone())
+        assert torch.equal(eager[0], again[0]) and torch.equal(eager[1], again[1])
