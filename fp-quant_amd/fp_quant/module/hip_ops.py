@@ -533,7 +533,10 @@ def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: i
     if act_global_scale is not None:
         gs = cached_on(act_global_scale, "_fpq_host", (act_global_scale._version, act_global_scale.data_ptr()),
                        lambda: float(act_global_scale))
-    return (rot, gs, stream, _capture_id.value, tuple(x_shape))
+    # the operand layout the GEMM will ask for is part of the key: the packed form can be made from the
+    # row-major one but not the other way round
+    want_packed = act_global_scale is None and packed_linear_eligible(x_shape[0], x_shape[1], "abs_max")
+    return (rot, gs, stream, _capture_id.value, tuple(x_shape), want_packed)
 
 
 def _publish(qa: QuantizedActivations, src: torch.Tensor, key, keep) -> None:
