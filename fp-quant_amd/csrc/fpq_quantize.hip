@@ -11,6 +11,7 @@
 
 #include "../../include/fpq.h"
 #include "fpq_device.h"
+#include "fpq_gemm_epilogue.h"  // LdsLimitOnce
 
 namespace fpq {
 
@@ -464,12 +465,23 @@ __device__ __forceinline__ uint32_t fix_zero_nibbles(uint32_t w) {
 // 2 * row + chunk, so the lane pairing of a 128-wide rotation is unchanged): the loads are 256-byte
 // row segments, and every 16-byte half of a lane's codes is exactly one lane slot of a packed
 // kilobyte block, so codes are stored straight from registers in two 512-byte runs per store.
-template <int EPL, int G, int FMT, int ROT, int ZERO, bool PACKED = false>
+//
+// PRO != kProNone (PACKED only) applies a producer's arithmetic to the values as they leave LDS (see
+// Prologue): kProRmsNorm scales by the row's 1/rms and the column's weight (16-byte loads that hit
+// the L1: a wave touches two 128-byte pieces of the weight) and can write the bf16 result;
+// kProSiluMul streams a second tile (the multiplier) through LDS next to the first and looks the
+// activation up in an LDS copy of the silu table's busy part (|g| in [2^-14, 128)), the rest in the
+// global table.
+constexpr uint32_t kSiluLdsFirst = 113u << 7;         // bf16 magnitude bits of 2^-14
+constexpr uint32_t kSiluLdsCount = 21u * 128u;        // magnitudes up to (not including) 2^7
+
+template <int EPL, int G, int FMT, int ROT, int ZERO, bool PACKED = false, int PRO = kProNone>
 __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
     const uint8_t* __restrict__ x, uint8_t* __restrict__ codes, uint8_t* __restrict__ scales,
     uint32_t n_chunks, uint32_t chunks_per_row, uint32_t rows, uint32_t scale_rows,
-    uint32_t scale_stride, float norm, const float* __restrict__ global_scale) {
+    uint32_t scale_stride, float norm, const float* __restrict__ global_scale, Prologue pro) {
   static_assert(!PACKED || (FMT == kFmtMx && EPL == 64), "packed output: MXFP4 with 64-element chunks");
+  static_assert(PRO == kProNone || PACKED, "prologues exist for the packed output only");
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
   constexpr int NG = EPL / GROUP;        // groups (= scale bytes) per chunk
   constexpr int PIECES = EPL / 8;        // 16-byte input pieces per chunk
@@ -479,12 +491,26 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
   constexpr int CW = EPL / 8;            // code dwords per chunk
   constexpr int CQ = CW / 4;             // 16-byte code pieces per chunk
   __shared__ __attribute__((aligned(128))) uint8_t smem[4][TILE];
+  // kProSiluMul: the second tile of every wave and the table copy live in dynamic LDS (together
+  // with the static part they exceed the 64 KB a kernel gets without asking); kProRmsNorm: a tile
+  // per wave for regrouping the by-product
+  extern __shared__ __attribute__((aligned(128))) uint8_t dyn_lds[];
+  uint16_t* silu_lds = (uint16_t*)(dyn_lds + 4 * TILE);
   __shared__ float2 lut[128];
+  if (PRO == kProSiluMul) {
+    for (uint32_t i = threadIdx.x; i < 2u * kSiluLdsCount; i += 256u) {
+      const uint32_t sgn = i >= kSiluLdsCount ? 1u : 0u;
+      silu_lds[i] = g_silu_table[(sgn << 15) | (kSiluLdsFirst + i - sgn * kSiluLdsCount)];
+    }
+    __syncthreads();
+  }
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t lane = threadIdx.x & 63u;
   uint8_t* my = smem[wave];
   const uint32_t my_base = (uint32_t)(uintptr_t)my;
+  uint8_t* my2 = dyn_lds + (PRO != kProNone ? wave : 0) * TILE;
+  const uint32_t my2_base = (uint32_t)(uintptr_t)my2;
 
   float gs = 1.0f, rg = 1.0f;
   bool nv_fast = true;
@@ -513,12 +539,17 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
   auto sw = [](uint32_t b) -> uint32_t { return PIECES == 8 ? ((b & 7u) ^ ((b >> 3) & 1u)) : (b % PIECES); };
   const uint32_t b_lo = lane / PIECES, j_lo = lane % PIECES;
   constexpr int NV_OFF = PIECES == 8 ? 2 : 4;  // distinct swizzle phases over the instruction index
-  const uint32_t row_bytes = chunks_per_row * CB;
+  // bytes from one row to the next (a prologue's inputs may sit in wider buffers)
+  const uint32_t row_bytes = PRO == kProNone ? chunks_per_row * CB : pro.ld_first * 16u;
+  const uint32_t row_bytes2 = PRO == kProSiluMul ? pro.ld_second * 16u : 0u;
   // PACKED: chunk b of the tile is row b / 2 of the row tile, chunk b % 2 of the pair
   const uint32_t b_off = PACKED ? (b_lo >> 1) * row_bytes + (b_lo & 1u) * CB : b_lo * CB;
-  uint32_t voff[NV_OFF];
+  uint32_t voff[NV_OFF], voff2[PRO == kProSiluMul ? NV_OFF : 1];
 #pragma unroll
-  for (int m = 0; m < NV_OFF; ++m) voff[m] = b_off + ((j_lo ^ sw(CPI * m + b_lo)) * 16u);
+  for (int m = 0; m < NV_OFF; ++m) {
+    voff[m] = b_off + ((j_lo ^ sw(CPI * m + b_lo)) * 16u);
+    if (PRO == kProSiluMul) voff2[m] = voff[m] - (b_lo >> 1) * row_bytes + (b_lo >> 1) * row_bytes2;
+  }
   const uint32_t rd_base = lane * CB, l_sw = sw(lane);
 
   const uint32_t pairs = chunks_per_row / 2u;  // PACKED: tiles per row tile
@@ -528,8 +559,11 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
     const uint32_t rt = PACKED ? tile / pairs : 0u, pr = PACKED ? tile - rt * pairs : 0u;
     // chunks (row-major) or rows (PACKED) of this tile that exist
     const uint32_t valid = PACKED ? min(32u, rows - rt * 32u) : min(64u, n_chunks - tile * 64u);
-    const uint8_t* src = PACKED ? x + ((size_t)rt * 32u * chunks_per_row + 2u * pr) * CB
+    const uint8_t* src = PACKED ? x + (size_t)rt * 32u * row_bytes + (size_t)(2u * pr) * CB
                                 : x + (size_t)tile * TILE;
+    const uint8_t* src2 = PRO == kProSiluMul
+                              ? (const uint8_t*)pro.second + (size_t)rt * 32u * row_bytes2 + (size_t)(2u * pr) * CB
+                              : nullptr;
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
       // The lane offset is an unsigned 32-bit addend to a scalar base, so it must never be
@@ -539,8 +573,13 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
       if (PACKED) {
         const bool instr_valid = (uint32_t)(CPI / 2 * i) < valid;          // wave-uniform
         const uint8_t* base_i = instr_valid ? src + (size_t)(CPI / 2 * i) * row_bytes : src;
-        if (CPI / 2 * i + (b_lo >> 1) >= valid) off = (b_lo & 1u) * CB + j_lo * 16u;
+        const bool past = CPI / 2 * i + (b_lo >> 1) >= valid;
+        if (past) off = (b_lo & 1u) * CB + j_lo * 16u;
         lds_dma16_nt(base_i, off, my_base + i * 1024u);
+        if (PRO == kProSiluMul) {
+          const uint8_t* base2_i = instr_valid ? src2 + (size_t)(CPI / 2 * i) * row_bytes2 : src2;
+          lds_dma16_nt(base2_i, past ? off : voff2[i % NV_OFF], my2_base + i * 1024u);
+        }
       } else {
         const bool instr_valid = (uint32_t)(CPI * i) < valid;                // wave-uniform
         const uint8_t* base_i = instr_valid ? src + i * 1024 : src;          // scalar address arithmetic
@@ -551,14 +590,70 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
     wait_vmem();
 
     // this lane's chunk: out of LDS, rotated
+    // prologue operands of this lane: its row (clamped: padding rows of the last row tile compute on
+    // a valid row's data and are zeroed before the store) and its first 8-element column chunk
+    const uint32_t p_row = PRO == kProNone ? 0u : min(rt * 32u + (lane >> 1), rows - 1u);
+    const uint32_t p_cc = PRO == kProNone ? 0u : (2u * pr + (lane & 1u)) * (uint32_t)PIECES;
+    const float p_rs = PRO == kProRmsNorm ? pro.row_scale[p_row] : 0.0f;
+    const bool p_store = PRO != kProNone && pro.out != nullptr && (lane >> 1) < valid;
     auto load_rotate = [&](float (&v)[EPL]) {
 #pragma unroll
     for (int k = 0; k < PIECES; ++k) {
       const uint4 raw = *(const uint4*)(my + rd_base + ((k ^ l_sw) * 16u));
-      v[8 * k + 0] = bf16_lo(raw.x); v[8 * k + 1] = bf16_hi(raw.x);
-      v[8 * k + 2] = bf16_lo(raw.y); v[8 * k + 3] = bf16_hi(raw.y);
-      v[8 * k + 4] = bf16_lo(raw.z); v[8 * k + 5] = bf16_hi(raw.z);
-      v[8 * k + 6] = bf16_lo(raw.w); v[8 * k + 7] = bf16_hi(raw.w);
+      float e[8];
+      unpack8(raw, e);
+      if (PRO != kProNone) {
+        float q[8];
+        if (PRO == kProRmsNorm) {
+          unpack8(pro.col_scale[p_cc + k], q);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) e[i] = bf16_rne(e[i] * p_rs);
+        } else {
+          unpack8(*(const uint4*)(my2 + rd_base + ((k ^ l_sw) * 16u)), q);
+          const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const uint32_t bits = (i & 1) ? (w[i >> 1] >> 16) : (w[i >> 1] & 0xffffu);
+            const uint32_t idx = (bits & 0x7fffu) - kSiluLdsFirst;
+            uint32_t t;
+            if (idx < kSiluLdsCount) {
+              t = silu_lds[(bits >> 15) * kSiluLdsCount + idx];
+            } else {
+              t = g_silu_table[bits];
+            }
+            e[i] = __uint_as_float(t << 16);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) e[i] = bf16_rne(e[i] * q[i]);
+        if (PRO == kProRmsNorm ? pro.out != nullptr : p_store) {
+          const uint4 packed8 =
+              make_uint4((__float_as_uint(e[0]) >> 16) | (__float_as_uint(e[1]) & 0xffff0000u),
+                         (__float_as_uint(e[2]) >> 16) | (__float_as_uint(e[3]) & 0xffff0000u),
+                         (__float_as_uint(e[4]) >> 16) | (__float_as_uint(e[5]) & 0xffff0000u),
+                         (__float_as_uint(e[6]) >> 16) | (__float_as_uint(e[7]) & 0xffff0000u));
+          if (PRO == kProRmsNorm) {
+            // parked in the wave's second LDS tile at the input's (swizzled) place, stored below
+            *(uint4*)(my2 + rd_base + ((k ^ l_sw) * 16u)) = packed8;
+          } else {
+            pro.out[(size_t)p_row * chunks_per_row * PIECES + p_cc + k] = packed8;
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[8 * k + i] = e[i];
+    }
+    if (PRO == kProRmsNorm && pro.out != nullptr) {
+      // the by-product leaves as 256-byte row segments: store i covers rows 4 i .. 4 i + 3 of the
+      // tile, 16 lanes per row (the two chunks of the row, 8 pieces each)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t r = 4u * i + (lane >> 4), ls = 2u * r + ((lane >> 3) & 1u), kk = lane & 7u;
+        const uint4 o = *(const uint4*)(my2 + ls * CB + ((kk ^ sw(ls)) * 16u));
+        if (r < valid) {
+          pro.out[((size_t)rt * 32u + r) * chunks_per_row * PIECES + (size_t)(2u * pr) * PIECES + (lane & 15u)] = o;
+        }
+      }
     }
     if (ROT == FPQ_ROT_HADAMARD || ROT == FPQ_ROT_GSR) {
 #pragma unroll
@@ -783,7 +878,7 @@ static int launch_stream(const void* x, int64_t rows, int64_t cols, float norm, 
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint8_t*)x, (uint8_t*)codes,
                        (uint8_t*)scales, (uint32_t)n_chunks, (uint32_t)(cols / EPL), (uint32_t)rows,
-                       (uint32_t)scale_rows, (uint32_t)scale_stride, norm, gsp);
+                       (uint32_t)scale_rows, (uint32_t)scale_stride, norm, gsp, Prologue{});
   };
   if (zero_policy == FPQ_ZERO_REFERENCE) {
     go(quantize_stream_kernel<EPL, G, FMT, ROT, kZeroReference>);
@@ -793,23 +888,34 @@ static int launch_stream(const void* x, int64_t rows, int64_t cols, float norm, 
   return (int)hipGetLastError();
 }
 
-template <int G, int ROT>
+constexpr int kSiluDynLds = 4 * 64 * 128 + 2 * (int)kSiluLdsCount * 2;  // second tiles + table copy
+
+template <int G, int ROT, int PRO = kProNone>
 static int launch_stream_packed(const void* x, int64_t rows, int64_t cols, float norm, void* codes,
-                                void* scales, int zero_policy, hipStream_t stream) {
+                                void* scales, int zero_policy, hipStream_t stream,
+                                const Prologue& pro = Prologue{}) {
   const int64_t n_tiles = ((rows + 31) / 32) * (cols / 128);
   int64_t blocks = (n_tiles + 3) / 4;
   if (blocks > 1024) blocks = 1024;
   const dim3 grid((unsigned)blocks), block(256);
+  // kProRmsNorm: one more tile per wave, in which the bf16 by-product is regrouped into row segments
+  constexpr int kDyn = PRO == kProSiluMul ? kSiluDynLds : PRO == kProRmsNorm ? 4 * 64 * 128 : 0;
+  int status = 0;
   auto go = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint8_t*)x, (uint8_t*)codes,
+    if (kDyn) {
+      static LdsLimitOnce limit;
+      if ((status = limit.ensure((const void*)kernel, kDyn)) != 0) return;
+    }
+    hipLaunchKernelGGL(kernel, grid, block, kDyn, stream, (const uint8_t*)x, (uint8_t*)codes,
                        (uint8_t*)scales, (uint32_t)(rows * cols / 64), (uint32_t)(cols / 64),
-                       (uint32_t)rows, 0u, 0u, norm, (const float*)nullptr);
+                       (uint32_t)rows, 0u, 0u, norm, (const float*)nullptr, pro);
   };
   if (zero_policy == FPQ_ZERO_REFERENCE) {
-    go(quantize_stream_kernel<64, G, kFmtMx, ROT, kZeroReference, true>);
+    go(quantize_stream_kernel<64, G, kFmtMx, ROT, kZeroReference, true, PRO>);
   } else {
-    go(quantize_stream_kernel<64, G, kFmtMx, ROT, kZeroSigned, true>);
+    go(quantize_stream_kernel<64, G, kFmtMx, ROT, kZeroSigned, true, PRO>);
   }
+  if (status) return status;
   return (int)hipGetLastError();
 }
 
@@ -1014,6 +1120,60 @@ static int dispatch_prologue(const void* x, int64_t ld_first, const void* second
   return FPQ_E_ROTATION;
 }
 
+// The same with the packed operand layout as output (streaming kernel; cols % 256 == 0).
+template <int PRO>
+static int dispatch_prologue_packed(const void* x, int64_t ld_first, const void* second, int64_t ld_second,
+                                    const float* row_scale, const void* col_scale, void* out, int64_t rows,
+                                    int64_t cols, int rot_kind, int g, float norm, void* codes, void* scales,
+                                    int zero_policy, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (rows < 0 || cols < 0) return FPQ_E_SHAPE;
+  if (rows == 0 || cols == 0) return FPQ_OK;
+  if (!x || !codes || !scales) return FPQ_E_NULL;
+  if (PRO == kProRmsNorm && (!row_scale || !col_scale)) return FPQ_E_NULL;
+  if (PRO == kProSiluMul && !second) return FPQ_E_NULL;
+  if (zero_policy != FPQ_ZERO_REFERENCE && zero_policy != FPQ_ZERO_SIGNED) return FPQ_E_POLICY;
+  if (rot_kind == FPQ_ROT_IDENTITY) g = 32;
+  if (rot_kind != FPQ_ROT_IDENTITY && rot_kind != FPQ_ROT_HADAMARD) {
+    return (rot_kind == FPQ_ROT_GSR || rot_kind == FPQ_ROT_GENERAL) ? FPQ_E_UNSUPPORTED : FPQ_E_ROTATION;
+  }
+  if (g != 16 && g != 32 && g != 64 && g != 128) return FPQ_E_ROTATION;
+  if (cols % 256 != 0) return FPQ_E_SHAPE;
+  if (ld_first < cols || ld_first % 8 != 0) return FPQ_E_SHAPE;
+  if (PRO == kProSiluMul && (ld_second < cols || ld_second % 8 != 0)) return FPQ_E_SHAPE;
+  // 32-bit byte offsets inside a row tile, 32-bit chunk counts
+  if (rows * cols >= (int64_t)1 << 34 || ld_first >= (int64_t)1 << 24 || ld_second >= (int64_t)1 << 24) {
+    return FPQ_E_SHAPE;
+  }
+  if (((uintptr_t)x & 15u) || ((uintptr_t)second & 15u) || ((uintptr_t)col_scale & 15u) ||
+      ((uintptr_t)out & 15u) || ((uintptr_t)row_scale & 3u) || ((uintptr_t)codes & 15u) ||
+      ((uintptr_t)scales & 3u)) {
+    return FPQ_E_ALIGN;
+  }
+  if (PRO == kProSiluMul) {
+    if (const int st = ensure_silu_table(stream)) return st;
+  }
+  Prologue pro;
+  pro.row_scale = row_scale;
+  pro.col_scale = (const uint4*)col_scale;
+  pro.second = (const uint4*)second;
+  pro.out = (uint4*)out;
+  pro.chunks_per_row = (uint32_t)(cols / 8);
+  pro.ld_first = (uint32_t)(ld_first / 8);
+  pro.ld_second = (uint32_t)(ld_second / 8);
+#define FPQ_LAUNCH_PRO_PACKED(GG, RR) \
+  return launch_stream_packed<GG, RR, PRO>(x, rows, cols, norm, codes, scales, zero_policy, stream, pro)
+  if (rot_kind == FPQ_ROT_IDENTITY) FPQ_LAUNCH_PRO_PACKED(32, FPQ_ROT_IDENTITY);
+  switch (g) {
+    case 16: FPQ_LAUNCH_PRO_PACKED(16, FPQ_ROT_HADAMARD);
+    case 32: FPQ_LAUNCH_PRO_PACKED(32, FPQ_ROT_HADAMARD);
+    case 64: FPQ_LAUNCH_PRO_PACKED(64, FPQ_ROT_HADAMARD);
+    case 128: FPQ_LAUNCH_PRO_PACKED(128, FPQ_ROT_HADAMARD);
+  }
+#undef FPQ_LAUNCH_PRO_PACKED
+  return FPQ_E_ROTATION;
+}
+
 // 1 / sqrt(mean(x^2) + eps) of every row, one wave per row.  Fixed summation order: squares of 8
 // consecutive elements left to right; lane l accumulates the octets l, l + 64, ... in that order;
 // the 64 lane sums combine by the butterfly a += a[lane ^ m], m = 1, 2, ..., 32.
@@ -1203,6 +1363,24 @@ extern "C" int fpq_silu_mul_quantize_nv(const void* gate, int64_t ld_gate, const
                                                                rows, cols, rot_kind, g, norm, global_scale, codes,
                                                                scales, scale_rows, scale_stride, zero_policy,
                                                                stream);
+}
+
+extern "C" int fpq_rmsnorm_quantize_mx_packed(const void* x, int64_t ld, const float* inv_rms, const void* weight,
+                                              int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                                              void* normed, void* packed_codes, void* packed_scales,
+                                              int zero_policy, void* stream) {
+  return fpq::dispatch_prologue_packed<fpq::kProRmsNorm>(x, ld, nullptr, 0, inv_rms, weight, normed, rows, cols,
+                                                         rot_kind, g, norm, packed_codes, packed_scales,
+                                                         zero_policy, stream);
+}
+
+extern "C" int fpq_silu_mul_quantize_mx_packed(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                                               int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                                               void* product, void* packed_codes, void* packed_scales,
+                                               int zero_policy, void* stream) {
+  return fpq::dispatch_prologue_packed<fpq::kProSiluMul>(gate, ld_gate, up, ld_up, nullptr, nullptr, product, rows,
+                                                         cols, rot_kind, g, norm, packed_codes, packed_scales,
+                                                         zero_policy, stream);
 }
 
 extern "C" int fpq_rotated_absmax(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,

@@ -39,6 +39,8 @@ _SIGNATURES = {
     "fpq_rmsnorm_quantize_mx": ([_P, _I64, _P, _P, _I64, _I64, _I, _I, _F, _P, _P, _P, _I64, _I64, _I, _P], _I),
     "fpq_rmsnorm_quantize_nv": ([_P, _I64, _P, _P, _I64, _I64, _I, _I, _F, _P, _P, _P, _P, _I64, _I64, _I, _P], _I),
     "fpq_silu_mul_quantize_mx": ([_P, _I64, _P, _I64, _I64, _I64, _I, _I, _F, _P, _P, _P, _I64, _I64, _I, _P], _I),
+    "fpq_rmsnorm_quantize_mx_packed": ([_P, _I64, _P, _P, _I64, _I64, _I, _I, _F, _P, _P, _P, _I, _P], _I),
+    "fpq_silu_mul_quantize_mx_packed": ([_P, _I64, _P, _I64, _I64, _I64, _I, _I, _F, _P, _P, _P, _I, _P], _I),
     "fpq_silu_mul_quantize_nv": ([_P, _I64, _P, _I64, _I64, _I64, _I, _I, _F, _P, _P, _P, _P, _I64, _I64, _I, _P], _I),
     "fpq_packed_scales_bytes_nv": ([_I64, _I64], _I64),
     "fpq_pack_nvf4": ([_P, _P, _I64, _I64, _I64, _P, _P, _P], _I),

@@ -664,9 +664,21 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
     fpq_<entry>_quantize_{mx,nv}; None if the library has no fused kernel for this rotation."""
     lib = _engine.lib()
     group = 16 if nvfp4 else 32
+    optr = out.data_ptr() if out is not None else None
+    if not nvfp4 and packed_linear_eligible(rows, cols, "abs_max"):
+        # straight into the operand layout of the packed GEMM (streaming kernel)
+        pc = torch.empty(lib.fpq_packed_codes_bytes(rows, cols), dtype=torch.uint8, device=dev)
+        ps = torch.empty(lib.fpq_packed_scales_bytes(rows, cols), dtype=torch.uint8, device=dev)
+        st = getattr(lib, f"fpq_{entry}_quantize_mx_packed")(*head, rows, cols, kind, h.shape[0], norm, optr,
+                                                             pc.data_ptr(), ps.data_ptr(), ZERO_NIBBLE_POLICY, stream)
+        if st == _engine.E_UNSUPPORTED:
+            return None
+        _engine.check(st, f"fpq_{entry}_quantize_mx_packed")
+        qa = QuantizedActivations(rows, cols, nvfp4)
+        qa.mx_packed = (pc, ps)
+        return qa
     codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=dev)
     scales = torch.empty(rows, cols // group, dtype=torch.uint8, device=dev)
-    optr = out.data_ptr() if out is not None else None
     tail = (optr, codes.data_ptr(), scales.data_ptr(), rows, cols // group, ZERO_NIBBLE_POLICY, stream)
     if nvfp4:
         gs = as_f32_scalar(act_global_scale)

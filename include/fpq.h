@@ -196,6 +196,15 @@ int fpq_silu_mul_quantize_nv(const void* gate, int64_t ld_gate, const void* up, 
                              int64_t rows, int64_t cols, int rot_kind, int g, float norm,
                              const float* global_scale, void* product, void* codes, void* scales,
                              int64_t scale_rows, int64_t scale_stride, int zero_policy, void* stream);
+/* The MXFP4 ones writing the packed operand layout (as fpq_quantize_mx_packed; cols % 256 == 0). */
+int fpq_rmsnorm_quantize_mx_packed(const void* x, int64_t ld, const float* inv_rms, const void* weight,
+                                   int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                                   void* normed, void* packed_codes, void* packed_scales, int zero_policy,
+                                   void* stream);
+int fpq_silu_mul_quantize_mx_packed(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                                    int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                                    void* product, void* packed_codes, void* packed_scales, int zero_policy,
+                                    void* stream);
 
 /*
  * *amax = max(*amax, max |rotate(x)|) as fp32, with the rotation of the quantize entry points

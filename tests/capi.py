@@ -238,3 +238,35 @@ def fused_quantize(kind, fmt, a, b, g=128, rot="hadamard", norm=None, global_sca
     _engine.check(st, f"fpq_{kind}_quantize")
     torch.cuda.synchronize()
     return codes.cpu(), scales.cpu(), (out.cpu() if out is not None else None)
+
+
+def fused_quantize_packed(kind, a, b, g=128, rot="hadamard", norm=None, eps=1e-5, want_out=True, ld_a=None,
+                          ld_b=None, zero_policy=_engine.ZERO_REFERENCE, fill=0xCD):
+    """fused_quantize for MXFP4 with the packed operand layout as output.  Returns CPU
+    (packed codes, packed scales, out or None)."""
+    lib = _engine.lib()
+    rows, cols = a.shape
+    ld_a = cols if ld_a is None else ld_a
+    ld_b = cols if ld_b is None else ld_b
+    a_dev = _strided(a, ld_a)
+    cb, sb = packed_sizes(rows, cols)
+    pc = torch.full((cb,), fill, dtype=torch.uint8, device="cuda")
+    ps = torch.full((sb,), fill, dtype=torch.uint8, device="cuda")
+    out = torch.full((rows, cols), float("nan"), dtype=torch.bfloat16, device="cuda") if want_out else None
+    optr = out.data_ptr() if out is not None else None
+    if norm is None:
+        norm = float(torch.tensor(g ** -0.5, dtype=torch.bfloat16))
+    stream = torch.cuda.current_stream().cuda_stream
+    if kind == "rmsnorm":
+        w = b.to("cuda").contiguous()
+        inv = torch.empty(rows, dtype=torch.float32, device="cuda")
+        _engine.check(lib.fpq_row_inv_rms(a_dev.data_ptr(), ld_a, rows, cols, eps, inv.data_ptr(), stream), "fpq_row_inv_rms")
+        st = lib.fpq_rmsnorm_quantize_mx_packed(a_dev.data_ptr(), ld_a, inv.data_ptr(), w.data_ptr(), rows, cols,
+                                                ROT[rot], g, norm, optr, pc.data_ptr(), ps.data_ptr(), zero_policy, stream)
+    else:
+        b_dev = _strided(b, ld_b)
+        st = lib.fpq_silu_mul_quantize_mx_packed(a_dev.data_ptr(), ld_a, b_dev.data_ptr(), ld_b, rows, cols, ROT[rot],
+                                                 g, norm, optr, pc.data_ptr(), ps.data_ptr(), zero_policy, stream)
+    _engine.check(st, f"fpq_{kind}_quantize_mx_packed")
+    torch.cuda.synchronize()
+    return pc.cpu(), ps.cpu(), (out.cpu() if out is not None else None)

@@ -76,6 +76,55 @@ def test_silu_mul_quantize_bit_exact(fmt, rot, g, rows, cols):
     del both
 
 
+PACKED_CASES = [("hadamard", 16), ("hadamard", 32), ("hadamard", 64), ("hadamard", 128), ("identity", 32)]
+
+
+@pytest.mark.parametrize("rot,g", PACKED_CASES)
+@pytest.mark.parametrize("kind", ["rmsnorm", "silu_mul"])
+@pytest.mark.parametrize("rows,cols", [(1, 256), (70, 512), (300, 1024)])
+def test_fused_quantize_packed_bit_exact(kind, rot, g, rows, cols):
+    """The streaming kernel with a prologue: packed codes and scales (ragged last row tile, strided
+    inputs, extreme exponents that take the slow path) and the bf16 by-product."""
+    from tests.test_packed_gpu import pack_by_definition
+    a = make_student_t(rows, cols, seed=rows + g) * 2
+    if kind == "rmsnorm":
+        gen = torch.Generator().manual_seed(cols)
+        b = (1 + 0.3 * torch.randn(cols, generator=gen)).to(torch.bfloat16)
+        if rows > 8:
+            b[64:96] = 0.0                           # a zero group in every row
+            a[5] *= 2.0 ** -60                       # (normalisation undoes the row's magnitude)
+        want_v = O.rmsnorm(a, b, 1e-5)
+    else:
+        b = make_outlier_normal(rows, cols, seed=cols + g)
+        a[0, :8] = torch.tensor([-300.0, 300.0, 0.0, -0.0, -88.5, 88.5, -20.0, 1e-30]).to(torch.bfloat16)
+        if rows > 8:
+            b[3, 64:96] = 0.0
+            b[7] *= 2.0 ** -110                      # exponents outside the fast range
+            b[9] *= 2.0 ** 100
+        want_v = O.silu_mul(a, b)
+    okind = O.ROT_HADAMARD if rot == "hadamard" else O.ROT_IDENTITY
+    wc, ws, _ = O.quantize_mx(want_v, okind, g, float(O.hadamard_matrix(g)[0, 0]))
+    want_c, want_s = pack_by_definition(wc, ws, cols)
+    lds = dict(ld_a=cols + 64, ld_b=2 * cols) if rows == 70 else {}
+    pc, ps, out = capi.fused_quantize_packed(kind, a, b, g=g, rot=rot, **lds)
+    assert torch.equal(out.view(torch.int16), want_v.view(torch.int16))
+    assert torch.equal(pc, want_c) and torch.equal(ps, want_s)
+    pc2, ps2, none = capi.fused_quantize_packed(kind, a, b, g=g, rot=rot, want_out=False)
+    assert none is None and torch.equal(pc2, want_c) and torch.equal(ps2, want_s)
+
+
+def test_fused_quantize_packed_full_size_matches_generic_kernel():
+    """A down_proj-sized input: the streaming fused kernel equals the generic fused kernel re-tiled."""
+    from tests.test_packed_gpu import pack_by_definition
+    rows, cols = 512, 14336
+    gate = make_student_t(rows, cols, seed=1) * 2
+    up = make_outlier_normal(rows, cols, seed=2)
+    codes, scales, _ = capi.fused_quantize("silu_mul", "mxfp4", gate, up, g=128, want_out=False)
+    want_c, want_s = pack_by_definition(codes, scales, cols)
+    pc, ps, _ = capi.fused_quantize_packed("silu_mul", gate, up, g=128, want_out=False)
+    assert torch.equal(pc, want_c) and torch.equal(ps, want_s)
+
+
 def test_fused_quantize_argument_checks():
     from fp_quant import _engine
     lib = _engine.lib()
@@ -149,7 +198,7 @@ def test_fused_norm_and_mlp_match_the_oracle_composition(fmt, g, tokens):
         y = block.input_layernorm(x)
         assert torch.equal(y, want_y)
         slot = hip_ops._shared_activations[0]
-        assert slot.ref() is y and slot.row_major is not None
+        assert slot.ref() is y and (slot.row_major is not None or slot.mx_packed is not None)
         assert torch.equal(block.self_attn.q_proj(y), want_q)
         assert torch.equal(block.self_attn.k_proj(y), want_k)
         assert hip_ops._shared_activations[0] is slot         # both projections used the norm's quantization
