@@ -102,6 +102,66 @@ def bench_quantize(torch, fmt, rows, cols, g, steps, warmup, seed, packed=False)
     }
 
 
+def bench_fused_producers(torch, steps, warmup):
+    """The quantizers fused with the producer of their input at Llama-3.1-8B prefill sizes (8192 tokens), MXFP4
+    Hadamard-128, packed output, through the C ABI: RMSNorm (row statistic + fused kernel, with the bf16
+    by-product) over [8192, 4096] and SiLU(gate)*up over [8192, 14336].  Algorithmic bytes: inputs once, codes,
+    scales, by-product."""
+    from fp_quant import _engine
+    lib = _engine.lib()
+    dev = torch.device("cuda:0")
+    norm = float(torch.tensor(128 ** -0.5, dtype=torch.bfloat16))
+    stream = torch.cuda.current_stream().cuda_stream
+    out = {}
+
+    def packed(rows, cols):
+        return (torch.empty(lib.fpq_packed_codes_bytes(rows, cols), dtype=torch.uint8, device=dev),
+                torch.empty(lib.fpq_packed_scales_bytes(rows, cols), dtype=torch.uint8, device=dev))
+
+    rows, cols = 8192, 4096
+    n_buf = 8
+    xs = [outlier_normal(torch, rows, cols, 10 + i).to(dev) for i in range(2)]
+    xs = [xs[i % 2].roll(i, 0).contiguous() for i in range(n_buf)]
+    w = (1 + 0.1 * torch.randn(cols)).to(torch.bfloat16).to(dev)
+    inv = torch.empty(rows, dtype=torch.float32, device=dev)
+    y = torch.empty(rows, cols, dtype=torch.bfloat16, device=dev)
+    pc, ps = packed(rows, cols)
+
+    def run_norm(i):
+        st = lib.fpq_row_inv_rms(xs[i].data_ptr(), cols, rows, cols, 1e-5, inv.data_ptr(), stream)
+        st = st or lib.fpq_rmsnorm_quantize_mx_packed(xs[i].data_ptr(), cols, inv.data_ptr(), w.data_ptr(), rows, cols,
+                                                      0, 128, norm, y.data_ptr(), pc.data_ptr(), ps.data_ptr(), 0, stream)
+        if st != 0:
+            _engine.check(st, "bench rmsnorm_quantize")
+
+    wall, ev = time_kernel(torch, run_norm, n_buf, steps, warmup)
+    algo = rows * cols * (2 + 2 + 0.5 + 1.0 / 32)
+    out["rmsnorm_quantize"] = {"workload": f"rmsnorm_quantize_mx_packed_{rows}x{cols}_had128 (+ bf16 by-product)",
+                               "kernels_us": round(ev * 1e3, 2), "GB/s": round(algo / (ev * 1e-3) / 1e9, 1),
+                               "hbm_frac": round(algo / (ev * 1e-3) / 8e12, 4)}
+    del xs, y
+
+    cols = 14336
+    n_buf = 3
+    g0 = student_t(torch, rows, cols, 20).to(dev)
+    gates = [g0.roll(i, 0).contiguous() for i in range(n_buf)]
+    ups = [g0.roll(i + 1, 1).contiguous() for i in range(n_buf)]
+    pc, ps = packed(rows, cols)
+
+    def run_silu(i):
+        st = lib.fpq_silu_mul_quantize_mx_packed(gates[i].data_ptr(), cols, ups[i].data_ptr(), cols, rows, cols, 0, 128,
+                                                 norm, None, pc.data_ptr(), ps.data_ptr(), 0, stream)
+        if st != 0:
+            _engine.check(st, "bench silu_mul_quantize")
+
+    wall, ev = time_kernel(torch, run_silu, n_buf, steps, warmup)
+    algo = rows * cols * (2 + 2 + 0.5 + 1.0 / 32)
+    out["silu_mul_quantize"] = {"workload": f"silu_mul_quantize_mx_packed_{rows}x{cols}_had128",
+                                "kernel_us": round(ev * 1e3, 2), "GB/s": round(algo / (ev * 1e-3) / 1e9, 1),
+                                "hbm_frac": round(algo / (ev * 1e-3) / 8e12, 4)}
+    return out
+
+
 def bench_linear(torch, fmt, m, n, k, g, steps, warmup, seed):
     """Quantize activations + W4A4 GEMM (the body of FPQuantLinear.forward) through the C ABI.
     Weights are quantized once outside the timed region; activations rotate through buffers."""
@@ -412,7 +472,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="comma list of workloads to run (for profiling one kernel): "
                     "nvfp4_quantize, mxfp4_quantize, mxfp4_linear_M2048, mxfp4_linear_M128, mxfp4_linear_M16, "
-                    "mxfp4_linear_M1, nvfp4_linear, mfma_ceiling, e2e_llama (whole-model forward, not part of the default run)")
+                    "mxfp4_linear_M1, nvfp4_linear, mfma_ceiling, fused_producers, e2e_llama (whole-model forward); the last "
+                    "three are not part of the default run")
     ap.add_argument("--e2e-layers", type=int, default=32, help="decoder layers of the --only e2e_llama model")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB device copy (known traffic) to scale rocprofv3 byte counters")
@@ -455,6 +516,8 @@ def main():
             out["e2e_llama"] = bench_e2e_llama(torch, layers=args.e2e_layers)
         if "mfma_ceiling" in only:
             out["mfma_ceiling"] = bench_mfma_ceiling(torch)
+        if "fused_producers" in only:
+            out["fused_producers"] = bench_fused_producers(torch, args.steps, args.warmup)
         print(json.dumps({"only": only, "steps": args.steps, "results": out}))
         return
 
