@@ -321,6 +321,29 @@ def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=
     finally:
         torch.set_default_dtype(old_dtype)
     model.eval()
+    sweep = ((1, 32), (8, 128), (16, 128), (64, 128), (prefill_batch, seq))   # (batch, sequence) prefill points
+
+    def prefill_sweep():
+        """Best-of-3 prefill milliseconds per (batch, seq) point: the reference's end-to-end plot is the ratio
+        of these between the bf16 and the MXFP4 model (assets/inference_speedup_*.png, batch x seq sweep)."""
+        res = {}
+        with torch.no_grad():
+            for b, sl in sweep:
+                ids = torch.randint(0, cfg.vocab_size, (b, sl), generator=torch.Generator().manual_seed(b * sl)).to(dev)
+                best = None
+                for rep in range(4):
+                    e0 = torch.cuda.Event(enable_timing=True)
+                    e1 = torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    model(input_ids=ids, use_cache=False, logits_to_keep=1)
+                    e1.record()
+                    torch.cuda.synchronize()
+                    if rep:
+                        best = e0.elapsed_time(e1) if best is None else min(best, e0.elapsed_time(e1))
+                res[f"{b}x{sl}"] = round(best, 3)
+        return res
+
+    bf16_ms = prefill_sweep()   # the unquantized model: nn.Linear in bf16 (hipBLASLt)
     qcfg = fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype.MXFP4, forward_method="abs_max",
                                   backward_dtype=fp_quant.FPQuantDtype.BF16, hadamard_group_size=128)
     fp_quant.replace_quantize_with_fp_quant_linear(model, qcfg)
@@ -396,12 +419,17 @@ def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=
                 torch.cuda.empty_cache()
 
     measure(out, True)
+    mx_ms = prefill_sweep()
     # the same model with the RMSNorms and the SiLU*up of every block fused into the quantizers that consume
     # them (one fused kernel instead of PyTorch's elementwise operators followed by a quantizer)
     from fp_quant.utils import fuse_producers
     fused = {"patched_modules": fuse_producers(model)}
     measure(fused, False)
     out["fused_producers"] = fused
+    fused_ms = prefill_sweep()
+    out["prefill_sweep_ms"] = {"bf16": bf16_ms, "mxfp4": mx_ms, "mxfp4_fused_producers": fused_ms,
+                               "speedup_vs_bf16": {k: round(bf16_ms[k] / mx_ms[k], 2) for k in bf16_ms},
+                               "speedup_vs_bf16_fused": {k: round(bf16_ms[k] / fused_ms[k], 2) for k in bf16_ms}}
     return out
 
 
