@@ -517,7 +517,6 @@ class QuantizedActivations:
 
 
 _shared_activations = {}   # device index -> QuantizedActivations of the latest call
-_capture_id = ctypes.c_ulonglong()
 
 
 def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: int):
@@ -527,7 +526,8 @@ def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: i
     copy of the scale (read once per buffer); an unrecognised rotation matrix only matches itself."""
     if not SHARE_ACT_QUANT:
         return None
-    _engine.check(_engine.lib().fpq_stream_capture_id(stream, ctypes.byref(_capture_id)), "fpq_stream_capture_id")
+    capture_id = ctypes.c_ulonglong()   # per call: host threads may run layers concurrently
+    _engine.check(_engine.lib().fpq_stream_capture_id(stream, ctypes.byref(capture_id)), "fpq_stream_capture_id")
     rot = (kind, norm, h.shape[0]) if kind != _engine.ROT_GENERAL else (kind, id(h), h._version)
     gs = None
     if act_global_scale is not None:
@@ -536,7 +536,7 @@ def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: i
     # the operand layout the GEMM will ask for is part of the key: the packed form can be made from the
     # row-major one but not the other way round
     want_packed = act_global_scale is None and packed_linear_eligible(x_shape[0], x_shape[1], "abs_max")
-    return (rot, gs, stream, _capture_id.value, tuple(x_shape), want_packed)
+    return (rot, gs, stream, capture_id.value, tuple(x_shape), want_packed)
 
 
 def _publish(qa: QuantizedActivations, src: torch.Tensor, key, keep) -> None:
