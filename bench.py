@@ -162,6 +162,22 @@ def bench_fused_producers(torch, steps, warmup):
     return out
 
 
+def bench_hbm_probe(torch, steps, warmup):
+    """What plain data movement reaches on this GPU, for judging the HBM-bound kernels: a device-to-device copy
+    (bytes read + bytes written per second) moving as many bytes as the NVFP4 quantize workload (86 MB) and at
+    256 MiB."""
+    dev = torch.device("cuda:0")
+    out = {}
+    for name, nbytes in (("copy_43MB", 43 << 20), ("copy_256MiB", 256 << 20)):
+        n_buf = max(2, (640 << 20) // nbytes)
+        src = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 256) for _ in range(n_buf)]
+        dst = [torch.empty_like(b) for b in src]
+        wall, ev = time_kernel(torch, lambda i: dst[i].copy_(src[i]), n_buf, steps, warmup)
+        out[name] = {"us": round(ev * 1e3, 2), "GB/s": round(2 * nbytes / (ev * 1e-3) / 1e9, 1)}
+        del src, dst
+    return out
+
+
 def bench_linear(torch, fmt, m, n, k, g, steps, warmup, seed):
     """Quantize activations + W4A4 GEMM (the body of FPQuantLinear.forward) through the C ABI.
     Weights are quantized once outside the timed region; activations rotate through buffers."""
@@ -500,8 +516,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="comma list of workloads to run (for profiling one kernel): "
                     "nvfp4_quantize, mxfp4_quantize, mxfp4_linear_M2048, mxfp4_linear_M128, mxfp4_linear_M16, "
-                    "mxfp4_linear_M1, nvfp4_linear, mfma_ceiling, fused_producers, e2e_llama (whole-model forward); the last "
-                    "three are not part of the default run")
+                    "mxfp4_linear_M1, nvfp4_linear, mfma_ceiling, hbm_probe, fused_producers, e2e_llama (whole-model "
+                    "forward); the last four are not part of the default run")
     ap.add_argument("--e2e-layers", type=int, default=32, help="decoder layers of the --only e2e_llama model")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB device copy (known traffic) to scale rocprofv3 byte counters")
@@ -544,6 +560,8 @@ def main():
             out["e2e_llama"] = bench_e2e_llama(torch, layers=args.e2e_layers)
         if "mfma_ceiling" in only:
             out["mfma_ceiling"] = bench_mfma_ceiling(torch)
+        if "hbm_probe" in only:
+            out["hbm_probe"] = bench_hbm_probe(torch, args.steps, args.warmup)
         if "fused_producers" in only:
             out["fused_producers"] = bench_fused_producers(torch, args.steps, args.warmup)
         print(json.dumps({"only": only, "steps": args.steps, "results": out}))
