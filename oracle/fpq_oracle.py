@@ -48,7 +48,6 @@ unpinned) have no fixtures in the reference: bit parity against QuTLASS itself i
 """
 from __future__ import annotations
 
-import math
 from typing import Optional, Tuple
 
 import numpy as np
