@@ -318,7 +318,8 @@ def bench_mfma_ceiling(torch, seed=4, iters=192):
     return out
 
 
-def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=(1, 32, 64), decode_steps=8):
+def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=(1, 32, 64), decode_steps=8,
+                    fmt="mxfp4"):
     """Forward passes of a random-weight Llama-3.1-8B-architecture model (transformers' LlamaForCausalLM) whose
     linears (all but lm_head) were replaced by MXFP4 FPQuantLinear with Hadamard-128: prefill tokens/s, decode
     tokens/s against a `seq`-token bf16 KV cache, and the share of GPU time spent inside the quantized linears
@@ -360,8 +361,9 @@ def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=
         return res
 
     bf16_ms = prefill_sweep()   # the unquantized model: nn.Linear in bf16 (hipBLASLt)
-    qcfg = fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype.MXFP4, forward_method="abs_max",
-                                  backward_dtype=fp_quant.FPQuantDtype.BF16, hadamard_group_size=128)
+    qcfg = fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype(fmt), forward_method="abs_max",
+                                  backward_dtype=fp_quant.FPQuantDtype.BF16,
+                                  hadamard_group_size=128 if fmt == "mxfp4" else 16)
     fp_quant.replace_quantize_with_fp_quant_linear(model, qcfg)
     qlinears = [m for m in model.modules() if isinstance(m, fp_quant.FPQuantLinear)]
     spans = []
@@ -400,7 +402,8 @@ def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=
             h.remove()
         return best, share
 
-    out = {"model": f"Llama-3.1-8B architecture, {layers} layers, random weights, MXFP4 W4A4 Hadamard-128",
+    out = {"model": f"Llama-3.1-8B architecture, {layers} layers, random weights, "
+                    + ("MXFP4 W4A4 Hadamard-128" if fmt == "mxfp4" else "NVFP4 W4A4 Hadamard-16"),
            "quantized_linears": len(qlinears)}
 
     def measure(out, with_share):
@@ -443,7 +446,7 @@ def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=
     measure(fused, False)
     out["fused_producers"] = fused
     fused_ms = prefill_sweep()
-    out["prefill_sweep_ms"] = {"bf16": bf16_ms, "mxfp4": mx_ms, "mxfp4_fused_producers": fused_ms,
+    out["prefill_sweep_ms"] = {"bf16": bf16_ms, fmt: mx_ms, fmt + "_fused_producers": fused_ms,
                                "speedup_vs_bf16": {k: round(bf16_ms[k] / mx_ms[k], 2) for k in bf16_ms},
                                "speedup_vs_bf16_fused": {k: round(bf16_ms[k] / fused_ms[k], 2) for k in bf16_ms}}
     return out
@@ -519,6 +522,7 @@ def main():
                     "mxfp4_linear_M1, nvfp4_linear, mfma_ceiling, hbm_probe, fused_producers, e2e_llama (whole-model "
                     "forward); the last four are not part of the default run")
     ap.add_argument("--e2e-layers", type=int, default=32, help="decoder layers of the --only e2e_llama model")
+    ap.add_argument("--e2e-format", default="mxfp4", choices=("mxfp4", "nvfp4"), help="format of the --only e2e_llama model")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB device copy (known traffic) to scale rocprofv3 byte counters")
     args = ap.parse_args()
@@ -557,7 +561,7 @@ def main():
             out["nvfp4_linear"] = bench_linear(torch, "nvfp4", 4096, 24576, 4096, 16, max(10, args.steps // 10),
                                                max(2, args.warmup // 10), seed=3)
         if "e2e_llama" in only:
-            out["e2e_llama"] = bench_e2e_llama(torch, layers=args.e2e_layers)
+            out["e2e_llama"] = bench_e2e_llama(torch, layers=args.e2e_layers, fmt=args.e2e_format)
         if "mfma_ceiling" in only:
             out["mfma_ceiling"] = bench_mfma_ceiling(torch)
         if "hbm_probe" in only:
