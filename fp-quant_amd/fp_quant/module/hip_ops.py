@@ -22,6 +22,17 @@ HAS_HIP_ENGINE = _engine.available()
 # zero-nibble policy used by the operators (see include/fpq.h)
 ZERO_NIBBLE_POLICY = _engine.ZERO_REFERENCE
 
+def _version(t: torch.Tensor) -> int:
+    """The tensor's in-place modification counter, the key of everything cached per tensor.  Tensors
+    created under torch.inference_mode() have none: they get a constant (parameters and buffers made
+    that way are not written to afterwards; activations made that way are never shared, see
+    _sharing_key)."""
+    try:
+        return t._version
+    except RuntimeError:
+        return -1
+
+
 def _sylvester(g: int) -> torch.Tensor:
     idx = torch.arange(g)
     anded = idx[:, None] & idx[None, :]
@@ -36,7 +47,7 @@ def classify_rotation(h: torch.Tensor) -> Tuple[int, float]:
     itself (with its version counter), so the one device->host copy it needs happens once per
     matrix and can never be confused with another tensor that later reuses the same memory."""
     hit = getattr(h, "_fpq_rotation", None)
-    if hit is not None and hit[0] == h._version:
+    if hit is not None and hit[0] == _version(h):
         return hit[1], hit[2]
     g = h.shape[0]
     if h.dim() != 2 or h.shape[1] != g:
@@ -55,7 +66,7 @@ def classify_rotation(h: torch.Tensor) -> Tuple[int, float]:
             if torch.equal(hf, signed[:, torch.argsort(changes)]):
                 kind, norm = _engine.ROT_GSR, n
     try:
-        h._fpq_rotation = (h._version, kind, norm)
+        h._fpq_rotation = (_version(h), kind, norm)
     except AttributeError:  # objects that refuse attributes: classify again next time
         pass
     return kind, norm
@@ -67,11 +78,11 @@ def as_bf16(h: torch.Tensor) -> torch.Tensor:
     if h.dtype == torch.bfloat16 and h.is_contiguous():
         return h
     hit = getattr(h, "_fpq_bf16", None)
-    if hit is not None and hit[0] == h._version:
+    if hit is not None and hit[0] == _version(h):
         return hit[1]
     conv = h.detach().to(torch.bfloat16).contiguous()
     try:
-        h._fpq_bf16 = (h._version, conv)
+        h._fpq_bf16 = (_version(h), conv)
     except AttributeError:
         pass
     return conv
@@ -319,7 +330,7 @@ def nv_packed_eligible(m: int, n: int, k: int) -> bool:
 
 def packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """Packed copy of a weight, cached on the code tensor until either tensor is written to."""
-    key = (wq.data_ptr(), wq._version, ws.data_ptr(), ws._version, tuple(wq.shape), nvfp4)
+    key = (wq.data_ptr(), _version(wq), ws.data_ptr(), _version(ws), tuple(wq.shape), nvfp4)
     hit = getattr(wq, "_fpq_packed", None)
     if hit is not None and hit[0] == key:
         return hit[1], hit[2]
@@ -471,7 +482,7 @@ def cached_on(t: torch.Tensor, slot: str, key, make):
 def linear_alpha(weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor) -> torch.Tensor:
     """fp32 one-element `1 / (wgs * ags)` evaluated in the buffers' dtype as the reference does
     (linear_fns.py:505; bf16 buffers round 1/9 to 0.111328125), cached until a buffer changes."""
-    key = (weight_global_scale._version, act_global_scale._version, act_global_scale.data_ptr(),
+    key = (_version(weight_global_scale), _version(act_global_scale), act_global_scale.data_ptr(),
            weight_global_scale.data_ptr())
     return cached_on(weight_global_scale, "_fpq_alpha", key,
                      lambda: (1.0 / (weight_global_scale * act_global_scale)).float().reshape(1).contiguous())
@@ -480,7 +491,7 @@ def linear_alpha(weight_global_scale: torch.Tensor, act_global_scale: torch.Tens
 def as_f32_scalar(t: torch.Tensor) -> torch.Tensor:
     if t.dtype == torch.float32 and t.is_contiguous():
         return t
-    return cached_on(t, "_fpq_f32", (t._version, t.data_ptr()), lambda: t.detach().float().contiguous())
+    return cached_on(t, "_fpq_f32", (_version(t), t.data_ptr()), lambda: t.detach().float().contiguous())
 
 
 # Several layers that consume one tensor (q/k/v projections, gate/up projections) would rotate and
@@ -524,14 +535,14 @@ def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: i
     None when nothing may be shared.  Layers own separate but equal rotation and global-scale
     buffers, so those are compared by value: (kind, norm, size) of a recognised rotation, the host
     copy of the scale (read once per buffer); an unrecognised rotation matrix only matches itself."""
-    if not SHARE_ACT_QUANT:
-        return None
+    if not SHARE_ACT_QUANT or torch.is_inference_mode_enabled():
+        return None   # in inference mode in-place writes to the source could not be noticed
     capture_id = ctypes.c_ulonglong()   # per call: host threads may run layers concurrently
     _engine.check(_engine.lib().fpq_stream_capture_id(stream, ctypes.byref(capture_id)), "fpq_stream_capture_id")
-    rot = (kind, norm, h.shape[0]) if kind != _engine.ROT_GENERAL else (kind, id(h), h._version)
+    rot = (kind, norm, h.shape[0]) if kind != _engine.ROT_GENERAL else (kind, id(h), _version(h))
     gs = None
     if act_global_scale is not None:
-        gs = cached_on(act_global_scale, "_fpq_host", (act_global_scale._version, act_global_scale.data_ptr()),
+        gs = cached_on(act_global_scale, "_fpq_host", (_version(act_global_scale), act_global_scale.data_ptr()),
                        lambda: float(act_global_scale))
     # the operand layout the GEMM will ask for is part of the key: the packed form can be made from the
     # row-major one but not the other way round
@@ -540,13 +551,13 @@ def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: i
 
 
 def _publish(qa: QuantizedActivations, src: torch.Tensor, key, keep) -> None:
-    qa.ref, qa.version, qa.key, qa.keep = weakref.ref(src), src._version, key, keep
+    qa.ref, qa.version, qa.key, qa.keep = weakref.ref(src), _version(src), key, keep
     _shared_activations[src.device.index] = qa
 
 
 def _lookup(src: torch.Tensor, key) -> Optional[QuantizedActivations]:
     qa = _shared_activations.get(src.device.index)
-    if qa is not None and qa.ref() is src and qa.version == src._version and qa.key == key:
+    if qa is not None and qa.ref() is src and qa.version == _version(src) and qa.key == key:
         return qa
     return None
 

@@ -268,3 +268,17 @@ def test_fused_block_is_graph_capturable(fmt, g, m):
         eager = step(static_x)
         again = step(static_x.clone())
         assert torch.equal(eager[0], again[0]) and torch.equal(eager[1], again[1])
+
+
+def test_fused_llama_in_inference_mode():
+    """Under torch.inference_mode() the fused modules still run (the MLP hands its quantized input
+    over directly; the norm's quantization is not shared) and give the no_grad logits."""
+    from fp_quant.utils import fuse_producers
+    model = _tiny_llama("mxfp4", 128, seed=5)
+    fuse_producers(model)
+    ids = torch.randint(0, 128, (2, 40), generator=torch.Generator().manual_seed(3)).cuda()
+    with torch.no_grad():
+        want = model(ids).logits
+    with torch.inference_mode():
+        got = model(ids).logits
+    assert torch.equal(got, want)

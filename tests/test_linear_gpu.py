@@ -320,3 +320,35 @@ def test_layers_sharing_an_input_share_its_quantization(fmt, g, m):
         layers[0](x2)
         got5 = scaled(x2)
         assert torch.equal(got5, want5) and not torch.equal(got5, unshared(x2, [_quantized_linear(fmt, g, k, 256, 8)])[0])
+
+
+@pytest.mark.parametrize("fmt,g,m", [("mxfp4", 128, 3), ("mxfp4", 32, 200), ("nvfp4", 16, 70)])
+def test_inference_mode(fmt, g, m):
+    """torch.inference_mode(): tensors made there carry no version counter, so nothing is cached on or
+    shared through them; results equal the no_grad ones, also for a layer built inside the mode."""
+    from fp_quant.module import hip_ops
+    lin = _quantized_linear(fmt, g, 512, 256, 21, bias=True)
+    other = _quantized_linear(fmt, g, 512, 128, 22)
+    x = torch.randn(m, 512, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        want, want_other = lin(x), other(x)
+    with torch.inference_mode():
+        hip_ops._shared_activations.clear()
+        xi = x * 1.0                                   # an inference tensor
+        assert xi.is_inference()
+        got, got_other = lin(xi), other(xi)
+        assert not hip_ops._shared_activations         # nothing shared: writes to xi could not be noticed
+        xi.mul_(2.0)
+        twice = lin(xi)
+    assert torch.equal(got, want) and torch.equal(got_other, want_other)
+    with torch.no_grad():
+        assert torch.equal(twice, lin(x * 2.0))
+    with torch.inference_mode():
+        import fp_quant
+        torch.manual_seed(21)
+        inner = fp_quant.FPQuantLinear(512, 256, _cfg(fmt, g), bias=True, device="cuda", dtype=torch.bfloat16)
+        inner.weight.data.normal_(0, 0.02)
+        inner.bias.data.normal_()
+        inner.pre_forward()
+        assert inner.qweight.is_inference()
+        assert torch.equal(inner(x), want) and torch.equal(inner(x), want)
