@@ -92,6 +92,16 @@ def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+# the current stream's handle without building a torch.cuda.Stream object (several microseconds per call)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _current_stream(device_index: int) -> int:
+    if _raw_stream is not None:
+        return _raw_stream(device_index)
+    return torch.cuda.current_stream().cuda_stream
+
+
 def _require_cuda(*tensors: torch.Tensor) -> None:
     for t in tensors:
         if not t.is_cuda:
@@ -508,10 +518,12 @@ SHARE_ACT_QUANT = os.environ.get("FPQ_SHARE_ACT_QUANT", "1") != "0"
 class QuantizedActivations:
     """Rotated and quantized activations of one [m, k] tensor, in whichever operand layouts have
     been asked for so far (row-major codes/scales, packed MXFP4, packed NVFP4)."""
-    __slots__ = ("m", "k", "nvfp4", "ref", "version", "key", "keep", "mx_packed", "row_major", "nv_packed")
+    __slots__ = ("m", "k", "nvfp4", "packed_gemm", "ref", "version", "key", "keep", "mx_packed", "row_major",
+                 "nv_packed")
 
-    def __init__(self, m: int, k: int, nvfp4: bool):
+    def __init__(self, m: int, k: int, nvfp4: bool, packed_gemm: bool):
         self.m, self.k, self.nvfp4 = m, k, nvfp4
+        self.packed_gemm = packed_gemm   # MXFP4: the GEMM runs on packed operands (decided once per call)
         self.ref = self.key = self.keep = None
         self.version = 0
         self.mx_packed = self.row_major = self.nv_packed = None
@@ -530,7 +542,7 @@ class QuantizedActivations:
 _shared_activations = {}   # device index -> QuantizedActivations of the latest call
 
 
-def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: int):
+def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: int, want_packed: bool):
     """What two calls must agree on, besides the source tensor, to share quantized activations, or
     None when nothing may be shared.  Layers own separate but equal rotation and global-scale
     buffers, so those are compared by value: (kind, norm, size) of a recognised rotation, the host
@@ -546,7 +558,6 @@ def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: i
                        lambda: float(act_global_scale))
     # the operand layout the GEMM will ask for is part of the key: the packed form can be made from the
     # row-major one but not the other way round
-    want_packed = act_global_scale is None and packed_linear_eligible(x_shape[0], x_shape[1], "abs_max")
     return (rot, gs, stream, capture_id.value, tuple(x_shape), want_packed)
 
 
@@ -563,15 +574,16 @@ def _lookup(src: torch.Tensor, key) -> Optional[QuantizedActivations]:
 
 
 def quantize_activations(x_flat: torch.Tensor, h: torch.Tensor, kind: int, norm: float,
-                         act_global_scale: Optional[torch.Tensor], nvfp4: bool, stream: int) -> QuantizedActivations:
+                         act_global_scale: Optional[torch.Tensor], nvfp4: bool, stream: int,
+                         want_packed: bool) -> QuantizedActivations:
     """Rotate and quantize bf16 [m, k]: MXFP4 straight into the packed layout when the packed GEMM will
     run, row-major otherwise (NVFP4 always; its packed form is made on demand)."""
     lib = _engine.lib()
     m, k = x_flat.shape
     dev = x_flat.device
     g = h.shape[0]
-    qa = QuantizedActivations(m, k, nvfp4)
-    if not nvfp4 and packed_linear_eligible(m, k, "abs_max"):
+    qa = QuantizedActivations(m, k, nvfp4, want_packed)
+    if want_packed:
         pc = torch.empty(lib.fpq_packed_codes_bytes(m, k), dtype=torch.uint8, device=dev)
         ps = torch.empty(lib.fpq_packed_scales_bytes(m, k), dtype=torch.uint8, device=dev)
         st = lib.fpq_quantize_mx_packed(x_flat.data_ptr(), m, k, kind, g, norm, pc.data_ptr(), ps.data_ptr(),
@@ -622,7 +634,7 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
                                ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
         _engine.check(st, "fpq_gemm_nvf4")
         return y
-    if packed_linear_eligible(m, k, "abs_max"):
+    if qa.packed_gemm:
         pc, ps = qa.packed()
         wp, wsp = packed_weight(wq, ws)
         st = lib.fpq_gemm_mxf4_packed(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(), alpha.data_ptr(),
@@ -650,16 +662,17 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
     if torch.cuda.current_device() != dev.index:
         with torch.cuda.device(dev):
             return linear_w4a4(x_flat, hadamard_matrix, wq, ws, alpha, act_global_scale, bias, nvfp4, shared_source)
-    stream = torch.cuda.current_stream().cuda_stream
+    stream = _current_stream(dev.index)
     h = as_bf16(hadamard_matrix)
     kind, norm = classify_rotation(h)
+    want_packed = not nvfp4 and packed_linear_eligible(x_flat.shape[0], x_flat.shape[1], "abs_max")
     qa = key = None
     if shared_source is not None:
-        key = _sharing_key(x_flat.shape, h, kind, norm, act_global_scale if nvfp4 else None, stream)
+        key = _sharing_key(x_flat.shape, h, kind, norm, act_global_scale if nvfp4 else None, stream, want_packed)
         if key is not None:
             qa = _lookup(shared_source, key)
     if qa is None:
-        qa = quantize_activations(x_flat, h, kind, norm, act_global_scale, nvfp4, stream)
+        qa = quantize_activations(x_flat, h, kind, norm, act_global_scale, nvfp4, stream, want_packed)
         if key is not None:
             _publish(qa, shared_source, key, h)
     return linear_on(qa, wq, ws, alpha, bias, stream)
@@ -676,7 +689,8 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
     lib = _engine.lib()
     group = 16 if nvfp4 else 32
     optr = out.data_ptr() if out is not None else None
-    if not nvfp4 and packed_linear_eligible(rows, cols, "abs_max"):
+    want_packed = not nvfp4 and packed_linear_eligible(rows, cols, "abs_max")
+    if want_packed:
         # straight into the operand layout of the packed GEMM (streaming kernel)
         pc = torch.empty(lib.fpq_packed_codes_bytes(rows, cols), dtype=torch.uint8, device=dev)
         ps = torch.empty(lib.fpq_packed_scales_bytes(rows, cols), dtype=torch.uint8, device=dev)
@@ -685,7 +699,7 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
         if st == _engine.E_UNSUPPORTED:
             return None
         _engine.check(st, f"fpq_{entry}_quantize_mx_packed")
-        qa = QuantizedActivations(rows, cols, nvfp4)
+        qa = QuantizedActivations(rows, cols, nvfp4, True)
         qa.mx_packed = (pc, ps)
         return qa
     codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=dev)
@@ -699,7 +713,7 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
     if st == _engine.E_UNSUPPORTED:
         return None
     _engine.check(st, f"fpq_{entry}_quantize")
-    qa = QuantizedActivations(rows, cols, nvfp4)
+    qa = QuantizedActivations(rows, cols, nvfp4, False)
     qa.row_major = (codes, scales)
     return qa
 
@@ -718,7 +732,7 @@ def rmsnorm_quantize(x: torch.Tensor, weight: torch.Tensor, eps: float, hadamard
         return None
     dev = x.device
     with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream().cuda_stream
+        stream = _current_stream(dev.index)
         h = as_bf16(hadamard_matrix)
         kind, norm = classify_rotation(h)
         if kind not in (_engine.ROT_HADAMARD, _engine.ROT_IDENTITY) or cols % max(h.shape[0], 32) != 0:
@@ -734,7 +748,7 @@ def rmsnorm_quantize(x: torch.Tensor, weight: torch.Tensor, eps: float, hadamard
         if qa is None:
             return None
         y = y.view(x.shape)
-        key = _sharing_key(x_flat.shape, h, kind, norm, act_global_scale if nvfp4 else None, stream)
+        key = _sharing_key(x_flat.shape, h, kind, norm, act_global_scale if nvfp4 else None, stream, qa.packed_gemm)
         if key is not None:
             _publish(qa, y, key, h)
     return y
@@ -752,7 +766,7 @@ def silu_mul_quantize(gate: torch.Tensor, up: torch.Tensor, hadamard_matrix: tor
         return None
     dev = gate.device
     with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream().cuda_stream
+        stream = _current_stream(dev.index)
         h = as_bf16(hadamard_matrix)
         kind, norm = classify_rotation(h)
         if kind not in (_engine.ROT_HADAMARD, _engine.ROT_IDENTITY) or cols % max(h.shape[0], 32) != 0:

@@ -176,7 +176,7 @@ class FPQuantLinear(nn.Module):
         fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16 and bias.is_contiguous()) else None
         with torch.cuda.device(self.qweight.device):
             y = hip_ops.linear_on(activations, self.qweight, self.scales, alpha, fused_bias,
-                                  torch.cuda.current_stream().cuda_stream)
+                                  hip_ops._current_stream(self.qweight.device.index))
         y = y.unflatten(dim=0, sizes=tuple(leading_shape))
         if bias is not None and fused_bias is None:
             y += bias
