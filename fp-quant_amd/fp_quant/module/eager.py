@@ -1,0 +1,334 @@
+"""The eager (non-traced) body of FPQuantLinear.forward and what hangs off it.
+
+* `linear_w4a4`: activation rotate+quantize and W4A4 GEMM of one linear with as little host work
+  as possible (same kernels and results as the `fp_quant::*` operators of hip_ops, which tracing
+  uses; the reference's counterpart is FPQuant4x16NoMasterFn.forward,
+  inference_lib/src/fp_quant/module/linear_fns.py:482-534).
+* `QuantizedActivations` and the sharing slot: layers that consume the same tensor quantize it once
+  (the reference keeps one activation quantizer per such group, src/utils/llama_utils.py:30,103).
+* `rmsnorm_quantize`, `silu_mul_quantize`: the quantizers fused with the producer of their input.
+"""
+import ctypes
+import os
+import weakref
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _engine
+from .hip_ops import (
+    ZERO_NIBBLE_POLICY,
+    _current_stream,
+    _version,
+    as_bf16,
+    classify_rotation,
+    nv_packed_eligible,
+    pack_mxf4,
+    pack_nvf4,
+    packed_linear_eligible,
+    packed_weight,
+    quantize_mx_packed,
+)
+
+
+def cached_on(t: torch.Tensor, slot: str, key, make):
+    """`make()` remembered on tensor `t` under attribute `slot` while `key` stays the same."""
+    hit = getattr(t, slot, None)
+    if hit is not None and hit[0] == key:
+        return hit[1]
+    val = make()
+    try:
+        setattr(t, slot, (key, val))
+    except (AttributeError, RuntimeError):
+        pass
+    return val
+
+
+def linear_alpha(weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor) -> torch.Tensor:
+    """fp32 one-element `1 / (wgs * ags)` evaluated in the buffers' dtype as the reference does
+    (linear_fns.py:505; bf16 buffers round 1/9 to 0.111328125), cached until a buffer changes."""
+    key = (_version(weight_global_scale), _version(act_global_scale), act_global_scale.data_ptr(),
+           weight_global_scale.data_ptr())
+    return cached_on(weight_global_scale, "_fpq_alpha", key,
+                     lambda: (1.0 / (weight_global_scale * act_global_scale)).float().reshape(1).contiguous())
+
+
+def as_f32_scalar(t: torch.Tensor) -> torch.Tensor:
+    if t.dtype == torch.float32 and t.is_contiguous():
+        return t
+    return cached_on(t, "_fpq_f32", (_version(t), t.data_ptr()), lambda: t.detach().float().contiguous())
+
+
+# Several layers that consume one tensor (q/k/v projections, gate/up projections) would rotate and
+# quantize it once each.  The quantized activations of the latest call are kept per device and reused
+# while the next call passes the very same tensor object, unmodified (its version counter), with an
+# equal rotation and global scale, on the same stream and in the same graph capture (or both outside
+# any: work recorded during a capture has not run when the capture ends).  The source is held weakly,
+# so a freed tensor whose address is reused can never match.  Producers fused with the quantizer
+# (rmsnorm_quantize, silu_mul_quantize) leave their result in the same slot for the layers that
+# follow.  FPQ_SHARE_ACT_QUANT=0 turns the sharing off.
+SHARE_ACT_QUANT = os.environ.get("FPQ_SHARE_ACT_QUANT", "1") != "0"
+
+
+class QuantizedActivations:
+    """Rotated and quantized activations of one [m, k] tensor, in whichever operand layouts have
+    been asked for so far (row-major codes/scales, packed MXFP4, packed NVFP4)."""
+    __slots__ = ("m", "k", "nvfp4", "packed_gemm", "ref", "version", "key", "keep", "mx_packed", "row_major",
+                 "nv_packed")
+
+    def __init__(self, m: int, k: int, nvfp4: bool, packed_gemm: bool):
+        self.m, self.k, self.nvfp4 = m, k, nvfp4
+        self.packed_gemm = packed_gemm   # MXFP4: the GEMM runs on packed operands (decided once per call)
+        self.ref = self.key = self.keep = None
+        self.version = 0
+        self.mx_packed = self.row_major = self.nv_packed = None
+
+    def packed(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Codes and scales in the packed GEMM layout (re-tiled from the row-major ones if need be)."""
+        if self.nvfp4:
+            if self.nv_packed is None:
+                self.nv_packed = pack_nvf4(self.row_major[0], self.row_major[1], self.m, self.k)
+            return self.nv_packed
+        if self.mx_packed is None:
+            self.mx_packed = pack_mxf4(self.row_major[0], self.row_major[1], self.m, self.k)
+        return self.mx_packed
+
+
+_shared_activations = {}   # device index -> QuantizedActivations of the latest call
+
+
+def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: int, want_packed: bool):
+    """What two calls must agree on, besides the source tensor, to share quantized activations, or
+    None when nothing may be shared.  Layers own separate but equal rotation and global-scale
+    buffers, so those are compared by value: (kind, norm, size) of a recognised rotation, the host
+    copy of the scale (read once per buffer); an unrecognised rotation matrix only matches itself."""
+    if not SHARE_ACT_QUANT or torch.is_inference_mode_enabled():
+        return None   # in inference mode in-place writes to the source could not be noticed
+    capture_id = ctypes.c_ulonglong()   # per call: host threads may run layers concurrently
+    _engine.check(_engine.lib().fpq_stream_capture_id(stream, ctypes.byref(capture_id)), "fpq_stream_capture_id")
+    rot = (kind, norm, h.shape[0]) if kind != _engine.ROT_GENERAL else (kind, id(h), _version(h))
+    gs = None
+    if act_global_scale is not None:
+        gs = cached_on(act_global_scale, "_fpq_host", (_version(act_global_scale), act_global_scale.data_ptr()),
+                       lambda: float(act_global_scale))
+    # the operand layout the GEMM will ask for is part of the key: the packed form can be made from the
+    # row-major one but not the other way round
+    return (rot, gs, stream, capture_id.value, tuple(x_shape), want_packed)
+
+
+def _publish(qa: QuantizedActivations, src: torch.Tensor, key, keep) -> None:
+    qa.ref, qa.version, qa.key, qa.keep = weakref.ref(src), _version(src), key, keep
+    _shared_activations[src.device.index] = qa
+
+
+def _lookup(src: torch.Tensor, key) -> Optional[QuantizedActivations]:
+    qa = _shared_activations.get(src.device.index)
+    if qa is not None and qa.ref() is src and qa.version == _version(src) and qa.key == key:
+        return qa
+    return None
+
+
+def quantize_activations(x_flat: torch.Tensor, h: torch.Tensor, kind: int, norm: float,
+                         act_global_scale: Optional[torch.Tensor], nvfp4: bool, stream: int,
+                         want_packed: bool) -> QuantizedActivations:
+    """Rotate and quantize bf16 [m, k]: MXFP4 straight into the packed layout when the packed GEMM will
+    run, row-major otherwise (NVFP4 always; its packed form is made on demand)."""
+    lib = _engine.lib()
+    m, k = x_flat.shape
+    dev = x_flat.device
+    g = h.shape[0]
+    qa = QuantizedActivations(m, k, nvfp4, want_packed)
+    if want_packed:
+        pc = torch.empty(lib.fpq_packed_codes_bytes(m, k), dtype=torch.uint8, device=dev)
+        ps = torch.empty(lib.fpq_packed_scales_bytes(m, k), dtype=torch.uint8, device=dev)
+        st = lib.fpq_quantize_mx_packed(x_flat.data_ptr(), m, k, kind, g, norm, pc.data_ptr(), ps.data_ptr(),
+                                        ZERO_NIBBLE_POLICY, stream)
+        if st == _engine.E_UNSUPPORTED:
+            pc, ps = quantize_mx_packed(x_flat, h)
+        else:
+            _engine.check(st, "fpq_quantize_mx_packed")
+        qa.mx_packed = (pc, ps)
+        return qa
+    group = 16 if nvfp4 else 32
+    codes = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
+    scales = torch.empty(m, k // group, dtype=torch.uint8, device=dev)
+    if nvfp4:
+        gs = as_f32_scalar(act_global_scale)
+        st = lib.fpq_quantize_nv(x_flat.data_ptr(), m, k, kind, g, norm, h.data_ptr(), gs.data_ptr(),
+                                 codes.data_ptr(), scales.data_ptr(), m, k // group, ZERO_NIBBLE_POLICY, stream)
+        _engine.check(st, "fpq_quantize_nv")
+    else:
+        st = lib.fpq_quantize_mx(x_flat.data_ptr(), m, k, kind, g, norm, h.data_ptr(), codes.data_ptr(),
+                                 scales.data_ptr(), m, k // group, ZERO_NIBBLE_POLICY, stream)
+        _engine.check(st, "fpq_quantize_mx")
+    qa.row_major = (codes, scales)
+    return qa
+
+
+def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alpha: torch.Tensor,
+              bias: Optional[torch.Tensor], stream: int) -> torch.Tensor:
+    """bf16 [m, n] = alpha * dq(activations) @ dq(w).T (+ bias) on quantized activations, with the
+    kernel and operand layout the shape calls for."""
+    lib = _engine.lib()
+    m, k = qa.m, qa.k
+    n = wq.shape[0]
+    if wq.shape[1] * 2 != k:
+        raise ValueError(f"inner dimensions differ: x has K={k}, w has K={wq.shape[1] * 2}")
+    y = torch.empty(m, n, dtype=torch.bfloat16, device=wq.device)
+    b_ptr = bias.data_ptr() if bias is not None else None
+    if qa.nvfp4:
+        if nv_packed_eligible(m, n, k):
+            xp, xsp = qa.packed()
+            wp, wsp = packed_weight(wq, ws, True)
+            st = lib.fpq_gemm_nvf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
+                                          alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
+            _engine.check(st, "fpq_gemm_nvf4_packed")
+            return y
+        codes, scales = qa.row_major
+        st = lib.fpq_gemm_nvf4(codes.data_ptr(), scales.data_ptr(), scales.shape[-1], wq.data_ptr(), ws.data_ptr(),
+                               ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
+        _engine.check(st, "fpq_gemm_nvf4")
+        return y
+    if qa.packed_gemm:
+        pc, ps = qa.packed()
+        wp, wsp = packed_weight(wq, ws)
+        st = lib.fpq_gemm_mxf4_packed(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(), alpha.data_ptr(),
+                                      b_ptr, y.data_ptr(), m, n, k, stream)
+        _engine.check(st, "fpq_gemm_mxf4_packed")
+        return y
+    codes, scales = qa.row_major
+    st = lib.fpq_gemm_mxf4(codes.data_ptr(), scales.data_ptr(), scales.shape[-1], wq.data_ptr(), ws.data_ptr(),
+                           ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
+    _engine.check(st, "fpq_gemm_mxf4")
+    return y
+
+
+def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.Tensor, ws: torch.Tensor,
+                alpha: torch.Tensor, act_global_scale: torch.Tensor, bias: Optional[torch.Tensor],
+                nvfp4: bool, shared_source: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Activation rotate+quantize and W4A4 GEMM of one linear with as little host work as possible:
+    the eager (non-traced) body of FPQuantLinear.forward.  Same kernels and results as the
+    fused_quantize_* and matmul_* operators; `x_flat` bf16 [M, K] contiguous on the GPU, `alpha`
+    fp32 [1], `bias` bf16 [N] or None.  `shared_source` is the tensor object `x_flat` was derived
+    from: consecutive calls with the same, unmodified object reuse its quantized form."""
+    if not x_flat.is_cuda:
+        raise ValueError("fp_quant HIP operators need tensors on a GPU; there is no CPU path")
+    dev = x_flat.device
+    if torch.cuda.current_device() != dev.index:
+        with torch.cuda.device(dev):
+            return linear_w4a4(x_flat, hadamard_matrix, wq, ws, alpha, act_global_scale, bias, nvfp4, shared_source)
+    stream = _current_stream(dev.index)
+    h = as_bf16(hadamard_matrix)
+    kind, norm = classify_rotation(h)
+    want_packed = not nvfp4 and packed_linear_eligible(x_flat.shape[0], x_flat.shape[1], "abs_max")
+    qa = key = None
+    if shared_source is not None:
+        key = _sharing_key(x_flat.shape, h, kind, norm, act_global_scale if nvfp4 else None, stream, want_packed)
+        if key is not None:
+            qa = _lookup(shared_source, key)
+    if qa is None:
+        qa = quantize_activations(x_flat, h, kind, norm, act_global_scale, nvfp4, stream, want_packed)
+        if key is not None:
+            _publish(qa, shared_source, key, h)
+    return linear_on(qa, wq, ws, alpha, bias, stream)
+
+
+### Quantizers fused with the producer of their input
+
+
+def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tensor, kind: int, norm: float,
+                    act_global_scale: Optional[torch.Tensor], nvfp4: bool, out: Optional[torch.Tensor],
+                    stream: int, dev) -> Optional[QuantizedActivations]:
+    """Common tail of the fused producers: allocate row-major codes/scales and call
+    fpq_<entry>_quantize_{mx,nv}; None if the library has no fused kernel for this rotation."""
+    lib = _engine.lib()
+    group = 16 if nvfp4 else 32
+    optr = out.data_ptr() if out is not None else None
+    want_packed = not nvfp4 and packed_linear_eligible(rows, cols, "abs_max")
+    if want_packed:
+        # straight into the operand layout of the packed GEMM (streaming kernel)
+        pc = torch.empty(lib.fpq_packed_codes_bytes(rows, cols), dtype=torch.uint8, device=dev)
+        ps = torch.empty(lib.fpq_packed_scales_bytes(rows, cols), dtype=torch.uint8, device=dev)
+        st = getattr(lib, f"fpq_{entry}_quantize_mx_packed")(*head, rows, cols, kind, h.shape[0], norm, optr,
+                                                             pc.data_ptr(), ps.data_ptr(), ZERO_NIBBLE_POLICY, stream)
+        if st == _engine.E_UNSUPPORTED:
+            return None
+        _engine.check(st, f"fpq_{entry}_quantize_mx_packed")
+        qa = QuantizedActivations(rows, cols, nvfp4, True)
+        qa.mx_packed = (pc, ps)
+        return qa
+    codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=dev)
+    scales = torch.empty(rows, cols // group, dtype=torch.uint8, device=dev)
+    tail = (optr, codes.data_ptr(), scales.data_ptr(), rows, cols // group, ZERO_NIBBLE_POLICY, stream)
+    if nvfp4:
+        gs = as_f32_scalar(act_global_scale)
+        st = getattr(lib, f"fpq_{entry}_quantize_nv")(*head, rows, cols, kind, h.shape[0], norm, gs.data_ptr(), *tail)
+    else:
+        st = getattr(lib, f"fpq_{entry}_quantize_mx")(*head, rows, cols, kind, h.shape[0], norm, *tail)
+    if st == _engine.E_UNSUPPORTED:
+        return None
+    _engine.check(st, f"fpq_{entry}_quantize")
+    qa = QuantizedActivations(rows, cols, nvfp4, False)
+    qa.row_major = (codes, scales)
+    return qa
+
+
+def rmsnorm_quantize(x: torch.Tensor, weight: torch.Tensor, eps: float, hadamard_matrix: torch.Tensor,
+                     act_global_scale: Optional[torch.Tensor], nvfp4: bool) -> Optional[torch.Tensor]:
+    """RMSNorm of bf16 `x` over its last dimension, y = bf16(weight * bf16(x / rms)), in one pass
+    that also leaves y rotated and quantized for the layers that consume it next (they find it
+    through the sharing slot when called with the returned tensor).  None if this rotation has no
+    fused kernel; the caller then normalises as usual."""
+    if not x.is_cuda or x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        return None
+    x_flat = x.contiguous().view(-1, x.shape[-1])
+    rows, cols = x_flat.shape
+    if rows == 0 or weight.numel() != cols:
+        return None
+    dev = x.device
+    with torch.cuda.device(dev):
+        stream = _current_stream(dev.index)
+        h = as_bf16(hadamard_matrix)
+        kind, norm = classify_rotation(h)
+        if kind not in (_engine.ROT_HADAMARD, _engine.ROT_IDENTITY) or cols % max(h.shape[0], 32) != 0:
+            return None
+        lib = _engine.lib()
+        inv = torch.empty(rows, dtype=torch.float32, device=dev)
+        _engine.check(lib.fpq_row_inv_rms(x_flat.data_ptr(), cols, rows, cols, eps, inv.data_ptr(), stream),
+                      "fpq_row_inv_rms")
+        y = torch.empty_like(x_flat)
+        w = weight.contiguous()
+        qa = _fused_quantize("rmsnorm", (x_flat.data_ptr(), cols, inv.data_ptr(), w.data_ptr()), rows, cols, h, kind,
+                             norm, act_global_scale, nvfp4, y, stream, dev)
+        if qa is None:
+            return None
+        y = y.view(x.shape)
+        key = _sharing_key(x_flat.shape, h, kind, norm, act_global_scale if nvfp4 else None, stream, qa.packed_gemm)
+        if key is not None:
+            _publish(qa, y, key, h)
+    return y
+
+
+def silu_mul_quantize(gate: torch.Tensor, up: torch.Tensor, hadamard_matrix: torch.Tensor,
+                      act_global_scale: Optional[torch.Tensor], nvfp4: bool) -> Optional[QuantizedActivations]:
+    """Quantized bf16(silu(gate)) * up without materialising the product; gate and up are bf16 with a
+    contiguous last dimension (two tensors, or two column halves of one).  None if not fusable."""
+    if (not gate.is_cuda or gate.dtype != torch.bfloat16 or up.dtype != torch.bfloat16 or gate.shape != up.shape
+            or gate.dim() != 2 or gate.stride(1) != 1 or up.stride(1) != 1):
+        return None
+    rows, cols = gate.shape
+    if rows == 0:
+        return None
+    dev = gate.device
+    with torch.cuda.device(dev):
+        stream = _current_stream(dev.index)
+        h = as_bf16(hadamard_matrix)
+        kind, norm = classify_rotation(h)
+        if kind not in (_engine.ROT_HADAMARD, _engine.ROT_IDENTITY) or cols % max(h.shape[0], 32) != 0:
+            return None
+        ld_g = gate.stride(0) if rows > 1 else cols
+        ld_u = up.stride(0) if rows > 1 else cols
+        if ld_g % 8 or ld_u % 8 or ld_g < cols or ld_u < cols or gate.data_ptr() % 16 or up.data_ptr() % 16:
+            return None
+        return _fused_quantize("silu_mul", (gate.data_ptr(), ld_g, up.data_ptr(), ld_u), rows, cols, h, kind, norm,
+                               act_global_scale, nvfp4, None, stream, dev)

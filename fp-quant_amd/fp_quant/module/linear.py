@@ -10,7 +10,7 @@ import torch
 from torch import nn
 
 from ..utils import FPQuantConfig, FPQuantDtype, validate_config
-from . import hip_ops
+from . import eager, hip_ops
 from .linear_fns import FPQuant4x16NoMasterFn, forward_quantize
 
 _SCALE_GROUP = {FPQuantDtype.MXFP4: 32, FPQuantDtype.NVFP4: 16}
@@ -170,12 +170,12 @@ class FPQuantLinear(nn.Module):
 
     def forward_quantized(self, activations, leading_shape) -> torch.Tensor:
         """The GEMM (+ bias) of `forward` on activations that a fused producer has already rotated and
-        quantized for this layer (`hip_ops.QuantizedActivations`); returns [*leading_shape, out]."""
-        alpha = hip_ops.linear_alpha(self.weight_global_scale, self.act_global_scale)
+        quantized for this layer (`eager.QuantizedActivations`); returns [*leading_shape, out]."""
+        alpha = eager.linear_alpha(self.weight_global_scale, self.act_global_scale)
         bias = self.bias
         fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16 and bias.is_contiguous()) else None
         with torch.cuda.device(self.qweight.device):
-            y = hip_ops.linear_on(activations, self.qweight, self.scales, alpha, fused_bias,
+            y = eager.linear_on(activations, self.qweight, self.scales, alpha, fused_bias,
                                   hip_ops._current_stream(self.qweight.device.index))
         y = y.unflatten(dim=0, sizes=tuple(leading_shape))
         if bias is not None and fused_bias is None:

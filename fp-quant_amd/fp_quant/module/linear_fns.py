@@ -18,11 +18,10 @@ from .hip_ops import (
     matmul_mxf4_bf16_tn_op,
     matmul_nvf4_bf16_tn_bias_op,
     matmul_nvf4_bf16_tn_op,
-    linear_alpha,
     linear_mxf4_packed_op,
-    linear_w4a4,
     packed_linear_eligible,
 )
+from .eager import linear_alpha, linear_w4a4
 
 
 def forward_quantize(

@@ -24,10 +24,10 @@ from torch import nn
 from .config import FPQuantDtype
 
 
-def _hip_ops():
-    from ..module import hip_ops
+def _eager():
+    from ..module import eager
 
-    return hip_ops
+    return eager
 
 
 def _is_real_quant_linear(layer) -> bool:
@@ -68,7 +68,7 @@ def fuse_rmsnorm(norm: nn.Module, consumer) -> bool:
     def forward(self, hidden_states):
         layer = peer[0]
         if _fusable_call(hidden_states) and self.weight.dtype == torch.bfloat16:
-            y = _hip_ops().rmsnorm_quantize(hidden_states, self.weight, self.variance_epsilon,
+            y = _eager().rmsnorm_quantize(hidden_states, self.weight, self.variance_epsilon,
                                             layer.forward_hadamard_matrix, layer.act_global_scale,
                                             layer.config.forward_dtype == FPQuantDtype.NVFP4)
             if y is not None:
@@ -99,7 +99,7 @@ def fuse_gated_mlp(mlp: nn.Module) -> bool:
         up = self.up_proj(x)
         down = self.down_proj
         inter = gate.shape[-1]
-        qa = _hip_ops().silu_mul_quantize(gate.reshape(-1, inter), up.reshape(-1, inter),
+        qa = _eager().silu_mul_quantize(gate.reshape(-1, inter), up.reshape(-1, inter),
                                           down.forward_hadamard_matrix, down.act_global_scale,
                                           down.config.forward_dtype == FPQuantDtype.NVFP4)
         if qa is None:

@@ -179,7 +179,7 @@ def _tiny_llama(fmt, g, seed=0):
 def test_fused_norm_and_mlp_match_the_oracle_composition(fmt, g, tokens):
     """A fused RMSNorm returns the oracle's bf16 tensor and its consumers give what they give when
     handed that tensor unfused; the fused MLP equals down_proj on the oracle's silu*up."""
-    from fp_quant.module import hip_ops
+    from fp_quant.module import eager, hip_ops
     from fp_quant.utils import fuse_producers, unfuse_producers
     model = _tiny_llama(fmt, g)
     block = model.model.layers[1]
@@ -194,23 +194,23 @@ def test_fused_norm_and_mlp_match_the_oracle_composition(fmt, g, tokens):
 
         assert fuse_producers(model) == 6                     # two norms and one MLP per block
         assert sorted(model.state_dict()) == sorted(_tiny_llama(fmt, g).state_dict())
-        hip_ops._shared_activations.clear()
+        eager._shared_activations.clear()
         y = block.input_layernorm(x)
         assert torch.equal(y, want_y)
-        slot = hip_ops._shared_activations[0]
+        slot = eager._shared_activations[0]
         assert slot.ref() is y and (slot.row_major is not None or slot.mx_packed is not None)
         assert torch.equal(block.self_attn.q_proj(y), want_q)
         assert torch.equal(block.self_attn.k_proj(y), want_k)
-        assert hip_ops._shared_activations[0] is slot         # both projections used the norm's quantization
+        assert eager._shared_activations[0] is slot         # both projections used the norm's quantization
         assert torch.equal(block.mlp(x), want_mlp)
 
         # a consumer that does not match (other tensor) still computes its own quantization
         assert torch.equal(block.self_attn.q_proj(want_y.clone()), want_q)
 
         unfuse_producers(model)
-        hip_ops._shared_activations.clear()
+        eager._shared_activations.clear()
         block.input_layernorm(x)
-        assert 0 not in hip_ops._shared_activations
+        assert 0 not in eager._shared_activations
 
 
 @pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])

@@ -69,7 +69,7 @@ def test_linear_matches_oracle_pipeline(fmt, g, bias):
 def test_other_transform_inits(init):
     """transform_init identity / gsr go through the same operators (matrix recognised on the host)."""
     import fp_quant
-    from fp_quant.module import hip_ops
+    from fp_quant.module import eager, hip_ops
     from fp_quant import _engine
     gen = torch.Generator().manual_seed(5)
     w = (torch.randn(64, 256, generator=gen) * 0.02).to(torch.bfloat16)
@@ -90,7 +90,7 @@ def test_other_transform_inits(init):
 
 
 def test_general_matrix_through_the_operator():
-    from fp_quant.module import hip_ops
+    from fp_quant.module import eager, hip_ops
     gen = torch.Generator().manual_seed(6)
     q, _ = torch.linalg.qr(torch.randn(32, 32, generator=gen))
     h = q.to(torch.bfloat16)
@@ -147,7 +147,7 @@ def test_state_dict_roundtrip_without_pre_forward():
 
 
 def test_operators_have_fake_impls_and_compile():
-    from fp_quant.module import hip_ops
+    from fp_quant.module import eager, hip_ops
     x = torch.randn(32, 256, device="cuda", dtype=torch.bfloat16)
     h = O.hadamard_matrix(32).cuda()
 
@@ -269,33 +269,33 @@ def test_layers_sharing_an_input_share_its_quantization(fmt, g, m):
     """q/k/v-style layers called with the same tensor object reuse the quantized activations of the
     first call; outputs are bit-identical to unshared calls, and any change of the input (in-place
     write, another tensor, another rotation or global scale) quantizes again."""
-    from fp_quant.module import hip_ops
+    from fp_quant.module import eager, hip_ops
     k = 512
     layers = [_quantized_linear(fmt, g, k, n, seed) for seed, n in enumerate((256, 128, 384))]
     x = torch.randn(2, m, k, device="cuda", dtype=torch.bfloat16)
 
     def unshared(inp, lins):
-        hip_ops.SHARE_ACT_QUANT = False
+        eager.SHARE_ACT_QUANT = False
         try:
             return [lin(inp) for lin in lins]
         finally:
-            hip_ops.SHARE_ACT_QUANT = True
+            eager.SHARE_ACT_QUANT = True
 
     want = unshared(x, layers)
-    hip_ops._shared_activations.clear()
+    eager._shared_activations.clear()
     got0 = layers[0](x)
-    slot = hip_ops._shared_activations[0]
+    slot = eager._shared_activations[0]
     filled = [f for f in ("mx_packed", "row_major", "nv_packed") if getattr(slot, f) is not None]
     assert filled
     got = [got0] + [lin(x) for lin in layers[1:]]
-    assert hip_ops._shared_activations[0] is slot          # the later calls found the first call's entry
+    assert eager._shared_activations[0] is slot          # the later calls found the first call's entry
     for a, b in zip(got, want):
         assert torch.equal(a, b)
 
     # in-place write: same object, new version -> quantized again
     x.mul_(-1.5)
     want2 = unshared(x, layers[:2])
-    assert torch.equal(layers[0](x), want2[0]) and hip_ops._shared_activations[0] is not slot
+    assert torch.equal(layers[0](x), want2[0]) and eager._shared_activations[0] is not slot
     assert torch.equal(layers[1](x), want2[1])
 
     # a new tensor (very likely at the freed address) never matches the dead one
@@ -326,18 +326,18 @@ def test_layers_sharing_an_input_share_its_quantization(fmt, g, m):
 def test_inference_mode(fmt, g, m):
     """torch.inference_mode(): tensors made there carry no version counter, so nothing is cached on or
     shared through them; results equal the no_grad ones, also for a layer built inside the mode."""
-    from fp_quant.module import hip_ops
+    from fp_quant.module import eager, hip_ops
     lin = _quantized_linear(fmt, g, 512, 256, 21, bias=True)
     other = _quantized_linear(fmt, g, 512, 128, 22)
     x = torch.randn(m, 512, device="cuda", dtype=torch.bfloat16)
     with torch.no_grad():
         want, want_other = lin(x), other(x)
     with torch.inference_mode():
-        hip_ops._shared_activations.clear()
+        eager._shared_activations.clear()
         xi = x * 1.0                                   # an inference tensor
         assert xi.is_inference()
         got, got_other = lin(xi), other(xi)
-        assert not hip_ops._shared_activations         # nothing shared: writes to xi could not be noticed
+        assert not eager._shared_activations         # nothing shared: writes to xi could not be noticed
         xi.mul_(2.0)
         twice = lin(xi)
     assert torch.equal(got, want) and torch.equal(got_other, want_other)
