@@ -496,6 +496,10 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
   // per wave for regrouping the by-product
   extern __shared__ __attribute__((aligned(128))) uint8_t dyn_lds[];
   uint16_t* silu_lds = (uint16_t*)(dyn_lds + 4 * TILE);
+  // lookups go through a pointer that names the LDS address space, so that they are LDS reads and
+  // not flat loads (which take the texture path)
+  typedef __attribute__((address_space(3))) const uint16_t lds_u16;
+  lds_u16* silu_tab = (lds_u16*)silu_lds;
   __shared__ float2 lut[128];
   if (PRO == kProSiluMul) {
     for (uint32_t i = threadIdx.x; i < 2u * kSiluLdsCount; i += 256u) {
@@ -614,13 +618,12 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
             const uint32_t bits = (i & 1) ? (w[i >> 1] >> 16) : (w[i >> 1] & 0xffffu);
+            // the LDS read is unconditional (index clamped) and the rare global read separate, so that
+            // neither turns into a flat load through a pointer that could be either
             const uint32_t idx = (bits & 0x7fffu) - kSiluLdsFirst;
-            uint32_t t;
-            if (idx < kSiluLdsCount) {
-              t = silu_lds[(bits >> 15) * kSiluLdsCount + idx];
-            } else {
-              t = g_silu_table[bits];
-            }
+            const bool in_lds = idx < kSiluLdsCount;
+            uint32_t t = silu_tab[(bits >> 15) * kSiluLdsCount + (in_lds ? idx : 0u)];
+            if (!in_lds) t = g_silu_table[bits];
             e[i] = __uint_as_float(t << 16);
           }
         }
