@@ -460,7 +460,7 @@ __device__ __forceinline__ uint32_t fix_zero_nibbles(uint32_t w) {
 }
 
 //
-// PACKED (MXFP4, EPL = 64 only) writes the operand layout of fpq_gemm_mxf4_packed instead of
+// PACKED (EPL = 64 only) writes the operand layout of fpq_gemm_mxf4_packed / fpq_gemm_nvf4_packed instead of
 // row-major codes and scales.  A wave tile is then 32 rows x two neighbouring chunks (lane =
 // 2 * row + chunk, so the lane pairing of a 128-wide rotation is unchanged): the loads are 256-byte
 // row segments, and every 16-byte half of a lane's codes is exactly one lane slot of a packed
@@ -480,8 +480,8 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
     const uint8_t* __restrict__ x, uint8_t* __restrict__ codes, uint8_t* __restrict__ scales,
     uint32_t n_chunks, uint32_t chunks_per_row, uint32_t rows, uint32_t scale_rows,
     uint32_t scale_stride, float norm, const float* __restrict__ global_scale, Prologue pro) {
-  static_assert(!PACKED || (FMT == kFmtMx && EPL == 64), "packed output: MXFP4 with 64-element chunks");
-  static_assert(PRO == kProNone || PACKED, "prologues exist for the packed output only");
+  static_assert(!PACKED || EPL == 64, "packed output: 64-element chunks");
+  static_assert(PRO == kProNone || (PACKED && FMT == kFmtMx), "prologues exist for the packed MXFP4 output only");
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
   constexpr int NG = EPL / GROUP;        // groups (= scale bytes) per chunk
   constexpr int PIECES = EPL / 8;        // 16-byte input pieces per chunk
@@ -773,7 +773,7 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
           float a = 0.0f;
 #pragma unroll
           for (int i = 0; i < GROUP; ++i) a = __builtin_fmaxf(a, __builtin_fabsf(u[gi * GROUP + i]));
-          const GroupScale g = mx_group_scale(a);
+          const GroupScale g = FMT == kFmtMx ? mx_group_scale(a) : nv_group_scale(a, gs, rg);
 #pragma unroll
           for (int d = 0; d < GROUP / 8; ++d) {
             uint32_t w = 0u;
@@ -782,6 +782,7 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
               const float xv = u[gi * GROUP + d * 8 + h];
               float q = scale_element(xv, g);
               if (ZERO == kZeroSigned) q = __builtin_copysignf(q, xv);
+              if (FMT == kFmtNv) q = g.zero ? 0.0f : q;
               w |= e2m1_code<ZERO>(q) << (4 * h);
             }
             cw[gi * (GROUP / 8) + d] = w;
@@ -804,10 +805,20 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
       // of a row holds bytes q and q + 1 of both dwords: the even lane stores the half-word of
       // K half 0, the odd lane that of K half 1.
       const uint32_t other = (uint32_t)__builtin_amdgcn_mov_dpp((int)sbytes, 0xB1, 0xF, 0xF, true);
-      const uint32_t hw = ksl == 0u ? ((sbytes & 0xffu) | ((other & 0xffu) << 8))
-                                    : (((other >> 8) & 0xffu) | (sbytes & 0xff00u));
-      uint8_t* sblk = scales + ((size_t)rt * (chunks_per_row / 4u) + (pr >> 1)) * 256u;
-      *(uint16_t*)(sblk + (ksl * 32u + r) * 4u + 2u * (pr & 1u)) = (uint16_t)hw;
+      if (FMT == kFmtMx) {
+        const uint32_t hw = ksl == 0u ? ((sbytes & 0xffu) | ((other & 0xffu) << 8))
+                                      : (((other >> 8) & 0xffu) | (sbytes & 0xff00u));
+        uint8_t* sblk = scales + ((size_t)rt * (chunks_per_row / 4u) + (pr >> 1)) * 256u;
+        *(uint16_t*)(sblk + (ksl * 32u + r) * 4u + 2u * (pr & 1u)) = (uint16_t)hw;
+      } else {
+        // NVFP4: four E4M3 bytes per lane, two per K half.  The 8 bytes of (kh, r) in block
+        // (rt, ks / 4) hold bytes 2 q, 2 q + 1 for K step q = ks % 4, so the lane pair of a row owns
+        // one dword of each K half: the even lane stores that of K half 0, the odd lane that of 1.
+        const uint32_t dw = ksl == 0u ? ((sbytes & 0xffffu) | (other << 16))
+                                      : ((other >> 16) | (sbytes & 0xffff0000u));
+        uint8_t* sblk = scales + ((size_t)rt * (chunks_per_row / 4u) + (pr >> 1)) * 512u;
+        *(uint32_t*)(sblk + (ksl * 32u + r) * 8u + 4u * (pr & 1u)) = dw;
+      }
       asm volatile("" ::: "memory");
       continue;
     }
@@ -893,10 +904,10 @@ static int launch_stream(const void* x, int64_t rows, int64_t cols, float norm, 
 
 constexpr int kSiluDynLds = 4 * 64 * 128 + 2 * (int)kSiluLdsCount * 2;  // second tiles + table copy
 
-template <int G, int ROT, int PRO = kProNone>
+template <int G, int ROT, int PRO = kProNone, int FMT = kFmtMx>
 static int launch_stream_packed(const void* x, int64_t rows, int64_t cols, float norm, void* codes,
                                 void* scales, int zero_policy, hipStream_t stream,
-                                const Prologue& pro = Prologue{}) {
+                                const Prologue& pro = Prologue{}, const float* gsp = nullptr) {
   const int64_t n_tiles = ((rows + 31) / 32) * (cols / 128);
   int64_t blocks = (n_tiles + 3) / 4;
   if (blocks > 1024) blocks = 1024;
@@ -911,23 +922,25 @@ static int launch_stream_packed(const void* x, int64_t rows, int64_t cols, float
     }
     hipLaunchKernelGGL(kernel, grid, block, kDyn, stream, (const uint8_t*)x, (uint8_t*)codes,
                        (uint8_t*)scales, (uint32_t)(rows * cols / 64), (uint32_t)(cols / 64),
-                       (uint32_t)rows, 0u, 0u, norm, (const float*)nullptr, pro);
+                       (uint32_t)rows, 0u, 0u, norm, gsp, pro);
   };
   if (zero_policy == FPQ_ZERO_REFERENCE) {
-    go(quantize_stream_kernel<64, G, kFmtMx, ROT, kZeroReference, true, PRO>);
+    go(quantize_stream_kernel<64, G, FMT, ROT, kZeroReference, true, PRO>);
   } else {
-    go(quantize_stream_kernel<64, G, kFmtMx, ROT, kZeroSigned, true, PRO>);
+    go(quantize_stream_kernel<64, G, FMT, ROT, kZeroSigned, true, PRO>);
   }
   if (status) return status;
   return (int)hipGetLastError();
 }
 
+template <int FMT>
 static int dispatch_packed(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
-                           void* codes, void* scales, int zero_policy, void* stream_) {
+                           const float* gsp, void* codes, void* scales, int zero_policy, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   if (rows < 0 || cols < 0) return FPQ_E_SHAPE;
   if (rows == 0 || cols == 0) return FPQ_OK;
   if (!x || !codes || !scales) return FPQ_E_NULL;
+  if (FMT == kFmtNv && !gsp) return FPQ_E_NULL;
   if (zero_policy != FPQ_ZERO_REFERENCE && zero_policy != FPQ_ZERO_SIGNED) return FPQ_E_POLICY;
   if (rot_kind == FPQ_ROT_IDENTITY) g = 32;
   if (g != 16 && g != 32 && g != 64 && g != 128) return FPQ_E_ROTATION;
@@ -935,7 +948,8 @@ static int dispatch_packed(const void* x, int64_t rows, int64_t cols, int rot_ki
   if (rows * cols >= (int64_t)1 << 34) return FPQ_E_SHAPE;
   if (((uintptr_t)x & 15u) || ((uintptr_t)codes & 15u) || ((uintptr_t)scales & 3u)) return FPQ_E_ALIGN;
 #define FPQ_LAUNCH_PACKED(GG, RR) \
-  return launch_stream_packed<GG, RR>(x, rows, cols, norm, codes, scales, zero_policy, stream)
+  return launch_stream_packed<GG, RR, kProNone, FMT>(x, rows, cols, norm, codes, scales, zero_policy, stream, \
+                                                     Prologue{}, gsp)
   if (rot_kind == FPQ_ROT_IDENTITY) {
     FPQ_LAUNCH_PACKED(32, FPQ_ROT_IDENTITY);
   } else if (rot_kind == FPQ_ROT_HADAMARD) {
@@ -1303,8 +1317,15 @@ extern "C" int fpq_quantize_mx_quest(const void* x, int64_t rows, int64_t cols, 
 extern "C" int fpq_quantize_mx_packed(const void* x, int64_t rows, int64_t cols, int rot_kind, int g,
                                       float norm, void* packed_codes, void* packed_scales,
                                       int zero_policy, void* stream) {
-  return fpq::dispatch_packed(x, rows, cols, rot_kind, g, norm, packed_codes, packed_scales, zero_policy,
-                              stream);
+  return fpq::dispatch_packed<fpq::kFmtMx>(x, rows, cols, rot_kind, g, norm, nullptr, packed_codes, packed_scales,
+                                           zero_policy, stream);
+}
+
+extern "C" int fpq_quantize_nv_packed(const void* x, int64_t rows, int64_t cols, int rot_kind, int g,
+                                      float norm, const float* global_scale, void* packed_codes,
+                                      void* packed_scales, int zero_policy, void* stream) {
+  return fpq::dispatch_packed<fpq::kFmtNv>(x, rows, cols, rot_kind, g, norm, global_scale, packed_codes,
+                                           packed_scales, zero_policy, stream);
 }
 
 extern "C" int fpq_quantize_nv(const void* x, int64_t rows, int64_t cols, int rot_kind, int g,

@@ -73,15 +73,18 @@ SHARE_ACT_QUANT = os.environ.get("FPQ_SHARE_ACT_QUANT", "1") != "0"
 class QuantizedActivations:
     """Rotated and quantized activations of one [m, k] tensor, in whichever operand layouts have
     been asked for so far (row-major codes/scales, packed MXFP4, packed NVFP4)."""
-    __slots__ = ("m", "k", "nvfp4", "packed_gemm", "ref", "version", "key", "keep", "mx_packed", "row_major",
-                 "nv_packed")
+    __slots__ = ("m", "k", "nvfp4", "ref", "version", "key", "keep", "mx_packed", "row_major", "nv_packed")
 
-    def __init__(self, m: int, k: int, nvfp4: bool, packed_gemm: bool):
+    def __init__(self, m: int, k: int, nvfp4: bool):
         self.m, self.k, self.nvfp4 = m, k, nvfp4
-        self.packed_gemm = packed_gemm   # MXFP4: the GEMM runs on packed operands (decided once per call)
         self.ref = self.key = self.keep = None
         self.version = 0
         self.mx_packed = self.row_major = self.nv_packed = None
+
+    def serves(self, want_packed: bool) -> bool:
+        """Whether a GEMM on packed (or on row-major) operands can run from what is held: the packed
+        form can be made from the row-major one, not the other way round."""
+        return want_packed or self.row_major is not None
 
     def packed(self) -> Tuple[torch.Tensor, torch.Tensor]:
         """Codes and scales in the packed GEMM layout (re-tiled from the row-major ones if need be)."""
@@ -97,7 +100,7 @@ class QuantizedActivations:
 _shared_activations = {}   # device index -> QuantizedActivations of the latest call
 
 
-def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: int, want_packed: bool):
+def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: int):
     """What two calls must agree on, besides the source tensor, to share quantized activations, or
     None when nothing may be shared.  Layers own separate but equal rotation and global-scale
     buffers, so those are compared by value: (kind, norm, size) of a recognised rotation, the host
@@ -111,9 +114,7 @@ def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: i
     if act_global_scale is not None:
         gs = cached_on(act_global_scale, "_fpq_host", (_version(act_global_scale), act_global_scale.data_ptr()),
                        lambda: float(act_global_scale))
-    # the operand layout the GEMM will ask for is part of the key: the packed form can be made from the
-    # row-major one but not the other way round
-    return (rot, gs, stream, capture_id.value, tuple(x_shape), want_packed)
+    return (rot, gs, stream, capture_id.value, tuple(x_shape))
 
 
 def _publish(qa: QuantizedActivations, src: torch.Tensor, key, keep) -> None:
@@ -121,9 +122,10 @@ def _publish(qa: QuantizedActivations, src: torch.Tensor, key, keep) -> None:
     _shared_activations[src.device.index] = qa
 
 
-def _lookup(src: torch.Tensor, key) -> Optional[QuantizedActivations]:
+def _lookup(src: torch.Tensor, key, want_packed: bool) -> Optional[QuantizedActivations]:
     qa = _shared_activations.get(src.device.index)
-    if qa is not None and qa.ref() is src and qa.version == _version(src) and qa.key == key:
+    if (qa is not None and qa.ref() is src and qa.version == _version(src) and qa.key == key
+            and qa.serves(want_packed)):
         return qa
     return None
 
@@ -137,8 +139,8 @@ def quantize_activations(x_flat: torch.Tensor, h: torch.Tensor, kind: int, norm:
     m, k = x_flat.shape
     dev = x_flat.device
     g = h.shape[0]
-    qa = QuantizedActivations(m, k, nvfp4, want_packed)
-    if want_packed:
+    qa = QuantizedActivations(m, k, nvfp4)
+    if want_packed and not nvfp4:
         pc = torch.empty(lib.fpq_packed_codes_bytes(m, k), dtype=torch.uint8, device=dev)
         ps = torch.empty(lib.fpq_packed_scales_bytes(m, k), dtype=torch.uint8, device=dev)
         st = lib.fpq_quantize_mx_packed(x_flat.data_ptr(), m, k, kind, g, norm, pc.data_ptr(), ps.data_ptr(),
@@ -149,6 +151,16 @@ def quantize_activations(x_flat: torch.Tensor, h: torch.Tensor, kind: int, norm:
             _engine.check(st, "fpq_quantize_mx_packed")
         qa.mx_packed = (pc, ps)
         return qa
+    if nvfp4 and want_packed:
+        pc = torch.empty(lib.fpq_packed_codes_bytes(m, k), dtype=torch.uint8, device=dev)
+        ps = torch.empty(lib.fpq_packed_scales_bytes_nv(m, k), dtype=torch.uint8, device=dev)
+        gs = as_f32_scalar(act_global_scale)
+        st = lib.fpq_quantize_nv_packed(x_flat.data_ptr(), m, k, kind, g, norm, gs.data_ptr(), pc.data_ptr(),
+                                        ps.data_ptr(), ZERO_NIBBLE_POLICY, stream)
+        if st != _engine.E_UNSUPPORTED:
+            _engine.check(st, "fpq_quantize_nv_packed")
+            qa.nv_packed = (pc, ps)
+            return qa
     group = 16 if nvfp4 else 32
     codes = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
     scales = torch.empty(m, k // group, dtype=torch.uint8, device=dev)
@@ -165,10 +177,16 @@ def quantize_activations(x_flat: torch.Tensor, h: torch.Tensor, kind: int, norm:
     return qa
 
 
+def wants_packed(m: int, n: int, k: int, nvfp4: bool) -> bool:
+    """Whether the GEMM of an [m, k] x [n, k] linear runs on packed operands."""
+    return nv_packed_eligible(m, n, k) if nvfp4 else packed_linear_eligible(m, k, "abs_max")
+
+
 def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alpha: torch.Tensor,
-              bias: Optional[torch.Tensor], stream: int) -> torch.Tensor:
+              bias: Optional[torch.Tensor], stream: int, use_packed: Optional[bool] = None) -> torch.Tensor:
     """bf16 [m, n] = alpha * dq(activations) @ dq(w).T (+ bias) on quantized activations, with the
-    kernel and operand layout the shape calls for."""
+    kernel and operand layout the shape calls for (`use_packed`: the caller's decision, if it has
+    made it already)."""
     lib = _engine.lib()
     m, k = qa.m, qa.k
     n = wq.shape[0]
@@ -176,8 +194,12 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
         raise ValueError(f"inner dimensions differ: x has K={k}, w has K={wq.shape[1] * 2}")
     y = torch.empty(m, n, dtype=torch.bfloat16, device=wq.device)
     b_ptr = bias.data_ptr() if bias is not None else None
+    if use_packed is None:
+        use_packed = wants_packed(m, n, k, qa.nvfp4)
+    if not qa.serves(use_packed):
+        raise ValueError("these activations were quantized into the packed layout only")
     if qa.nvfp4:
-        if nv_packed_eligible(m, n, k):
+        if use_packed:
             xp, xsp = qa.packed()
             wp, wsp = packed_weight(wq, ws, True)
             st = lib.fpq_gemm_nvf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
@@ -189,7 +211,7 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
                                ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
         _engine.check(st, "fpq_gemm_nvf4")
         return y
-    if qa.packed_gemm:
+    if use_packed:
         pc, ps = qa.packed()
         wp, wsp = packed_weight(wq, ws)
         st = lib.fpq_gemm_mxf4_packed(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(), alpha.data_ptr(),
@@ -220,17 +242,18 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
     stream = _current_stream(dev.index)
     h = as_bf16(hadamard_matrix)
     kind, norm = classify_rotation(h)
-    want_packed = not nvfp4 and packed_linear_eligible(x_flat.shape[0], x_flat.shape[1], "abs_max")
+    m, k = x_flat.shape
+    want_packed = wants_packed(m, wq.shape[0], k, nvfp4)
     qa = key = None
     if shared_source is not None:
-        key = _sharing_key(x_flat.shape, h, kind, norm, act_global_scale if nvfp4 else None, stream, want_packed)
+        key = _sharing_key(x_flat.shape, h, kind, norm, act_global_scale if nvfp4 else None, stream)
         if key is not None:
-            qa = _lookup(shared_source, key)
+            qa = _lookup(shared_source, key, want_packed)
     if qa is None:
         qa = quantize_activations(x_flat, h, kind, norm, act_global_scale, nvfp4, stream, want_packed)
         if key is not None:
             _publish(qa, shared_source, key, h)
-    return linear_on(qa, wq, ws, alpha, bias, stream)
+    return linear_on(qa, wq, ws, alpha, bias, stream, want_packed)
 
 
 ### Quantizers fused with the producer of their input
@@ -254,7 +277,7 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
         if st == _engine.E_UNSUPPORTED:
             return None
         _engine.check(st, f"fpq_{entry}_quantize_mx_packed")
-        qa = QuantizedActivations(rows, cols, nvfp4, True)
+        qa = QuantizedActivations(rows, cols, nvfp4)
         qa.mx_packed = (pc, ps)
         return qa
     codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=dev)
@@ -268,7 +291,7 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
     if st == _engine.E_UNSUPPORTED:
         return None
     _engine.check(st, f"fpq_{entry}_quantize")
-    qa = QuantizedActivations(rows, cols, nvfp4, False)
+    qa = QuantizedActivations(rows, cols, nvfp4)
     qa.row_major = (codes, scales)
     return qa
 
@@ -303,7 +326,7 @@ def rmsnorm_quantize(x: torch.Tensor, weight: torch.Tensor, eps: float, hadamard
         if qa is None:
             return None
         y = y.view(x.shape)
-        key = _sharing_key(x_flat.shape, h, kind, norm, act_global_scale if nvfp4 else None, stream, qa.packed_gemm)
+        key = _sharing_key(x_flat.shape, h, kind, norm, act_global_scale if nvfp4 else None, stream)
         if key is not None:
             _publish(qa, y, key, h)
     return y

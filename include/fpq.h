@@ -236,6 +236,15 @@ int fpq_pack_nvf4(const void* codes, const void* scales, int64_t scale_stride, i
 int fpq_gemm_nvf4_packed(const void* xq_packed, const void* xs_packed, const void* wq_packed,
                          const void* ws_packed, const float* alpha, const void* bias, void* y,
                          int64_t M, int64_t N, int64_t K, void* stream);
+/*
+ * fpq_quantize_nv writing the packed layout directly (same codes and scale bytes; rows past `rows`
+ * in the last 32-row tile get zero codes and zero scale bytes).  cols % 256 == 0; rotations as for
+ * fpq_quantize_mx_packed, others return FPQ_E_UNSUPPORTED (quantize row-major, then fpq_pack_nvf4).
+ * Same reference counterpart as fpq_quantize_nv (qutlass_ops.py:74-105).
+ */
+int fpq_quantize_nv_packed(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                           const float* global_scale, void* packed_codes, void* packed_scales,
+                           int zero_policy, void* stream);
 
 /*
  * Measurement hook: `blocks` workgroups of four waves run `iters` x 16 FP4 32x32x64 block-scaled

@@ -270,3 +270,21 @@ def fused_quantize_packed(kind, a, b, g=128, rot="hadamard", norm=None, eps=1e-5
     _engine.check(st, f"fpq_{kind}_quantize_mx_packed")
     torch.cuda.synchronize()
     return pc.cpu(), ps.cpu(), (out.cpu() if out is not None else None)
+
+
+def quantize_nv_packed(x_bf16, global_scale, rot="hadamard", g=16, norm=None, zero_policy=_engine.ZERO_REFERENCE,
+                       fill=0xCD):
+    """Run fpq_quantize_nv_packed; returns CPU uint8 (packed codes, packed scales)."""
+    lib = _engine.lib()
+    x = x_bf16.to("cuda").contiguous()
+    rows, cols = x.shape
+    pc = torch.full((lib.fpq_packed_codes_bytes(rows, cols),), fill, dtype=torch.uint8, device="cuda")
+    ps = torch.full((lib.fpq_packed_scales_bytes_nv(rows, cols),), fill, dtype=torch.uint8, device="cuda")
+    if norm is None:
+        norm = float(torch.tensor(g ** -0.5, dtype=torch.bfloat16))
+    gs = torch.tensor([global_scale], dtype=torch.float32, device="cuda")
+    st = lib.fpq_quantize_nv_packed(x.data_ptr(), rows, cols, ROT[rot], g, norm, gs.data_ptr(), pc.data_ptr(),
+                                    ps.data_ptr(), zero_policy, torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_quantize_nv_packed")
+    torch.cuda.synchronize()
+    return pc.cpu(), ps.cpu()

@@ -187,6 +187,36 @@ def test_gemm_nv_packed_matches_oracle(m, n, k, bias):
     assert exact > 0.97
 
 
+@pytest.mark.parametrize("rot,g", [("hadamard", 16), ("hadamard", 32), ("hadamard", 64), ("hadamard", 128),
+                                   ("identity", 16), ("gsr", 32)])
+@pytest.mark.parametrize("policy", [0, 1])
+def test_quantize_nv_packed_bit_exact(rot, g, policy):
+    rows, cols = 70, 512  # ragged last row tile
+    x = make_outlier_normal(rows, cols, 13 * g + len(rot))
+    x[3, 64:96] = 0.0            # zero groups
+    x[5, :32] = -0.0
+    x[7] *= 2.0 ** -20           # E4M3 scales that underflow to zero
+    okind = {"hadamard": O.ROT_HADAMARD, "identity": O.ROT_IDENTITY, "gsr": O.ROT_GSR}[rot]
+    norm = float(O.hadamard_matrix(g)[0, 0])
+    for gs in (40.0, 2.0 ** 70):  # the second takes the generic per-element path
+        wc, ws, _ = O.quantize_nv(x, gs, okind, g, norm, zero_nibble=policy)
+        want_c, want_s = pack_nv_by_definition(wc, ws, cols)
+        pc, ps = capi.quantize_nv_packed(x, gs, rot=rot, g=g, norm=norm, zero_policy=policy)
+        assert torch.equal(pc, want_c)
+        assert torch.equal(ps, want_s)
+
+
+def test_quantize_nv_packed_large_matches_row_major_path():
+    gen = torch.Generator().manual_seed(6)
+    x = (torch.randn(1000, 4096, generator=gen) * 3).to(torch.bfloat16)
+    rc, rs = capi.quantize(x, "nvfp4", g=16, global_scale=25.0)
+    want_c, want_s = pack_nv_by_definition(rc, rs, 4096)
+    pc, ps = capi.quantize_nv_packed(x, 25.0, g=16)
+    assert torch.equal(pc, want_c) and torch.equal(ps, want_s)
+    with pytest.raises(ValueError):
+        capi.quantize_nv_packed(torch.zeros(32, 384, dtype=torch.bfloat16), 1.0)   # cols % 256 != 0
+
+
 def test_nvfp4_linear_mid_m_runs_packed_and_matches_oracle(monkeypatch):
     import fp_quant
     from fp_quant.module import hip_ops
