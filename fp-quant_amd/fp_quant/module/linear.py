@@ -13,9 +13,6 @@ from ..utils import FPQuantConfig, FPQuantDtype, validate_config
 from . import eager, hip_ops
 from .linear_fns import FPQuant4x16NoMasterFn, forward_quantize
 
-_SCALE_GROUP = {FPQuantDtype.MXFP4: 32, FPQuantDtype.NVFP4: 16}
-
-
 def _sylvester_signs(n: int) -> torch.Tensor:
     """+-1 Sylvester-Hadamard matrix, entry (i, j) = (-1)^popcount(i & j) (== scipy.linalg.hadamard)."""
     h = torch.ones(1, 1, dtype=torch.float64)
@@ -69,7 +66,7 @@ class FPQuantLinear(nn.Module):
             raise ValueError(
                 "libfpq_hip.so is not built or failed to load; build it with `python fp-quant_amd/build.py`"
             )
-        group = _SCALE_GROUP.get(config.forward_dtype)
+        group = config.forward_dtype.scale_group if config.forward_dtype in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4) else None
         if group is None:
             raise ValueError(f"Unsupported forward dtype: {config.forward_dtype}")
 
@@ -132,7 +129,7 @@ class FPQuantLinear(nn.Module):
             self.weight, self.forward_hadamard_matrix, self.weight_global_scale,
             cfg.forward_dtype, cfg.forward_method,
         )
-        group = _SCALE_GROUP[cfg.forward_dtype]
+        group = cfg.forward_dtype.scale_group
         rows, cols = self.weight.shape[0], self.weight.shape[1] // group
         scales = scales.view(dtype=torch.uint8)[:rows, :cols].contiguous()  # drop the op's padding
         self.qweight = nn.Parameter(weight_q, requires_grad=False)

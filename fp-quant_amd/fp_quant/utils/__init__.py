@@ -1,7 +1,20 @@
+"""Configuration, model surgery, producer fusion and export helpers of the fp_quant package."""
+from . import config, export, fuse, replace
 from .config import FPQuantConfig, FPQuantDtype, validate_config
-from .replace import (
-    finalize_master_weights,
-    replace_quantize_with_fp_quant_linear,
-    replace_with_fp_quant_linear,
-)
 from .fuse import fuse_producers, unfuse_producers
+from .replace import finalize_master_weights, replace_quantize_with_fp_quant_linear, replace_with_fp_quant_linear
+
+__all__ = [
+    "FPQuantConfig",
+    "FPQuantDtype",
+    "validate_config",
+    "replace_with_fp_quant_linear",
+    "replace_quantize_with_fp_quant_linear",
+    "finalize_master_weights",
+    "fuse_producers",
+    "unfuse_producers",
+    "config",
+    "export",
+    "fuse",
+    "replace",
+]

@@ -212,17 +212,14 @@ def rtn_export(
 
 
 def quantization_config_dict(config: FPQuantConfig) -> Dict[str, object]:
-    """`quantization_config` entry of the saved model config (src/quantization/qconfig.py:3-21)."""
-    return {
-        "forward_dtype": config.forward_dtype.value,
-        "backward_dtype": "bf16",
-        "forward_method": "abs_max",
-        "hadamard_group_size": config.hadamard_group_size,
-        "modules_to_not_convert": list(config.modules_to_not_convert),
-        "quant_method": "fp_quant",
-        "store_master_weights": False,
-        "pseudoquantization": False,
-    }
+    """`quantization_config` entry of the saved model config (src/quantization/qconfig.py:3-21): the
+    inference configuration of what was exported."""
+    entry = config.to_dict()
+    entry.update(backward_dtype="bf16", forward_method="abs_max", store_master_weights=False,
+                 pseudoquantization=False)
+    if config.transform_init == "hadamard":   # the reference's entry has no such key; only say what differs
+        del entry["transform_init"]
+    return entry
 
 
 def save_realquant_checkpoint(

@@ -120,3 +120,25 @@ def test_replace_with_meta_init_and_skip_rule():
     assert all(not p.requires_grad for p in fl.parameters())
     model2, replaced2 = fp_quant.replace_with_fp_quant_linear(nn.Sequential(nn.ReLU()), cfg)
     assert not replaced2
+
+
+def test_config_dict_round_trip_and_scale_groups():
+    import fp_quant
+    D = fp_quant.FPQuantDtype
+    assert D.MXFP4.scale_group == 32 and D.NVFP4.scale_group == 16 and D.BF16.scale_group == 0
+    # the entry the reference writes for an exported checkpoint (src/quantization/qconfig.py:9-18)
+    entry = {"forward_dtype": "nvfp4", "backward_dtype": "bf16", "forward_method": "abs_max",
+             "hadamard_group_size": 16, "modules_to_not_convert": ["lm_head"], "quant_method": "fp_quant",
+             "store_master_weights": False, "pseudoquantization": False}
+    cfg = fp_quant.FPQuantConfig.from_dict(entry)
+    assert cfg.forward_dtype is D.NVFP4 and cfg.backward_dtype is D.BF16 and cfg.hadamard_group_size == 16
+    assert cfg.transform_init == "hadamard" and cfg.modules_to_not_convert == ["lm_head"]
+    back = cfg.to_dict()
+    assert {k: back[k] for k in entry} == entry and back["transform_init"] == "hadamard"
+    # enum members pass through, unknown keys are dropped, defaults stay defaults
+    cfg2 = fp_quant.FPQuantConfig.from_dict({"forward_dtype": D.MXFP4, "something_else": 1})
+    assert cfg2 == fp_quant.FPQuantConfig()
+    from fp_quant.utils import export
+    assert "transform_init" not in export.quantization_config_dict(cfg)
+    cfg.transform_init = "gsr"
+    assert export.quantization_config_dict(cfg)["transform_init"] == "gsr"
