@@ -67,7 +67,8 @@ __device__ __forceinline__ void wave_tile_store(const v16f (&acc)[TN][TM], uint8
                                                 uint16_t* __restrict__ y,
                                                 const uint16_t* __restrict__ bias,
                                                 const float* __restrict__ alpha_p, int n0, int m0,
-                                                int wave, int lane, int M, int N) {
+                                                int wave, int lane, int M, int N,
+                                                const uint16_t* __restrict__ residual = nullptr) {
   const int r32 = lane & 31, kh = lane >> 5;
   const float alpha = *alpha_p;
   constexpr int WT_N = TN * 32, WT_M = TM * 32;      // this wave's part of the workgroup tile
@@ -109,17 +110,35 @@ __device__ __forceinline__ void wave_tile_store(const v16f (&acc)[TN][TM], uint8
   for (int p = 0; p < WT_M / kRpi; ++p) {
     const int ml = p * kRpi + rr;
     if (cc * 16 >= kRowBytes) continue;
-    const uint4 v = *(const uint4*)(stg + ml * kStride + cc * 16);
+    uint4 v = *(const uint4*)(stg + ml * kStride + cc * 16);
     const int m = m0 + ml, n = n0 + cc * 8;
     if (m >= M || n >= N) continue;
     uint16_t* dst = y + (size_t)m * N + n;
     if (vec_ok && n + 7 < N) {
+      if (residual) {  // a separate bf16 add after the GEMM: one more rounding
+        const uint4 rv = *(const uint4*)(residual + (size_t)m * N + n);
+        const uint32_t a[4] = {v.x, v.y, v.z, v.w}, b[4] = {rv.x, rv.y, rv.z, rv.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          o[u] = pack_bf16x2(__uint_as_float(a[u] << 16) + __uint_as_float(b[u] << 16),
+                             __uint_as_float(a[u] & 0xffff0000u) + __uint_as_float(b[u] & 0xffff0000u));
+        v = make_uint4(o[0], o[1], o[2], o[3]);
+      }
       *(uint4*)dst = v;
     } else {
       const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (n + u < N) dst[u] = (uint16_t)(w[u >> 1] >> (16 * (u & 1)));
+      for (int u = 0; u < 8; ++u) {
+        if (n + u < N) {
+          uint32_t h = (w[u >> 1] >> (16 * (u & 1))) & 0xffffu;
+          if (residual) {
+            const float sum = __uint_as_float(h << 16) + __uint_as_float((uint32_t)residual[(size_t)m * N + n + u] << 16);
+            h = pack_bf16x2(sum, 0.0f) & 0xffffu;
+          }
+          dst[u] = (uint16_t)h;
+        }
+      }
     }
   }
 }

@@ -124,7 +124,8 @@ template <int NT, int KW, int MT, int WN, int WM, bool NV = false, int RING = kR
 __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_kernel(
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p,
-    const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int tiles_m) {
+    const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int tiles_m,
+    const uint16_t* __restrict__ residual) {
   constexpr int BN = NT * 32, BM = MT * 32;
   constexpr int NW = WN * WM;           // waves
   static_assert(NW == 4 && NT <= KW && KW % 4 == 0 && MT % 4 == 0 && NT % WN == 0 && MT % WM == 0,
@@ -353,7 +354,7 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
 #undef FPQ_TAKE_SCALES
 
   wave_tile_store<TN, TM, packed_lds_alloc(kBlocks, NV, RING, TN * 32, TM * 32), NW>(acc, smem, y, bias, alpha_p, n_blk + wn * TN * 32, m_blk + wm * TM * 32,
-                                          wave, lane, M, N);
+                                          wave, lane, M, N, residual);
 }
 
 }  // namespace fpq
@@ -361,7 +362,8 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
 namespace fpq {
 template <int NT, int KW, int MT, int WN, int WM, bool NV, int RING = kRing>
 static int launch_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
-                         const void* bias, void* y, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
+                         const void* bias, void* y, int64_t M, int64_t N, int64_t K, hipStream_t stream,
+                         const void* residual) {
   constexpr int kLds = packed_lds_alloc(KW + MT, NV, RING, NT / WN * 32, MT / WM * 32);
   const int tiles_m = (int)((M + MT * 32 - 1) / (MT * 32)), tiles_n = (int)((N + NT * 32 - 1) / (NT * 32));
   static LdsLimitOnce lds_limit;
@@ -369,13 +371,14 @@ static int launch_packed(const void* xq, const void* xs, const void* wq, const v
   hipLaunchKernelGGL((gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV, RING>), dim3((unsigned)(tiles_m * tiles_n)),
                      dim3(256), kLds, stream, (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq,
                      (const uint8_t*)ws, alpha, (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K,
-                     tiles_m);
+                     tiles_m, (const uint16_t*)residual);
   return (int)hipGetLastError();
 }
 
 template <bool NV>
 static int gemm_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
-                       const void* bias, void* y, int64_t M, int64_t N, int64_t K, void* stream);
+                       const void* bias, void* y, int64_t M, int64_t N, int64_t K, void* stream,
+                       const void* residual = nullptr);
 
 template <bool NV>
 static int pack_operand(const void* codes, const void* scales, int64_t scale_stride, int64_t rows, int64_t K,
@@ -406,7 +409,8 @@ static int pack_operand(const void* codes, const void* scales, int64_t scale_str
 namespace fpq {
 template <bool NV>
 static int gemm_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
-                       const void* bias, void* y, int64_t M, int64_t N, int64_t K, void* stream) {
+                       const void* bias, void* y, int64_t M, int64_t N, int64_t K, void* stream,
+                       const void* residual) {
   if (M < 0 || N < 0 || K < 0) return FPQ_E_SHAPE;
   if (M == 0 || N == 0) return FPQ_OK;
   if (!xq || !xs || !wq || !ws || !alpha || !y) return FPQ_E_NULL;
@@ -417,16 +421,16 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
   if (((M + 31) / 32) * 32 * (K / sdiv) >= ((int64_t)1 << 32) || ((N + 31) / 32) * 32 * (K / sdiv) >= ((int64_t)1 << 32))
     return FPQ_E_SHAPE;
   if (((uintptr_t)xq & 15u) || ((uintptr_t)wq & 15u) || ((uintptr_t)xs & 15u) || ((uintptr_t)ws & 15u) ||
-      ((uintptr_t)y & 15u))
+      ((uintptr_t)y & 15u) || ((uintptr_t)residual & 15u))
     return FPQ_E_ALIGN;
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
   if (big_tiles < FPQ_PACKED_SMALL_BELOW)
-    return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
+    return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual);
 #if FPQ_PACKED_HALF_TILES
   if (!NV || FPQ_PACKED_HALF_TILES > 1)
-    return launch_packed<8, 8, 4, 2, 2, NV, 4>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
+    return launch_packed<8, 8, 4, 2, 2, NV, 4>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual);
 #endif
-  return launch_packed<8, 8, 8, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream);
+  return launch_packed<8, 8, 8, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual);
 }
 }  // namespace fpq
 
@@ -456,6 +460,13 @@ extern "C" int fpq_gemm_mxf4_packed(const void* xq, const void* xs, const void* 
                                     const float* alpha, const void* bias, void* y, int64_t M,
                                     int64_t N, int64_t K, void* stream) {
   return fpq::gemm_packed<false>(xq, xs, wq, ws, alpha, bias, y, M, N, K, stream);
+}
+
+extern "C" int fpq_gemm_mxf4_packed_residual(const void* xq, const void* xs, const void* wq, const void* ws,
+                                             const float* alpha, const void* bias, const void* residual, void* y,
+                                             int64_t M, int64_t N, int64_t K, void* stream) {
+  if (!residual) return FPQ_E_NULL;
+  return fpq::gemm_packed<false>(xq, xs, wq, ws, alpha, bias, y, M, N, K, stream, residual);
 }
 
 extern "C" int fpq_gemm_nvf4_packed(const void* xq, const void* xs, const void* wq, const void* ws,

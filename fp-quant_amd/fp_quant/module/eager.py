@@ -183,10 +183,12 @@ def wants_packed(m: int, n: int, k: int, nvfp4: bool) -> bool:
 
 
 def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alpha: torch.Tensor,
-              bias: Optional[torch.Tensor], stream: int, use_packed: Optional[bool] = None) -> torch.Tensor:
+              bias: Optional[torch.Tensor], stream: int, use_packed: Optional[bool] = None,
+              residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """bf16 [m, n] = alpha * dq(activations) @ dq(w).T (+ bias) on quantized activations, with the
     kernel and operand layout the shape calls for (`use_packed`: the caller's decision, if it has
-    made it already)."""
+    made it already).  `residual` (bf16 [m, n]) is added as a separate bf16 addition would add it:
+    inside the packed MXFP4 kernel's epilogue, by a PyTorch addition after the other kernels."""
     lib = _engine.lib()
     m, k = qa.m, qa.k
     n = wq.shape[0]
@@ -194,6 +196,9 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
         raise ValueError(f"inner dimensions differ: x has K={k}, w has K={wq.shape[1] * 2}")
     y = torch.empty(m, n, dtype=torch.bfloat16, device=wq.device)
     b_ptr = bias.data_ptr() if bias is not None else None
+    if residual is not None and (residual.dtype != torch.bfloat16 or residual.numel() != m * n
+                                 or not residual.is_contiguous() or residual.device != wq.device):
+        raise ValueError("residual must be a contiguous bfloat16 tensor of the output's size on the same device")
     if use_packed is None:
         use_packed = wants_packed(m, n, k, qa.nvfp4)
     if not qa.serves(use_packed):
@@ -205,29 +210,39 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
             st = lib.fpq_gemm_nvf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
                                           alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
             _engine.check(st, "fpq_gemm_nvf4_packed")
-            return y
-        codes, scales = qa.row_major
-        st = lib.fpq_gemm_nvf4(codes.data_ptr(), scales.data_ptr(), scales.shape[-1], wq.data_ptr(), ws.data_ptr(),
-                               ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
-        _engine.check(st, "fpq_gemm_nvf4")
+        else:
+            codes, scales = qa.row_major
+            st = lib.fpq_gemm_nvf4(codes.data_ptr(), scales.data_ptr(), scales.shape[-1], wq.data_ptr(),
+                                   ws.data_ptr(), ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
+            _engine.check(st, "fpq_gemm_nvf4")
+        if residual is not None:
+            y += residual
         return y
     if use_packed:
         pc, ps = qa.packed()
         wp, wsp = packed_weight(wq, ws)
-        st = lib.fpq_gemm_mxf4_packed(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(), alpha.data_ptr(),
-                                      b_ptr, y.data_ptr(), m, n, k, stream)
+        if residual is not None:
+            st = lib.fpq_gemm_mxf4_packed_residual(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
+                                                   alpha.data_ptr(), b_ptr, residual.data_ptr(), y.data_ptr(),
+                                                   m, n, k, stream)
+        else:
+            st = lib.fpq_gemm_mxf4_packed(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
+                                          alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
         _engine.check(st, "fpq_gemm_mxf4_packed")
         return y
     codes, scales = qa.row_major
     st = lib.fpq_gemm_mxf4(codes.data_ptr(), scales.data_ptr(), scales.shape[-1], wq.data_ptr(), ws.data_ptr(),
                            ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
     _engine.check(st, "fpq_gemm_mxf4")
+    if residual is not None:
+        y += residual
     return y
 
 
 def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.Tensor, ws: torch.Tensor,
                 alpha: torch.Tensor, act_global_scale: torch.Tensor, bias: Optional[torch.Tensor],
-                nvfp4: bool, shared_source: Optional[torch.Tensor] = None) -> torch.Tensor:
+                nvfp4: bool, shared_source: Optional[torch.Tensor] = None,
+                residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Activation rotate+quantize and W4A4 GEMM of one linear with as little host work as possible:
     the eager (non-traced) body of FPQuantLinear.forward.  Same kernels and results as the
     fused_quantize_* and matmul_* operators; `x_flat` bf16 [M, K] contiguous on the GPU, `alpha`
@@ -238,7 +253,8 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
     dev = x_flat.device
     if torch.cuda.current_device() != dev.index:
         with torch.cuda.device(dev):
-            return linear_w4a4(x_flat, hadamard_matrix, wq, ws, alpha, act_global_scale, bias, nvfp4, shared_source)
+            return linear_w4a4(x_flat, hadamard_matrix, wq, ws, alpha, act_global_scale, bias, nvfp4, shared_source,
+                               residual)
     stream = _current_stream(dev.index)
     h = as_bf16(hadamard_matrix)
     kind, norm = classify_rotation(h)
@@ -253,7 +269,7 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
         qa = quantize_activations(x_flat, h, kind, norm, act_global_scale, nvfp4, stream, want_packed)
         if key is not None:
             _publish(qa, shared_source, key, h)
-    return linear_on(qa, wq, ws, alpha, bias, stream, want_packed)
+    return linear_on(qa, wq, ws, alpha, bias, stream, want_packed, residual)
 
 
 ### Quantizers fused with the producer of their input

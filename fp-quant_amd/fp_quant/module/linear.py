@@ -6,6 +6,8 @@ inference branch of `forward()` of the reference module
 the reference work unchanged.  Training branches (master weights, quantized backward) and
 pseudo-quantization are not part of this engine and raise.
 """
+from typing import Optional
+
 import torch
 from torch import nn
 
@@ -137,6 +139,11 @@ class FPQuantLinear(nn.Module):
         self.weight = None
         self.dqweight = None
 
+    # A tensor of the output's shape that the next forward adds to its result (inside the GEMM
+    # where the kernel can) and then clears; set by a fused decoder block around its attention call.
+    # It stays set when the forward cannot take it (autograd), and the block then adds it itself.
+    _fpq_residual: Optional[torch.Tensor] = None
+
     def forward(self, x) -> torch.Tensor:
         cfg = self.config
         if (
@@ -148,6 +155,12 @@ class FPQuantLinear(nn.Module):
             # no autograd graph to build (inference): call the forward directly
             fn = (FPQuant4x16NoMasterFn.apply if (torch.is_grad_enabled() and x.requires_grad)
                   else _no_master_forward)
+            extra = ()
+            residual = self._fpq_residual
+            if (residual is not None and fn is _no_master_forward and not residual.requires_grad
+                    and residual.shape[:-1] == x.shape[:-1] and residual.shape[-1] == self.out_features):
+                self._fpq_residual = None
+                extra = (residual,)
             return fn(
                 x,
                 self.qweight,
@@ -158,6 +171,7 @@ class FPQuantLinear(nn.Module):
                 self.forward_hadamard_matrix,
                 cfg.forward_dtype,
                 cfg.forward_method,
+                *extra,
             )
         raise ValueError(
             f"Forward dtype: {cfg.forward_dtype}, backward dtype: {cfg.backward_dtype}, "
@@ -165,16 +179,22 @@ class FPQuantLinear(nn.Module):
             f"{cfg.pseudoquantization} isn't supported yet."
         )
 
-    def forward_quantized(self, activations, leading_shape) -> torch.Tensor:
+    def forward_quantized(self, activations, leading_shape, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
         """The GEMM (+ bias) of `forward` on activations that a fused producer has already rotated and
-        quantized for this layer (`eager.QuantizedActivations`); returns [*leading_shape, out]."""
+        quantized for this layer (`eager.QuantizedActivations`); returns [*leading_shape, out].
+        `residual` ([*leading_shape, out], bf16) is added to the result as a separate bf16 addition
+        would add it, inside the GEMM where the kernel can."""
         alpha = eager.linear_alpha(self.weight_global_scale, self.act_global_scale)
         bias = self.bias
         fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16 and bias.is_contiguous()) else None
+        in_gemm = residual is not None and (bias is None or fused_bias is not None)
         with torch.cuda.device(self.qweight.device):
             y = eager.linear_on(activations, self.qweight, self.scales, alpha, fused_bias,
-                                  hip_ops._current_stream(self.qweight.device.index))
+                                  hip_ops._current_stream(self.qweight.device.index),
+                                  residual=residual.contiguous().flatten(end_dim=-2) if in_gemm else None)
         y = y.unflatten(dim=0, sizes=tuple(leading_shape))
         if bias is not None and fused_bias is None:
             y += bias
+        if residual is not None and not in_gemm:
+            y += residual
         return y

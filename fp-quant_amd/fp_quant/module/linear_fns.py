@@ -70,8 +70,12 @@ class FPQuant4x16NoMasterFn(Function):
         forward_hadamard_matrix: torch.Tensor,
         dtype: FPQuantDtype,
         forward_method: str,
+        residual: Optional[torch.Tensor] = None,
     ):
+        """`residual` (not in the reference's signature): a tensor of the output's shape added to
+        the result as a separate bf16 addition would, inside the GEMM where the kernel can."""
         x_flat = x.contiguous().flatten(end_dim=-2)
+        res_flat = residual.contiguous().flatten(end_dim=-2) if residual is not None else None
         if (not torch.compiler.is_compiling() and forward_method == "abs_max"
                 and dtype in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4)
                 and weight_q.is_contiguous() and weight_scales.is_contiguous()):
@@ -80,10 +84,13 @@ class FPQuant4x16NoMasterFn(Function):
             fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16 and bias.is_contiguous()) else None
             y = linear_w4a4(x_flat.to(torch.bfloat16), forward_hadamard_matrix, weight_q, weight_scales,
                             linear_alpha(weight_global_scale, act_global_scale), act_global_scale, fused_bias,
-                            dtype == FPQuantDtype.NVFP4, shared_source=x)
+                            dtype == FPQuantDtype.NVFP4, shared_source=x,
+                            residual=res_flat if (bias is None or fused_bias is not None) else None)
             y = y.unflatten(dim=0, sizes=x.shape[:-1])
             if bias is not None and fused_bias is None:
                 y += bias
+                if residual is not None:
+                    y += residual
             return y
         if (dtype == FPQuantDtype.MXFP4 and x_flat.is_cuda
                 and packed_linear_eligible(x_flat.shape[0], x_flat.shape[1], forward_method)):
@@ -95,6 +102,8 @@ class FPQuant4x16NoMasterFn(Function):
             y = y.unflatten(dim=0, sizes=x.shape[:-1])
             if bias is not None and fused_bias is None:
                 y += bias
+            if residual is not None:
+                y = y + residual
             return y
         x_q, x_scales, _ = forward_quantize(
             x_flat, forward_hadamard_matrix, act_global_scale, dtype, forward_method
@@ -106,6 +115,8 @@ class FPQuant4x16NoMasterFn(Function):
         y = y.unflatten(dim=0, sizes=x.shape[:-1])
         if bias is not None and fused_bias is None:
             y += bias
+        if residual is not None:
+            y = y + residual
         return y
 
     @staticmethod

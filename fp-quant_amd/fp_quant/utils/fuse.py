@@ -8,15 +8,21 @@ keep one activation quantizer per such group).  With those projections being FPQ
 * each RMSNorm computes its bf16 output and the rotated, quantized form of it in one kernel; the
   projections that are then called with that output find the quantized form and go straight to
   their GEMM;
-* the MLP quantizes bf16(silu(gate)) * up directly from `gate` and `up`, without writing the product.
+* the MLP quantizes bf16(silu(gate)) * up directly from `gate` and `up`, without writing the product;
+* the two `residual + hidden_states` additions of the block happen in the epilogues of the `o_proj`
+  and `down_proj` GEMMs (blocks whose forward is, statement for statement, the one of transformers'
+  LlamaDecoderLayer; others keep their additions).
 
 Results are those of the unfused modules with one bf16 rounding per PyTorch operator (normalise,
 scale by the weight; silu, multiply); parameters, buffers and state-dict keys are untouched.  Calls
 that cannot take the fused kernels (tracing, CPU tensors, other dtypes, training, rotations without
 a fused kernel) run the original forward.
 """
+import ast
+import inspect
+import textwrap
 import types
-from typing import Optional
+from typing import Dict, Optional
 
 import torch
 from torch import nn
@@ -92,9 +98,11 @@ def fuse_gated_mlp(mlp: nn.Module) -> bool:
         return True
     unfused = mlp.forward
 
-    def forward(self, x):
-        if not _fusable_call(x):
-            return unfused(x)
+    def forward(self, x, residual=None):
+        """`residual`: added to the result (a fused decoder block passes its skip connection)."""
+        if not _fusable_call(x) or (residual is not None and not _fusable_call(residual)):
+            y = unfused(x)
+            return y if residual is None else residual + y
         gate = self.gate_proj(x)
         up = self.up_proj(x)
         down = self.down_proj
@@ -103,17 +111,125 @@ def fuse_gated_mlp(mlp: nn.Module) -> bool:
                                           down.forward_hadamard_matrix, down.act_global_scale,
                                           down.config.forward_dtype == FPQuantDtype.NVFP4)
         if qa is None:
-            return down(self.act_fn(gate) * up)
-        return down.forward_quantized(qa, gate.shape[:-1])
+            y = down(self.act_fn(gate) * up)
+            return y if residual is None else residual + y
+        return down.forward_quantized(qa, gate.shape[:-1], residual)
 
     mlp._fpq_unfused_forward = unfused
     mlp.forward = types.MethodType(forward, mlp)
     return True
 
 
+# The decoder block forward whose additions fuse_residual_adds moves into the GEMMs, one entry per
+# statement as ast.unparse prints it; entry 2 (the attention call) is checked structurally.
+_BLOCK_STATEMENTS = (
+    "residual = hidden_states",
+    "hidden_states = self.input_layernorm(hidden_states)",
+    None,
+    "hidden_states = residual + hidden_states",
+    "residual = hidden_states",
+    "hidden_states = self.post_attention_layernorm(hidden_states)",
+    "hidden_states = self.mlp(hidden_states)",
+    "hidden_states = residual + hidden_states",
+    "return hidden_states",
+)
+
+
+def _attention_call_defaults(block: nn.Module) -> Optional[Dict[str, object]]:
+    """If the class's forward is exactly the statements above, with the attention called as
+    `hidden_states, _ = self.self_attn(hidden_states=hidden_states, <p>=<p> for every other
+    parameter p of forward, **kwargs)`: the defaults of those parameters.  None otherwise."""
+    fn = type(block).forward
+    try:
+        tree = ast.parse(textwrap.dedent(inspect.getsource(fn)))
+        params = inspect.signature(fn).parameters
+    except (OSError, TypeError, SyntaxError, ValueError):
+        return None
+    body = tree.body[0].body if tree.body and isinstance(tree.body[0], ast.FunctionDef) else []
+    if body and isinstance(body[0], ast.Expr) and isinstance(getattr(body[0], "value", None), ast.Constant):
+        body = body[1:]   # docstring
+    if len(body) != len(_BLOCK_STATEMENTS):
+        return None
+    for stmt, want in zip(body, _BLOCK_STATEMENTS):
+        if want is not None and ast.unparse(stmt) != want:
+            return None
+    call = body[2]
+    if not (isinstance(call, ast.Assign) and len(call.targets) == 1
+            and ast.unparse(call.targets[0]) in ("(hidden_states, _)", "hidden_states, _")
+            and isinstance(call.value, ast.Call) and ast.unparse(call.value.func) == "self.self_attn"
+            and not call.value.args):
+        return None
+    names = list(params)
+    if len(names) < 2 or names[0] != "self" or names[1] != "hidden_states":
+        return None
+    defaults: Dict[str, object] = {}
+    var_keyword = None
+    for name in names[2:]:
+        p = params[name]
+        if p.kind == inspect.Parameter.VAR_KEYWORD:
+            var_keyword = name
+        elif p.kind in (inspect.Parameter.POSITIONAL_OR_KEYWORD, inspect.Parameter.KEYWORD_ONLY) \
+                and p.default is not inspect.Parameter.empty:
+            defaults[name] = p.default
+        else:
+            return None
+    passed = {}
+    for kw in call.value.keywords:
+        if kw.arg is None:
+            if not (isinstance(kw.value, ast.Name) and kw.value.id == var_keyword):
+                return None
+            var_keyword = None
+        elif not (isinstance(kw.value, ast.Name) and kw.value.id == kw.arg):
+            return None
+        else:
+            passed[kw.arg] = True
+    if var_keyword is not None or set(passed) != set(defaults) | {"hidden_states"}:
+        return None
+    return defaults
+
+
+def fuse_residual_adds(block: nn.Module) -> bool:
+    """Move the two `residual + hidden_states` additions of a decoder block into the GEMMs of
+    `self_attn.o_proj` and `mlp.down_proj`.  Needs the MLP patched by fuse_gated_mlp, `o_proj` an
+    FPQuantLinear, and the block's forward to be the Llama one statement for statement (checked on
+    its source); False otherwise.  Each addition that a GEMM cannot take (small batches, NVFP4,
+    autograd) is done by PyTorch as before, so results do not depend on which path ran."""
+    mlp, attn = getattr(block, "mlp", None), getattr(block, "self_attn", None)
+    o_proj = getattr(attn, "o_proj", None)
+    if getattr(mlp, "_fpq_unfused_forward", None) is None or not _is_real_quant_linear(o_proj):
+        return False
+    if getattr(block, "_fpq_unfused_forward", None) is not None:
+        return True
+    if "forward" in vars(block):   # already patched by someone else
+        return False
+    defaults = _attention_call_defaults(block)
+    if defaults is None:
+        return False
+    unfused = block.forward
+
+    def forward(self, hidden_states, *args, **kwargs):
+        if args or not isinstance(hidden_states, torch.Tensor) or not _fusable_call(hidden_states):
+            return unfused(hidden_states, *args, **kwargs)
+        out_proj = self.self_attn.o_proj
+        normed = self.input_layernorm(hidden_states)
+        out_proj._fpq_residual = hidden_states
+        try:
+            attn_out, _ = self.self_attn(hidden_states=normed, **{**defaults, **kwargs})
+        finally:
+            pending = out_proj._fpq_residual
+            out_proj._fpq_residual = None
+        if pending is not None:   # o_proj did not take it
+            attn_out = hidden_states + attn_out
+        return self.mlp(self.post_attention_layernorm(attn_out), residual=attn_out)
+
+    block._fpq_unfused_forward = unfused
+    block.forward = types.MethodType(forward, block)
+    return True
+
+
 def fuse_producers(model: nn.Module) -> int:
-    """Apply fuse_rmsnorm / fuse_gated_mlp to every decoder block of `model` that has the Llama
-    layout (`input_layernorm`, `self_attn.q_proj`, `post_attention_layernorm`, `mlp.gate_proj`).
+    """Apply fuse_rmsnorm / fuse_gated_mlp / fuse_residual_adds to every decoder block of `model` that
+    has the Llama layout (`input_layernorm`, `self_attn.q_proj`, `post_attention_layernorm`, `mlp.gate_proj`).
     Call it after the linears have been replaced and quantized.  Returns the number of patches."""
     count = 0
     for block in model.modules():
@@ -123,6 +239,7 @@ def fuse_producers(model: nn.Module) -> int:
         count += int(fuse_rmsnorm(getattr(block, "input_layernorm", None), getattr(attn, "q_proj", None)))
         count += int(fuse_rmsnorm(getattr(block, "post_attention_layernorm", None), getattr(mlp, "gate_proj", None)))
         count += int(fuse_gated_mlp(mlp))
+        count += int(fuse_residual_adds(block))
     return count
 
 
@@ -131,5 +248,8 @@ def unfuse_producers(model: nn.Module) -> None:
     for module in model.modules():
         unfused: Optional[object] = getattr(module, "_fpq_unfused_forward", None)
         if unfused is not None:
-            module.forward = unfused
+            if getattr(unfused, "__func__", None) is type(module).forward:
+                vars(module).pop("forward", None)   # back to the class's method
+            else:
+                module.forward = unfused
             module._fpq_unfused_forward = None

@@ -217,6 +217,18 @@ int fpq_rotated_absmax(const void* x, int64_t rows, int64_t cols, int rot_kind, 
                        const void* h, float* amax, void* stream);
 
 /*
+ * fpq_gemm_mxf4_packed followed by the addition of a bf16 [M, N] tensor in the same kernel:
+ *   y = bf16(bf16(alpha * acc (+ bias)) + residual)   -- the rounding of a separate bf16 add.
+ * For the output projections of a decoder block, whose result the reference's models add to the
+ * residual stream right away (src/utils/llama_utils.py:60-71 computes the projection, the block
+ * adds).  `residual` may be `y` itself (every element is read before it is written).
+ */
+int fpq_gemm_mxf4_packed_residual(const void* xq_packed, const void* xs_packed, const void* wq_packed,
+                                  const void* ws_packed, const float* alpha, const void* bias,
+                                  const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                                  void* stream);
+
+/*
  * Test hook: E2M1 codes of n fp32 values exactly as the quantize kernels round them
  * (out[i] in 0..15, one byte per value).  Used to check the device rounding exhaustively.
  */

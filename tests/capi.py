@@ -96,16 +96,25 @@ def quantize_packed(x_bf16, rot="hadamard", g=128, norm=None, zero_policy=_engin
     return pc.cpu(), ps.cpu()
 
 
-def gemm_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=None):
-    """fpq_gemm_mxf4_packed on packed operands; bf16 [M, N] on the CPU."""
+def gemm_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=None, residual=None, in_place=False):
+    """fpq_gemm_mxf4_packed (with `residual`: fpq_gemm_mxf4_packed_residual, `in_place`: writing over
+    the residual tensor) on packed operands; bf16 [M, N] on the CPU."""
     lib = _engine.lib()
     xp, xsp, wp, wsp = (t.to("cuda").contiguous() for t in (xp, xsp, wp, wsp))
     y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     a = torch.tensor([alpha], dtype=torch.float32, device="cuda")
     b = bias.to("cuda").contiguous() if bias is not None else None
-    st = lib.fpq_gemm_mxf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(), a.data_ptr(),
-                                  b.data_ptr() if b is not None else None, y.data_ptr(), m, n, k,
-                                  torch.cuda.current_stream().cuda_stream)
+    bp = b.data_ptr() if b is not None else None
+    stream = torch.cuda.current_stream().cuda_stream
+    if residual is None:
+        st = lib.fpq_gemm_mxf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(), a.data_ptr(),
+                                      bp, y.data_ptr(), m, n, k, stream)
+    else:
+        r = residual.to("cuda").contiguous().clone()
+        if in_place:
+            y = r
+        st = lib.fpq_gemm_mxf4_packed_residual(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
+                                               a.data_ptr(), bp, r.data_ptr(), y.data_ptr(), m, n, k, stream)
     _engine.check(st, "fpq_gemm_mxf4_packed")
     torch.cuda.synchronize()
     return y.cpu()

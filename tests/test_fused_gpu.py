@@ -192,7 +192,7 @@ def test_fused_norm_and_mlp_match_the_oracle_composition(fmt, g, tokens):
         h = O.silu_mul(gate.cpu().view(-1, 512), up.cpu().view(-1, 512)).view(gate.shape).cuda()
         want_mlp = block.mlp.down_proj(h)
 
-        assert fuse_producers(model) == 6                     # two norms and one MLP per block
+        assert fuse_producers(model) == 8                     # two norms, the MLP, the additions per block
         assert sorted(model.state_dict()) == sorted(_tiny_llama(fmt, g).state_dict())
         eager._shared_activations.clear()
         y = block.input_layernorm(x)
@@ -223,7 +223,7 @@ def test_fused_llama_matches_unfused(fmt, g):
     with torch.no_grad():
         want = model(ids).logits.float()
         want1 = model(ids[:, :1]).logits.float()
-        assert fuse_producers(model) == 6
+        assert fuse_producers(model) == 8
         got = model(ids).logits.float()
         got1 = model(ids[:, :1]).logits.float()
     for a, b in ((got, want), (got1, want1)):
@@ -282,3 +282,65 @@ def test_fused_llama_in_inference_mode():
     with torch.inference_mode():
         got = model(ids).logits
     assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])
+@pytest.mark.parametrize("shape", [(2, 48), (1, 200), (2, 3)])
+def test_residual_adds_in_the_gemm_change_nothing(fmt, g, shape):
+    """Moving the block's two additions into the o_proj / down_proj GEMMs (or, where the GEMM cannot
+    take them, adding afterwards) gives bit for bit the block with PyTorch's additions."""
+    from fp_quant.utils import fuse
+    model = _tiny_llama(fmt, g, seed=7)
+    for block in model.model.layers:
+        assert fuse.fuse_rmsnorm(block.input_layernorm, block.self_attn.q_proj)
+        assert fuse.fuse_rmsnorm(block.post_attention_layernorm, block.mlp.gate_proj)
+        assert fuse.fuse_gated_mlp(block.mlp)
+    ids = torch.randint(0, 128, shape, generator=torch.Generator().manual_seed(4)).cuda()
+    with torch.no_grad():
+        want = model(ids, output_hidden_states=True)
+        want_tokens = model.generate(ids[:, :3], max_new_tokens=5, do_sample=False)
+        for block in model.model.layers:
+            assert fuse.fuse_residual_adds(block)
+        got = model(ids, output_hidden_states=True)
+        for a, b in zip(got.hidden_states, want.hidden_states):
+            assert torch.equal(a, b)
+        assert torch.equal(got.logits, want.logits)
+        assert all(b.self_attn.o_proj._fpq_residual is None for b in model.model.layers)
+        # generation (KV cache, one-token steps) takes the same tokens
+        assert torch.equal(model.generate(ids[:, :3], max_new_tokens=5, do_sample=False), want_tokens)
+        fuse.unfuse_producers(model)
+        assert all("forward" not in vars(b) for b in model.model.layers)
+        assert fuse.fuse_producers(model) == 8
+
+
+def test_pending_residual_of_a_linear():
+    """A tensor left in `_fpq_residual` is added by the next forward and cleared; a forward that
+    builds an autograd graph leaves it alone; a shape that does not fit is not taken."""
+    import fp_quant
+    torch.manual_seed(11)
+    lin = torch.nn.Linear(512, 384, bias=True, device="cuda", dtype=torch.bfloat16)
+    layer = fp_quant.FPQuantLinear(512, 384, bias=True, config=_cfg("mxfp4", 128), device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        layer.weight.copy_(lin.weight)
+        layer.bias.copy_(lin.bias)
+    layer.pre_forward()
+    for m in (4, 96):
+        x = torch.randn(m, 512, device="cuda", dtype=torch.bfloat16)
+        res = torch.randn(m, 384, device="cuda", dtype=torch.bfloat16)
+        with torch.no_grad():
+            plain = layer(x)
+            layer._fpq_residual = res
+            got = layer(x)
+            assert layer._fpq_residual is None
+            assert torch.equal(got, plain + res)
+            assert torch.equal(layer(x), plain)
+            layer._fpq_residual = res[:, :100]
+            assert torch.equal(layer(x), plain) and layer._fpq_residual is not None
+            layer._fpq_residual = None
+    # the fused block's forward falls back to the original one when a graph is being built
+    model = _tiny_llama("mxfp4", 128, seed=8)
+    from fp_quant.utils import fuse_producers
+    fuse_producers(model)
+    emb = torch.randn(1, 8, 256, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    with pytest.raises(NotImplementedError):
+        model(inputs_embeds=emb).logits.sum().backward()

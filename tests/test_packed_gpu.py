@@ -187,6 +187,28 @@ def test_gemm_nv_packed_matches_oracle(m, n, k, bias):
     assert exact > 0.97
 
 
+@pytest.mark.parametrize("m,n,k", [(32, 32, 256), (65, 100, 256), (300, 520, 768), (256, 4096, 512), (2048, 1024, 512)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_gemm_packed_residual_equals_gemm_then_add(m, n, k, bias):
+    """The residual epilogue is the separate bf16 addition, bit for bit, for every tile shape and at
+    ragged edges (N not a multiple of 8 takes the element-wise stores); also when written in place."""
+    g = torch.Generator().manual_seed(3 * m + n + k)
+    xq = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=g)
+    wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=g)
+    xs = torch.randint(118, 134, (m, k // 32), dtype=torch.uint8, generator=g)
+    ws = torch.randint(118, 134, (n, k // 32), dtype=torch.uint8, generator=g)
+    b = torch.randn(n, generator=g).to(torch.bfloat16) if bias else None
+    res = (torch.randn(m, n, generator=g) * 20).to(torch.bfloat16)
+    xp, xsp = pack_by_definition(xq, xs, k)
+    wp, wsp = pack_by_definition(wq, ws, k)
+    plain = capi.gemm_packed(xp, xsp, wp, wsp, m, n, k, 0.111328125, bias=b)
+    want = plain + res                                   # torch's bf16 add: one rounding of the fp32 sum
+    got = capi.gemm_packed(xp, xsp, wp, wsp, m, n, k, 0.111328125, bias=b, residual=res)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    got2 = capi.gemm_packed(xp, xsp, wp, wsp, m, n, k, 0.111328125, bias=b, residual=res, in_place=True)
+    assert torch.equal(got2.view(torch.int16), want.view(torch.int16))
+
+
 @pytest.mark.parametrize("rot,g", [("hadamard", 16), ("hadamard", 32), ("hadamard", 64), ("hadamard", 128),
                                    ("identity", 16), ("gsr", 32)])
 @pytest.mark.parametrize("policy", [0, 1])
