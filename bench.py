@@ -319,7 +319,7 @@ def bench_mfma_ceiling(torch, seed=4, iters=192):
 
 
 def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=(1, 32, 64), decode_steps=8,
-                    fmt="mxfp4"):
+                    fmt="mxfp4", compiled_decode=False):
     """Forward passes of a random-weight Llama-3.1-8B-architecture model (transformers' LlamaForCausalLM) whose
     linears (all but lm_head) were replaced by MXFP4 FPQuantLinear with Hadamard-128: prefill tokens/s, decode
     tokens/s against a `seq`-token bf16 KV cache, and the share of GPU time spent inside the quantized linears
@@ -439,6 +439,8 @@ def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=
 
     measure(out, True)
     mx_ms = prefill_sweep()
+    if compiled_decode:
+        out["decode_compiled"] = compiled_decode_ms(torch, model, cfg, seq, decode_batches, decode_steps, gen)
     # the same model with the RMSNorms and the SiLU*up of every block fused into the quantizers that consume
     # them (one fused kernel instead of PyTorch's elementwise operators followed by a quantizer)
     from fp_quant.utils import fuse_producers
@@ -450,6 +452,41 @@ def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=
                                "speedup_vs_bf16": {k: round(bf16_ms[k] / mx_ms[k], 2) for k in bf16_ms},
                                "speedup_vs_bf16_fused": {k: round(bf16_ms[k] / fused_ms[k], 2) for k in bf16_ms}}
     return out
+
+
+def compiled_decode_ms(torch, model, cfg, seq, batches, steps, gen):
+    """Decode the way the reference's README recommends for speed (README.md:39): the model's forward under
+    torch.compile(mode="reduce-overhead", fullgraph=True), i.e. replayed as one HIP graph per step, over
+    transformers' StaticCache holding `seq` tokens.  The quantize / GEMM operators enter the graph as
+    custom operators; the prefill stays eager."""
+    from transformers import StaticCache
+    dev = torch.device("cuda:0")
+    res = {}
+    with torch.no_grad():
+        for b in batches:
+            ids = torch.randint(0, cfg.vocab_size, (b, seq), generator=gen).to(dev)
+            tok = torch.randint(0, cfg.vocab_size, (b, 1), generator=gen).to(dev)
+            cache = StaticCache(config=cfg, max_cache_len=seq + 4 * steps + 16)
+            model(input_ids=ids, past_key_values=cache, use_cache=True, logits_to_keep=1)
+            torch._dynamo.reset()
+            fwd = torch.compile(model.forward, mode="reduce-overhead", fullgraph=True)
+            for _ in range(4):                       # compile, graph warm-up, capture, first replay
+                fwd(input_ids=tok, past_key_values=cache, use_cache=True)
+            best = None
+            for _ in range(2):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    fwd(input_ids=tok, past_key_values=cache, use_cache=True)
+                torch.cuda.synchronize()
+                ms = (time.perf_counter() - t0) * 1e3 / steps
+                best = ms if best is None else min(best, ms)
+            res[f"batch{b}"] = {"kv_tokens": seq, "ms_per_step": round(best, 3),
+                                "tokens_per_s": round(b / (best * 1e-3), 1)}
+            del cache, fwd
+            torch._dynamo.reset()
+            torch.cuda.empty_cache()
+    return res
 
 
 def cpu_baseline_quantize(torch, fmt, rows, cols, g, seed, sample_rows):
@@ -523,6 +560,8 @@ def main():
                     "forward); the last four are not part of the default run")
     ap.add_argument("--e2e-layers", type=int, default=32, help="decoder layers of the --only e2e_llama model")
     ap.add_argument("--e2e-format", default="mxfp4", choices=("mxfp4", "nvfp4"), help="format of the --only e2e_llama model")
+    ap.add_argument("--e2e-compiled-decode", action="store_true",
+                    help="--only e2e_llama: also time decode under torch.compile(mode='reduce-overhead') with a static cache")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB device copy (known traffic) to scale rocprofv3 byte counters")
     args = ap.parse_args()
@@ -561,7 +600,8 @@ def main():
             out["nvfp4_linear"] = bench_linear(torch, "nvfp4", 4096, 24576, 4096, 16, max(10, args.steps // 10),
                                                max(2, args.warmup // 10), seed=3)
         if "e2e_llama" in only:
-            out["e2e_llama"] = bench_e2e_llama(torch, layers=args.e2e_layers, fmt=args.e2e_format)
+            out["e2e_llama"] = bench_e2e_llama(torch, layers=args.e2e_layers, fmt=args.e2e_format,
+                                               compiled_decode=args.e2e_compiled_decode)
         if "mfma_ceiling" in only:
             out["mfma_ceiling"] = bench_mfma_ceiling(torch)
         if "hbm_probe" in only:

@@ -27,36 +27,42 @@ from .hip_ops import (
     pack_nvf4,
     packed_linear_eligible,
     packed_weight,
+    packed_weight_ready,
     quantize_mx_packed,
 )
 
 
-def cached_on(t: torch.Tensor, slot: str, key, make):
-    """`make()` remembered on tensor `t` under attribute `slot` while `key` stays the same."""
+def cached_on(t: torch.Tensor, slot: str, key, make, remember: bool = True):
+    """`make()` remembered on tensor `t` under attribute `slot` while `key` stays the same.
+    `remember=False` uses what is remembered but stores nothing new: for callers that may be running
+    inside a compiler's graph memory pool, where a tensor that outlives the call is an error."""
     hit = getattr(t, slot, None)
     if hit is not None and hit[0] == key:
         return hit[1]
     val = make()
-    try:
-        setattr(t, slot, (key, val))
-    except (AttributeError, RuntimeError):
-        pass
+    if remember:
+        try:
+            setattr(t, slot, (key, val))
+        except (AttributeError, RuntimeError):
+            pass
     return val
 
 
-def linear_alpha(weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor) -> torch.Tensor:
+def linear_alpha(weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor,
+                 remember: bool = True) -> torch.Tensor:
     """fp32 one-element `1 / (wgs * ags)` evaluated in the buffers' dtype as the reference does
     (linear_fns.py:505; bf16 buffers round 1/9 to 0.111328125), cached until a buffer changes."""
     key = (_version(weight_global_scale), _version(act_global_scale), act_global_scale.data_ptr(),
            weight_global_scale.data_ptr())
     return cached_on(weight_global_scale, "_fpq_alpha", key,
-                     lambda: (1.0 / (weight_global_scale * act_global_scale)).float().reshape(1).contiguous())
+                     lambda: (1.0 / (weight_global_scale * act_global_scale)).float().reshape(1).contiguous(),
+                     remember)
 
 
-def as_f32_scalar(t: torch.Tensor) -> torch.Tensor:
+def as_f32_scalar(t: torch.Tensor, remember: bool = True) -> torch.Tensor:
     if t.dtype == torch.float32 and t.is_contiguous():
         return t
-    return cached_on(t, "_fpq_f32", (_version(t), t.data_ptr()), lambda: t.detach().float().contiguous())
+    return cached_on(t, "_fpq_f32", (_version(t), t.data_ptr()), lambda: t.detach().float().contiguous(), remember)
 
 
 # Several layers that consume one tensor (q/k/v projections, gate/up projections) would rotate and
@@ -64,9 +70,11 @@ def as_f32_scalar(t: torch.Tensor) -> torch.Tensor:
 # while the next call passes the very same tensor object, unmodified (its version counter), with an
 # equal rotation and global scale, on the same stream and in the same graph capture (or both outside
 # any: work recorded during a capture has not run when the capture ends).  The source is held weakly,
-# so a freed tensor whose address is reused can never match.  Producers fused with the quantizer
-# (rmsnorm_quantize, silu_mul_quantize) leave their result in the same slot for the layers that
-# follow.  FPQ_SHARE_ACT_QUANT=0 turns the sharing off.
+# so a freed tensor whose address is reused can never match, and the entry goes away with it.
+# Producers fused with the quantizer (rmsnorm_quantize, silu_mul_quantize) leave their result in the
+# same slot for the layers that follow.  The version counter only sees writes made through PyTorch:
+# compiled callers (whose generated kernels overwrite reused buffers behind it) never share, and a
+# stack that updates activations in place with raw-pointer kernels must set FPQ_SHARE_ACT_QUANT=0.
 SHARE_ACT_QUANT = os.environ.get("FPQ_SHARE_ACT_QUANT", "1") != "0"
 
 
@@ -118,8 +126,17 @@ def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: i
 
 
 def _publish(qa: QuantizedActivations, src: torch.Tensor, key, keep) -> None:
-    qa.ref, qa.version, qa.key, qa.keep = weakref.ref(src), _version(src), key, keep
-    _shared_activations[src.device.index] = qa
+    dev = src.device.index
+
+    def source_died(ref, dev=dev):
+        # nobody can ask for this tensor's quantized form any more: give the memory back now (a graph
+        # capture's memory pool must hold nothing but the captured step's outputs when it ends)
+        slot = _shared_activations.get(dev)
+        if slot is not None and slot.ref is ref:
+            del _shared_activations[dev]
+
+    qa.ref, qa.version, qa.key, qa.keep = weakref.ref(src, source_died), _version(src), key, keep
+    _shared_activations[dev] = qa
 
 
 def _lookup(src: torch.Tensor, key, want_packed: bool) -> Optional[QuantizedActivations]:
@@ -132,7 +149,7 @@ def _lookup(src: torch.Tensor, key, want_packed: bool) -> Optional[QuantizedActi
 
 def quantize_activations(x_flat: torch.Tensor, h: torch.Tensor, kind: int, norm: float,
                          act_global_scale: Optional[torch.Tensor], nvfp4: bool, stream: int,
-                         want_packed: bool) -> QuantizedActivations:
+                         want_packed: bool, remember: bool = True) -> QuantizedActivations:
     """Rotate and quantize bf16 [m, k]: MXFP4 straight into the packed layout when the packed GEMM will
     run, row-major otherwise (NVFP4 always; its packed form is made on demand)."""
     lib = _engine.lib()
@@ -154,7 +171,7 @@ def quantize_activations(x_flat: torch.Tensor, h: torch.Tensor, kind: int, norm:
     if nvfp4 and want_packed:
         pc = torch.empty(lib.fpq_packed_codes_bytes(m, k), dtype=torch.uint8, device=dev)
         ps = torch.empty(lib.fpq_packed_scales_bytes_nv(m, k), dtype=torch.uint8, device=dev)
-        gs = as_f32_scalar(act_global_scale)
+        gs = as_f32_scalar(act_global_scale, remember)
         st = lib.fpq_quantize_nv_packed(x_flat.data_ptr(), m, k, kind, g, norm, gs.data_ptr(), pc.data_ptr(),
                                         ps.data_ptr(), ZERO_NIBBLE_POLICY, stream)
         if st != _engine.E_UNSUPPORTED:
@@ -165,7 +182,7 @@ def quantize_activations(x_flat: torch.Tensor, h: torch.Tensor, kind: int, norm:
     codes = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
     scales = torch.empty(m, k // group, dtype=torch.uint8, device=dev)
     if nvfp4:
-        gs = as_f32_scalar(act_global_scale)
+        gs = as_f32_scalar(act_global_scale, remember)
         st = lib.fpq_quantize_nv(x_flat.data_ptr(), m, k, kind, g, norm, h.data_ptr(), gs.data_ptr(),
                                  codes.data_ptr(), scales.data_ptr(), m, k // group, ZERO_NIBBLE_POLICY, stream)
         _engine.check(st, "fpq_quantize_nv")
@@ -242,7 +259,7 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
 def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.Tensor, ws: torch.Tensor,
                 alpha: torch.Tensor, act_global_scale: torch.Tensor, bias: Optional[torch.Tensor],
                 nvfp4: bool, shared_source: Optional[torch.Tensor] = None,
-                residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+                residual: Optional[torch.Tensor] = None, remember: bool = True) -> torch.Tensor:
     """Activation rotate+quantize and W4A4 GEMM of one linear with as little host work as possible:
     the eager (non-traced) body of FPQuantLinear.forward.  Same kernels and results as the
     fused_quantize_* and matmul_* operators; `x_flat` bf16 [M, K] contiguous on the GPU, `alpha`
@@ -254,22 +271,66 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
     if torch.cuda.current_device() != dev.index:
         with torch.cuda.device(dev):
             return linear_w4a4(x_flat, hadamard_matrix, wq, ws, alpha, act_global_scale, bias, nvfp4, shared_source,
-                               residual)
+                               residual, remember)
     stream = _current_stream(dev.index)
     h = as_bf16(hadamard_matrix)
     kind, norm = classify_rotation(h)
     m, k = x_flat.shape
     want_packed = wants_packed(m, wq.shape[0], k, nvfp4)
+    if want_packed and not remember and not packed_weight_ready(wq, ws, nvfp4):
+        want_packed = False   # no packed copy of the weight yet and none may be kept: row-major kernels
     qa = key = None
     if shared_source is not None:
         key = _sharing_key(x_flat.shape, h, kind, norm, act_global_scale if nvfp4 else None, stream)
         if key is not None:
             qa = _lookup(shared_source, key, want_packed)
-    if qa is None:
-        qa = quantize_activations(x_flat, h, kind, norm, act_global_scale, nvfp4, stream, want_packed)
+    if qa is not None:
+        if nvfp4:
+            as_f32_scalar(act_global_scale)   # remembered now: a later traced call must not have to create it
+    else:
+        qa = quantize_activations(x_flat, h, kind, norm, act_global_scale, nvfp4, stream, want_packed, remember)
         if key is not None:
             _publish(qa, shared_source, key, h)
     return linear_on(qa, wq, ws, alpha, bias, stream, want_packed, residual)
+
+
+@torch.library.custom_op("fp_quant::linear_w4a4_op", mutates_args=())
+def linear_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.Tensor, ws: torch.Tensor,
+                   weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor,
+                   bias: Optional[torch.Tensor], nvfp4: bool) -> torch.Tensor:
+    """The whole abs-max forward of one layer as ONE operator, for traced callers (torch.compile):
+    inside it runs exactly what an eager call runs (linear_w4a4: cached alpha, packed or row-major
+    kernels by shape; no sharing of quantized activations between layers), so a compiled model gives the eager model's
+    bits and a captured step holds two kernels per layer instead of the reference's operator chain
+    (quantize, four tiny kernels for alpha, GEMM; linear_fns.py:496-514).  The global scales are read
+    when the operator runs; a HIP graph recorded around it replays the alpha it was recorded with."""
+    x = x_flat if x_flat.is_contiguous() else x_flat.contiguous()
+    if x.dtype != torch.bfloat16 or x.dim() != 2:
+        raise ValueError("x_flat must be a 2-D bfloat16 tensor")
+    if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_contiguous()):
+        raise ValueError("bias must be a contiguous bfloat16 vector")
+    # Nothing created here may outlive the call (the compiler may be running it inside its graph
+    # memory pool): what `prime` or eager calls have remembered is used, nothing new is remembered.
+    # No shared_source: compiler-generated kernels rewrite reused buffers without touching the
+    # version counter that sharing relies on.
+    alpha = linear_alpha(weight_global_scale, act_global_scale, remember=False)
+    return linear_w4a4(x, hadamard_matrix, wq.contiguous(), ws.contiguous(), alpha, act_global_scale, bias, nvfp4,
+                       remember=False)
+
+
+def prime(hadamard_matrix: torch.Tensor, weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor) -> None:
+    """Compute and remember a layer's per-call constants (rotation kind, alpha, fp32 global scale) now,
+    in ordinary memory: afterwards neither a traced call nor a graph capture has to create them."""
+    if not weight_global_scale.is_cuda or hadamard_matrix.device != weight_global_scale.device:
+        return
+    classify_rotation(as_bf16(hadamard_matrix))
+    linear_alpha(weight_global_scale, act_global_scale)
+    as_f32_scalar(act_global_scale)
+
+
+@linear_w4a4_op.register_fake
+def _(x_flat, hadamard_matrix, wq, ws, weight_global_scale, act_global_scale, bias, nvfp4):
+    return x_flat.new_empty((x_flat.shape[0], wq.shape[0]), dtype=torch.bfloat16)
 
 
 ### Quantizers fused with the producer of their input

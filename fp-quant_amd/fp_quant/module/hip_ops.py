@@ -136,6 +136,20 @@ def packed_linear_eligible(rows: int, k: int, forward_method: str) -> bool:
     return forward_method == "abs_max" and rows >= PACKED_LINEAR_MIN_M and k % 256 == 0 and packed_weights_enabled()
 
 
+@torch.library.custom_op("fp_quant::linear_alpha_op", mutates_args=())
+def linear_alpha_op(weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor) -> torch.Tensor:
+    """fp32 [1]: `1 / (weight_global_scale * act_global_scale)` with the product and the reciprocal
+    each rounded to the buffers' dtype, as eager PyTorch evaluates the reference's expression
+    (linear_fns.py:505).  An operator so that a compiler cannot fuse the chain and drop the
+    intermediate roundings (bf16 buffers: 1/9 becomes 0.111328125, fused in fp32 it would not)."""
+    return (1.0 / (weight_global_scale * act_global_scale)).float().reshape(1)
+
+
+@linear_alpha_op.register_fake
+def _(weight_global_scale, act_global_scale):
+    return weight_global_scale.new_empty((1,), dtype=torch.float32)
+
+
 @torch.library.custom_op("fp_quant::linear_mxf4_packed_op", mutates_args=())
 def linear_mxf4_packed_op(
     x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, w: torch.Tensor, ws: torch.Tensor,
@@ -336,9 +350,19 @@ def nv_packed_eligible(m: int, n: int, k: int) -> bool:
             and ((m + 255) // 256) * ((n + 255) // 256) < 100)
 
 
+def _packed_weight_key(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool):
+    return (wq.data_ptr(), _version(wq), ws.data_ptr(), _version(ws), tuple(wq.shape), nvfp4)
+
+
+def packed_weight_ready(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False) -> bool:
+    """Whether packed_weight would find its cached copy."""
+    hit = getattr(wq, "_fpq_packed", None)
+    return hit is not None and hit[0] == _packed_weight_key(wq, ws, nvfp4)
+
+
 def packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """Packed copy of a weight, cached on the code tensor until either tensor is written to."""
-    key = (wq.data_ptr(), _version(wq), ws.data_ptr(), _version(ws), tuple(wq.shape), nvfp4)
+    key = _packed_weight_key(wq, ws, nvfp4)
     hit = getattr(wq, "_fpq_packed", None)
     if hit is not None and hit[0] == key:
         return hit[1], hit[2]

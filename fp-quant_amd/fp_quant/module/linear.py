@@ -91,6 +91,7 @@ class FPQuantLinear(nn.Module):
         g = config.hadamard_group_size
         self.register_buffer("forward_hadamard_matrix", torch.empty(g, g, **factory))
         self.register_buffer("backward_hadamard_matrix", torch.empty(g, g, **factory))
+        self.register_load_state_dict_post_hook(FPQuantLinear._prime)
 
     @torch.no_grad()
     def pre_forward(self):
@@ -138,6 +139,14 @@ class FPQuantLinear(nn.Module):
         self.scales = nn.Parameter(scales, requires_grad=False)
         self.weight = None
         self.dqweight = None
+        self._prime()
+
+    def _prime(self, *_):
+        """Per-call constants (rotation kind, alpha, fp32 global scale) computed now rather than inside
+        the first forward, which may be a traced one or a graph capture; also run after load_state_dict."""
+        h, wgs, ags = self.forward_hadamard_matrix, self.weight_global_scale, self.act_global_scale
+        if all(isinstance(t, torch.Tensor) and t.is_cuda for t in (h, wgs, ags)):
+            eager.prime(h, wgs, ags)
 
     # A tensor of the output's shape that the next forward adds to its result (inside the GEMM
     # where the kernel can) and then clears; set by a fused decoder block around its attention call.

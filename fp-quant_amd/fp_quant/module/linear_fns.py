@@ -14,6 +14,7 @@ from .hip_ops import (
     as_bf16,
     fused_quantize_mx_op,
     fused_quantize_nv_op,
+    linear_alpha_op,
     matmul_mxf4_bf16_tn_bias_op,
     matmul_mxf4_bf16_tn_op,
     matmul_nvf4_bf16_tn_bias_op,
@@ -21,7 +22,7 @@ from .hip_ops import (
     linear_mxf4_packed_op,
     packed_linear_eligible,
 )
-from .eager import linear_alpha, linear_w4a4
+from .eager import linear_alpha, linear_w4a4, linear_w4a4_op
 
 
 def forward_quantize(
@@ -92,13 +93,25 @@ class FPQuant4x16NoMasterFn(Function):
                 if residual is not None:
                     y += residual
             return y
+        if (forward_method == "abs_max" and dtype in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4) and x_flat.is_cuda
+                and weight_q.is_contiguous() and weight_scales.is_contiguous()):
+            # traced callers: the eager body above as one operator
+            fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16 and bias.is_contiguous()) else None
+            y = linear_w4a4_op(x_flat.to(torch.bfloat16), forward_hadamard_matrix, weight_q, weight_scales,
+                               weight_global_scale, act_global_scale, fused_bias, dtype == FPQuantDtype.NVFP4)
+            y = y.unflatten(dim=0, sizes=x.shape[:-1])
+            if bias is not None and fused_bias is None:
+                y += bias
+            if residual is not None:
+                y = y + residual
+            return y
         if (dtype == FPQuantDtype.MXFP4 and x_flat.is_cuda
                 and packed_linear_eligible(x_flat.shape[0], x_flat.shape[1], forward_method)):
             # large batches: quantize and multiply on operands in the matrix units' own order
-            alpha = 1.0 / (weight_global_scale * act_global_scale)
+            alpha = linear_alpha_op(weight_global_scale, act_global_scale)
             fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16) else None
             y = linear_mxf4_packed_op(x_flat.to(torch.bfloat16), as_bf16(forward_hadamard_matrix), weight_q,
-                                      weight_scales, alpha.float(), fused_bias)
+                                      weight_scales, alpha, fused_bias)
             y = y.unflatten(dim=0, sizes=x.shape[:-1])
             if bias is not None and fused_bias is None:
                 y += bias
@@ -109,7 +122,7 @@ class FPQuant4x16NoMasterFn(Function):
             x_flat, forward_hadamard_matrix, act_global_scale, dtype, forward_method
         )
         # evaluated in the buffers' dtype, as the reference does (bf16 buffers round 1/9)
-        alpha = 1.0 / (weight_global_scale * act_global_scale)
+        alpha = linear_alpha_op(weight_global_scale, act_global_scale)
         fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16) else None
         y = forward_gemm(x_q, weight_q, x_scales, weight_scales, alpha, dtype, fused_bias)
         y = y.unflatten(dim=0, sizes=x.shape[:-1])

@@ -344,3 +344,35 @@ def test_pending_residual_of_a_linear():
     emb = torch.randn(1, 8, 256, device="cuda", dtype=torch.bfloat16, requires_grad=True)
     with pytest.raises(NotImplementedError):
         model(inputs_embeds=emb).logits.sum().backward()
+
+
+@pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])
+def test_compiled_static_cache_decode_matches_eager(fmt, g):
+    """The reference README's recipe for fast generation: model.forward under
+    torch.compile(mode="reduce-overhead", fullgraph=True) over a static KV cache, i.e. every decode step one
+    replayed HIP graph holding this library's operators.  With the compiler told to keep PyTorch's bf16
+    roundings between elementwise operators (emulate_precision_casts) the logits of every step equal the
+    eager model's bit for bit."""
+    import torch._inductor.config as inductor_config
+    from transformers import StaticCache
+    model = _tiny_llama(fmt, g, seed=9)
+    cfg = model.config
+    ids = torch.randint(0, 128, (2, 24), generator=torch.Generator().manual_seed(6)).cuda()
+    toks = torch.randint(0, 128, (5, 2, 1), generator=torch.Generator().manual_seed(7)).cuda()
+
+    def fresh_cache():
+        cache = StaticCache(config=cfg, max_cache_len=64)
+        model(input_ids=ids, past_key_values=cache, use_cache=True)
+        return cache
+
+    with torch.no_grad():
+        cache = fresh_cache()
+        want = [model(input_ids=t, past_key_values=cache, use_cache=True).logits.clone() for t in toks]
+        cache = fresh_cache()
+        torch._dynamo.reset()
+        with inductor_config.patch(emulate_precision_casts=True):
+            step = torch.compile(model.forward, mode="reduce-overhead", fullgraph=True)
+            got = [step(input_ids=t, past_key_values=cache, use_cache=True).logits.clone() for t in toks]
+    torch._dynamo.reset()
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert torch.equal(a, b), i

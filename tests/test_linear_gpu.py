@@ -161,6 +161,38 @@ def test_operators_have_fake_impls_and_compile():
     assert s0.shape == (128, 8) and s0.dtype == torch.float8_e8m0fnu
 
 
+@pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])
+def test_inductor_compiled_layers_match_eager(fmt, g):
+    """torch.compile(fullgraph=True) with the default (inductor) backend, which the reference's README
+    recommends for speed: chained layers, a residual addition, strided intermediates.  Every
+    elementwise step here is exact (relu, doubling, one addition), so compiled and eager outputs must
+    be bit-identical -- which also needs alpha to keep eager's bf16 roundings inside the compiled graph."""
+    import fp_quant
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up = nn.Linear(256, 512, bias=False)
+            self.down = nn.Linear(512, 256, bias=True)
+
+        def forward(self, x):
+            h = torch.relu(self.up(x)).view(x.shape[0], 4, 128).transpose(0, 1)
+            h = (h * 2.0).transpose(0, 1).reshape(x.shape[0], 512)      # reaches `down` through a strided view
+            return x + self.down(h)
+
+    torch.manual_seed(21)
+    net = Net().to(device="cuda", dtype=torch.bfloat16)
+    fp_quant.replace_quantize_with_fp_quant_linear(net, _cfg(fmt, g))
+    with torch.no_grad():
+        for rows in (1, 40, 300):       # split-K, packed 128x128 and packed-linear operator paths
+            x = torch.randn(rows, 256, device="cuda", dtype=torch.bfloat16)
+            want = net(x)
+            torch._dynamo.reset()
+            got = torch.compile(net, fullgraph=True)(x)
+            assert torch.equal(got, want), rows
+    torch._dynamo.reset()
+
+
 def test_unsupported_branches_raise():
     import fp_quant
     cfg = fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype.MXFP4, forward_method="abs_max",
