@@ -690,8 +690,8 @@ def main():
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline_linear(torch, 64, 14336, 4096, 128, seed=2)
-        line["cpu_baseline_quantize"] = cpu_baseline_quantize(torch, "nvfp4", 8192, 4096, 16, 1, 1024)
+        line["cpu_baseline"] = cpu_baseline_linear(torch, 2048, 14336, 4096, 128, seed=2)
+        line["cpu_baseline_quantize"] = cpu_baseline_quantize(torch, "nvfp4", 8192, 4096, 16, 1, 8192)
     print(json.dumps(line))
 
 
