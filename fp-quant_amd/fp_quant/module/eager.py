@@ -108,7 +108,7 @@ class QuantizedActivations:
 _shared_activations = {}   # device index -> QuantizedActivations of the latest call
 
 
-def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: int):
+def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: int, quest: bool = False):
     """What two calls must agree on, besides the source tensor, to share quantized activations, or
     None when nothing may be shared.  Layers own separate but equal rotation and global-scale
     buffers, so those are compared by value: (kind, norm, size) of a recognised rotation, the host
@@ -122,7 +122,7 @@ def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: i
     if act_global_scale is not None:
         gs = cached_on(act_global_scale, "_fpq_host", (_version(act_global_scale), act_global_scale.data_ptr()),
                        lambda: float(act_global_scale))
-    return (rot, gs, stream, capture_id.value, tuple(x_shape))
+    return (rot, gs, stream, capture_id.value, tuple(x_shape), quest)
 
 
 def _publish(qa: QuantizedActivations, src: torch.Tensor, key, keep) -> None:
@@ -149,7 +149,7 @@ def _lookup(src: torch.Tensor, key, want_packed: bool) -> Optional[QuantizedActi
 
 def quantize_activations(x_flat: torch.Tensor, h: torch.Tensor, kind: int, norm: float,
                          act_global_scale: Optional[torch.Tensor], nvfp4: bool, stream: int,
-                         want_packed: bool, remember: bool = True) -> QuantizedActivations:
+                         want_packed: bool, remember: bool = True, quest: bool = False) -> QuantizedActivations:
     """Rotate and quantize bf16 [m, k]: MXFP4 straight into the packed layout when the packed GEMM will
     run, row-major otherwise (NVFP4 always; its packed form is made on demand)."""
     lib = _engine.lib()
@@ -157,6 +157,15 @@ def quantize_activations(x_flat: torch.Tensor, h: torch.Tensor, kind: int, norm:
     dev = x_flat.device
     g = h.shape[0]
     qa = QuantizedActivations(m, k, nvfp4)
+    if quest:
+        # the quest rule (MXFP4) has a row-major kernel only; the packed form is made from it on demand
+        codes = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
+        scales = torch.empty(m, k // 32, dtype=torch.uint8, device=dev)
+        st = lib.fpq_quantize_mx_quest(x_flat.data_ptr(), m, k, kind, g, norm, h.data_ptr(), codes.data_ptr(),
+                                       scales.data_ptr(), m, k // 32, None, ZERO_NIBBLE_POLICY, stream)
+        _engine.check(st, "fpq_quantize_mx_quest")
+        qa.row_major = (codes, scales)
+        return qa
     if want_packed and not nvfp4:
         pc = torch.empty(lib.fpq_packed_codes_bytes(m, k), dtype=torch.uint8, device=dev)
         ps = torch.empty(lib.fpq_packed_scales_bytes(m, k), dtype=torch.uint8, device=dev)
@@ -259,7 +268,8 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
 def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.Tensor, ws: torch.Tensor,
                 alpha: torch.Tensor, act_global_scale: torch.Tensor, bias: Optional[torch.Tensor],
                 nvfp4: bool, shared_source: Optional[torch.Tensor] = None,
-                residual: Optional[torch.Tensor] = None, remember: bool = True) -> torch.Tensor:
+                residual: Optional[torch.Tensor] = None, remember: bool = True,
+                quest: bool = False) -> torch.Tensor:
     """Activation rotate+quantize and W4A4 GEMM of one linear with as little host work as possible:
     the eager (non-traced) body of FPQuantLinear.forward.  Same kernels and results as the
     fused_quantize_* and matmul_* operators; `x_flat` bf16 [M, K] contiguous on the GPU, `alpha`
@@ -271,7 +281,7 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
     if torch.cuda.current_device() != dev.index:
         with torch.cuda.device(dev):
             return linear_w4a4(x_flat, hadamard_matrix, wq, ws, alpha, act_global_scale, bias, nvfp4, shared_source,
-                               residual, remember)
+                               residual, remember, quest)
     stream = _current_stream(dev.index)
     h = as_bf16(hadamard_matrix)
     kind, norm = classify_rotation(h)
@@ -281,14 +291,15 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
         want_packed = False   # no packed copy of the weight yet and none may be kept: row-major kernels
     qa = key = None
     if shared_source is not None:
-        key = _sharing_key(x_flat.shape, h, kind, norm, act_global_scale if nvfp4 else None, stream)
+        key = _sharing_key(x_flat.shape, h, kind, norm, act_global_scale if nvfp4 else None, stream, quest)
         if key is not None:
             qa = _lookup(shared_source, key, want_packed)
     if qa is not None:
         if nvfp4:
             as_f32_scalar(act_global_scale)   # remembered now: a later traced call must not have to create it
     else:
-        qa = quantize_activations(x_flat, h, kind, norm, act_global_scale, nvfp4, stream, want_packed, remember)
+        qa = quantize_activations(x_flat, h, kind, norm, act_global_scale, nvfp4, stream, want_packed, remember,
+                                  quest)
         if key is not None:
             _publish(qa, shared_source, key, h)
     return linear_on(qa, wq, ws, alpha, bias, stream, want_packed, residual)
@@ -297,7 +308,7 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
 @torch.library.custom_op("fp_quant::linear_w4a4_op", mutates_args=())
 def linear_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.Tensor, ws: torch.Tensor,
                    weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor,
-                   bias: Optional[torch.Tensor], nvfp4: bool) -> torch.Tensor:
+                   bias: Optional[torch.Tensor], nvfp4: bool, quest: bool = False) -> torch.Tensor:
     """The whole abs-max forward of one layer as ONE operator, for traced callers (torch.compile):
     inside it runs exactly what an eager call runs (linear_w4a4: cached alpha, packed or row-major
     kernels by shape; no sharing of quantized activations between layers), so a compiled model gives the eager model's
@@ -315,7 +326,7 @@ def linear_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torc
     # version counter that sharing relies on.
     alpha = linear_alpha(weight_global_scale, act_global_scale, remember=False)
     return linear_w4a4(x, hadamard_matrix, wq.contiguous(), ws.contiguous(), alpha, act_global_scale, bias, nvfp4,
-                       remember=False)
+                       remember=False, quest=quest)
 
 
 def prime(hadamard_matrix: torch.Tensor, weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor) -> None:
@@ -329,7 +340,7 @@ def prime(hadamard_matrix: torch.Tensor, weight_global_scale: torch.Tensor, act_
 
 
 @linear_w4a4_op.register_fake
-def _(x_flat, hadamard_matrix, wq, ws, weight_global_scale, act_global_scale, bias, nvfp4):
+def _(x_flat, hadamard_matrix, wq, ws, weight_global_scale, act_global_scale, bias, nvfp4, quest=False):
     return x_flat.new_empty((x_flat.shape[0], wq.shape[0]), dtype=torch.bfloat16)
 
 

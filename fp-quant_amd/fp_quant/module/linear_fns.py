@@ -77,8 +77,10 @@ class FPQuant4x16NoMasterFn(Function):
         the result as a separate bf16 addition would, inside the GEMM where the kernel can."""
         x_flat = x.contiguous().flatten(end_dim=-2)
         res_flat = residual.contiguous().flatten(end_dim=-2) if residual is not None else None
-        if (not torch.compiler.is_compiling() and forward_method == "abs_max"
-                and dtype in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4)
+        # quest (MXFP4 only, validate_config) takes the same road when no clip mask is wanted
+        quest = forward_method == "quest" and dtype == FPQuantDtype.MXFP4 and not x.requires_grad
+        direct = ((forward_method == "abs_max" and dtype in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4)) or quest)
+        if (not torch.compiler.is_compiling() and direct
                 and weight_q.is_contiguous() and weight_scales.is_contiguous()):
             # eager calls: the same kernels as the operators below without two operator dispatches,
             # with alpha and the fp32 global scale computed once per layer instead of once per call
@@ -86,19 +88,18 @@ class FPQuant4x16NoMasterFn(Function):
             y = linear_w4a4(x_flat.to(torch.bfloat16), forward_hadamard_matrix, weight_q, weight_scales,
                             linear_alpha(weight_global_scale, act_global_scale), act_global_scale, fused_bias,
                             dtype == FPQuantDtype.NVFP4, shared_source=x,
-                            residual=res_flat if (bias is None or fused_bias is not None) else None)
+                            residual=res_flat if (bias is None or fused_bias is not None) else None, quest=quest)
             y = y.unflatten(dim=0, sizes=x.shape[:-1])
             if bias is not None and fused_bias is None:
                 y += bias
                 if residual is not None:
                     y += residual
             return y
-        if (forward_method == "abs_max" and dtype in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4) and x_flat.is_cuda
-                and weight_q.is_contiguous() and weight_scales.is_contiguous()):
+        if direct and x_flat.is_cuda and weight_q.is_contiguous() and weight_scales.is_contiguous():
             # traced callers: the eager body above as one operator
             fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16 and bias.is_contiguous()) else None
             y = linear_w4a4_op(x_flat.to(torch.bfloat16), forward_hadamard_matrix, weight_q, weight_scales,
-                               weight_global_scale, act_global_scale, fused_bias, dtype == FPQuantDtype.NVFP4)
+                               weight_global_scale, act_global_scale, fused_bias, dtype == FPQuantDtype.NVFP4, quest)
             y = y.unflatten(dim=0, sizes=x.shape[:-1])
             if bias is not None and fused_bias is None:
                 y += bias

@@ -82,3 +82,40 @@ def test_quest_operator_and_linear():
     assert ((y.double() - ref).abs() <= 2.0 ** -8 * ref.abs() + 1e-5 * mag).all()
     dense = x.cpu().double() @ w.double().T
     assert (y.double() - dense).norm() / dense.norm() < 0.3
+
+
+@pytest.mark.parametrize("m", [1, 30, 70, 300])
+def test_quest_module_equals_the_operator_chain(m):
+    """FPQuantLinear with forward_method="quest" (direct calls into the library, activations re-tiled
+    for the packed GEMM from 25 rows on) gives the bits of fused_quantize_mx_op followed by
+    matmul_mxf4_bf16_tn_op, eagerly, under torch.compile, and for layers sharing one input."""
+    import fp_quant
+    from fp_quant.module import hip_ops
+    cfg = fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype.MXFP4, forward_method="quest",
+                                 backward_dtype=fp_quant.FPQuantDtype.BF16, hadamard_group_size=128)
+    torch.manual_seed(31)
+    layers = []
+    for n in (192, 320):
+        lin = fp_quant.FPQuantLinear(512, n, cfg, bias=(n == 320), device="cuda", dtype=torch.bfloat16)
+        with torch.no_grad():
+            lin.weight.normal_(0, 0.05)
+            if lin.bias is not None:
+                lin.bias.normal_(0, 1)
+        lin.pre_forward()
+        layers.append(lin)
+    x = make_outlier_normal(m, 512, 9).cuda()
+    with torch.no_grad():
+        codes, scales, _ = hip_ops.fused_quantize_mx_op(x, layers[0].forward_hadamard_matrix, "quest", False)
+        alpha = torch.ones(1, dtype=torch.float32, device="cuda")
+        for lin in layers:                      # called one after the other with the same tensor: shared
+            want = hip_ops.matmul_mxf4_bf16_tn_op(codes, lin.qweight, scales, lin.scales.view(torch.float8_e8m0fnu), alpha)
+            if lin.bias is not None:
+                want = want + lin.bias
+            assert torch.equal(lin(x), want)
+            torch._dynamo.reset()
+            assert torch.equal(torch.compile(lin, fullgraph=True)(x), want)
+    torch._dynamo.reset()
+    # a forward that needs the clip mask (autograd) still goes through the operators and has no backward
+    xg = x.clone().requires_grad_(True)
+    with pytest.raises(NotImplementedError):
+        layers[0](xg).sum().backward()
