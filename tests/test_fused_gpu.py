@@ -376,3 +376,29 @@ def test_compiled_static_cache_decode_matches_eager(fmt, g):
     torch._dynamo.reset()
     for i, (a, b) in enumerate(zip(got, want)):
         assert torch.equal(a, b), i
+
+
+@pytest.mark.parametrize("arch", ["qwen3", "mistral"])
+def test_fuse_producers_on_other_llama_layout_models(arch):
+    """Qwen3 (the reference's headline family) and Mistral blocks have the Llama layout: every norm,
+    MLP and residual addition is patched, and the fused model follows the unfused one."""
+    import fp_quant
+    from fp_quant.utils import fuse_producers, unfuse_producers
+    if arch == "qwen3":
+        from transformers import Qwen3Config as Cfg, Qwen3ForCausalLM as Model
+    else:
+        from transformers import MistralConfig as Cfg, MistralForCausalLM as Model
+    torch.manual_seed(12)
+    cfg = Cfg(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+              num_key_value_heads=2, head_dim=64, vocab_size=128, max_position_embeddings=256)
+    model = Model(cfg).to(device="cuda", dtype=torch.bfloat16).eval()
+    fp_quant.replace_quantize_with_fp_quant_linear(model, _cfg("mxfp4", 128))
+    ids = torch.randint(0, 128, (2, 48), generator=torch.Generator().manual_seed(2)).cuda()
+    with torch.no_grad():
+        want = model(ids).logits.float()
+        assert fuse_producers(model) == 8
+        got = model(ids).logits.float()
+        assert float((got - want).norm() / want.norm()) < 0.02
+        assert model.generate(ids[:, :8], max_new_tokens=3, do_sample=False).shape == (2, 11)
+        unfuse_producers(model)
+        assert torch.equal(model(ids).logits.float(), want)
