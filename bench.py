@@ -275,6 +275,75 @@ def _time_linear(torch, run_linear, run_gemm, fmt, m, n, k, g, group, n_buf, ste
     }
 
 
+def bench_vendor_gemm(torch, steps, warmup, shapes=((2048, 14336, 4096), (8192, 14336, 4096), (8192, 4096, 14336))):
+    """The library GEMMs PyTorch-ROCm reaches (hipBLASLt) next to this repository's packed MXFP4 kernel, same
+    process, same shapes, operands of uniformly random codes (every kernel sees the same bytes): MXFP4 through
+    torch._scaled_mm (float4_e2m1fn_x2 operands, float8_e8m0fnu scales per 32), fp8 through torch._scaled_mm,
+    bf16 through F.linear.  Only timings are compared; the scale layouts the library kernels expect are not
+    reproduced, so their numerical results are not."""
+    from fp_quant import _engine
+    lib = _engine.lib()
+    dev = torch.device("cuda:0")
+
+    def timed(fn):
+        for _ in range(max(3, warmup)):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        best = None
+        for _ in range(3):
+            e0.record()
+            for _ in range(steps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / steps
+            best = us if best is None else min(best, us)
+        return best
+
+    out = {}
+    for m, n, k in shapes:
+        gen = torch.Generator(device=dev).manual_seed(m + n + k)
+        xq = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, device=dev, generator=gen)
+        wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev, generator=gen)
+        xs = torch.randint(118, 130, (m, k // 32), dtype=torch.uint8, device=dev, generator=gen)
+        ws = torch.randint(118, 130, (n, k // 32), dtype=torch.uint8, device=dev, generator=gen)
+        flops = 2.0 * m * n * k
+        res = {}
+        stream = torch.cuda.current_stream().cuda_stream
+        xp = torch.empty(lib.fpq_packed_codes_bytes(m, k), dtype=torch.uint8, device=dev)
+        xsp = torch.empty(lib.fpq_packed_scales_bytes(m, k), dtype=torch.uint8, device=dev)
+        wp = torch.empty(lib.fpq_packed_codes_bytes(n, k), dtype=torch.uint8, device=dev)
+        wsp = torch.empty(lib.fpq_packed_scales_bytes(n, k), dtype=torch.uint8, device=dev)
+        _engine.check(lib.fpq_pack_mxf4(xq.data_ptr(), xs.data_ptr(), k // 32, m, k, xp.data_ptr(), xsp.data_ptr(), stream), "pack")
+        _engine.check(lib.fpq_pack_mxf4(wq.data_ptr(), ws.data_ptr(), k // 32, n, k, wp.data_ptr(), wsp.data_ptr(), stream), "pack")
+        alpha = torch.tensor([1e-3], dtype=torch.float32, device=dev)
+        y = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+        us = timed(lambda: lib.fpq_gemm_mxf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
+                                                    alpha.data_ptr(), None, y.data_ptr(), m, n, k, stream))
+        res["this_repo_mxfp4_packed"] = {"us": round(us, 2), "TFLOP/s": round(flops / us / 1e6, 1)}
+        try:
+            a4, b4 = xq.view(torch.float4_e2m1fn_x2), wq.view(torch.float4_e2m1fn_x2)
+            sa, sb = xs.view(torch.float8_e8m0fnu), ws.view(torch.float8_e8m0fnu)
+            us = timed(lambda: torch._scaled_mm(a4, b4.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16))
+            res["hipblaslt_mxfp4_scaled_mm"] = {"us": round(us, 2), "TFLOP/s": round(flops / us / 1e6, 1)}
+        except Exception as e:   # not every PyTorch-ROCm build has the MXFP4 path
+            res["hipblaslt_mxfp4_scaled_mm"] = {"error": f"{type(e).__name__}: {str(e)[:160]}"}
+        xb = torch.randn(m, k, device=dev, dtype=torch.bfloat16, generator=gen)
+        wb = torch.randn(n, k, device=dev, dtype=torch.bfloat16, generator=gen)
+        try:
+            x8, w8 = xb.to(torch.float8_e4m3fn), wb.to(torch.float8_e4m3fn)
+            one = torch.ones((), device=dev)
+            us = timed(lambda: torch._scaled_mm(x8, w8.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16))
+            res["hipblaslt_fp8_scaled_mm"] = {"us": round(us, 2), "TFLOP/s": round(flops / us / 1e6, 1)}
+        except Exception as e:
+            res["hipblaslt_fp8_scaled_mm"] = {"error": f"{type(e).__name__}: {str(e)[:160]}"}
+        us = timed(lambda: torch.nn.functional.linear(xb, wb))
+        res["hipblaslt_bf16_linear"] = {"us": round(us, 2), "TFLOP/s": round(flops / us / 1e6, 1)}
+        out[f"M{m}_N{n}_K{k}"] = res
+    return out
+
+
 def bench_mfma_ceiling(torch, seed=4, iters=192):
     """Register-resident FP4 MFMA loop (no memory system): the matrix throughput and clock the chip
     sustains for all-zero operands and for operands with the bit statistics of quantized data, over
@@ -556,7 +625,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="comma list of workloads to run (for profiling one kernel): "
                     "nvfp4_quantize, mxfp4_quantize, mxfp4_linear_M2048, mxfp4_linear_M128, mxfp4_linear_M16, "
-                    "mxfp4_linear_M1, nvfp4_linear, mfma_ceiling, hbm_probe, fused_producers, e2e_llama (whole-model "
+                    "mxfp4_linear_M1, nvfp4_linear, mfma_ceiling, hbm_probe, vendor_gemm, fused_producers, e2e_llama (whole-model "
                     "forward); the last four are not part of the default run")
     ap.add_argument("--e2e-layers", type=int, default=32, help="decoder layers of the --only e2e_llama model")
     ap.add_argument("--e2e-format", default="mxfp4", choices=("mxfp4", "nvfp4"), help="format of the --only e2e_llama model")
@@ -606,6 +675,8 @@ def main():
             out["mfma_ceiling"] = bench_mfma_ceiling(torch)
         if "hbm_probe" in only:
             out["hbm_probe"] = bench_hbm_probe(torch, args.steps, args.warmup)
+        if "vendor_gemm" in only:
+            out["vendor_gemm"] = bench_vendor_gemm(torch, max(10, args.steps // 4), args.warmup)
         if "fused_producers" in only:
             out["fused_producers"] = bench_fused_producers(torch, args.steps, args.warmup)
         print(json.dumps({"only": only, "steps": args.steps, "results": out}))
