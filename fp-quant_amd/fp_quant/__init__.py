@@ -12,7 +12,7 @@ from .utils import (
     replace_with_fp_quant_linear,
 )
 
-__version__ = "0.1.0"
+__version__ = "0.3.2"   # the release of the reference package whose surface this mirrors (inference_lib/setup.py:5)
 __all__ = [
     "FPQuantLinear",
     "FPQuantConfig",
