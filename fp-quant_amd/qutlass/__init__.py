@@ -30,7 +30,7 @@ _spec = importlib.util.spec_from_file_location(
 _engine = importlib.util.module_from_spec(_spec)
 _spec.loader.exec_module(_engine)
 
-_ZERO_POLICY = 1 if os.environ.get("FPQ_ZERO_NIBBLE", "reference") == "signed" else 0
+_ZERO_POLICY = _engine.ZERO_REFERENCE   # every zero packs as 0x8, as the reference's exporter packs it
 _PACKED_MIN_M = 48   # from here on the MXFP4 GEMM runs on re-tiled operands (weights re-tiled once)
 
 
