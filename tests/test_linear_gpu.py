@@ -384,3 +384,47 @@ def test_inference_mode(fmt, g, m):
         inner.pre_forward()
         assert inner.qweight.is_inference()
         assert torch.equal(inner(x), want) and torch.equal(inner(x), want)
+
+
+def test_layers_called_from_two_threads_on_their_own_streams():
+    """Every call runs on the calling thread's current stream and shares nothing it should not:
+    two host threads, each with its own stream and inputs, calling the same layers concurrently,
+    get what a single thread gets."""
+    import threading
+    import fp_quant
+    torch.manual_seed(17)
+    lins = []
+    for fmt, g in (("mxfp4", 128), ("nvfp4", 16)):
+        lin = fp_quant.FPQuantLinear(512, 256, _cfg(fmt, g), bias=True, device="cuda", dtype=torch.bfloat16)
+        with torch.no_grad():
+            lin.weight.normal_(0, 0.05)
+            lin.bias.normal_(0, 1)
+        lin.pre_forward()
+        lins.append(lin)
+    inputs = [[torch.randn(m, 512, device="cuda", dtype=torch.bfloat16) for m in (1, 30, 70, 300)] for _ in range(2)]
+    with torch.no_grad():
+        want = [[[lin(x) for x in xs] for lin in lins] for xs in inputs]
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(t):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream), torch.no_grad():
+                for _ in range(25):
+                    for li, lin in enumerate(lins):
+                        for xi, x in enumerate(inputs[t]):
+                            y = lin(x)
+                            stream.synchronize()
+                            if not torch.equal(y, want[t][li][xi]):
+                                errors.append((t, li, xi))
+        except Exception as exc:   # surfaced below
+            errors.append(repr(exc))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=100)
+    assert not any(th.is_alive() for th in threads)
+    assert not errors, errors[:5]
