@@ -142,3 +142,39 @@ def test_config_dict_round_trip_and_scale_groups():
     assert "transform_init" not in export.quantization_config_dict(cfg)
     cfg.transform_init = "gsr"
     assert export.quantization_config_dict(cfg)["transform_init"] == "gsr"
+
+
+def test_everything_fails_loudly_without_the_library():
+    """No other backend exists: with the shared library missing, the loader, the module constructor
+    (the reference raises there when QuTLASS is absent, linear.py:57-60) and the qutlass stand-in all
+    raise instead of computing something else."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = r"""
+import sys
+sys.path.insert(0, sys.argv[1])
+import torch, fp_quant, qutlass
+from fp_quant import _engine
+assert not _engine.available()
+for what in ("loader", "module", "standin"):
+    try:
+        if what == "loader":
+            _engine.lib()
+        elif what == "module":
+            fp_quant.FPQuantLinear(64, 32, fp_quant.FPQuantConfig(forward_method="abs_max",
+                                   backward_dtype=fp_quant.FPQuantDtype.BF16), device="meta")
+        else:
+            qutlass._engine.lib()
+    except Exception as exc:
+        print(what, type(exc).__name__)
+    else:
+        print(what, "NO ERROR")
+"""
+    env = dict(os.environ, FPQ_LIBRARY_PATH="/nonexistent/libfpq_hip.so")
+    r = subprocess.run([sys.executable, "-c", code, os.path.join(root, "fp-quant_amd")], capture_output=True, text=True,
+                       env=env, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = dict(l.split(" ", 1) for l in r.stdout.strip().splitlines())
+    assert lines == {"loader": "FPQEngineError", "module": "ValueError", "standin": "FPQEngineError"}, r.stdout
