@@ -402,3 +402,35 @@ def test_fuse_producers_on_other_llama_layout_models(arch):
         assert model.generate(ids[:, :8], max_new_tokens=3, do_sample=False).shape == (2, 11)
         unfuse_producers(model)
         assert torch.equal(model(ids).logits.float(), want)
+
+
+@pytest.mark.parametrize("tokens", [4, 64])
+def test_fused_decoder_block_with_residual_epilogues_is_graph_capturable(tokens):
+    """The whole patched block (norm+quantize, attention, o_proj with the residual in its GEMM, fused MLP with
+    the residual in down_proj's GEMM) recorded into a HIP graph and replayed on new inputs."""
+    from fp_quant.utils import fuse_producers
+    model = _tiny_llama("mxfp4", 128, seed=13)
+    assert fuse_producers(model) == 8
+    block = model.model.layers[1]
+    pos = torch.arange(tokens, device="cuda").unsqueeze(0)
+    static_x = torch.randn(1, tokens, 256, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        emb = model.model.rotary_emb(static_x, position_ids=pos)
+
+        def step(x):
+            return block(x, position_embeddings=emb, attention_mask=None)
+
+        step(static_x)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_y = step(static_x)
+        for seed in range(3):
+            fresh = torch.randn(1, tokens, 256, device="cuda",
+                                generator=torch.Generator("cuda").manual_seed(seed)).to(torch.bfloat16)
+            want = step(fresh.clone())
+            static_x.copy_(fresh)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_y, want), seed
+    assert block.self_attn.o_proj._fpq_residual is None
