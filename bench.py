@@ -515,6 +515,8 @@ def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=
     from fp_quant.utils import fuse_producers
     fused = {"patched_modules": fuse_producers(model)}
     measure(fused, False)
+    if compiled_decode:   # the traced attention and MLP modules now call the group operators
+        fused["decode_compiled"] = compiled_decode_ms(torch, model, cfg, seq, decode_batches, decode_steps, gen)
     out["fused_producers"] = fused
     fused_ms = prefill_sweep()
     out["prefill_sweep_ms"] = {"bf16": bf16_ms, fmt: mx_ms, fmt + "_fused_producers": fused_ms,

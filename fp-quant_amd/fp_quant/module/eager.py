@@ -11,7 +11,7 @@
 import ctypes
 import os
 import weakref
-from typing import Optional, Tuple
+from typing import List, Optional, Tuple
 
 import torch
 
@@ -329,6 +329,79 @@ def linear_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torc
                        remember=False, quest=quest)
 
 
+# Traced callers, groups of layers.  A compiler cannot see that q/k/v (or gate/up) quantize the same
+# tensor, and the sharing slot is closed to it; these operators state the grouping instead.
+@torch.library.custom_op("fp_quant::linear_group_w4a4_op", mutates_args=())
+def linear_group_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wqs: List[torch.Tensor],
+                         wss: List[torch.Tensor], weight_global_scales: List[torch.Tensor],
+                         act_global_scales: List[torch.Tensor], biases: List[Optional[torch.Tensor]],
+                         nvfp4: bool) -> List[torch.Tensor]:
+    """Several layers on one input: the activations are rotated and quantized once (with the first
+    layer's rotation and activation scale, which the caller has checked to equal the others'), then
+    one GEMM per layer -- what consecutive eager calls do through the sharing slot."""
+    x = x_flat if x_flat.is_contiguous() else x_flat.contiguous()
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or not x.is_cuda:
+        raise ValueError("x_flat must be a 2-D bfloat16 tensor on a GPU")
+    n_layers = len(wqs)
+    if not (len(wss) == len(weight_global_scales) == len(act_global_scales) == len(biases) == n_layers) or not n_layers:
+        raise ValueError("one entry per layer is needed in every list")
+    dev = x.device
+    with torch.cuda.device(dev):
+        stream = _current_stream(dev.index)
+        h = as_bf16(hadamard_matrix)
+        kind, norm = classify_rotation(h)
+        m, k = x.shape
+        # a GEMM runs on packed operands where the shape calls for it and the packed weight exists
+        # already (nothing may be created and kept here); the activations are quantized straight into
+        # the packed layout only if every GEMM of the group wants them so (MXFP4), else row-major,
+        # from which the packed form is made on demand
+        packed = [wants_packed(m, wq.shape[0], k, nvfp4) and packed_weight_ready(wq, ws, nvfp4)
+                  for wq, ws in zip(wqs, wss)]
+        qa = quantize_activations(x, h, kind, norm, act_global_scales[0], nvfp4, stream,
+                                  all(packed) and not nvfp4, remember=False)
+        out = []
+        for i in range(n_layers):
+            bias = biases[i]
+            if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_contiguous()):
+                raise ValueError("bias must be a contiguous bfloat16 vector")
+            alpha = linear_alpha(weight_global_scales[i], act_global_scales[i], remember=False)
+            out.append(linear_on(qa, wqs[i].contiguous(), wss[i].contiguous(), alpha, bias, stream, packed[i]))
+    return out
+
+
+@linear_group_w4a4_op.register_fake
+def _(x_flat, hadamard_matrix, wqs, wss, weight_global_scales, act_global_scales, biases, nvfp4):
+    return [x_flat.new_empty((x_flat.shape[0], wq.shape[0]), dtype=torch.bfloat16) for wq in wqs]
+
+
+@torch.library.custom_op("fp_quant::silu_mul_linear_w4a4_op", mutates_args=())
+def silu_mul_linear_w4a4_op(gate: torch.Tensor, up: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.Tensor,
+                            ws: torch.Tensor, weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor,
+                            bias: Optional[torch.Tensor], nvfp4: bool) -> torch.Tensor:
+    """down(bf16(silu(gate)) * up) of a gated MLP: the product is quantized as it is formed
+    (silu_mul_quantize) and multiplied by the layer's weight; bf16 [m, n]."""
+    g2, u2 = gate.reshape(-1, gate.shape[-1]), up.reshape(-1, up.shape[-1])
+    wq, ws = wq.contiguous(), ws.contiguous()
+    # packed operands only where the packed weight exists already: nothing may be created and kept here
+    ready = packed_weight_ready(wq, ws, nvfp4)
+    qa = silu_mul_quantize(g2, u2, hadamard_matrix, act_global_scale, nvfp4, remember=False, allow_packed=ready)
+    if qa is None:
+        raise ValueError("no fused SiLU*up quantizer for these tensors (rotation, strides or alignment)")
+    if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_contiguous()):
+        raise ValueError("bias must be a contiguous bfloat16 vector")
+    dev = gate.device
+    with torch.cuda.device(dev):
+        alpha = linear_alpha(weight_global_scale, act_global_scale, remember=False)
+        use_packed = ready and wants_packed(qa.m, wq.shape[0], qa.k, nvfp4)
+        return linear_on(qa, wq, ws, alpha, bias, _current_stream(dev.index), use_packed)
+
+
+@silu_mul_linear_w4a4_op.register_fake
+def _(gate, up, hadamard_matrix, wq, ws, weight_global_scale, act_global_scale, bias, nvfp4):
+    rows = gate.numel() // gate.shape[-1]
+    return gate.new_empty((rows, wq.shape[0]), dtype=torch.bfloat16)
+
+
 def prime(hadamard_matrix: torch.Tensor, weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor) -> None:
     """Compute and remember a layer's per-call constants (rotation kind, alpha, fp32 global scale) now,
     in ordinary memory: afterwards neither a traced call nor a graph capture has to create them."""
@@ -349,13 +422,14 @@ def _(x_flat, hadamard_matrix, wq, ws, weight_global_scale, act_global_scale, bi
 
 def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tensor, kind: int, norm: float,
                     act_global_scale: Optional[torch.Tensor], nvfp4: bool, out: Optional[torch.Tensor],
-                    stream: int, dev) -> Optional[QuantizedActivations]:
+                    stream: int, dev, remember: bool = True,
+                    allow_packed: bool = True) -> Optional[QuantizedActivations]:
     """Common tail of the fused producers: allocate row-major codes/scales and call
     fpq_<entry>_quantize_{mx,nv}; None if the library has no fused kernel for this rotation."""
     lib = _engine.lib()
     group = 16 if nvfp4 else 32
     optr = out.data_ptr() if out is not None else None
-    want_packed = not nvfp4 and packed_linear_eligible(rows, cols, "abs_max")
+    want_packed = allow_packed and not nvfp4 and packed_linear_eligible(rows, cols, "abs_max")
     if want_packed:
         # straight into the operand layout of the packed GEMM (streaming kernel)
         pc = torch.empty(lib.fpq_packed_codes_bytes(rows, cols), dtype=torch.uint8, device=dev)
@@ -372,7 +446,7 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
     scales = torch.empty(rows, cols // group, dtype=torch.uint8, device=dev)
     tail = (optr, codes.data_ptr(), scales.data_ptr(), rows, cols // group, ZERO_NIBBLE_POLICY, stream)
     if nvfp4:
-        gs = as_f32_scalar(act_global_scale)
+        gs = as_f32_scalar(act_global_scale, remember)
         st = getattr(lib, f"fpq_{entry}_quantize_nv")(*head, rows, cols, kind, h.shape[0], norm, gs.data_ptr(), *tail)
     else:
         st = getattr(lib, f"fpq_{entry}_quantize_mx")(*head, rows, cols, kind, h.shape[0], norm, *tail)
@@ -421,7 +495,8 @@ def rmsnorm_quantize(x: torch.Tensor, weight: torch.Tensor, eps: float, hadamard
 
 
 def silu_mul_quantize(gate: torch.Tensor, up: torch.Tensor, hadamard_matrix: torch.Tensor,
-                      act_global_scale: Optional[torch.Tensor], nvfp4: bool) -> Optional[QuantizedActivations]:
+                      act_global_scale: Optional[torch.Tensor], nvfp4: bool,
+                      remember: bool = True, allow_packed: bool = True) -> Optional[QuantizedActivations]:
     """Quantized bf16(silu(gate)) * up without materialising the product; gate and up are bf16 with a
     contiguous last dimension (two tensors, or two column halves of one).  None if not fusable."""
     if (not gate.is_cuda or gate.dtype != torch.bfloat16 or up.dtype != torch.bfloat16 or gate.shape != up.shape
@@ -442,4 +517,4 @@ def silu_mul_quantize(gate: torch.Tensor, up: torch.Tensor, hadamard_matrix: tor
         if ld_g % 8 or ld_u % 8 or ld_g < cols or ld_u < cols or gate.data_ptr() % 16 or up.data_ptr() % 16:
             return None
         return _fused_quantize("silu_mul", (gate.data_ptr(), ld_g, up.data_ptr(), ld_u), rows, cols, h, kind, norm,
-                               act_global_scale, nvfp4, None, stream, dev)
+                               act_global_scale, nvfp4, None, stream, dev, remember, allow_packed)

@@ -13,6 +13,11 @@ keep one activation quantizer per such group).  With those projections being FPQ
   and `down_proj` GEMMs (blocks whose forward is, statement for statement, the one of transformers'
   LlamaDecoderLayer; others keep their additions).
 
+Under `torch.compile` the norms and additions are left to the compiler (it fuses them itself); what it
+cannot know is that q/k/v, and gate/up, quantize the same tensor: there the patched MLP and attention
+modules call group operators (one quantization, one GEMM per layer; SiLU*up fused into down_proj's
+quantizer), which a captured decode step replays as fewer kernels.
+
 Results are those of the unfused modules with one bf16 rounding per PyTorch operator (normalise,
 scale by the weight; silu, multiply); parameters, buffers and state-dict keys are untouched.  Calls
 that cannot take the fused kernels (tracing, CPU tensors, other dtypes, training, rotations without
@@ -50,6 +55,42 @@ def _is_real_quant_linear(layer) -> bool:
 def _fusable_call(x: torch.Tensor) -> bool:
     return (x.is_cuda and x.dtype == torch.bfloat16 and not torch.compiler.is_compiling()
             and not (torch.is_grad_enabled() and x.requires_grad))
+
+
+def _traceable_call(x: torch.Tensor) -> bool:
+    """A call being traced by a compiler that the group operators can serve."""
+    return (torch.compiler.is_compiling() and x.is_cuda and x.dtype == torch.bfloat16
+            and not (torch.is_grad_enabled() and x.requires_grad))
+
+
+def _quantize_alike(layers) -> bool:
+    """Whether these layers quantize an input identically (format, method, rotation, activation
+    scale), so that one quantization can serve them all, and take their bias inside the GEMM."""
+    first = layers[0]
+    for layer in layers:
+        a, b = first.config, layer.config
+        if (a.forward_dtype, a.forward_method, a.hadamard_group_size) != (b.forward_dtype, b.forward_method,
+                                                                          b.hadamard_group_size):
+            return False
+        if layer.in_features != first.in_features or layer.qweight.device != first.qweight.device:
+            return False
+        if not torch.equal(layer.forward_hadamard_matrix, first.forward_hadamard_matrix):
+            return False
+        if not torch.equal(layer.act_global_scale.float(), first.act_global_scale.float()):
+            return False
+        if layer.bias is not None and (layer.bias.dtype != torch.bfloat16 or not layer.bias.is_contiguous()):
+            return False
+    return True
+
+
+def _group_linear(layers, x: torch.Tensor):
+    """The outputs of `layers` on `x` from ONE operator (one quantization, one GEMM each)."""
+    first = layers[0]
+    outs = _eager().linear_group_w4a4_op(
+        x.reshape(-1, x.shape[-1]), first.forward_hadamard_matrix, [l.qweight for l in layers],
+        [l.scales for l in layers], [l.weight_global_scale for l in layers], [l.act_global_scale for l in layers],
+        [l.bias for l in layers], first.config.forward_dtype == FPQuantDtype.NVFP4)
+    return [o.view(*x.shape[:-1], o.shape[-1]) for o in outs]
 
 
 def _is_llama_rmsnorm(norm) -> bool:
@@ -97,9 +138,30 @@ def fuse_gated_mlp(mlp: nn.Module) -> bool:
     if getattr(mlp, "_fpq_unfused_forward", None) is not None:
         return True
     unfused = mlp.forward
+    down_proj = parts[2]
+    # what the traced form needs on top: gate/up quantize alike, a SiLU*up quantizer for down's rotation
+    traceable = False
+    if down_proj.forward_hadamard_matrix.is_cuda:
+        eager = _eager()
+        kind, _ = eager.classify_rotation(eager.as_bf16(down_proj.forward_hadamard_matrix))
+        g = down_proj.forward_hadamard_matrix.shape[0]
+        traceable = (_quantize_alike(parts[:2]) and kind in (eager._engine.ROT_HADAMARD, eager._engine.ROT_IDENTITY)
+                     and down_proj.in_features % max(g, 32) == 0
+                     and (down_proj.bias is None or (down_proj.bias.dtype == torch.bfloat16
+                                                     and down_proj.bias.is_contiguous())))
 
     def forward(self, x, residual=None):
         """`residual`: added to the result (a fused decoder block passes its skip connection)."""
+        if traceable and _traceable_call(x):
+            # two operators: gate and up from one quantization of x; SiLU*up quantized as it is
+            # formed and multiplied by down's weight
+            gate, up = _group_linear((self.gate_proj, self.up_proj), x)
+            down = self.down_proj
+            y = _eager().silu_mul_linear_w4a4_op(gate, up, down.forward_hadamard_matrix, down.qweight, down.scales,
+                                                 down.weight_global_scale, down.act_global_scale, down.bias,
+                                                 down.config.forward_dtype == FPQuantDtype.NVFP4)
+            y = y.view(*x.shape[:-1], y.shape[-1])
+            return y if residual is None else residual + y
         if not _fusable_call(x) or (residual is not None and not _fusable_call(residual)):
             y = unfused(x)
             return y if residual is None else residual + y
@@ -227,8 +289,82 @@ def fuse_residual_adds(block: nn.Module) -> bool:
     return True
 
 
+class _ProjectionCalls(ast.NodeTransformer):
+    """Replaces `self.<q|k|v>_proj(hidden_states)` by the names `__fpq_q`, `__fpq_k`, `__fpq_v`."""
+
+    def __init__(self):
+        self.seen = []
+
+    def visit_Call(self, node):
+        self.generic_visit(node)
+        f = node.func
+        if (isinstance(f, ast.Attribute) and isinstance(f.value, ast.Name) and f.value.id == "self"
+                and f.attr in ("q_proj", "k_proj", "v_proj") and len(node.args) == 1 and not node.keywords
+                and isinstance(node.args[0], ast.Name) and node.args[0].id == "hidden_states"):
+            self.seen.append(f.attr)
+            return ast.copy_location(ast.Name(id="__fpq_" + f.attr[0], ctx=ast.Load()), node)
+        return node
+
+
+def _qkv(attn, hidden_states):
+    """q, k and v projections of `hidden_states`: from one operator when a compiler is tracing
+    (which cannot see that the three layers quantize the same tensor), else three ordinary calls
+    (which share the quantization by themselves)."""
+    if attn._fpq_qkv_alike and _traceable_call(hidden_states):
+        return _group_linear((attn.q_proj, attn.k_proj, attn.v_proj), hidden_states)
+    return attn.q_proj(hidden_states), attn.k_proj(hidden_states), attn.v_proj(hidden_states)
+
+
+def fuse_qkv(attn: nn.Module) -> bool:
+    """Give a traced attention module one operator for its q/k/v projections.  The module's own
+    `forward` is kept: its source is re-compiled with the three calls `self.q_proj(hidden_states)`,
+    `self.k_proj(hidden_states)`, `self.v_proj(hidden_states)` -- which must sit in three consecutive
+    statements -- reading the results of one grouped call placed in front of them.  False (nothing
+    changed) if the forward does not have that shape or the layers do not quantize alike."""
+    layers = [getattr(attn, n, None) for n in ("q_proj", "k_proj", "v_proj")]
+    if not all(_is_real_quant_linear(l) for l in layers):
+        return False
+    if getattr(attn, "_fpq_unfused_forward", None) is not None:
+        return True
+    fn = type(attn).forward
+    if "forward" in vars(attn) or getattr(fn, "__closure__", None) or hasattr(fn, "__wrapped__"):
+        return False
+    try:
+        tree = ast.parse(textwrap.dedent(inspect.getsource(fn)))
+    except (OSError, TypeError, SyntaxError):
+        return False
+    fdef = tree.body[0] if tree.body and isinstance(tree.body[0], ast.FunctionDef) else None
+    if fdef is None or fdef.decorator_list or "super" in ast.unparse(fdef):
+        return False
+    hits = []
+    for i, stmt in enumerate(fdef.body):
+        rewriter = _ProjectionCalls()
+        fdef.body[i] = rewriter.visit(stmt)
+        if rewriter.seen:
+            hits.append((i, rewriter.seen))
+    if ([h[1] for h in hits] != [["q_proj"], ["k_proj"], ["v_proj"]]
+            or [h[0] for h in hits] != list(range(hits[0][0], hits[0][0] + 3))):
+        return False
+    # (the helper is reached through `self`: a name added to a copy of the module's globals would be
+    # invisible to a tracer that resolves globals through the module itself)
+    grouped = ast.parse("__fpq_q, __fpq_k, __fpq_v = self._fpq_qkv(hidden_states)").body[0]
+    fdef.body.insert(hits[0][0], grouped)
+    fdef.name = "forward"
+    ast.fix_missing_locations(tree)
+    namespace = dict(fn.__globals__)
+    try:
+        exec(compile(tree, f"<{type(attn).__qualname__}.forward with grouped q/k/v>", "exec"), namespace)
+    except Exception:
+        return False
+    attn._fpq_qkv_alike = _quantize_alike(layers)
+    attn._fpq_qkv = types.MethodType(_qkv, attn)
+    attn._fpq_unfused_forward = attn.forward
+    attn.forward = types.MethodType(namespace["forward"], attn)
+    return True
+
+
 def fuse_producers(model: nn.Module) -> int:
-    """Apply fuse_rmsnorm / fuse_gated_mlp / fuse_residual_adds to every decoder block of `model` that
+    """Apply fuse_rmsnorm / fuse_gated_mlp / fuse_residual_adds / fuse_qkv to every decoder block of `model` that
     has the Llama layout (`input_layernorm`, `self_attn.q_proj`, `post_attention_layernorm`, `mlp.gate_proj`).
     Call it after the linears have been replaced and quantized.  Returns the number of patches."""
     count = 0
@@ -240,6 +376,7 @@ def fuse_producers(model: nn.Module) -> int:
         count += int(fuse_rmsnorm(getattr(block, "post_attention_layernorm", None), getattr(mlp, "gate_proj", None)))
         count += int(fuse_gated_mlp(mlp))
         count += int(fuse_residual_adds(block))
+        count += int(fuse_qkv(attn))
     return count
 
 

@@ -192,7 +192,7 @@ def test_fused_norm_and_mlp_match_the_oracle_composition(fmt, g, tokens):
         h = O.silu_mul(gate.cpu().view(-1, 512), up.cpu().view(-1, 512)).view(gate.shape).cuda()
         want_mlp = block.mlp.down_proj(h)
 
-        assert fuse_producers(model) == 8                     # two norms, the MLP, the additions per block
+        assert fuse_producers(model) == 10                    # two norms, the MLP, the additions, q/k/v per block
         assert sorted(model.state_dict()) == sorted(_tiny_llama(fmt, g).state_dict())
         eager._shared_activations.clear()
         y = block.input_layernorm(x)
@@ -223,7 +223,7 @@ def test_fused_llama_matches_unfused(fmt, g):
     with torch.no_grad():
         want = model(ids).logits.float()
         want1 = model(ids[:, :1]).logits.float()
-        assert fuse_producers(model) == 8
+        assert fuse_producers(model) == 10
         got = model(ids).logits.float()
         got1 = model(ids[:, :1]).logits.float()
     for a, b in ((got, want), (got1, want1)):
@@ -310,7 +310,7 @@ def test_residual_adds_in_the_gemm_change_nothing(fmt, g, shape):
         assert torch.equal(model.generate(ids[:, :3], max_new_tokens=5, do_sample=False), want_tokens)
         fuse.unfuse_producers(model)
         assert all("forward" not in vars(b) for b in model.model.layers)
-        assert fuse.fuse_producers(model) == 8
+        assert fuse.fuse_producers(model) == 10
 
 
 def test_pending_residual_of_a_linear():
@@ -396,7 +396,7 @@ def test_fuse_producers_on_other_llama_layout_models(arch):
     ids = torch.randint(0, 128, (2, 48), generator=torch.Generator().manual_seed(2)).cuda()
     with torch.no_grad():
         want = model(ids).logits.float()
-        assert fuse_producers(model) == 8
+        assert fuse_producers(model) == 10
         got = model(ids).logits.float()
         assert float((got - want).norm() / want.norm()) < 0.02
         assert model.generate(ids[:, :8], max_new_tokens=3, do_sample=False).shape == (2, 11)
@@ -410,7 +410,7 @@ def test_fused_decoder_block_with_residual_epilogues_is_graph_capturable(tokens)
     the residual in down_proj's GEMM) recorded into a HIP graph and replayed on new inputs."""
     from fp_quant.utils import fuse_producers
     model = _tiny_llama("mxfp4", 128, seed=13)
-    assert fuse_producers(model) == 8
+    assert fuse_producers(model) == 10
     block = model.model.layers[1]
     pos = torch.arange(tokens, device="cuda").unsqueeze(0)
     static_x = torch.randn(1, tokens, 256, device="cuda", dtype=torch.bfloat16)
@@ -434,3 +434,57 @@ def test_fused_decoder_block_with_residual_epilogues_is_graph_capturable(tokens)
             torch.cuda.synchronize()
             assert torch.equal(static_y, want), seed
     assert block.self_attn.o_proj._fpq_residual is None
+
+
+@pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])
+@pytest.mark.parametrize("arch", ["llama", "qwen3"])
+def test_compiled_decode_with_grouped_operators_matches_eager(fmt, g, arch):
+    """fuse_producers before torch.compile: the traced attention calls one operator for q/k/v and the
+    traced MLP two (gate/up; SiLU*up -> down) instead of seven layer operators and an elementwise kernel.
+    Reference: the eager model with only its MLPs fused (the fused SiLU*up arithmetic is this library's, the
+    norms and additions are PyTorch's in both), under the compiler's emulate_precision_casts."""
+    import fp_quant
+    import torch._inductor.config as inductor_config
+    from torch._dynamo.utils import counters
+    from transformers import StaticCache
+    from fp_quant.utils import fuse
+    if arch == "llama":
+        model = _tiny_llama(fmt, g, seed=21)
+    else:
+        from transformers import Qwen3Config, Qwen3ForCausalLM
+        torch.manual_seed(21)
+        cfg = Qwen3Config(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                          num_key_value_heads=2, head_dim=64, vocab_size=128, max_position_embeddings=256)
+        model = Qwen3ForCausalLM(cfg).to(device="cuda", dtype=torch.bfloat16).eval()
+        fp_quant.replace_quantize_with_fp_quant_linear(model, _cfg(fmt, g))
+    cfg = model.config
+    for block in model.model.layers:
+        assert fuse.fuse_gated_mlp(block.mlp)
+    ids = torch.randint(0, 128, (2, 24), generator=torch.Generator().manual_seed(6)).cuda()
+    toks = torch.randint(0, 128, (4, 2, 1), generator=torch.Generator().manual_seed(7)).cuda()
+
+    def fresh_cache():
+        cache = StaticCache(config=cfg, max_cache_len=64)
+        model(input_ids=ids, past_key_values=cache, use_cache=True)
+        return cache
+
+    with torch.no_grad():
+        cache = fresh_cache()
+        want = [model(input_ids=t, past_key_values=cache, use_cache=True).logits.clone() for t in toks]
+        assert fuse.fuse_producers(model) == 10
+        assert all(b.self_attn._fpq_qkv_alike for b in model.model.layers)
+        eager_again = fresh_cache()      # the patched attention forward, called eagerly, changes nothing
+        assert torch.equal(model(input_ids=toks[0], past_key_values=eager_again, use_cache=True).logits, want[0])
+        fuse.unfuse_producers(model)
+        for block in model.model.layers:     # back to the reference configuration for the prefill
+            assert fuse.fuse_gated_mlp(block.mlp)
+        cache = fresh_cache()
+        assert fuse.fuse_producers(model) == 10
+        torch._dynamo.reset()
+        counters.clear()
+        with inductor_config.patch(emulate_precision_casts=True):
+            step = torch.compile(model.forward, mode="reduce-overhead", fullgraph=True)
+            got = [step(input_ids=t, past_key_values=cache, use_cache=True).logits.clone() for t in toks]
+    torch._dynamo.reset()
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert torch.equal(a, b), i
