@@ -428,3 +428,48 @@ def test_layers_called_from_two_threads_on_their_own_streams():
         th.join(timeout=100)
     assert not any(th.is_alive() for th in threads)
     assert not errors, errors[:5]
+
+
+@pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])
+def test_group_operators_equal_separate_layers(fmt, g):
+    """linear_group_w4a4_op (one quantization, one GEMM per layer) and silu_mul_linear_w4a4_op give the
+    bits of the layers called one by one -- with biases, for row-major and packed operand paths, and
+    whether or not a packed copy of a weight exists yet (a traced call may not create one)."""
+    import fp_quant
+    from fp_quant.module import eager
+    torch.manual_seed(41)
+    layers = []
+    for n, bias in ((256, True), (128, False), (384, True)):
+        lin = fp_quant.FPQuantLinear(512, n, _cfg(fmt, g), bias=bias, device="cuda", dtype=torch.bfloat16)
+        with torch.no_grad():
+            lin.weight.normal_(0, 0.05)
+            if bias:
+                lin.bias.normal_(0, 1)
+        lin.pre_forward()
+        layers.append(lin)
+    down = fp_quant.FPQuantLinear(256, 512, _cfg(fmt, g), bias=True, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        down.weight.normal_(0, 0.05)
+        down.bias.normal_(0, 1)
+    down.pre_forward()
+    nv = fmt == "nvfp4"
+
+    def group(x):
+        return eager.linear_group_w4a4_op(x, layers[0].forward_hadamard_matrix, [l.qweight for l in layers],
+                                          [l.scales for l in layers], [l.weight_global_scale for l in layers],
+                                          [l.act_global_scale for l in layers], [l.bias for l in layers], nv)
+
+    def mlp(gate, up):
+        return eager.silu_mul_linear_w4a4_op(gate, up, down.forward_hadamard_matrix, down.qweight, down.scales,
+                                             down.weight_global_scale, down.act_global_scale, down.bias, nv)
+
+    with torch.no_grad():
+        for round_ in range(2):          # second round: after eager calls have made the packed weights
+            for m in (3, 70, 300):
+                x = torch.randn(m, 512, device="cuda", dtype=torch.bfloat16)
+                got = group(x)
+                want = [l(x.clone()) for l in layers]
+                assert all(torch.equal(a, b) for a, b in zip(got, want)), (round_, m)
+                gate, up = torch.randn(2, m, 256, device="cuda", dtype=torch.bfloat16).unbind(0)
+                qa = eager.silu_mul_quantize(gate, up, down.forward_hadamard_matrix, down.act_global_scale, nv)
+                assert torch.equal(mlp(gate, up), down.forward_quantized(qa, (m,))), (round_, m)
