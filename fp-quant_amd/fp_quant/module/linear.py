@@ -151,6 +151,7 @@ class FPQuantLinear(nn.Module):
     # A tensor of the output's shape that the next forward adds to its result (inside the GEMM
     # where the kernel can) and then clears; set by a fused decoder block around its attention call.
     # It stays set when the forward cannot take it (autograd), and the block then adds it itself.
+    # Host-side state of the module: two threads must not run the same fused block at the same time.
     _fpq_residual: Optional[torch.Tensor] = None
 
     def forward(self, x) -> torch.Tensor:
