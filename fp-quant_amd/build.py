@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "fp_quant", "_lib")
 LIB = os.path.join(OUT_DIR, "libfpq_hip.so")
-SOURCES = ["fpq_capi.hip", "fpq_quantize.hip", "fpq_gemm.hip", "fpq_gemm_packed.hip"]
+SOURCES = ["fpq_capi.hip", "fpq_quantize.hip", "fpq_gemm.hip", "fpq_gemm_packed.hip", "fpq_gemm_stream.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-fhip-fp32-correctly-rounded-divide-sqrt", "-fno-gpu-flush-denormals-to-zero",

@@ -375,10 +375,17 @@ static int launch_packed(const void* xq, const void* xs, const void* wq, const v
   return (int)hipGetLastError();
 }
 
+// fpq_gemm_stream.hip: the weight-streaming kernel for at most 128 activation rows
+bool stream_eligible(int64_t M, int64_t N, int64_t K);
+int64_t gemm_mxf4_stream_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int gemm_mxf4_stream(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
+                     const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                     void* workspace, int64_t workspace_bytes, hipStream_t stream);
+
 template <bool NV>
 static int gemm_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                        const void* bias, void* y, int64_t M, int64_t N, int64_t K, void* stream,
-                       const void* residual = nullptr);
+                       const void* residual = nullptr, void* workspace = nullptr, int64_t workspace_bytes = 0);
 
 template <bool NV>
 static int pack_operand(const void* codes, const void* scales, int64_t scale_stride, int64_t rows, int64_t K,
@@ -410,8 +417,8 @@ namespace fpq {
 template <bool NV>
 static int gemm_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                        const void* bias, void* y, int64_t M, int64_t N, int64_t K, void* stream,
-                       const void* residual) {
-  if (M < 0 || N < 0 || K < 0) return FPQ_E_SHAPE;
+                       const void* residual, void* workspace, int64_t workspace_bytes) {
+  if (M < 0 || N < 0 || K < 0 || workspace_bytes < 0) return FPQ_E_SHAPE;
   if (M == 0 || N == 0) return FPQ_OK;
   if (!xq || !xs || !wq || !ws || !alpha || !y) return FPQ_E_NULL;
   if (K == 0 || K % 256 != 0) return FPQ_E_SHAPE;
@@ -423,6 +430,10 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
   if (((uintptr_t)xq & 15u) || ((uintptr_t)wq & 15u) || ((uintptr_t)xs & 15u) || ((uintptr_t)ws & 15u) ||
       ((uintptr_t)y & 15u) || ((uintptr_t)residual & 15u))
     return FPQ_E_ALIGN;
+  if ((uintptr_t)workspace & 255u) return FPQ_E_ALIGN;
+  if (!NV && stream_eligible(M, N, K))
+    return gemm_mxf4_stream(xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, workspace, workspace_bytes,
+                            (hipStream_t)stream);
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
   if (big_tiles < FPQ_PACKED_SMALL_BELOW)
     return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual);
@@ -467,6 +478,27 @@ extern "C" int fpq_gemm_mxf4_packed_residual(const void* xq, const void* xs, con
                                              int64_t M, int64_t N, int64_t K, void* stream) {
   if (!residual) return FPQ_E_NULL;
   return fpq::gemm_packed<false>(xq, xs, wq, ws, alpha, bias, y, M, N, K, stream, residual);
+}
+
+namespace fpq {
+int gemm_mxf4_packed_any(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
+                         const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                         void* workspace, int64_t workspace_bytes, void* stream) {
+  return gemm_packed<false>(xq, xs, wq, ws, alpha, bias, y, M, N, K, stream, residual, workspace,
+                            workspace ? workspace_bytes : 0);
+}
+}  // namespace fpq
+
+extern "C" int64_t fpq_gemm_mxf4_packed_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  return fpq::gemm_mxf4_stream_workspace_bytes(M, N, K);
+}
+
+extern "C" int fpq_gemm_mxf4_packed_splitk(const void* xq, const void* xs, const void* wq, const void* ws,
+                                           const float* alpha, const void* bias, const void* residual, void* y,
+                                           int64_t M, int64_t N, int64_t K, void* workspace,
+                                           int64_t workspace_bytes, void* stream) {
+  return fpq::gemm_mxf4_packed_any(xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, workspace, workspace_bytes,
+                                   stream);
 }
 
 extern "C" int fpq_gemm_nvf4_packed(const void* xq, const void* xs, const void* wq, const void* ws,

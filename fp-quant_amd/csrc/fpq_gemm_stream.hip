@@ -1,0 +1,338 @@
+// Weight-streaming MXFP4 GEMM on packed operands for at most 128 activation rows.
+//
+// With so few rows the time is the one pass over the weights (31 MB for the Llama-3-8B up/gate
+// projection: 3.9 us at 8 TB/s), so the kernel is built around bytes in flight, not around tiles:
+//   * a workgroup owns ONE 32-row weight tile and a range of K; nothing is staged through LDS:
+//     in the packed layout one operand of one 32x32x64 matrix instruction is one contiguous
+//     kilobyte, lane by lane, so a wave loads it straight into the registers the instruction reads;
+//   * the four waves take the 256-K blocks of the range in turn (wave w: blocks w, w + 4, ...) and
+//     every wave issues the loads of up to DB blocks before its first matrix instruction, so for
+//     K = 4096 and 32 rows the whole weight tile is requested at once;
+//   * activations (at most four 32-row tiles, padded rows are zero) are re-read by every workgroup
+//     and come from the L2;
+//   * the four partial tiles meet in LDS and are summed in the fixed order (w0 + w2) + (w1 + w3).
+// Shapes with few weight tiles (N = 4096: 128 workgroups for 256 CUs) or long K also split K
+// ACROSS workgroups: each stores its fp32 partial tile into a workspace, a per-tile counter tells
+// the last one to arrive, and that one adds the partials of all splits in split order (its own
+// included, read back from the workspace), so the result does not depend on the arrival order.
+// Counters are left at zero for the next launch.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+#include "../../include/fpq.h"
+#include "fpq_device.h"
+#include "fpq_gemm_epilogue.h"
+
+namespace fpq {
+
+typedef unsigned v4u_s __attribute__((ext_vector_type(4)));
+
+constexpr int kStreamCounters = 4096;                        // one per weight tile group
+constexpr int64_t kStreamCounterBytes = kStreamCounters * 4;  // they open the workspace
+constexpr int kStreamMaxRows = 128;
+
+// NT weight row tiles per workgroup, MT activation row tiles (exactly ceil(M / 32)), DB 256-K blocks
+// of loads in flight per wave, NW waves.  Every workgroup re-reads all activations, so with more
+// than 32 activation rows two weight tiles per workgroup halve what the L2 has to deliver.
+template <int NT, int MT, int DB, int NW>
+__global__ __launch_bounds__(64 * NW) void gemm_mxf4_stream_kernel(
+    const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
+    const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias,
+    const uint16_t* residual, uint16_t* y, int M, int N, int K, int bps, int ksplit,
+    float* partial, unsigned* counters) {
+  static_assert(NW == 4, "the partial sums meet in two rounds of two");
+  __shared__ v4f part[2][NT * MT][4][64];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int nu = K >> 6, nkb = K >> 8;
+  const int rtg = blockIdx.x, split = blockIdx.y;
+  const int rt_n = (N + 31) >> 5;
+  const int kb_begin = split * bps, kb_end = min(nkb, kb_begin + bps);
+  const int first = kb_begin + wave;                                   // this wave: first, first + NW, ...
+  const int nblk = kb_end > first ? (kb_end - first + NW - 1) / NW : 0;
+
+  // A weight tile past the last one (odd tile count, NT = 2) re-reads the last: nothing of it is stored.
+  const uint8_t* wcode[NT];
+  const uint8_t* wscale[NT];
+#pragma unroll
+  for (int i = 0; i < NT; ++i) {
+    const int rt = min(rtg * NT + i, rt_n - 1);
+    wcode[i] = wq + (size_t)rt * nu * 1024 + lane * 16;
+    wscale[i] = ws + (size_t)rt * nkb * 256 + lane * 4;
+  }
+  // Lanes whose activation row lies past M (last row tile only) read what the lane of row 0 in
+  // their K half reads: no further cache line is touched for rows that are never stored.
+  const int rows_last = M - 32 * (MT - 1);
+  const int xl = (lane & 31) < rows_last ? lane : (lane & 32);
+  const uint8_t* xcode[MT];
+  const uint8_t* xscale[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const int l = j == MT - 1 ? xl : lane;
+    xcode[j] = xq + (size_t)j * nu * 1024 + l * 16;
+    xscale[j] = xs + (size_t)j * nkb * 256 + l * 4;
+  }
+
+  v16f acc[NT * MT];
+#pragma unroll
+  for (int j = 0; j < NT * MT; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+
+  // A ring of DB blocks in registers.  Every load is unconditional (a block index past the wave's
+  // last one is clamped to it and its matrix instructions are skipped): with loads under branches
+  // the compiler can no longer count which of them are still in flight and waits for all.
+  uint4 a[DB][4][NT], b[DB][4][MT];
+  uint32_t sa[DB][NT], sb[DB][MT];
+  const int t_last = nblk > 0 ? nblk - 1 : 0;
+  auto load_block = [&](auto slot, int t) {
+    constexpr int s = decltype(slot)::value;
+    const int kb = min(first + NW * min(t, t_last), nkb - 1);
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const v4u_s ld = __builtin_nontemporal_load((const v4u_s*)(wcode[i] + (size_t)(kb * 4 + u) * 1024));
+        a[s][u][i] = make_uint4(ld.x, ld.y, ld.z, ld.w);
+      }
+      sa[s][i] = *(const uint32_t*)(wscale[i] + (size_t)kb * 256);
+    }
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) b[s][u][j] = *(const uint4*)(xcode[j] + (size_t)(kb * 4 + u) * 1024);
+      sb[s][j] = *(const uint32_t*)(xscale[j] + (size_t)kb * 256);
+    }
+  };
+  auto compute_block = [&](auto slot) {
+    constexpr int s = decltype(slot)::value;
+#define FPQ_STREAM_STEP(U)                                                                              \
+  _Pragma("unroll") for (int i = 0; i < NT; ++i) {                                                      \
+    const uint4 aq = a[s][U][i];                                                                        \
+    const v8i av = v8i{(int)aq.x, (int)aq.y, (int)aq.z, (int)aq.w, 0, 0, 0, 0};                         \
+    _Pragma("unroll") for (int j = 0; j < MT; ++j) {                                                    \
+      const uint4 bq = b[s][U][j];                                                                      \
+      const v8i bv = v8i{(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w, 0, 0, 0, 0};                       \
+      acc[i * MT + j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(                                \
+          av, bv, acc[i * MT + j], 4, 4, U, (int)sa[s][i], U, (int)sb[s][j]);                           \
+    }                                                                                                   \
+  }
+    FPQ_STREAM_STEP(0)
+    FPQ_STREAM_STEP(1)
+    FPQ_STREAM_STEP(2)
+    FPQ_STREAM_STEP(3)
+#undef FPQ_STREAM_STEP
+  };
+  auto for_slots = [&](auto&& f) {
+    f(std::integral_constant<int, 0>{});
+    if constexpr (DB > 1) f(std::integral_constant<int, 1>{});
+    if constexpr (DB > 2) f(std::integral_constant<int, 2>{});
+    if constexpr (DB > 3) f(std::integral_constant<int, 3>{});
+  };
+  static_assert(DB >= 1 && DB <= 4, "at most four blocks in flight");
+
+  for_slots([&](auto slot) { load_block(slot, decltype(slot)::value); });
+  int t0 = 0;
+  for (; t0 + 2 * DB <= nblk; t0 += DB) {   // steady state: the block DB ahead exists
+    for_slots([&](auto slot) {
+      compute_block(slot);
+      load_block(slot, t0 + DB + decltype(slot)::value);
+    });
+  }
+  for_slots([&](auto slot) {                // the ring's last full or partial content
+    if (t0 + decltype(slot)::value < nblk) compute_block(slot);
+  });
+  if (nblk - t0 > DB) {                     // up to DB - 1 blocks more
+    for_slots([&](auto slot) { load_block(slot, t0 + DB + decltype(slot)::value); });
+    for_slots([&](auto slot) {
+      if (t0 + DB + decltype(slot)::value < nblk) compute_block(slot);
+    });
+  }
+
+  // ---- the four K parts of the workgroup, summed in the fixed order (w0 + w2) + (w1 + w3)
+  auto put = [&](int slot) {
+#pragma unroll
+    for (int j = 0; j < NT * MT; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        part[slot][j][g][lane] = v4f{acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]};
+  };
+  auto take = [&](int slot) {
+#pragma unroll
+    for (int j = 0; j < NT * MT; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const v4f p = part[slot][j][g][lane];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[j][4 * g + q] += p[q];
+      }
+  };
+  if (wave >= 2) put(wave - 2);
+  __syncthreads();
+  if (wave < 2) take(wave);
+  __syncthreads();
+  if (wave == 1) put(0);
+  __syncthreads();
+  if (wave != 0) return;
+  take(0);
+
+  // ---- K split across workgroups: partial tiles through the workspace, last arrival finishes
+  if (ksplit > 1) {
+    // The parts of a tile run on different XCDs, whose L2 caches are not coherent with each other
+    // for ordinary accesses.  Device-scope fences would write back and invalidate whole caches
+    // (measured: 55 us for a 6 us kernel); instead every access to the workspace is a relaxed
+    // device-scope atomic, which the hardware performs at the point all XCDs agree on, and the
+    // wave waits for its stores to be acknowledged before it moves the counter.
+    constexpr int kTile = NT * MT * 16 * 64;  // floats per partial
+    float* mine = partial + ((size_t)rtg * ksplit + split) * kTile + lane;
+#pragma unroll
+    for (int j = 0; j < NT * MT; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        __hip_atomic_store(mine + (j * 16 + v) * 64, acc[j][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    unsigned arrived = 0;
+    if (lane == 0) arrived = __hip_atomic_fetch_add(counters + rtg, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    arrived = __builtin_amdgcn_readfirstlane(arrived);
+    if (arrived != (unsigned)(ksplit - 1)) return;
+    const float* all = partial + (size_t)rtg * ksplit * kTile + lane;
+    for (int s = 0; s < ksplit; ++s) {
+#pragma unroll
+      for (int j = 0; j < NT * MT; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const float p = __hip_atomic_load(all + (size_t)s * kTile + (j * 16 + v) * 64, __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT);
+          acc[j][v] = s == 0 ? p : acc[j][v] + p;
+        }
+    }
+    if (lane == 0) __hip_atomic_store(counters + rtg, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+
+  // ---- y[m][n] = bf16(alpha * acc) (+ bias) (+ residual, a further bf16 add): register 4g + q of
+  // tile (i, j) is m = 32 j + lane % 32, n = 32 (NT rtg + i) + 8 g + 4 (lane / 32) + q
+  const float alpha = *alpha_p;
+  const int r32 = lane & 31, kh = lane >> 5;
+  const bool vec_ok = (N & 3) == 0;
+#pragma unroll
+  for (int ig = 0; ig < NT * 4; ++ig) {
+    const int i = ig >> 2, g = ig & 3;
+    const int n = (rtg * NT + i) * 32 + 8 * g + 4 * kh;
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (n + q < N) bv[q] = __uint_as_float((uint32_t)bias[n + q] << 16);
+    }
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      const int m = j * 32 + r32;
+      if (m >= M || n >= N) continue;
+      const v16f& t = acc[i * MT + j];
+      uint32_t lo = pack_bf16x2(t[4 * g + 0] * alpha, t[4 * g + 1] * alpha);
+      uint32_t hi = pack_bf16x2(t[4 * g + 2] * alpha, t[4 * g + 3] * alpha);
+      if (bias) {
+        lo = pack_bf16x2(__uint_as_float(lo << 16) + bv[0], __uint_as_float(lo & 0xffff0000u) + bv[1]);
+        hi = pack_bf16x2(__uint_as_float(hi << 16) + bv[2], __uint_as_float(hi & 0xffff0000u) + bv[3]);
+      }
+      uint16_t* dst = y + (size_t)m * N + n;
+      if (vec_ok && n + 3 < N) {
+        if (residual) {
+          const uint2 rv = *(const uint2*)(residual + (size_t)m * N + n);
+          lo = pack_bf16x2(__uint_as_float(lo << 16) + __uint_as_float(rv.x << 16),
+                           __uint_as_float(lo & 0xffff0000u) + __uint_as_float(rv.x & 0xffff0000u));
+          hi = pack_bf16x2(__uint_as_float(hi << 16) + __uint_as_float(rv.y << 16),
+                           __uint_as_float(hi & 0xffff0000u) + __uint_as_float(rv.y & 0xffff0000u));
+        }
+        *(uint2*)dst = make_uint2(lo, hi);
+      } else {
+        const uint32_t w[2] = {lo, hi};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if (n + q >= N) continue;
+          uint32_t h = (w[q >> 1] >> (16 * (q & 1))) & 0xffffu;
+          if (residual)
+            h = pack_bf16x2(__uint_as_float(h << 16) + __uint_as_float((uint32_t)residual[(size_t)m * N + n + q] << 16), 0.0f) & 0xffffu;
+          dst[q] = (uint16_t)h;
+        }
+      }
+    }
+  }
+}
+
+struct StreamPlan {
+  bool use;    // false: the tile kernels of fpq_gemm_packed.hip serve the shape better
+  int nt;      // weight row tiles per workgroup
+  int ksplit;  // K parts (workgroups per group of weight tiles)
+  int bps;     // 256-K blocks per part
+};
+
+// Which shapes run here and how (all thresholds are measured break-even points on Llama-3-8B and
+// Qwen3-8B layer shapes).  Up to 32 activation rows: always, one weight tile per workgroup.  More
+// rows: one weight tile per workgroup while those fit one round of the 256 CUs; two per workgroup
+// for up to 64 rows; beyond that the 128x128 tile kernel, which shares activations through LDS.
+// K is split across workgroups only for at most 32 rows, when the weight tiles leave at least half
+// of the CUs idle and every part keeps at least 4096 of K (the exchange of partial tiles through
+// the workspace costs about as much as streaming 16 blocks); fewer parts if the workspace is small.
+static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_bytes) {
+  StreamPlan plan{false, 1, 1, 0};
+  if (M < 1 || M > kStreamMaxRows || N < 1 || K < 256 || K % 256 != 0) return plan;
+  const int64_t rt_m = (M + 31) / 32, tiles = (N + 31) / 32, nkb = K / 256;
+  if (rt_m == 1 || tiles <= 256) plan.nt = 1;
+  else if (rt_m == 2) plan.nt = 2;
+  else return plan;
+  plan.use = true;
+  const int64_t groups = (tiles + plan.nt - 1) / plan.nt;
+  int64_t ksplit = 1;
+  if (rt_m == 1 && workspace_bytes > kStreamCounterBytes && groups <= kStreamCounters) {
+    ksplit = 256 / groups;
+    if (ksplit > nkb / 16) ksplit = nkb / 16;
+    if (ksplit < 1) ksplit = 1;
+    while (ksplit > 1 && kStreamCounterBytes + ksplit * groups * 4096 > workspace_bytes) --ksplit;
+  }
+  const int64_t bps = (nkb + ksplit - 1) / ksplit;
+  plan.ksplit = (int)((nkb + bps - 1) / bps);  // no empty part
+  plan.bps = (int)bps;
+  return plan;
+}
+
+bool stream_eligible(int64_t M, int64_t N, int64_t K) { return stream_plan(M, N, K, 0).use; }
+
+int64_t gemm_mxf4_stream_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  const StreamPlan plan = stream_plan(M, N, K, (int64_t)1 << 62);
+  if (!plan.use || plan.ksplit <= 1) return 0;
+  const int64_t groups = ((N + 31) / 32 + plan.nt - 1) / plan.nt;
+  return kStreamCounterBytes + (int64_t)plan.ksplit * groups * plan.nt * ((M + 31) / 32) * 4096;
+}
+
+// Arguments are validated by the caller (gemm_packed); `workspace` is null or 256-byte aligned with
+// its first kStreamCounterBytes zero.
+int gemm_mxf4_stream(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
+                     const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                     void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+  const StreamPlan plan = stream_plan(M, N, K, workspace ? workspace_bytes : 0);
+  const dim3 grid((unsigned)(((N + 31) / 32 + plan.nt - 1) / plan.nt), (unsigned)plan.ksplit);
+  unsigned* counters = (unsigned*)workspace;
+  float* partial = workspace ? (float*)((uint8_t*)workspace + kStreamCounterBytes) : nullptr;
+#define FPQ_STREAM(NTT, MTT, DBB)                                                                       \
+  hipLaunchKernelGGL((gemm_mxf4_stream_kernel<NTT, MTT, DBB, 4>), grid, dim3(256), 0, stream, (const uint8_t*)xq, \
+                     (const uint8_t*)xs, (const uint8_t*)wq, (const uint8_t*)ws, alpha,                 \
+                     (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, (int)M, (int)N,    \
+                     (int)K, plan.bps, plan.ksplit, partial, counters)
+  const int mt = (int)((M + 31) / 32);
+  if (plan.nt == 1) {
+    switch (mt) {
+      case 1: FPQ_STREAM(1, 1, 4); break;
+      case 2: FPQ_STREAM(1, 2, 3); break;
+      case 3: FPQ_STREAM(1, 3, 2); break;
+      default: FPQ_STREAM(1, 4, 2); break;
+    }
+  } else {
+    FPQ_STREAM(2, 2, 2);
+  }
+#undef FPQ_STREAM
+  return (int)hipGetLastError();
+}
+
+}  // namespace fpq

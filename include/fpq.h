@@ -229,6 +229,27 @@ int fpq_gemm_mxf4_packed_residual(const void* xq_packed, const void* xs_packed, 
                                   void* stream);
 
 /*
+ * fpq_gemm_mxf4_packed (with `residual` non-null: fpq_gemm_mxf4_packed_residual) that may split K
+ * across workgroups.  With at most 128 activation rows the time is one pass over the weights, and a
+ * shape with few weight rows or a long K fills the chip only if several workgroups share one output
+ * tile: each stores its fp32 partial tile into `workspace`, and the last one to arrive (a counter
+ * per tile) adds the partials of all parts in part order, so the result is deterministic.  It is
+ * the counterpart of the small-M entry the reference keeps disabled (matmul_ada_mxf4_bf16_tn_op,
+ * qutlass_ops.py:133-146; linear_fns.py:55).
+ *   workspace        null (K stays whole) or a 256-byte aligned device buffer whose first 16384 bytes
+ *                    are zero before the first call; every call leaves them zero again.  Calls that
+ *                    share a workspace must not overlap (same stream, or ordered by events).
+ *   workspace_bytes  its size; fpq_gemm_mxf4_packed_workspace_bytes(M, N, K) is what the shape can
+ *                    use (0: it never splits).  A smaller buffer means fewer parts, not an error.
+ * Larger M runs the tile kernels of fpq_gemm_mxf4_packed and ignores the workspace.
+ */
+int64_t fpq_gemm_mxf4_packed_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int fpq_gemm_mxf4_packed_splitk(const void* xq_packed, const void* xs_packed, const void* wq_packed,
+                                const void* ws_packed, const float* alpha, const void* bias,
+                                const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                                void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * Test hook: E2M1 codes of n fp32 values exactly as the quantize kernels round them
  * (out[i] in 0..15, one byte per value).  Used to check the device rounding exhaustively.
  */
