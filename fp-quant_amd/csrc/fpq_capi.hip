@@ -15,6 +15,7 @@ extern "C" const char* fpq_status_string(int status) {
     case FPQ_E_ALIGN: return "a pointer is not aligned as documented";
     case FPQ_E_POLICY: return "unknown zero-nibble policy";
     case FPQ_E_UNSUPPORTED: return "no kernel in this build for the requested combination";
+    case FPQ_E_LIMIT: return "a size is beyond the stated maximum of this entry point";
     default: break;
   }
   if (status > 0) return hipGetErrorString((hipError_t)status);

@@ -19,6 +19,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "../../include/fpq.h"
@@ -335,4 +336,54 @@ int gemm_mxf4_stream(const void* xq, const void* xs, const void* wq, const void*
   return (int)hipGetLastError();
 }
 
+
+// ---- the entry point that allocates nothing -------------------------------------------------------
+// Counters and partial tiles of a split K live in this file-scope array instead of a caller-provided
+// workspace.  Every GPU the library runs on holds its own copy at its own address until the process
+// ends; the array's name is only a host-side handle, the device address comes from
+// hipGetSymbolAddress, once per device, and that address is what kernels and host code use.
+// A split needs at most 256 partial tiles of 4 KB (stream_plan: parts x weight tiles <= 256).
+constexpr int64_t kScratchBytes = kStreamCounterBytes + 256 * 4096;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device (looked up on the first call per device; two
+// threads racing on that first call store the same address).
+static int scratch_address(void** out) {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return (int)err;
+  if (device < 0 || device >= kMaxDevices) return FPQ_E_UNSUPPORTED;
+  void* ptr = g_scratch_ptr[device].load(std::memory_order_acquire);
+  if (!ptr) {
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return (int)err;
+    if (!ptr) return FPQ_E_UNSUPPORTED;
+    g_scratch_ptr[device].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return FPQ_OK;
+}
+
+// fpq_gemm_packed.hip: argument checks and dispatch shared with fpq_gemm_mxf4_packed_splitk
+int gemm_mxf4_packed_any(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
+                         const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                         void* workspace, int64_t workspace_bytes, void* stream);
+
 }  // namespace fpq
+
+extern "C" int64_t fpq_gemm_mxf4_packed_noalloc_max_rows(void) { return fpq::kStreamMaxRows; }
+
+extern "C" int fpq_gemm_mxf4_packed_noalloc(const void* xq, const void* xs, const void* wq, const void* ws,
+                                            const float* alpha, const void* bias, const void* residual,
+                                            void* y, int64_t M, int64_t N, int64_t K, void* stream) {
+  if (M > fpq::kStreamMaxRows) return FPQ_E_LIMIT;
+  if (fpq::gemm_mxf4_stream_workspace_bytes(M, N, K) > fpq::kScratchBytes) return FPQ_E_LIMIT;
+  void* ptr = nullptr;
+  const int st = fpq::scratch_address(&ptr);
+  if (st != FPQ_OK) return st;
+  return fpq::gemm_mxf4_packed_any(xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, ptr, fpq::kScratchBytes,
+                                   stream);
+}

@@ -30,6 +30,7 @@ extern "C" {
 #define FPQ_E_ALIGN -4       /* a pointer is not aligned as documented           */
 #define FPQ_E_POLICY -5      /* unknown zero-nibble policy or scale layout       */
 #define FPQ_E_UNSUPPORTED -6 /* valid request this build has no kernel for       */
+#define FPQ_E_LIMIT -7       /* a size is beyond the entry point's stated maximum */
 
 /* rotation kinds: how the [g, g] matrix of the reference (linear.py:24-41) is applied */
 #define FPQ_ROT_HADAMARD 0 /* +-norm Sylvester matrix: fp32 radix-2 butterflies, strides 1..g/2 */
@@ -248,6 +249,27 @@ int fpq_gemm_mxf4_packed_splitk(const void* xq_packed, const void* xs_packed, co
                                 const void* ws_packed, const float* alpha, const void* bias,
                                 const void* residual, void* y, int64_t M, int64_t N, int64_t K,
                                 void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * fpq_gemm_mxf4_packed_splitk for callers that cannot allocate or hold a workspace (code recorded
+ * into a HIP graph, tight serving loops, harnesses that forbid hipMalloc): the counters and partial
+ * tiles of a split K live in a file-scope device array of the library (1 064 960 bytes per GPU, held
+ * until the process ends) instead of a caller-provided buffer.  It has no counterpart in the
+ * reference.  Same arguments, results and status codes as fpq_gemm_mxf4_packed_splitk called with a
+ * workspace of that size, with these limits:
+ *   M <= fpq_gemm_mxf4_packed_noalloc_max_rows() (128), the weight-streaming regime; more rows
+ *   return FPQ_E_LIMIT (the tile kernels of fpq_gemm_mxf4_packed use no scratch memory at all);
+ *   a shape whose split would need more than the array holds returns FPQ_E_LIMIT.
+ * The call makes no hipMalloc/hipFree and launches the same kernels.  All calls on one GPU share
+ * that GPU's array: calls that may overlap on one GPU (different streams without an ordering
+ * event) race on it and must use fpq_gemm_mxf4_packed_splitk with their own workspaces.  The
+ * counters start at zero (static storage) and every call leaves them at zero.
+ */
+int64_t fpq_gemm_mxf4_packed_noalloc_max_rows(void);
+int fpq_gemm_mxf4_packed_noalloc(const void* xq_packed, const void* xs_packed, const void* wq_packed,
+                                 const void* ws_packed, const float* alpha, const void* bias,
+                                 const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                                 void* stream);
 
 /*
  * Test hook: E2M1 codes of n fp32 values exactly as the quantize kernels round them
