@@ -85,7 +85,7 @@ __device__ __forceinline__ uint32_t e8m0_encode(float t) {
 // ---------------------------------------------------------------------------------------------
 // Per-group scale parameters.  The element step is  v = fma(x, k1, x * k2)  on the fast path,
 // which yields the same E2M1 code as the correctly rounded quotient x / s for every x (proved
-// by exhaustion over all divisor mantissas on the host), or the IEEE quotient x / s itself on
+// by exhaustion over all divisor mantissas on the host: tests/div_equivalence.c), or the IEEE quotient x / s itself on
 // the slow path taken for extreme exponents.
 struct GroupScale {
   float k1;      // fast: RN(1/s)            slow: s

@@ -39,10 +39,14 @@ other (fp32 everywhere, bf16 only at the input and at the rotation matrix entrie
   keeps the sign bit of the scaled value (what a hardware cvt does).
 
 Pin status (each function below is checked in tests/test_oracle_*.py against closed
-forms, exhaustive tables, library casts or brute force; none needed an import of the
-reference): rotation, E8M0 exponent, E2M1 RNE, packing, E4M3 cast, E8M0 cast, GEMM, the quest
+forms, exhaustive tables, library casts or brute force): rotation, E8M0 exponent, E2M1 RNE, packing, E4M3 cast, E8M0 cast, GEMM, the quest
 scale (against numpy float64 statistics and a per-group Python loop) and clip mask; the two
 producers (silu_mul, rmsnorm) against float64 evaluations and torch's own operators.
+tests/test_reference_golden.py additionally pins quantize_mx, quantize_nv, nv_tracked_global_scale,
+e2m1_round_rne, e2m1_codes and pack_nibbles to bytes written by the reference's own modules
+(src/quantization/{quant_args,quant_ops,quantizer}.py, src/helpers.py, loaded by file path in the
+build container by tests/golden/make_reference_golden.py); the only difference is the documented
+zero-scale deviation above.
 The third-party kernels the reference calls for this path (QuTLASS, un-vendored, version
 unpinned) have no fixtures in the reference: bit parity against QuTLASS itself is unpinned.
 """

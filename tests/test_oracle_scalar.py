@@ -292,6 +292,62 @@ def test_quantize_mx_against_python_loop():
         assert codes[r].tolist() == c and scales[r].tolist() == s
 
 
+def _e4m3_grid():
+    """Every finite non-negative float8_e4m3fn value by its byte, from the format's definition."""
+    vals = []
+    for byte in range(127):                     # 0x7f is NaN
+        e, m = byte >> 3, byte & 7
+        vals.append((m / 8.0) * 2.0 ** -6 if e == 0 else (1 + m / 8.0) * 2.0 ** (e - 7))
+    return vals
+
+
+def _e4m3_nearest_byte(t, grid=_e4m3_grid()):
+    """Nearest E4M3 value of t >= 0 (already clamped to 448), ties to the even byte."""
+    best = min(range(127), key=lambda b: (abs(grid[b] - t), b % 2))
+    return best
+
+
+def _brute_quantize_nv_row(xr, gs):
+    """Per-element Python loop of the NVFP4 chain as quantizer.py:107-112,143-168 and rtn.py:187-188
+    write it, in numpy fp32 scalars, with the E4M3 cast as a nearest-value search."""
+    f32 = np.float32
+    grid = _e4m3_grid()
+    gs = f32(gs)
+    rg = f32(1.0) / gs
+    out_codes, out_scales = [], []
+    for g0 in range(0, len(xr), 16):
+        grp = [f32(v) for v in xr[g0:g0 + 16]]
+        a = max(abs(v) for v in grp)
+        sc0 = f32(f32(f32(2) * a) / f32(12))
+        t = min(f32(sc0 * gs), f32(448))
+        sc = f32(grid[_e4m3_nearest_byte(float(t))])
+        sw = f32(sc * rg)
+        if sw == 0:                                   # the documented deviation: byte 0, zero codes
+            out_scales.append(0)
+            out_codes += [8] * 16
+            continue
+        stored = _e4m3_nearest_byte(float(min(f32(sw * gs), f32(448))))
+        out_scales.append(stored)
+        for v in grp:
+            q = f32(v / sw)
+            c = _nearest_even_code(min(abs(float(q)), 100.0))
+            out_codes.append(c | (8 if (q < 0 or c == 0) else 0))
+    return out_codes, out_scales
+
+
+@pytest.mark.parametrize("gs", [3.0, 10.0, 0.0897435918450355, 1234.5])
+def test_quantize_nv_against_python_loop(gs):
+    gen = torch.Generator().manual_seed(21)
+    x = (torch.randn(6, 128, generator=gen) * torch.tensor([1, 30, 1e-3, 1e3, 0.2, 5]).view(6, 1)).to(torch.bfloat16)
+    x[0, :16] = 0
+    x[4, 16:32] = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0] * 2)
+    packed, scales, xr = O.quantize_nv(x, gs, O.ROT_HADAMARD, 16)
+    codes = O.unpack_nibbles(packed)
+    for r in range(6):
+        c, s = _brute_quantize_nv_row(xr[r].tolist(), gs)
+        assert codes[r].tolist() == c and scales[r].tolist() == s
+
+
 def test_quantize_roundtrip_error_bound():
     # dequant(code, stored)/3 reproduces the rotated input to within half an E2M1 step
     gen = torch.Generator().manual_seed(12)
