@@ -38,12 +38,34 @@ def outlier_normal(torch, rows, cols, seed, frac=0.005, mult=25.0):
     return torch.where(mask, x * mult, x).to(torch.bfloat16)
 
 
+SETTLE_MS = 30.0        # untimed GPU work before any timed region, so that short runs see settled clocks
+BLOCK_MIN_MS = 50.0     # GPU time a block-median measurement covers at least, per leg
+BLOCK_MIN_COUNT = 9
+
+
+def _settle(torch, fn, n_variants, chunk):
+    """Untimed launches until SETTLE_MS of GPU time have passed (the part's clock moves with load: the
+    first milliseconds after an idle period run at another frequency than a sustained loop)."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    spent, i = 0.0, 0
+    while spent < SETTLE_MS:
+        e0.record()
+        for _ in range(chunk):
+            fn(i % n_variants)
+            i += 1
+        e1.record()
+        torch.cuda.synchronize()
+        spent += e0.elapsed_time(e1)
+
+
 def time_kernel(torch, fn, n_variants, steps, warmup):
-    """Runs fn(i % n_variants) warmup+steps times on the current stream.  Returns
-    (wall ms per step, event ms per step)."""
+    """Runs fn(i % n_variants) warmup+steps times on the current stream (plus the untimed settling
+    launches above, before the timed region).  Returns (wall ms per step, event ms per step) over
+    EXACTLY `steps` timed steps."""
     for i in range(warmup):
         fn(i % n_variants)
     torch.cuda.synchronize()
+    _settle(torch, fn, n_variants, max(4, min(steps, 64)))
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
@@ -54,6 +76,39 @@ def time_kernel(torch, fn, n_variants, steps, warmup):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
     return wall, e0.elapsed_time(e1) / steps
+
+
+def time_blocks(torch, legs, n_variants, block):
+    """Interleaved block timing of several legs (name -> fn): blocks of `block` launches of each leg
+    in turn, HIP events around every block, until every leg has BLOCK_MIN_MS of GPU time and
+    BLOCK_MIN_COUNT blocks.  Returns name -> (median ms per launch, min, max, blocks).  Interleaving
+    makes the legs see the same clocks, the median discards the blocks a frequency change fell into."""
+    names = list(legs)
+    for nm in names:
+        _settle(torch, legs[nm], n_variants, block)
+    per = {nm: [] for nm in names}
+    total = {nm: 0.0 for nm in names}
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    i = 0
+    while min(total.values()) < BLOCK_MIN_MS or len(per[names[0]]) < BLOCK_MIN_COUNT:
+        for nm in names:
+            fn = legs[nm]
+            e0.record()
+            for _ in range(block):
+                fn(i % n_variants)
+                i += 1
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+            per[nm].append(ms / block)
+            total[nm] += ms
+        if len(per[names[0]]) >= 400:
+            break
+    out = {}
+    for nm in names:
+        v = sorted(per[nm])
+        out[nm] = (v[len(v) // 2], v[0], v[-1], len(v))
+    return out
 
 
 def bench_quantize(torch, fmt, rows, cols, g, steps, warmup, seed, packed=False):
@@ -90,12 +145,16 @@ def bench_quantize(torch, fmt, rows, cols, g, steps, warmup, seed, packed=False)
         if st != 0:
             _engine.check(st, "bench quantize")
 
-    wall, ev = time_kernel(torch, run, n_buf, steps, warmup)
+    wall, ev_steps = time_kernel(torch, run, n_buf, steps, warmup)
+    ev, ev_min, ev_max, blocks = time_blocks(torch, {"q": run}, n_buf, max(20, min(steps, 100)))["q"]
     algo_bytes = rows * cols * (2 + 0.5 + 1.0 / group)
     return {
         "workload": f"{fmt}_quantize_{rows}x{cols}_had{g}" + ("_packed" if packed else ""),
         "ms_per_step": wall,
         "kernel_ms": ev,
+        "kernel_ms_min": ev_min,
+        "kernel_ms_over_steps": ev_steps,
+        "blocks": blocks,
         "algo_bytes": algo_bytes,
         "gbps": algo_bytes / (ev * 1e-3) / 1e9,
         "buffers": n_buf,
@@ -178,7 +237,30 @@ def bench_hbm_probe(torch, steps, warmup):
     return out
 
 
-def bench_linear(torch, fmt, m, n, k, g, steps, warmup, seed):
+def check_linear_output(torch, x, y, w, wq, ws, m, n, k, g, alpha, rows=48, cols=192):
+    """Outside every timed region: a seeded sample of the output the timed kernels just wrote against the
+    CPU oracle (quantize the sampled activation rows, dequantize, fp64 matmul against the sampled weight
+    rows), with the tolerance of the GEMM tests.  The oracle is the checker here, never the thing timed."""
+    from oracle import fpq_oracle as O
+    gen = torch.Generator().manual_seed(m + n)
+    ri = torch.randperm(m, generator=gen)[:min(rows, m)].sort().values
+    ci = torch.randperm(n, generator=gen)[:min(cols, n)].sort().values
+    xq, xs, _ = O.quantize_mx(x[ri.to(x.device)].cpu(), O.ROT_HADAMARD, g)
+    wq_s, ws_s = wq[ci.to(wq.device)].cpu(), ws[ci.to(ws.device)].cpu()
+    wq_o, ws_o, _ = O.quantize_mx(w[ci.to(w.device)].cpu(), O.ROT_HADAMARD, g)
+    if not (torch.equal(wq_o, wq_s) and torch.equal(ws_o, ws_s)):
+        raise RuntimeError("bench: quantized weights differ from the oracle's")
+    ref, mag = O.gemm_ref(xq, xs, wq_s, ws_s, alpha, "mxfp4")
+    got = y[ri.to(y.device)][:, ci.to(y.device)].cpu()
+    tol = 2.0 ** -8 * ref.abs() + 1e-5 * mag + 1e-6
+    ok = bool(((got.double() - ref).abs() <= tol).all())
+    exact = float((got == ref.to(torch.bfloat16)).float().mean())
+    if not ok:
+        raise RuntimeError("bench: the timed MXFP4 linear's output differs from the oracle beyond the tolerance")
+    return {"sample": f"{len(ri)}x{len(ci)} outputs", "within_tolerance": ok, "equal_to_bf16_of_fp64": round(exact, 4)}
+
+
+def bench_linear(torch, fmt, m, n, k, g, steps, warmup, seed, check=False):
     """Quantize activations + W4A4 GEMM (the body of FPQuantLinear.forward) through the C ABI.
     Weights are quantized once outside the timed region; activations rotate through buffers."""
     from fp_quant import _engine
@@ -235,7 +317,11 @@ def bench_linear(torch, fmt, m, n, k, g, steps, warmup, seed):
             if st != 0:
                 _engine.check(st, "bench packed gemm")
 
-        return _time_linear(torch, run_linear, run_gemm, fmt, m, n, k, g, group, n_buf, steps, warmup, "packed")
+        res = _time_linear(torch, run_linear, run_gemm, fmt, m, n, k, g, group, n_buf, steps, warmup, "packed")
+        if check:
+            run_linear(0)
+            res["output_check"] = check_linear_output(torch, xs_[0], ys[0], w, wq, ws, m, n, k, g, float(alpha))
+        return res
 
     def run_linear(i):
         a, b, c, d = p[i]
@@ -252,22 +338,40 @@ def bench_linear(torch, fmt, m, n, k, g, steps, warmup, seed):
         if st != 0:
             _engine.check(st, "bench gemm")
 
-    return _time_linear(torch, run_linear, run_gemm, fmt, m, n, k, g, group, n_buf, steps, warmup, "row-major")
+    res = _time_linear(torch, run_linear, run_gemm, fmt, m, n, k, g, group, n_buf, steps, warmup, "row-major")
+    if check and fmt == "mxfp4":
+        run_linear(0)
+        res["output_check"] = check_linear_output(torch, xs_[0], ys[0], w, wq, ws, m, n, k, g, float(alpha))
+    return res
 
 
 def _time_linear(torch, run_linear, run_gemm, fmt, m, n, k, g, group, n_buf, steps, warmup, layout):
-    wall, ev = time_kernel(torch, run_linear, n_buf, steps, warmup)
-    _, ev_gemm = time_kernel(torch, run_gemm, n_buf, steps, warmup)
+    wall, ev_steps = time_kernel(torch, run_linear, n_buf, steps, warmup)
+    block = max(10, min(steps, 100))
+    consistent = False
+    for _ in range(3):   # the GEMM alone cannot take longer than quantize + the same GEMM
+        t = time_blocks(torch, {"linear": run_linear, "gemm": run_gemm}, n_buf, block)
+        ev, ev_gemm = t["linear"][0], t["gemm"][0]
+        if ev_gemm <= ev * 1.01:
+            consistent = True
+            break
     flops = 2.0 * m * n * k
     gemm_bytes = n * k / 2 + n * k / group + m * k / 2 + m * k / group + 2.0 * m * n
     return {
         "workload": f"{fmt}_linear_M{m}_N{n}_K{k}_had{g}",
         "ms_per_step": wall,
+        "linear_ms_over_steps": ev_steps,
         "linear_ms": ev,
         "gemm_ms": ev_gemm,
+        "gemm_ms_min": t["gemm"][1],
+        "gemm_ms_max": t["gemm"][2],
+        "blocks": t["gemm"][3],
+        "block_launches": block,
+        "timing_consistent": consistent,
         "flops": flops,
         "gemm_bytes": gemm_bytes,
         "linear_tflops": flops / (ev * 1e-3) / 1e12,
+        "linear_tflops_over_steps": flops / (ev_steps * 1e-3) / 1e12,
         "gemm_tflops": flops / (ev_gemm * 1e-3) / 1e12,
         "gemm_gbps": gemm_bytes / (ev_gemm * 1e-3) / 1e9,
         "buffers": n_buf,
@@ -388,7 +492,7 @@ def bench_mfma_ceiling(torch, seed=4, iters=192):
 
 
 def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=(1, 32, 64), decode_steps=8,
-                    fmt="mxfp4", compiled_decode=False):
+                    fmt="mxfp4", compiled_decode=False, compact=False):
     """Forward passes of a random-weight Llama-3.1-8B-architecture model (transformers' LlamaForCausalLM) whose
     linears (all but lm_head) were replaced by MXFP4 FPQuantLinear with Hadamard-128: prefill tokens/s, decode
     tokens/s against a `seq`-token bf16 KV cache, and the share of GPU time spent inside the quantized linears
@@ -429,7 +533,7 @@ def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=
                 res[f"{b}x{sl}"] = round(best, 3)
         return res
 
-    bf16_ms = prefill_sweep()   # the unquantized model: nn.Linear in bf16 (hipBLASLt)
+    bf16_ms = None if compact else prefill_sweep()   # the unquantized model: nn.Linear in bf16 (hipBLASLt)
     qcfg = fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype(fmt), forward_method="abs_max",
                                   backward_dtype=fp_quant.FPQuantDtype.BF16,
                                   hadamard_group_size=128 if fmt == "mxfp4" else 16)
@@ -507,7 +611,7 @@ def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=
                 torch.cuda.empty_cache()
 
     measure(out, True)
-    mx_ms = prefill_sweep()
+    mx_ms = None if compact else prefill_sweep()
     if compiled_decode:
         out["decode_compiled"] = compiled_decode_ms(torch, model, cfg, seq, decode_batches, decode_steps, gen)
     # the same model with the RMSNorms and the SiLU*up of every block fused into the quantizers that consume
@@ -518,6 +622,10 @@ def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=
     if compiled_decode:   # the traced attention and MLP modules now call the group operators
         fused["decode_compiled"] = compiled_decode_ms(torch, model, cfg, seq, decode_batches, decode_steps, gen)
     out["fused_producers"] = fused
+    if compact:
+        del model
+        torch.cuda.empty_cache()
+        return out
     fused_ms = prefill_sweep()
     out["prefill_sweep_ms"] = {"bf16": bf16_ms, fmt: mx_ms, fmt + "_fused_producers": fused_ms,
                                "speedup_vs_bf16": {k: round(bf16_ms[k] / mx_ms[k], 2) for k in bf16_ms},
@@ -625,6 +733,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-e2e", action="store_true", help="skip the compact whole-model leg of the default run")
     ap.add_argument("--only", default="", help="comma list of workloads to run (for profiling one kernel): "
                     "nvfp4_quantize, mxfp4_quantize, mxfp4_linear_M2048, mxfp4_linear_M128, mxfp4_linear_M16, "
                     "mxfp4_linear_M1, nvfp4_linear, mfma_ceiling, hbm_probe, vendor_gemm, fused_producers, e2e_llama (whole-model "
@@ -692,7 +801,7 @@ def main():
 
     linears = {}
     for m in (2048, 128, 16, 1):
-        linears[m] = bench_linear(torch, "mxfp4", m, 14336, 4096, 128, args.steps, args.warmup, seed=2)
+        linears[m] = bench_linear(torch, "mxfp4", m, 14336, 4096, 128, args.steps, args.warmup, seed=2, check=True)
     nv = bench_linear(torch, "nvfp4", 4096, 24576, 4096, 16, max(10, args.steps // 10), max(2, args.warmup // 10), seed=3)
 
     ceiling = bench_mfma_ceiling(torch)
@@ -708,7 +817,8 @@ def main():
             "workload": v["workload"], "gemm_us": round(v["gemm_ms"] * 1e3, 3),
             "linear_us": round(v["linear_ms"] * 1e3, 3), "gemm_TFLOP/s": round(v["gemm_tflops"], 2),
             "mfma_frac": round(v["gemm_tflops"] / FP4_PEAK_TFLOPS, 4),
-            "gemm_GB/s": round(v["gemm_gbps"], 2), "hbm_frac": round(v["gemm_gbps"] / HBM_PEAK_GBS, 4)}
+            "gemm_GB/s": round(v["gemm_gbps"], 2), "hbm_frac": round(v["gemm_gbps"] / HBM_PEAK_GBS, 4),
+            "operand_layout": v["operand_layout"], "output_check": v.get("output_check", {}).get("within_tolerance")}
     kernels["nvfp4_gemm_M4096_gate_up"] = {
         "workload": nv["workload"], "gemm_us": round(nv["gemm_ms"] * 1e3, 3),
         "gemm_TFLOP/s": round(nv["gemm_tflops"], 2),
@@ -717,10 +827,12 @@ def main():
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f)  # HBM bytes per launch measured with rocprofv3 --pmc (see profiles/)
+            traffic = json.load(f)  # HBM bytes per launch from an earlier rocprofv3 --pmc run (see profiles/)
+    traffic_source = ("profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, run by the "
+                      "builder and scaled by a 256 MiB copy; a constant, not measured in this run")
     line = {
         "metric": METRIC,
-        "value": round(head["linear_tflops"], 2),
+        "value": round(head["linear_tflops_over_steps"], 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -732,7 +844,12 @@ def main():
         "dtype": "fp4",
         "data": "synthetic",
         "config": {"workload": head["workload"] + " (activation rotate+quantize then W4A4 GEMM)",
-                   "rotating_buffers": head["buffers"]},
+                   "rotating_buffers": head["buffers"],
+                   "timing": f"value and ms_per_step: exactly --steps timed steps after --warmup steps and {SETTLE_MS:.0f} ms "
+                             f"of untimed settling launches; kernel figures: median of interleaved blocks of "
+                             f"{head['block_launches']} launches covering at least {BLOCK_MIN_MS:.0f} ms per leg",
+                   "value_median_blocks": round(head["linear_tflops"], 2),
+                   "output_check": head.get("output_check")},
         "roofline": {
             "kernel": "MXFP4 W4A4 GEMM, M=2048 N=14336 K=4096",
             "bound": "mfma",
@@ -741,7 +858,11 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(head["gemm_tflops"] / FP4_PEAK_TFLOPS, 4),
             "traffic": traffic.get("mxfp4_gemm_M2048"),
+            "traffic_source": traffic_source,
             "kernel_us": round(head["gemm_ms"] * 1e3, 3),
+            "kernel_us_min_max": [round(head["gemm_ms_min"] * 1e3, 3), round(head["gemm_ms_max"] * 1e3, 3)],
+            "linear_us": round(head["linear_ms"] * 1e3, 3),
+            "timing_consistent": head["timing_consistent"],
             "algorithmic_flops_per_launch": int(head["flops"]),
             "operand_layout": head["operand_layout"],
             # what the matrix pipes alone sustain (register-resident operands): the clock drops with
@@ -757,11 +878,32 @@ def main():
             "unit": "GB/s",
             "frac": round(quant["gbps"] / HBM_PEAK_GBS, 4),
             "traffic": traffic.get("nvfp4_quantize"),
+            "traffic_source": traffic_source,
             "kernel_us": round(quant["kernel_ms"] * 1e3, 3),
             "algorithmic_bytes_per_launch": int(quant["algo_bytes"]),
         },
         "kernels": kernels,
     }
+    if not args.no_e2e:
+        # BASELINE config 5 in compact form: the whole-model forward (see bench_e2e_llama); an error here
+        # (e.g. a transformers version without the model class) is recorded, the kernel figures stand
+        try:
+            e2e = bench_e2e_llama(torch, compact=True)
+            line["e2e"] = {
+                "model": e2e["model"],
+                "prefill_4x2048_tokens_per_s": e2e["prefill"]["tokens_per_s"],
+                "prefill_linear_time_share": e2e["prefill"]["linear_time_share"],
+                "decode_tokens_per_s": {k: v["tokens_per_s"] for k, v in e2e["decode"].items()},
+                "decode_linear_time_share": {k: v["linear_time_share"] for k, v in e2e["decode"].items()},
+                "fused_producers": {"prefill_4x2048_tokens_per_s": e2e["fused_producers"]["prefill"]["tokens_per_s"],
+                                    "decode_tokens_per_s": {k: v["tokens_per_s"] for k, v in
+                                                            e2e["fused_producers"]["decode"].items()}},
+                "note": "eager PyTorch model, bf16 KV cache of 2048 tokens, everything outside the linears is stock "
+                        "PyTorch-ROCm; python bench.py --only e2e_llama adds the bf16 comparison and the batch sweep",
+            }
+        except Exception as e:  # noqa: BLE001
+            line["e2e"] = {"error": f"{type(e).__name__}: {str(e)[:300]}"}
+        torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline_linear(torch, 2048, 14336, 4096, 128, seed=2)
         line["cpu_baseline_quantize"] = cpu_baseline_quantize(torch, "nvfp4", 8192, 4096, 16, 1, 8192)

@@ -51,7 +51,27 @@ struct Prologue {
   uint32_t chunks_per_row;  // cols / 8
   uint32_t ld_first;        // row stride of x in 8-element chunks
   uint32_t ld_second;       // row stride of `second` in 8-element chunks
+  uint32_t packed_rows;     // generic kernel only: 0 = row-major codes and scales; otherwise the row count
+                            // padded to a multiple of 32, and codes / scales are written in the packed
+                            // operand layout of the GEMMs (padded rows: zero codes, zero scale bytes)
 };
+
+// Packed operand layout, as 32-bit word / byte indices: the 4 code bytes of the 8-element chunk `cc`
+// of `row`, and the scale byte of its group (MXFP4: group of 32 = 4 chunks, NVFP4: 16 = 2 chunks).
+__device__ __forceinline__ uint32_t packed_code_word(uint32_t row, uint32_t cc, uint32_t chunks_per_row) {
+  const uint32_t rt = row >> 5, r = row & 31u, ks = cc >> 3, kh = (cc >> 2) & 1u;
+  return ((rt * (chunks_per_row >> 3) + ks) * 64u + kh * 32u + r) * 4u + (cc & 3u);
+}
+template <int FMT>
+__device__ __forceinline__ uint32_t packed_scale_byte(uint32_t row, uint32_t cc, uint32_t chunks_per_row) {
+  const uint32_t rt = row >> 5, r = row & 31u, kb = cc >> 5;
+  if (FMT == kFmtMx) {
+    const uint32_t gi = (cc >> 2) & 7u;   // group of the 256-K block: byte q = gi / 2 of lane slot kh = gi % 2
+    return ((rt * (chunks_per_row >> 5) + kb) * 64u + (gi & 1u) * 32u + r) * 4u + (gi >> 1);
+  }
+  const uint32_t gi = (cc >> 1) & 15u;    // gi = 4 q + 2 kh + b: byte 2 q + b of lane slot kh
+  return ((rt * (chunks_per_row >> 5) + kb) * 64u + ((gi >> 1) & 1u) * 32u + r) * 8u + 2u * (gi >> 2) + (gi & 1u);
+}
 
 __device__ __forceinline__ float bf16_rne(float v) {
   uint32_t b = __float_as_uint(v);
@@ -285,6 +305,16 @@ __device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint3
     packed |= e2m1_code<ZERO>(v) << (4 * i);
   }
 
+  if (!QUEST && pro.packed_rows != 0u) {
+    if (chunk < pro.packed_rows * chunks_per_row) {
+      const uint32_t row = chunk / chunks_per_row, cc = chunk - row * chunks_per_row;
+      codes[packed_code_word(row, cc, chunks_per_row)] = active ? packed : 0u;
+      if ((cc & (GROUP / 8 - 1)) == 0u) {
+        scales[packed_scale_byte<FMT>(row, cc, chunks_per_row)] = active ? (uint8_t)gs.byte : (uint8_t)0;
+      }
+    }
+    return;
+  }
   if (active) {
     codes[chunk] = packed;
     if ((chunk & (GROUP / 8 - 1)) == 0u) {
@@ -411,14 +441,17 @@ static int dispatch_quest(const void* x, int64_t rows, int64_t cols, int rot_kin
 template <int G, int FMT, int ROT>
 static int launch_lane8(const void* x, int64_t rows, int64_t cols, float norm, const float* gsp,
                         void* codes, void* scales, int64_t scale_rows, int64_t scale_stride,
-                        int zero_policy, hipStream_t stream, const void* h = nullptr) {
+                        int zero_policy, hipStream_t stream, const void* h = nullptr, bool packed = false) {
   const int64_t n_chunks = rows * cols / 8;
-  const dim3 grid((unsigned)((n_chunks + 255) / 256)), block(256);
+  Prologue pro{};
+  pro.packed_rows = packed ? (uint32_t)((rows + 31) / 32 * 32) : 0u;
+  const int64_t threads = packed ? (int64_t)pro.packed_rows * (cols / 8) : n_chunks;
+  const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
   auto args = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint4*)x, (uint32_t*)codes,
                        (uint8_t*)scales, (uint32_t)n_chunks, (uint32_t)(cols / 8), (uint32_t)rows,
                        (uint32_t)scale_rows, (uint32_t)scale_stride, norm, gsp, (const uint16_t*)h,
-                       (uint8_t*)nullptr, Prologue{});
+                       (uint8_t*)nullptr, pro);
   };
   if (zero_policy == FPQ_ZERO_REFERENCE) {
     args(quantize_lane8_kernel<G, FMT, ROT, kZeroReference>);
@@ -933,6 +966,8 @@ static int launch_stream_packed(const void* x, int64_t rows, int64_t cols, float
   return (int)hipGetLastError();
 }
 
+constexpr int64_t kPackedFewRows = 64;
+
 template <int FMT>
 static int dispatch_packed(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
                            const float* gsp, void* codes, void* scales, int zero_policy, void* stream_) {
@@ -947,9 +982,18 @@ static int dispatch_packed(const void* x, int64_t rows, int64_t cols, int rot_ki
   if (cols % 256 != 0) return FPQ_E_SHAPE;
   if (rows * cols >= (int64_t)1 << 34) return FPQ_E_SHAPE;
   if (((uintptr_t)x & 15u) || ((uintptr_t)codes & 15u) || ((uintptr_t)scales & 3u)) return FPQ_E_ALIGN;
-#define FPQ_LAUNCH_PACKED(GG, RR) \
-  return launch_stream_packed<GG, RR, kProNone, FMT>(x, rows, cols, norm, codes, scales, zero_policy, stream, \
-                                                     Prologue{}, gsp)
+  // A few rows (decode): the generic kernel spreads a row over 512 lanes and finishes sooner than the
+  // streaming kernel, whose wave tile is 32 rows deep; it writes the same packed bytes.
+  const bool few = rows <= kPackedFewRows;
+  constexpr int64_t kGroupCols = FMT == kFmtMx ? 32 : 16;
+#define FPQ_LAUNCH_PACKED(GG, RR)                                                                                 \
+  {                                                                                                               \
+    if (few)                                                                                                      \
+      return launch_lane8<GG, FMT, RR>(x, rows, cols, norm, gsp, codes, scales, rows, cols / kGroupCols,          \
+                                       zero_policy, stream, nullptr, true);                                       \
+    return launch_stream_packed<GG, RR, kProNone, FMT>(x, rows, cols, norm, codes, scales, zero_policy, stream,   \
+                                                       Prologue{}, gsp);                                          \
+  }
   if (rot_kind == FPQ_ROT_IDENTITY) {
     FPQ_LAUNCH_PACKED(32, FPQ_ROT_IDENTITY);
   } else if (rot_kind == FPQ_ROT_HADAMARD) {
@@ -1040,7 +1084,8 @@ static int launch_lane8_prologue(const void* x, int64_t rows, int64_t cols, floa
                                  void* codes, void* scales, int64_t scale_rows, int64_t scale_stride,
                                  int zero_policy, hipStream_t stream, const Prologue& pro) {
   const int64_t n_chunks = rows * cols / 8;
-  const dim3 grid((unsigned)((n_chunks + 255) / 256)), block(256);
+  const int64_t threads = pro.packed_rows ? (int64_t)pro.packed_rows * (cols / 8) : n_chunks;
+  const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
   auto args = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint4*)x, (uint32_t*)codes,
                        (uint8_t*)scales, (uint32_t)n_chunks, (uint32_t)(cols / 8), (uint32_t)rows,
@@ -1115,7 +1160,7 @@ static int dispatch_prologue(const void* x, int64_t ld_first, const void* second
   if (PRO == kProSiluMul) {
     if (const int st = ensure_silu_table(stream)) return st;
   }
-  Prologue pro;
+  Prologue pro{};
   pro.row_scale = row_scale;
   pro.col_scale = (const uint4*)col_scale;
   pro.second = (const uint4*)second;
@@ -1170,7 +1215,7 @@ static int dispatch_prologue_packed(const void* x, int64_t ld_first, const void*
   if (PRO == kProSiluMul) {
     if (const int st = ensure_silu_table(stream)) return st;
   }
-  Prologue pro;
+  Prologue pro{};
   pro.row_scale = row_scale;
   pro.col_scale = (const uint4*)col_scale;
   pro.second = (const uint4*)second;
@@ -1178,8 +1223,16 @@ static int dispatch_prologue_packed(const void* x, int64_t ld_first, const void*
   pro.chunks_per_row = (uint32_t)(cols / 8);
   pro.ld_first = (uint32_t)(ld_first / 8);
   pro.ld_second = (uint32_t)(ld_second / 8);
-#define FPQ_LAUNCH_PRO_PACKED(GG, RR) \
-  return launch_stream_packed<GG, RR, PRO>(x, rows, cols, norm, codes, scales, zero_policy, stream, pro)
+  pro.packed_rows = 0u;
+  const bool few = rows <= kPackedFewRows;
+  if (few) pro.packed_rows = (uint32_t)((rows + 31) / 32 * 32);
+#define FPQ_LAUNCH_PRO_PACKED(GG, RR)                                                                          \
+  {                                                                                                            \
+    if (few)                                                                                                   \
+      return launch_lane8_prologue<GG, kFmtMx, RR, PRO>(x, rows, cols, norm, nullptr, codes, scales, rows,     \
+                                                        cols / 32, zero_policy, stream, pro);                  \
+    return launch_stream_packed<GG, RR, PRO>(x, rows, cols, norm, codes, scales, zero_policy, stream, pro);    \
+  }
   if (rot_kind == FPQ_ROT_IDENTITY) FPQ_LAUNCH_PRO_PACKED(32, FPQ_ROT_IDENTITY);
   switch (g) {
     case 16: FPQ_LAUNCH_PRO_PACKED(16, FPQ_ROT_HADAMARD);

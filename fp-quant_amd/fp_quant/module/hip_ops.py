@@ -311,8 +311,9 @@ def rotated_absmax(x: torch.Tensor, hadamard_matrix: torch.Tensor, amax: Optiona
 PACKED_MIN_M = 48          # GEMM operator on row-major operands (pays for re-tiling the activations)
 NV_PACKED_MIN_M = 65       # NVFP4 fused linear: from here on (and while the 128x128 tiles apply) packed;
 #                            below, the split-K weight-streaming kernel on row-major operands is faster
-PACKED_LINEAR_MIN_M = 25   # fused linear: activations are quantized straight into the packed layout
-#                            (below, the weight-streaming split-K kernel on row-major operands is faster)
+# fused linear: activations are quantized straight into the packed layout; the weight-streaming
+# kernel on packed operands serves the few-row (decode) calls; FPQ_PACKED_MIN_ROWS raises the bar
+PACKED_LINEAR_MIN_M = int(os.environ.get("FPQ_PACKED_MIN_ROWS", "1"))
 
 
 def packed_weights_enabled() -> bool:

@@ -81,7 +81,7 @@ PACKED_CASES = [("hadamard", 16), ("hadamard", 32), ("hadamard", 64), ("hadamard
 
 @pytest.mark.parametrize("rot,g", PACKED_CASES)
 @pytest.mark.parametrize("kind", ["rmsnorm", "silu_mul"])
-@pytest.mark.parametrize("rows,cols", [(1, 256), (70, 512), (300, 1024)])
+@pytest.mark.parametrize("rows,cols", [(1, 256), (20, 768), (70, 512), (300, 1024)])
 def test_fused_quantize_packed_bit_exact(kind, rot, g, rows, cols):
     """The streaming kernel with a prologue: packed codes and scales (ragged last row tile, strided
     inputs, extreme exponents that take the slow path) and the bf16 by-product."""
@@ -105,7 +105,7 @@ def test_fused_quantize_packed_bit_exact(kind, rot, g, rows, cols):
     okind = O.ROT_HADAMARD if rot == "hadamard" else O.ROT_IDENTITY
     wc, ws, _ = O.quantize_mx(want_v, okind, g, float(O.hadamard_matrix(g)[0, 0]))
     want_c, want_s = pack_by_definition(wc, ws, cols)
-    lds = dict(ld_a=cols + 64, ld_b=2 * cols) if rows == 70 else {}
+    lds = dict(ld_a=cols + 64, ld_b=2 * cols) if rows in (20, 70) else {}
     pc, ps, out = capi.fused_quantize_packed(kind, a, b, g=g, rot=rot, **lds)
     assert torch.equal(out.view(torch.int16), want_v.view(torch.int16))
     assert torch.equal(pc, want_c) and torch.equal(ps, want_s)

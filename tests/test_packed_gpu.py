@@ -50,13 +50,15 @@ CASES = [("hadamard", 128), ("hadamard", 64), ("hadamard", 32), ("hadamard", 16)
 
 @pytest.mark.parametrize("rot,g", CASES)
 @pytest.mark.parametrize("policy", [_engine.ZERO_REFERENCE, _engine.ZERO_SIGNED])
-def test_quantize_packed_bit_exact(rot, g, policy):
-    rows, cols = 70, 512  # ragged last row tile
+@pytest.mark.parametrize("rows", [70, 1, 13, 24, 64, 65])   # up to 64 rows: the generic kernel writes the packed layout
+def test_quantize_packed_bit_exact(rot, g, policy, rows):
+    cols = 512  # 70 rows: ragged last row tile
     x = make_outlier_normal(rows, cols, 11 * g + len(rot))
-    x[3, 64:96] = 0.0            # a zero group
-    x[5, :32] = -0.0
-    x[7] *= 2.0 ** -110          # exponents outside the fast range
-    x[9] *= 2.0 ** 105
+    x[3 % rows, 64:96] = 0.0     # a zero group
+    x[5 % rows, :32] = -0.0
+    if rows > 9:
+        x[7] *= 2.0 ** -110      # exponents outside the fast range
+        x[9] *= 2.0 ** 105
     okind = {"hadamard": O.ROT_HADAMARD, "identity": O.ROT_IDENTITY, "gsr": O.ROT_GSR}[rot]
     norm = float(O.hadamard_matrix(g)[0, 0])
     wc, ws, _ = O.quantize_mx(x, okind, g, norm, zero_nibble=policy)
@@ -212,12 +214,14 @@ def test_gemm_packed_residual_equals_gemm_then_add(m, n, k, bias):
 @pytest.mark.parametrize("rot,g", [("hadamard", 16), ("hadamard", 32), ("hadamard", 64), ("hadamard", 128),
                                    ("identity", 16), ("gsr", 32)])
 @pytest.mark.parametrize("policy", [0, 1])
-def test_quantize_nv_packed_bit_exact(rot, g, policy):
-    rows, cols = 70, 512  # ragged last row tile
+@pytest.mark.parametrize("rows", [70, 1, 13, 64])
+def test_quantize_nv_packed_bit_exact(rot, g, policy, rows):
+    cols = 512  # 70 rows: ragged last row tile
     x = make_outlier_normal(rows, cols, 13 * g + len(rot))
-    x[3, 64:96] = 0.0            # zero groups
-    x[5, :32] = -0.0
-    x[7] *= 2.0 ** -20           # E4M3 scales that underflow to zero
+    x[3 % rows, 64:96] = 0.0     # zero groups
+    x[5 % rows, :32] = -0.0
+    if rows > 7:
+        x[7] *= 2.0 ** -20       # E4M3 scales that underflow to zero
     okind = {"hadamard": O.ROT_HADAMARD, "identity": O.ROT_IDENTITY, "gsr": O.ROT_GSR}[rot]
     norm = float(O.hadamard_matrix(g)[0, 0])
     for gs in (40.0, 2.0 ** 70):  # the second takes the generic per-element path
