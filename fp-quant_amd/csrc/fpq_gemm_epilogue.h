@@ -58,6 +58,87 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
 }
 
+// The epilogue for a wave tile that lies inside the output (no row or column of it is cut off) with
+// N a multiple of 8 and an 8-byte aligned bias: same values as wave_tile_store below with as few
+// instructions as possible, because a workgroup's four waves issue them alone -- one instruction every
+// few cycles per wave, with the matrix pipes idle.  Bias values are fetched with 8-byte loads before
+// the barrier, the staging addresses are one register plus immediates, the global addresses one
+// uniform base plus a 32-bit lane offset, and nothing is bounds-checked.
+template <int TN, int TM, int NWAVES, bool BIAS, bool RESID>
+__device__ __forceinline__ void wave_tile_store_interior(const v16f (&acc)[TN][TM], uint8_t* smem,
+                                                         uint16_t* __restrict__ y,
+                                                         const uint16_t* __restrict__ bias, float alpha,
+                                                         int n0, int m0, int wave, int lane, int N,
+                                                         const uint16_t* __restrict__ residual) {
+  const int r32 = lane & 31, kh = lane >> 5;
+  constexpr int WT_N = TN * 32, WT_M = TM * 32;
+  constexpr int kRowBytes = WT_N * 2;
+  constexpr int kStride = kRowBytes + 16;
+  uint2 braw[BIAS ? TN * 4 : 1];
+  if (BIAS) {
+#pragma unroll
+    for (int ig = 0; ig < TN * 4; ++ig) braw[ig] = *(const uint2*)(bias + n0 + ig * 8 + 4 * kh);
+  }
+  __syncthreads();                                   // every wave is done reading operands
+  uint8_t* stg = smem + wave * (WT_M * kStride);
+  uint8_t* lane_w = stg + r32 * kStride + kh * 8;
+#pragma unroll
+  for (int i = 0; i < TN; ++i) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+#pragma unroll
+      for (int j = 0; j < TM; ++j) {
+        uint32_t lo = pack_bf16x2(acc[i][j][4 * g + 0] * alpha, acc[i][j][4 * g + 1] * alpha);
+        uint32_t hi = pack_bf16x2(acc[i][j][4 * g + 2] * alpha, acc[i][j][4 * g + 3] * alpha);
+        if (BIAS) {
+          const uint2 b = braw[i * 4 + g];
+          lo = pack_bf16x2(__uint_as_float(lo << 16) + __uint_as_float(b.x << 16),
+                           __uint_as_float(lo & 0xffff0000u) + __uint_as_float(b.x & 0xffff0000u));
+          hi = pack_bf16x2(__uint_as_float(hi << 16) + __uint_as_float(b.y << 16),
+                           __uint_as_float(hi & 0xffff0000u) + __uint_as_float(b.y & 0xffff0000u));
+        }
+        *(uint2*)(lane_w + j * 32 * kStride + (i * 32 + 8 * g) * 2) = make_uint2(lo, hi);
+      }
+    }
+  }
+  constexpr int kLpr = kRowBytes / 16 <= 16 ? 16 : 32;
+  constexpr int kRpi = 64 / kLpr;
+  constexpr int kIters = WT_M / kRpi;
+  constexpr int kBatch = kIters % 8 == 0 ? 8 : (kIters % 4 == 0 ? 4 : 1);
+  static_assert(kRowBytes / 16 <= 32 && WT_M % kRpi == 0, "unsupported wave tile shape");
+  const int rr = lane / kLpr, cc = lane % kLpr;
+  if (cc * 16 >= kRowBytes) return;
+  const uint8_t* lane_r = stg + rr * kStride + cc * 16;
+  uint8_t* gbase = (uint8_t*)(y + (size_t)m0 * N + n0);                       // uniform
+  const uint8_t* rbase = (const uint8_t*)(residual + (size_t)m0 * N + n0);    // uniform (unused without RESID)
+  const uint32_t goff = (uint32_t)(rr * N + cc * 8) * 2u;                     // < WT_M * N * 2 < 2^31
+  const uint32_t gstep = (uint32_t)(kRpi * N) * 2u;
+#pragma unroll
+  for (int p0 = 0; p0 < kIters; p0 += kBatch) {
+    uint4 vb[kBatch], rb[RESID ? kBatch : 1];
+#pragma unroll
+    for (int q = 0; q < kBatch; ++q) vb[q] = *(const uint4*)(lane_r + (p0 + q) * kRpi * kStride);
+    if (RESID) {
+#pragma unroll
+      for (int q = 0; q < kBatch; ++q) rb[q] = *(const uint4*)(rbase + goff + (uint32_t)(p0 + q) * gstep);
+    }
+#pragma unroll
+    for (int q = 0; q < kBatch; ++q) {
+      uint4 v = vb[q];
+      if (RESID) {  // a separate bf16 add after the GEMM: one more rounding
+        const uint32_t a[4] = {v.x, v.y, v.z, v.w}, b[4] = {rb[q].x, rb[q].y, rb[q].z, rb[q].w};
+        uint32_t o[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          o[u] = pack_bf16x2(__uint_as_float(a[u] << 16) + __uint_as_float(b[u] << 16),
+                             __uint_as_float(a[u] & 0xffff0000u) + __uint_as_float(b[u] & 0xffff0000u));
+        v = make_uint4(o[0], o[1], o[2], o[3]);
+      }
+      *(uint4*)(gbase + goff + (uint32_t)(p0 + q) * gstep) = v;
+    }
+  }
+}
+
 // Epilogue of the LDS-tiled kernels.  A wave owns TN x TM accumulator tiles of 32 x 32; register
 // v of tile (i, j) is y[m][n] with m = j*32 + r32 and n = i*32 + 8*(v/4) + 4*kh + v%4 relative to
 // the wave's origin (m0, n0).  The wave's part goes through its share of the (now idle) LDS as
@@ -75,6 +156,17 @@ __device__ __forceinline__ void wave_tile_store(const v16f (&acc)[TN][TM], uint8
   constexpr int kRowBytes = WT_N * 2;
   constexpr int kStride = kRowBytes + 16;            // bytes per staged row (+16: spread banks)
   static_assert(NWAVES * WT_M * kStride <= LDS_BYTES, "epilogue staging does not fit in LDS");
+  // wave-uniform: the whole wave tile is inside the output and the vector paths apply
+  if (m0 + WT_M <= M && n0 + WT_N <= N && (N & 7) == 0 && ((uintptr_t)bias & 7u) == 0) {
+    if (bias) {
+      if (residual) wave_tile_store_interior<TN, TM, NWAVES, true, true>(acc, smem, y, bias, alpha, n0, m0, wave, lane, N, residual);
+      else wave_tile_store_interior<TN, TM, NWAVES, true, false>(acc, smem, y, bias, alpha, n0, m0, wave, lane, N, residual);
+    } else {
+      if (residual) wave_tile_store_interior<TN, TM, NWAVES, false, true>(acc, smem, y, bias, alpha, n0, m0, wave, lane, N, residual);
+      else wave_tile_store_interior<TN, TM, NWAVES, false, false>(acc, smem, y, bias, alpha, n0, m0, wave, lane, N, residual);
+    }
+    return;
+  }
   __syncthreads();                                   // every wave is done reading operands
   uint8_t* stg = smem + wave * (WT_M * kStride);
 #pragma unroll
@@ -106,37 +198,47 @@ __device__ __forceinline__ void wave_tile_store(const v16f (&acc)[TN][TM], uint8
   static_assert(kRowBytes / 16 <= 32 && WT_M % kRpi == 0, "unsupported wave tile shape");
   const int rr = lane / kLpr, cc = lane % kLpr;
   const bool vec_ok = (N & 7) == 0;
-#pragma unroll 4
-  for (int p = 0; p < WT_M / kRpi; ++p) {
-    const int ml = p * kRpi + rr;
-    if (cc * 16 >= kRowBytes) continue;
-    uint4 v = *(const uint4*)(stg + ml * kStride + cc * 16);
-    const int m = m0 + ml, n = n0 + cc * 8;
-    if (m >= M || n >= N) continue;
-    uint16_t* dst = y + (size_t)m * N + n;
-    if (vec_ok && n + 7 < N) {
-      if (residual) {  // a separate bf16 add after the GEMM: one more rounding
-        const uint4 rv = *(const uint4*)(residual + (size_t)m * N + n);
-        const uint32_t a[4] = {v.x, v.y, v.z, v.w}, b[4] = {rv.x, rv.y, rv.z, rv.w};
-        uint32_t o[4];
+  // Batches of kBatch rows-per-instruction groups: all LDS reads of a batch are issued before its
+  // first store, so the stores do not each wait for an LDS round trip.
+  constexpr int kIters = WT_M / kRpi;
+  constexpr int kBatch = kIters % 8 == 0 ? 8 : (kIters % 4 == 0 ? 4 : 1);
+  if (cc * 16 >= kRowBytes) return;
+#pragma unroll 1
+  for (int p0 = 0; p0 < kIters; p0 += kBatch) {
+    uint4 vb[kBatch];
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
-          o[u] = pack_bf16x2(__uint_as_float(a[u] << 16) + __uint_as_float(b[u] << 16),
-                             __uint_as_float(a[u] & 0xffff0000u) + __uint_as_float(b[u] & 0xffff0000u));
-        v = make_uint4(o[0], o[1], o[2], o[3]);
-      }
-      *(uint4*)dst = v;
-    } else {
-      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    for (int q = 0; q < kBatch; ++q) vb[q] = *(const uint4*)(stg + ((p0 + q) * kRpi + rr) * kStride + cc * 16);
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        if (n + u < N) {
-          uint32_t h = (w[u >> 1] >> (16 * (u & 1))) & 0xffffu;
-          if (residual) {
-            const float sum = __uint_as_float(h << 16) + __uint_as_float((uint32_t)residual[(size_t)m * N + n + u] << 16);
-            h = pack_bf16x2(sum, 0.0f) & 0xffffu;
+    for (int q = 0; q < kBatch; ++q) {
+      uint4 v = vb[q];
+      const int ml = (p0 + q) * kRpi + rr;
+      const int m = m0 + ml, n = n0 + cc * 8;
+      if (m >= M || n >= N) continue;
+      uint16_t* dst = y + (size_t)m * N + n;
+      if (vec_ok && n + 7 < N) {
+        if (residual) {  // a separate bf16 add after the GEMM: one more rounding
+          const uint4 rv = *(const uint4*)(residual + (size_t)m * N + n);
+          const uint32_t a[4] = {v.x, v.y, v.z, v.w}, b[4] = {rv.x, rv.y, rv.z, rv.w};
+          uint32_t o[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            o[u] = pack_bf16x2(__uint_as_float(a[u] << 16) + __uint_as_float(b[u] << 16),
+                               __uint_as_float(a[u] & 0xffff0000u) + __uint_as_float(b[u] & 0xffff0000u));
+          v = make_uint4(o[0], o[1], o[2], o[3]);
+        }
+        *(uint4*)dst = v;
+      } else {
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (n + u < N) {
+            uint32_t h = (w[u >> 1] >> (16 * (u & 1))) & 0xffffu;
+            if (residual) {
+              const float sum = __uint_as_float(h << 16) + __uint_as_float((uint32_t)residual[(size_t)m * N + n + u] << 16);
+              h = pack_bf16x2(sum, 0.0f) & 0xffffu;
+            }
+            dst[u] = (uint16_t)h;
           }
-          dst[u] = (uint16_t)h;
         }
       }
     }
