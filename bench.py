@@ -491,6 +491,83 @@ def bench_mfma_ceiling(torch, seed=4, iters=192):
     return out
 
 
+def bench_power(torch, seconds=3.0):
+    """Socket power and per-XCD clocks (amd-smi) while one kernel runs back to back for `seconds`: the packed
+    MXFP4 GEMM at M=2048 N=14336 K=4096 on quantized Gaussian data, the register-resident MFMA loop on the same
+    operand bits and on zeros, and a plain 256 MiB copy.  Shows which limit the GEMM runs at: the package power
+    cap (the clock the firmware grants falls) or the matrix pipes' own throttle (power below the cap)."""
+    import re
+    import subprocess
+    import threading
+    from fp_quant import _engine
+    lib = _engine.lib()
+    dev = torch.device("cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+    norm = float(torch.tensor(128 ** -0.5, dtype=torch.bfloat16))
+    m, n, k = 2048, 14336, 4096
+    gen = torch.Generator().manual_seed(2)
+    w = (torch.randn(n, k, generator=gen) * 0.02).to(torch.bfloat16).to(dev)
+    x = torch.randn(m, k, generator=gen).to(torch.bfloat16).to(dev)
+
+    def quantize(t, rows):
+        pc = torch.empty(lib.fpq_packed_codes_bytes(rows, k), dtype=torch.uint8, device=dev)
+        ps = torch.empty(lib.fpq_packed_scales_bytes(rows, k), dtype=torch.uint8, device=dev)
+        _engine.check(lib.fpq_quantize_mx_packed(t.data_ptr(), rows, k, 0, 128, norm, pc.data_ptr(), ps.data_ptr(), 0, st),
+                      "quantize")
+        return pc, ps
+
+    wp, ws = quantize(w, n)
+    xp, xs = quantize(x, m)
+    alpha = torch.tensor([0.111328125], device=dev)
+    y = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    blocks = torch.cuda.get_device_properties(0).multi_processor_count
+    words = wp.view(torch.int32)[:blocks * 256 * 32].contiguous()
+    zeros = torch.zeros_like(words)
+    sink = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+    clocks = torch.empty(blocks * 2, dtype=torch.int64, device=dev)
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 256)
+    dst = torch.empty_like(src)
+    legs = {
+        "mxfp4_gemm_M2048": lambda: lib.fpq_gemm_mxf4_packed(xp.data_ptr(), xs.data_ptr(), wp.data_ptr(), ws.data_ptr(),
+                                                             alpha.data_ptr(), None, y.data_ptr(), m, n, k, st),
+        "mfma_only_quantized_bits": lambda: lib.fpq_test_mfma_rate(words.data_ptr(), blocks, 192, sink.data_ptr(),
+                                                                   clocks.data_ptr(), st),
+        "mfma_only_zeros": lambda: lib.fpq_test_mfma_rate(zeros.data_ptr(), blocks, 192, sink.data_ptr(),
+                                                          clocks.data_ptr(), st),
+        "copy_256MiB": lambda: dst.copy_(src),
+    }
+
+    def sample():
+        try:
+            out = subprocess.run(["amd-smi", "metric", "-p", "-c"], capture_output=True, text=True, timeout=20).stdout
+        except Exception as e:  # noqa: BLE001
+            return {"error": f"{type(e).__name__}: {e}"}
+        watts = re.search(r"SOCKET_POWER:\s*(\d+)\s*W", out)
+        clk = [int(v) for v in re.findall(r"GFX_\d+:\s*CLK:\s*(\d+)\s*MHz", out)]
+        return {"socket_power_W": int(watts.group(1)) if watts else None,
+                "xcd_clock_MHz_min_max": [min(clk), max(clk)] if clk else None}
+
+    res = {}
+    for name, fn in legs.items():
+        got = []
+
+        def sampler():
+            time.sleep(seconds * 0.5)
+            got.append(sample())
+
+        th = threading.Thread(target=sampler)
+        th.start()
+        launches, t0 = 0, time.perf_counter()
+        while th.is_alive() or time.perf_counter() - t0 < seconds:
+            for _ in range(200):
+                fn()
+            torch.cuda.synchronize()
+            launches += 200
+        th.join()
+        res[name] = dict(got[0], us_per_launch=round((time.perf_counter() - t0) / launches * 1e6, 2))
+    return res
+
+
 def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=(1, 32, 64), decode_steps=8,
                     fmt="mxfp4", compiled_decode=False, compact=False):
     """Forward passes of a random-weight Llama-3.1-8B-architecture model (transformers' LlamaForCausalLM) whose
@@ -736,8 +813,8 @@ def main():
     ap.add_argument("--no-e2e", action="store_true", help="skip the compact whole-model leg of the default run")
     ap.add_argument("--only", default="", help="comma list of workloads to run (for profiling one kernel): "
                     "nvfp4_quantize, mxfp4_quantize, mxfp4_linear_M2048, mxfp4_linear_M128, mxfp4_linear_M16, "
-                    "mxfp4_linear_M1, nvfp4_linear, mfma_ceiling, hbm_probe, vendor_gemm, fused_producers, e2e_llama (whole-model "
-                    "forward); the last four are not part of the default run")
+                    "mxfp4_linear_M1, nvfp4_linear, mfma_ceiling, hbm_probe, vendor_gemm, fused_producers, power (socket power and clocks by "
+                    "kernel), e2e_llama (whole-model forward); from hbm_probe on they are not part of the default run")
     ap.add_argument("--e2e-layers", type=int, default=32, help="decoder layers of the --only e2e_llama model")
     ap.add_argument("--e2e-format", default="mxfp4", choices=("mxfp4", "nvfp4"), help="format of the --only e2e_llama model")
     ap.add_argument("--e2e-compiled-decode", action="store_true",
@@ -784,6 +861,8 @@ def main():
                                                compiled_decode=args.e2e_compiled_decode)
         if "mfma_ceiling" in only:
             out["mfma_ceiling"] = bench_mfma_ceiling(torch)
+        if "power" in only:
+            out["power"] = bench_power(torch)
         if "hbm_probe" in only:
             out["hbm_probe"] = bench_hbm_probe(torch, args.steps, args.warmup)
         if "vendor_gemm" in only:

@@ -29,6 +29,21 @@ extern "C" int fpq_device_supported(int device) {
   return strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 0;
 }
 
+namespace fpq {
+int ensure_silu_table(hipStream_t stream);   // fpq_quantize.hip
+int scratch_address(void** out);             // fpq_gemm_stream.hip
+}  // namespace fpq
+
+extern "C" int fpq_prepare_device(void* stream) {
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  const hipError_t err = hipStreamIsCapturing((hipStream_t)stream, &cap);
+  if (err != hipSuccess) return (int)err;
+  if (cap != hipStreamCaptureStatusNone) return FPQ_E_UNSUPPORTED;   // it has to run, not be recorded
+  if (const int st = fpq::ensure_silu_table((hipStream_t)stream)) return st;
+  void* scratch = nullptr;
+  return fpq::scratch_address(&scratch);
+}
+
 extern "C" int fpq_stream_capture_id(void* stream, unsigned long long* id) {
   if (!id) return FPQ_E_NULL;
   hipStreamCaptureStatus status = hipStreamCaptureStatusNone;

@@ -351,7 +351,7 @@ static std::atomic<void*> g_scratch_ptr[kMaxDevices];
 
 // Device address of `scratch` on the current device (looked up on the first call per device; two
 // threads racing on that first call store the same address).
-static int scratch_address(void** out) {
+int scratch_address(void** out) {   // also called by fpq_prepare_device (fpq_capi.hip)
   int device = -1;
   hipError_t err = hipGetDevice(&device);
   if (err != hipSuccess) return (int)err;

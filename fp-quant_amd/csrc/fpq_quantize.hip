@@ -1103,7 +1103,7 @@ static int launch_lane8_prologue(const void* x, int64_t rows, int64_t cols, floa
 // Fills g_silu_table once per device.  The first call on a device builds the table on the caller's
 // stream and waits for it, so that calls on other streams can rely on it afterwards; while a stream
 // is being captured the build is recorded into the capture instead and nothing is remembered.
-static int ensure_silu_table(hipStream_t stream) {
+int ensure_silu_table(hipStream_t stream) {   // also called by fpq_prepare_device (fpq_capi.hip)
   static std::atomic<uint64_t> built{0};  // bit d: device d holds the table (devices >= 64 rebuild every call)
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);

@@ -50,6 +50,7 @@ _SIGNATURES = {
     "fpq_gemm_mxf4_packed_workspace_bytes": ([_I64, _I64, _I64], _I64),
     "fpq_gemm_mxf4_packed_splitk": ([_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P, _I64, _P], _I),
     "fpq_gemm_mxf4_packed_residual": ([_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _I),
+    "fpq_prepare_device": ([_P], _I),
     "fpq_gemm_mxf4_packed_noalloc_max_rows": ([], _I64),
     "fpq_gemm_mxf4_packed_noalloc": ([_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _I),
 }
@@ -103,3 +104,60 @@ def check(status: int, what: str) -> None:
     if status < 0:
         raise ValueError(f"{what}: {msg} (fpq status {status})")
     raise RuntimeError(f"{what}: HIP error {status}: {msg}")
+
+
+# ---- rotation matrices: shared by the fp_quant operators and the qutlass stand-in -------------------------
+def tensor_version(t):
+    """The tensor's in-place modification counter, or None for tensors created under
+    torch.inference_mode(), which have none."""
+    try:
+        return t._version
+    except RuntimeError:
+        return None
+
+
+def sylvester_signs(g: int):
+    """+-1 entries of the Sylvester Hadamard matrix of size g (scipy.linalg.hadamard order)."""
+    import torch
+    idx = torch.arange(g)
+    anded = idx[:, None] & idx[None, :]
+    pop = torch.zeros_like(anded)
+    for b in range(8):
+        pop += (anded >> b) & 1
+    return (1 - 2 * (pop & 1)).to(torch.float32)
+
+
+def classify_rotation(h):
+    """(rotation kind, norm) of a [g, g] matrix: the Hadamard / identity / sequency-ordered matrices the
+    reference builds (inference_lib/src/fp_quant/module/linear.py:24-41) are applied as butterflies,
+    anything else as a matrix product.  The result is remembered on the tensor object itself, keyed by
+    its storage address and modification counter, so the one device->host copy it needs happens once
+    per matrix; a tensor without a counter (made under torch.inference_mode()) is classified on every call."""
+    import torch
+    version = tensor_version(h)
+    key = (h.data_ptr(), version)
+    hit = getattr(h, "_fpq_rotation", None)
+    if version is not None and hit is not None and hit[0] == key:
+        return hit[1], hit[2]
+    g = h.shape[0]
+    if h.dim() != 2 or h.shape[1] != g:
+        raise ValueError(f"rotation matrix must be square, got {tuple(h.shape)}")
+    hf = h.detach().to(device="cpu", dtype=torch.float32)
+    kind, norm = ROT_GENERAL, 0.0
+    if torch.equal(hf, torch.eye(g)):
+        kind, norm = ROT_IDENTITY, 1.0
+    elif g in (16, 32, 64, 128) and float(hf[0, 0]) != 0.0:
+        n = float(hf[0, 0])
+        signed = sylvester_signs(g) * n
+        if torch.equal(hf, signed):
+            kind, norm = ROT_HADAMARD, n
+        else:
+            changes = torch.diff(signed, dim=0).ne(0).sum(dim=0)
+            if torch.equal(hf, signed[:, torch.argsort(changes)]):
+                kind, norm = ROT_GSR, n
+    if version is not None:
+        try:
+            h._fpq_rotation = (key, kind, norm)
+        except AttributeError:  # objects that refuse attributes: classify again next time
+            pass
+    return kind, norm

@@ -410,6 +410,25 @@ def prime(hadamard_matrix: torch.Tensor, weight_global_scale: torch.Tensor, act_
     classify_rotation(as_bf16(hadamard_matrix))
     linear_alpha(weight_global_scale, act_global_scale)
     as_f32_scalar(act_global_scale)
+    prepare_device(weight_global_scale.device)
+
+
+_prepared_devices = set()
+
+
+def prepare_device(device: torch.device) -> None:
+    """The library's per-device set-up (silu lookup table, scratch address), once per device and outside
+    any graph capture, so that no later call has to build it on a stream that is being recorded."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index in _prepared_devices:
+        return
+    with torch.cuda.device(index):
+        stream = _current_stream(index)
+        st = _engine.lib().fpq_prepare_device(stream)
+    if st == _engine.E_UNSUPPORTED:   # called under a capture: a later call outside one does it
+        return
+    _engine.check(st, "fpq_prepare_device")
+    _prepared_devices.add(index)
 
 
 @linear_w4a4_op.register_fake

@@ -20,54 +20,31 @@ HAS_HIP_ENGINE = _engine.available()
 # zero-nibble policy used by the operators (see include/fpq.h)
 ZERO_NIBBLE_POLICY = _engine.ZERO_REFERENCE
 
-def _version(t: torch.Tensor) -> int:
-    """The tensor's in-place modification counter, the key of everything cached per tensor.  Tensors
-    created under torch.inference_mode() have none: they get a constant (parameters and buffers made
-    that way are not written to afterwards; activations made that way are never shared, see
-    _sharing_key)."""
-    try:
-        return t._version
-    except RuntimeError:
-        return -1
+def _version(t: torch.Tensor):
+    """Cache key part for everything remembered per tensor: the in-place modification counter, or for
+    tensors created under torch.inference_mode() (which have none) a marker -- what is remembered for
+    those is only dropped by drop_tensor_caches, which FPQuantLinear runs after load_state_dict."""
+    v = _engine.tensor_version(t)
+    return "no-counter" if v is None else v
 
 
-def _sylvester(g: int) -> torch.Tensor:
-    idx = torch.arange(g)
-    anded = idx[:, None] & idx[None, :]
-    pop = torch.zeros_like(anded)
-    for b in range(8):
-        pop += (anded >> b) & 1
-    return (1 - 2 * (pop & 1)).to(torch.float32)
+_TENSOR_CACHES = ("_fpq_rotation", "_fpq_bf16", "_fpq_packed", "_fpq_alpha", "_fpq_f32", "_fpq_host")
 
 
-def classify_rotation(h: torch.Tensor) -> Tuple[int, float]:
-    """(rotation kind, norm) of a [g, g] matrix.  The result is remembered on the tensor object
-    itself (with its version counter), so the one device->host copy it needs happens once per
-    matrix and can never be confused with another tensor that later reuses the same memory."""
-    hit = getattr(h, "_fpq_rotation", None)
-    if hit is not None and hit[0] == _version(h):
-        return hit[1], hit[2]
-    g = h.shape[0]
-    if h.dim() != 2 or h.shape[1] != g:
-        raise ValueError(f"rotation matrix must be square, got {tuple(h.shape)}")
-    hf = h.detach().to(device="cpu", dtype=torch.float32)
-    kind, norm = _engine.ROT_GENERAL, 0.0
-    if torch.equal(hf, torch.eye(g)):
-        kind, norm = _engine.ROT_IDENTITY, 1.0
-    elif g in (16, 32, 64, 128) and float(hf[0, 0]) != 0.0:
-        n = float(hf[0, 0])
-        signed = _sylvester(g) * n
-        if torch.equal(hf, signed):
-            kind, norm = _engine.ROT_HADAMARD, n
-        else:
-            changes = torch.diff(signed, dim=0).ne(0).sum(dim=0)
-            if torch.equal(hf, signed[:, torch.argsort(changes)]):
-                kind, norm = _engine.ROT_GSR, n
-    try:
-        h._fpq_rotation = (_version(h), kind, norm)
-    except AttributeError:  # objects that refuse attributes: classify again next time
-        pass
-    return kind, norm
+def drop_tensor_caches(*tensors) -> None:
+    """Forget everything remembered on these tensors (packed weights, alpha, converted copies): for
+    callers that rewrote their storage in a way the modification counter does not see."""
+    for t in tensors:
+        if isinstance(t, torch.Tensor):
+            for name in _TENSOR_CACHES:
+                if hasattr(t, name):
+                    try:
+                        delattr(t, name)
+                    except AttributeError:
+                        pass
+
+
+classify_rotation = _engine.classify_rotation
 
 
 def as_bf16(h: torch.Tensor) -> torch.Tensor:

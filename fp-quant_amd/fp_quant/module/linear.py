@@ -145,6 +145,9 @@ class FPQuantLinear(nn.Module):
         """Per-call constants (rotation kind, alpha, fp32 global scale) computed now rather than inside
         the first forward, which may be a traced one or a graph capture; also run after load_state_dict."""
         h, wgs, ags = self.forward_hadamard_matrix, self.weight_global_scale, self.act_global_scale
+        # whatever was remembered about the old contents goes (in-place copies under torch.inference_mode()
+        # leave no trace in a tensor's modification counter)
+        hip_ops.drop_tensor_caches(h, wgs, ags, getattr(self, "qweight", None), getattr(self, "scales", None))
         if all(isinstance(t, torch.Tensor) and t.is_cuda for t in (h, wgs, ags)):
             eager.prime(h, wgs, ags)
 

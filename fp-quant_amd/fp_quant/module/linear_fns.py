@@ -80,56 +80,38 @@ class FPQuant4x16NoMasterFn(Function):
         # quest (MXFP4 only, validate_config) takes the same road when no clip mask is wanted
         quest = forward_method == "quest" and dtype == FPQuantDtype.MXFP4 and not x.requires_grad
         direct = ((forward_method == "abs_max" and dtype in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4)) or quest)
-        if (not torch.compiler.is_compiling() and direct
-                and weight_q.is_contiguous() and weight_scales.is_contiguous()):
-            # eager calls: the same kernels as the operators below without two operator dispatches,
-            # with alpha and the fp32 global scale computed once per layer instead of once per call
-            fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16 and bias.is_contiguous()) else None
+        plain = weight_q.is_contiguous() and weight_scales.is_contiguous()
+        # a bias the kernels can add in their epilogue; any other is added afterwards, like the reference's `y += bias`
+        fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16 and bias.is_contiguous()) else None
+        residual_done = False
+        if direct and plain and not torch.compiler.is_compiling():
+            # eager calls: the kernels of the operators below without operator dispatch, with alpha and the
+            # fp32 global scale computed once per layer; the residual rides in the GEMM when nothing has to
+            # be added between the GEMM and it
+            res_in = res_flat if (bias is None or fused_bias is not None) else None
             y = linear_w4a4(x_flat.to(torch.bfloat16), forward_hadamard_matrix, weight_q, weight_scales,
                             linear_alpha(weight_global_scale, act_global_scale), act_global_scale, fused_bias,
-                            dtype == FPQuantDtype.NVFP4, shared_source=x,
-                            residual=res_flat if (bias is None or fused_bias is not None) else None, quest=quest)
-            y = y.unflatten(dim=0, sizes=x.shape[:-1])
-            if bias is not None and fused_bias is None:
-                y += bias
-                if residual is not None:
-                    y += residual
-            return y
-        if direct and x_flat.is_cuda and weight_q.is_contiguous() and weight_scales.is_contiguous():
+                            dtype == FPQuantDtype.NVFP4, shared_source=x, residual=res_in, quest=quest)
+            residual_done = res_in is not None
+        elif direct and plain and x_flat.is_cuda:
             # traced callers: the eager body above as one operator
-            fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16 and bias.is_contiguous()) else None
             y = linear_w4a4_op(x_flat.to(torch.bfloat16), forward_hadamard_matrix, weight_q, weight_scales,
                                weight_global_scale, act_global_scale, fused_bias, dtype == FPQuantDtype.NVFP4, quest)
-            y = y.unflatten(dim=0, sizes=x.shape[:-1])
-            if bias is not None and fused_bias is None:
-                y += bias
-            if residual is not None:
-                y = y + residual
-            return y
-        if (dtype == FPQuantDtype.MXFP4 and x_flat.is_cuda
+        elif (dtype == FPQuantDtype.MXFP4 and x_flat.is_cuda
                 and packed_linear_eligible(x_flat.shape[0], x_flat.shape[1], forward_method)):
-            # large batches: quantize and multiply on operands in the matrix units' own order
-            alpha = linear_alpha_op(weight_global_scale, act_global_scale)
-            fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16) else None
+            # quantize and multiply on operands in the matrix units' own order
             y = linear_mxf4_packed_op(x_flat.to(torch.bfloat16), as_bf16(forward_hadamard_matrix), weight_q,
-                                      weight_scales, alpha, fused_bias)
-            y = y.unflatten(dim=0, sizes=x.shape[:-1])
-            if bias is not None and fused_bias is None:
-                y += bias
-            if residual is not None:
-                y = y + residual
-            return y
-        x_q, x_scales, _ = forward_quantize(
-            x_flat, forward_hadamard_matrix, act_global_scale, dtype, forward_method
-        )
-        # evaluated in the buffers' dtype, as the reference does (bf16 buffers round 1/9)
-        alpha = linear_alpha_op(weight_global_scale, act_global_scale)
-        fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16) else None
-        y = forward_gemm(x_q, weight_q, x_scales, weight_scales, alpha, dtype, fused_bias)
+                                      weight_scales, linear_alpha_op(weight_global_scale, act_global_scale), fused_bias)
+        else:
+            # the reference's operator chain (quest with a clip mask, strided weights, CPU tensors raise in the operators)
+            x_q, x_scales, _ = forward_quantize(x_flat, forward_hadamard_matrix, act_global_scale, dtype, forward_method)
+            # alpha is evaluated in the buffers' dtype, as the reference does (bf16 buffers round 1/9)
+            y = forward_gemm(x_q, weight_q, x_scales, weight_scales,
+                             linear_alpha_op(weight_global_scale, act_global_scale), dtype, fused_bias)
         y = y.unflatten(dim=0, sizes=x.shape[:-1])
         if bias is not None and fused_bias is None:
             y += bias
-        if residual is not None:
+        if residual is not None and not residual_done:
             y = y + residual
         return y
 

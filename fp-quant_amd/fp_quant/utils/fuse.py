@@ -18,8 +18,12 @@ cannot know is that q/k/v, and gate/up, quantize the same tensor: there the patc
 modules call group operators (one quantization, one GEMM per layer; SiLU*up fused into down_proj's
 quantizer), which a captured decode step replays as fewer kernels.
 
-Results are those of the unfused modules with one bf16 rounding per PyTorch operator (normalise,
-scale by the weight; silu, multiply); parameters, buffers and state-dict keys are untouched.  Calls
+Results follow the operator sequence of the unfused modules with one bf16 rounding per PyTorch operator
+(normalise, scale by the weight; silu, multiply), evaluated with correctly rounded fp32 arithmetic in a
+fixed order.  They are bit-identical to that definition, not to PyTorch's own kernels: torch's rsqrt and
+exp are not correctly rounded, so a few elements per million differ by one bf16 step from the unfused
+model (the whole-model test bounds the difference of the logits, it does not require equality).
+Parameters, buffers and state-dict keys are untouched.  Calls
 that cannot take the fused kernels (tracing, CPU tensors, other dtypes, training, rotations without
 a fused kernel) run the original forward.
 """

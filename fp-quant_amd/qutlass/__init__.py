@@ -44,44 +44,7 @@ def _need_gpu(*tensors: torch.Tensor) -> None:
             raise ValueError("these kernels need tensors on a GPU; there is no CPU path")
 
 
-def _sylvester(g: int) -> torch.Tensor:
-    i = torch.arange(g)
-    anded = i[:, None] & i[None, :]
-    pop = torch.zeros_like(anded)
-    for b in range(8):
-        pop += (anded >> b) & 1
-    return 1.0 - 2.0 * (pop & 1).float()
-
-
-def _rotation(h: torch.Tensor) -> Tuple[int, float]:
-    """(rotation kind, norm) of the [g, g] matrix: the Hadamard / identity / sequency-ordered
-    matrices the reference builds (linear.py:24-41) are applied as butterflies, anything else as a
-    matrix product.  Remembered on the tensor object with its version counter."""
-    hit = getattr(h, "_fpq_rotation", None)
-    version = getattr(h, "_version", -1) if not h.is_inference() else -1
-    if hit is not None and hit[0] == version and version >= 0:
-        return hit[1], hit[2]
-    g = h.shape[0]
-    if h.dim() != 2 or h.shape[1] != g:
-        raise ValueError(f"rotation matrix must be square, got {tuple(h.shape)}")
-    hf = h.detach().to(device="cpu", dtype=torch.float32)
-    kind, norm = _engine.ROT_GENERAL, 0.0
-    if torch.equal(hf, torch.eye(g)):
-        kind, norm = _engine.ROT_IDENTITY, 1.0
-    elif g in (16, 32, 64, 128) and float(hf[0, 0]) != 0.0:
-        n = float(hf[0, 0])
-        signed = _sylvester(g) * n
-        if torch.equal(hf, signed):
-            kind, norm = _engine.ROT_HADAMARD, n
-        else:
-            changes = torch.diff(signed, dim=0).ne(0).sum(dim=0)
-            if torch.equal(hf, signed[:, torch.argsort(changes)]):
-                kind, norm = _engine.ROT_GSR, n
-    try:
-        h._fpq_rotation = (version, kind, norm)
-    except AttributeError:
-        pass
-    return kind, norm
+_rotation = _engine.classify_rotation   # (rotation kind, norm) of a [g, g] matrix, remembered per tensor
 
 
 def _padded(rows: int, groups: int) -> Tuple[int, int]:

@@ -4,9 +4,16 @@
  * Every entry point takes raw device pointers, sizes and a HIP stream (passed as void*, 0 = the
  * null stream), launches asynchronously on that stream and returns an int status:
  *   0  success;  <0  invalid argument (FPQ_E_*);  >0  a hipError_t reported by the runtime.
- * No entry point allocates device memory, synchronises the stream or keeps mutable global state;
- * all of them may be called from any host thread.  Scalars the reference passes as one-element
- * tensors (alpha, global scale) stay device pointers so no host sync is introduced.
+ * No entry point allocates device memory, and all of them may be called from any host thread.
+ * Scalars the reference passes as one-element tensors (alpha, global scale) stay device pointers
+ * so no host sync is introduced.  Two pieces of per-device state exist, both set up by
+ * fpq_prepare_device (or by the first call that needs them):
+ *   - a 128 KB lookup table of bf16 silu values used by fpq_silu_mul_quantize_*: the first such
+ *     call on a device fills it on the caller's stream and WAITS for that stream once; if that
+ *     first call is being captured into a graph, the fill is recorded into the capture and
+ *     repeated by every later first call until one runs outside a capture;
+ *   - the device address of the scratch array of fpq_gemm_mxf4_packed_noalloc.
+ * Apart from that no entry point synchronises a stream or keeps mutable global state.
  *
  * Each declaration cites the reference interface it stands in for (paths relative to the
  * reference checkout, inference_lib/src/fp_quant/module/).
@@ -49,6 +56,13 @@ const char* fpq_status_string(int status);
 
 /* 1 if `device` is a gfx950 GPU this library has code for, 0 if not, <0 / >0 on error. */
 int fpq_device_supported(int device);
+
+/*
+ * Sets up the per-device state described at the top for the current device, on `stream`, and waits
+ * for it: call it once per device before capturing graphs or entering a loop that must not block.
+ * Returns FPQ_E_UNSUPPORTED if `stream` is being captured.  Idempotent and cheap after the first call.
+ */
+int fpq_prepare_device(void* stream);
 
 /*
  * *id = 0 if `stream` is not being captured into a graph, else a value unique to the capture in

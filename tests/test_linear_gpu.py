@@ -473,3 +473,46 @@ def test_group_operators_equal_separate_layers(fmt, g):
                 gate, up = torch.randn(2, m, 256, device="cuda", dtype=torch.bfloat16).unbind(0)
                 qa = eager.silu_mul_quantize(gate, up, down.forward_hadamard_matrix, down.act_global_scale, nv)
                 assert torch.equal(mlp(gate, up), down.forward_quantized(qa, (m,))), (round_, m)
+
+
+@pytest.mark.parametrize("fmt,g,m", [("mxfp4", 128, 4), ("mxfp4", 128, 200), ("nvfp4", 16, 100)])
+def test_load_state_dict_onto_tensors_without_a_modification_counter(fmt, g, m):
+    """A layer built under torch.inference_mode() holds tensors without a modification counter; a
+    load_state_dict into it (an in-place copy nothing records) must still reach the packed weights,
+    alpha and the other per-tensor copies the layer keeps."""
+    import fp_quant
+    gen = torch.Generator().manual_seed(77)
+    k, n = 512, 256
+    x = torch.randn(m, k, generator=gen).to(torch.bfloat16).cuda()
+
+    def make(scale):
+        lin = fp_quant.FPQuantLinear(k, n, _cfg(fmt, g), bias=False, device="cuda", dtype=torch.bfloat16)
+        lin.weight.data = (torch.randn(n, k, generator=gen) * scale).to(torch.bfloat16).cuda()
+        lin.pre_forward()
+        return lin
+
+    with torch.inference_mode():
+        a, b = make(0.02), make(0.05)
+        ya, yb = a(x), b(x)                       # both now hold their packed weights and alpha
+        assert not torch.equal(ya, yb)
+        sd = {key: v.clone() for key, v in b.state_dict().items()}
+        sd["act_global_scale"] = sd["act_global_scale"] * 2   # a different alpha as well: exactly half of b's
+        a.load_state_dict(sd)
+        if fmt == "mxfp4":
+            assert torch.equal(a(x), yb * 0.5)                # same codes, alpha halved (a power of two: exact)
+        else:
+            assert not torch.equal(a(x), ya)                  # NVFP4 activations are scaled by it before rounding
+            c = make(0.02)
+            c.load_state_dict(sd)
+            assert torch.equal(a(x), c(x))
+
+
+def test_prepare_device_entry_point():
+    from fp_quant import _engine
+    lib = _engine.lib()
+    s = torch.cuda.Stream()
+    assert lib.fpq_prepare_device(s.cuda_stream) == 0
+    assert lib.fpq_prepare_device(s.cuda_stream) == 0          # idempotent
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        assert lib.fpq_prepare_device(s.cuda_stream) == _engine.E_UNSUPPORTED   # must run, not be recorded
