@@ -58,6 +58,46 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
 }
 
+// Output of a GEMM whose weight operand is several layers' weights laid end to end along N: columns
+// [end[i-1], end[i]) of the product go to y[i], a dense [M, end[i] - end[i-1]] matrix of its own
+// (end[-1] = 0).  count == 0: one output [M, N].  Every boundary is a multiple of kSegmentAlign, so
+// that no workgroup tile of any kernel lies across one.
+constexpr int kMaxSegments = 4;
+constexpr int kSegmentAlign = 256;
+struct OutSegments {
+  int count;
+  int end[kMaxSegments];
+  uint16_t* y[kMaxSegments];
+};
+
+// Where a tile whose first column is n0 (workgroup- or wave-uniform) is stored: the output matrix,
+// its width, the tile's first column in it, and the bias moved to the matrix's first column.
+struct OutView {
+  uint16_t* y;
+  const uint16_t* bias;
+  int n0, N;
+};
+__device__ __forceinline__ OutView out_view(const OutSegments& seg, uint16_t* y, const uint16_t* bias, int n0,
+                                            int N) {
+  OutView v{y, bias, n0, N};
+  if (seg.count > 0) {
+    int start = 0, stop = seg.end[0];
+    uint16_t* ys = seg.y[0];
+#pragma unroll
+    for (int i = 1; i < kMaxSegments; ++i)
+      if (i < seg.count && n0 >= seg.end[i - 1]) {
+        start = seg.end[i - 1];
+        stop = seg.end[i];
+        ys = seg.y[i];
+      }
+    v.y = ys;
+    v.bias = bias ? bias + start : bias;
+    v.n0 = n0 - start;
+    v.N = stop - start;
+  }
+  return v;
+}
+
 // The epilogue for a wave tile that lies inside the output (no row or column of it is cut off) with
 // N a multiple of 8 and an 8-byte aligned bias: same values as wave_tile_store below with as few
 // instructions as possible, because a workgroup's four waves issue them alone -- one instruction every

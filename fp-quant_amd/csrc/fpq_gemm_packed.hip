@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int tiles_m,
-    const uint16_t* __restrict__ residual) {
+    const uint16_t* __restrict__ residual, const OutSegments seg) {
   constexpr int BN = NT * 32, BM = MT * 32;
   constexpr int NW = WN * WM;           // waves
   static_assert(NW == 4 && NT <= KW && KW % 4 == 0 && MT % 4 == 0 && NT % WN == 0 && MT % WM == 0,
@@ -353,8 +353,9 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
 #undef FPQ_MFMA_ROW
 #undef FPQ_TAKE_SCALES
 
-  wave_tile_store<TN, TM, packed_lds_alloc(kBlocks, NV, RING, TN * 32, TM * 32), NW>(acc, smem, y, bias, alpha_p, n_blk + wn * TN * 32, m_blk + wm * TM * 32,
-                                          wave, lane, M, N, residual);
+  const OutView out = out_view(seg, y, bias, n_blk + wn * TN * 32, N);
+  wave_tile_store<TN, TM, packed_lds_alloc(kBlocks, NV, RING, TN * 32, TM * 32), NW>(
+      acc, smem, out.y, out.bias, alpha_p, out.n0, m_blk + wm * TM * 32, wave, lane, M, out.N, residual);
 }
 
 }  // namespace fpq
@@ -363,7 +364,7 @@ namespace fpq {
 template <int NT, int KW, int MT, int WN, int WM, bool NV, int RING = kRing>
 static int launch_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                          const void* bias, void* y, int64_t M, int64_t N, int64_t K, hipStream_t stream,
-                         const void* residual) {
+                         const void* residual, const OutSegments& seg) {
   constexpr int kLds = packed_lds_alloc(KW + MT, NV, RING, NT / WN * 32, MT / WM * 32);
   const int tiles_m = (int)((M + MT * 32 - 1) / (MT * 32)), tiles_n = (int)((N + NT * 32 - 1) / (NT * 32));
   static LdsLimitOnce lds_limit;
@@ -371,7 +372,7 @@ static int launch_packed(const void* xq, const void* xs, const void* wq, const v
   hipLaunchKernelGGL((gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV, RING>), dim3((unsigned)(tiles_m * tiles_n)),
                      dim3(256), kLds, stream, (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq,
                      (const uint8_t*)ws, alpha, (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K,
-                     tiles_m, (const uint16_t*)residual);
+                     tiles_m, (const uint16_t*)residual, seg);
   return (int)hipGetLastError();
 }
 
@@ -380,12 +381,13 @@ bool stream_eligible(int64_t M, int64_t N, int64_t K);
 int64_t gemm_mxf4_stream_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int gemm_mxf4_stream(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                      const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
-                     void* workspace, int64_t workspace_bytes, hipStream_t stream);
+                     void* workspace, int64_t workspace_bytes, const OutSegments& seg, hipStream_t stream);
 
 template <bool NV>
 static int gemm_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                        const void* bias, void* y, int64_t M, int64_t N, int64_t K, void* stream,
-                       const void* residual = nullptr, void* workspace = nullptr, int64_t workspace_bytes = 0);
+                       const void* residual = nullptr, void* workspace = nullptr, int64_t workspace_bytes = 0,
+                       const OutSegments& seg = OutSegments{});
 
 template <bool NV>
 static int pack_operand(const void* codes, const void* scales, int64_t scale_stride, int64_t rows, int64_t K,
@@ -417,7 +419,7 @@ namespace fpq {
 template <bool NV>
 static int gemm_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                        const void* bias, void* y, int64_t M, int64_t N, int64_t K, void* stream,
-                       const void* residual, void* workspace, int64_t workspace_bytes) {
+                       const void* residual, void* workspace, int64_t workspace_bytes, const OutSegments& seg) {
   if (M < 0 || N < 0 || K < 0 || workspace_bytes < 0) return FPQ_E_SHAPE;
   if (M == 0 || N == 0) return FPQ_OK;
   if (!xq || !xs || !wq || !ws || !alpha || !y) return FPQ_E_NULL;
@@ -433,15 +435,15 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
   if ((uintptr_t)workspace & 255u) return FPQ_E_ALIGN;
   if (!NV && stream_eligible(M, N, K))
     return gemm_mxf4_stream(xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, workspace, workspace_bytes,
-                            (hipStream_t)stream);
+                            seg, (hipStream_t)stream);
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
   if (big_tiles < FPQ_PACKED_SMALL_BELOW)
-    return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual);
+    return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);
 #if FPQ_PACKED_HALF_TILES
   if (!NV || FPQ_PACKED_HALF_TILES > 1)
-    return launch_packed<8, 8, 4, 2, 2, NV, 4>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual);
+    return launch_packed<8, 8, 4, 2, 2, NV, 4>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);
 #endif
-  return launch_packed<8, 8, 8, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual);
+  return launch_packed<8, 8, 8, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);
 }
 }  // namespace fpq
 
@@ -499,6 +501,25 @@ extern "C" int fpq_gemm_mxf4_packed_splitk(const void* xq, const void* xs, const
                                            int64_t workspace_bytes, void* stream) {
   return fpq::gemm_mxf4_packed_any(xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, workspace, workspace_bytes,
                                    stream);
+}
+
+extern "C" int fpq_gemm_mxf4_packed_multi(const void* xq, const void* xs, const void* wq, const void* ws,
+                                          const float* alpha, const void* bias, void* const* ys,
+                                          const int64_t* ns, int64_t count, int64_t M, int64_t K, void* stream) {
+  if (count < 1 || count > fpq::kMaxSegments) return FPQ_E_SHAPE;
+  if (!ys || !ns) return FPQ_E_NULL;
+  fpq::OutSegments seg{};
+  int64_t N = 0;
+  for (int64_t i = 0; i < count; ++i) {
+    if (ns[i] < 1 || ns[i] % fpq::kSegmentAlign != 0 || N + ns[i] > (1 << 24)) return FPQ_E_SHAPE;
+    if (M > 0 && !ys[i]) return FPQ_E_NULL;
+    if ((uintptr_t)ys[i] & 15u) return FPQ_E_ALIGN;
+    N += ns[i];
+    seg.end[i] = (int)N;
+    seg.y[i] = (uint16_t*)ys[i];
+  }
+  seg.count = (int)count;
+  return fpq::gemm_packed<false>(xq, xs, wq, ws, alpha, bias, ys[0], M, N, K, stream, nullptr, nullptr, 0, seg);
 }
 
 extern "C" int fpq_gemm_nvf4_packed(const void* xq, const void* xs, const void* wq, const void* ws,

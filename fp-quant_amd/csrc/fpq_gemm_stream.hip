@@ -42,7 +42,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_mxf4_stream_kernel(
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias,
     const uint16_t* residual, uint16_t* y, int M, int N, int K, int bps, int ksplit,
-    float* partial, unsigned* counters) {
+    float* partial, unsigned* counters, const OutSegments seg) {
   static_assert(NW == 4, "the partial sums meet in two rounds of two");
   __shared__ v4f part[2][NT * MT][4][64];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -215,11 +215,14 @@ __global__ __launch_bounds__(64 * NW) void gemm_mxf4_stream_kernel(
   // tile (i, j) is m = 32 j + lane % 32, n = 32 (NT rtg + i) + 8 g + 4 (lane / 32) + q
   const float alpha = *alpha_p;
   const int r32 = lane & 31, kh = lane >> 5;
-  const bool vec_ok = (N & 3) == 0;
 #pragma unroll
   for (int ig = 0; ig < NT * 4; ++ig) {
     const int i = ig >> 2, g = ig & 3;
     const int n = (rtg * NT + i) * 32 + 8 * g + 4 * kh;
+    // the matrix this weight tile's columns are stored to (bias is indexed by the product's column n)
+    const OutView out = out_view(seg, y, nullptr, (rtg * NT + i) * 32, N);
+    const int ldy = out.N, nl = out.n0 + 8 * g + 4 * kh;
+    const bool vec_ok = (ldy & 3) == 0;
     float bv[4] = {0.f, 0.f, 0.f, 0.f};
     if (bias) {
 #pragma unroll
@@ -237,9 +240,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_mxf4_stream_kernel(
         lo = pack_bf16x2(__uint_as_float(lo << 16) + bv[0], __uint_as_float(lo & 0xffff0000u) + bv[1]);
         hi = pack_bf16x2(__uint_as_float(hi << 16) + bv[2], __uint_as_float(hi & 0xffff0000u) + bv[3]);
       }
-      uint16_t* dst = y + (size_t)m * N + n;
+      uint16_t* dst = out.y + (size_t)m * ldy + nl;
       if (vec_ok && n + 3 < N) {
-        if (residual) {
+        if (residual) {   // never together with segments: one output, ldy == N and nl == n
           const uint2 rv = *(const uint2*)(residual + (size_t)m * N + n);
           lo = pack_bf16x2(__uint_as_float(lo << 16) + __uint_as_float(rv.x << 16),
                            __uint_as_float(lo & 0xffff0000u) + __uint_as_float(rv.x & 0xffff0000u));
@@ -311,7 +314,7 @@ int64_t gemm_mxf4_stream_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 // its first kStreamCounterBytes zero.
 int gemm_mxf4_stream(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                      const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
-                     void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+                     void* workspace, int64_t workspace_bytes, const OutSegments& seg, hipStream_t stream) {
   const StreamPlan plan = stream_plan(M, N, K, workspace ? workspace_bytes : 0);
   const dim3 grid((unsigned)(((N + 31) / 32 + plan.nt - 1) / plan.nt), (unsigned)plan.ksplit);
   unsigned* counters = (unsigned*)workspace;
@@ -320,7 +323,7 @@ int gemm_mxf4_stream(const void* xq, const void* xs, const void* wq, const void*
   hipLaunchKernelGGL((gemm_mxf4_stream_kernel<NTT, MTT, DBB, 4>), grid, dim3(256), 0, stream, (const uint8_t*)xq, \
                      (const uint8_t*)xs, (const uint8_t*)wq, (const uint8_t*)ws, alpha,                 \
                      (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, (int)M, (int)N,    \
-                     (int)K, plan.bps, plan.ksplit, partial, counters)
+                     (int)K, plan.bps, plan.ksplit, partial, counters, seg)
   const int mt = (int)((M + 31) / 32);
   if (plan.nt == 1) {
     switch (mt) {

@@ -28,6 +28,7 @@ from .hip_ops import (
     packed_linear_eligible,
     packed_weight,
     packed_weight_ready,
+    packed_weights_enabled,
     quantize_mx_packed,
 )
 
@@ -210,21 +211,32 @@ def wants_packed(m: int, n: int, k: int, nvfp4: bool) -> bool:
 
 def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alpha: torch.Tensor,
               bias: Optional[torch.Tensor], stream: int, use_packed: Optional[bool] = None,
-              residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+              residual: Optional[torch.Tensor] = None,
+              packed: Optional[Tuple[torch.Tensor, torch.Tensor, int]] = None) -> torch.Tensor:
     """bf16 [m, n] = alpha * dq(activations) @ dq(w).T (+ bias) on quantized activations, with the
     kernel and operand layout the shape calls for (`use_packed`: the caller's decision, if it has
     made it already).  `residual` (bf16 [m, n]) is added as a separate bf16 addition would add it:
     inside the packed MXFP4 kernel's epilogue, by a PyTorch addition after the other kernels."""
     lib = _engine.lib()
     m, k = qa.m, qa.k
-    n = wq.shape[0]
-    if wq.shape[1] * 2 != k:
-        raise ValueError(f"inner dimensions differ: x has K={k}, w has K={wq.shape[1] * 2}")
-    y = torch.empty(m, n, dtype=torch.bfloat16, device=wq.device)
+    if packed is not None:   # packed MXFP4 weights of `n` rows handed in directly (a WeightGroup): wq, ws unused
+        wp, wsp, n = packed
+        if qa.nvfp4 or wp.numel() * 2 != n * k:
+            raise ValueError("packed weights need MXFP4 activations with the same inner dimension")
+        use_packed = True
+    else:
+        n = wq.shape[0]
+        if wq.shape[1] * 2 != k:
+            raise ValueError(f"inner dimensions differ: x has K={k}, w has K={wq.shape[1] * 2}")
+        wp = wsp = None
+    dev = wp.device if packed is not None else wq.device
+    y = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
     b_ptr = bias.data_ptr() if bias is not None else None
     if residual is not None and (residual.dtype != torch.bfloat16 or residual.numel() != m * n
-                                 or not residual.is_contiguous() or residual.device != wq.device):
+                                 or not residual.is_contiguous()):
         raise ValueError("residual must be a contiguous bfloat16 tensor of the output's size on the same device")
+    if residual is not None and residual.device != dev:
+        raise ValueError("residual must be on the weights' device")
     if use_packed is None:
         use_packed = wants_packed(m, n, k, qa.nvfp4)
     if not qa.serves(use_packed):
@@ -246,7 +258,8 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
         return y
     if use_packed:
         pc, ps = qa.packed()
-        wp, wsp = packed_weight(wq, ws)
+        if packed is None:
+            wp, wsp = packed_weight(wq, ws)
         if residual is not None:
             st = lib.fpq_gemm_mxf4_packed_residual(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
                                                    alpha.data_ptr(), b_ptr, residual.data_ptr(), y.data_ptr(),
@@ -327,6 +340,148 @@ def linear_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torc
     alpha = linear_alpha(weight_global_scale, act_global_scale, remember=False)
     return linear_w4a4(x, hadamard_matrix, wq.contiguous(), ws.contiguous(), alpha, act_global_scale, bias, nvfp4,
                        remember=False, quest=quest)
+
+
+# Layers fed by one tensor (q/k/v, gate/up) as ONE GEMM.  In the packed layout a weight is a sequence of
+# 32-row tiles, so the packed weights of several layers with the same K, laid end to end, are the packed
+# weight of their concatenation along N: one launch computes [m, n_1 + n_2 + ...] and the layers' outputs
+# are column slices of it.  The layers' own packed copies become views into the concatenated buffers, so
+# no 4-bit weight is held a further time.  MXFP4 only (the NVFP4 packed kernel serves mid-sized batches only).
+class WeightGroup:
+    __slots__ = ("key", "wp", "wsp", "bias", "n", "splits", "k")
+
+
+def _member_key(wq: torch.Tensor, ws: torch.Tensor, bias: Optional[torch.Tensor]):
+    return (wq.data_ptr(), _version(wq), ws.data_ptr(), _version(ws), tuple(wq.shape),
+            None if bias is None else (bias.data_ptr(), _version(bias)))
+
+
+def weight_group(members, create: bool = False) -> Optional[WeightGroup]:
+    """The WeightGroup of `members` = [(qweight, scales, bias or None), ...] (MXFP4, row-major, same K, every
+    N a multiple of 32, biases all absent or all contiguous bf16), remembered on the first member's qweight
+    until a member is written to; built now if `create`, else None when there is none."""
+    first = members[0][0]
+    key = tuple(_member_key(*m) for m in members)
+    hit = getattr(first, "_fpq_group", None)
+    if hit is not None and hit.key == key:
+        return hit
+    if not create or not packed_weights_enabled():
+        return None
+    k2 = first.shape[1]
+    dev = first.device
+    have_bias = [m[2] is not None for m in members]
+    for wq, ws, bias in members:
+        if (wq.dtype != torch.uint8 or ws.dtype != torch.uint8 or not wq.is_cuda or wq.device != dev
+                or not wq.is_contiguous() or not ws.is_contiguous() or wq.dim() != 2 or wq.shape[1] != k2
+                or wq.shape[0] % 32 != 0 or (k2 * 2) % 256 != 0 or ws.shape != (wq.shape[0], k2 * 2 // 32)):
+            return None
+        if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_contiguous() or bias.device != dev):
+            return None
+    if any(have_bias) and not all(have_bias):
+        return None
+    lib = _engine.lib()
+    k = k2 * 2
+    splits = [m[0].shape[0] for m in members]
+    n = sum(splits)
+    group = WeightGroup()
+    group.key, group.n, group.splits, group.k = key, n, splits, k
+    with torch.cuda.device(dev):
+        stream = _current_stream(dev.index)
+        group.wp = torch.empty(lib.fpq_packed_codes_bytes(n, k), dtype=torch.uint8, device=dev)
+        group.wsp = torch.empty(lib.fpq_packed_scales_bytes(n, k), dtype=torch.uint8, device=dev)
+        row = 0
+        for wq, ws, _ in members:
+            rows = wq.shape[0]
+            c0, c1 = lib.fpq_packed_codes_bytes(row, k), lib.fpq_packed_codes_bytes(row + rows, k)
+            s0, s1 = lib.fpq_packed_scales_bytes(row, k), lib.fpq_packed_scales_bytes(row + rows, k)
+            pc, ps = group.wp[c0:c1], group.wsp[s0:s1]
+            st = lib.fpq_pack_mxf4(wq.data_ptr(), ws.data_ptr(), ws.shape[1], rows, k, pc.data_ptr(), ps.data_ptr(), stream)
+            _engine.check(st, "fpq_pack_mxf4")
+            # the member's own packed copy: these views (same key as hip_ops.packed_weight uses)
+            wq._fpq_packed = ((wq.data_ptr(), _version(wq), ws.data_ptr(), _version(ws), tuple(wq.shape), False), pc, ps)
+            row += rows
+    group.bias = torch.cat([m[2] for m in members]).contiguous() if all(have_bias) else None
+    try:
+        first._fpq_group = group
+    except (AttributeError, RuntimeError):
+        pass
+    return group
+
+
+def linear_on_group(qa: QuantizedActivations, wp: torch.Tensor, wsp: torch.Tensor, splits: List[int],
+                    alpha: torch.Tensor, bias: Optional[torch.Tensor], stream: int) -> List[torch.Tensor]:
+    """ONE GEMM of quantized activations with the packed MXFP4 weights of several layers laid end to end
+    (`splits`: the layers' output features); returns the layers' outputs, bf16 [m, n_i] each.  Every
+    layer gets a dense matrix of its own from the kernel when all n_i are multiples of 256; else the
+    outputs are column ranges of one [m, sum n_i] matrix (rows keep the full stride)."""
+    m, k, n = qa.m, qa.k, sum(splits)
+    if qa.nvfp4 or wp.numel() * 2 != n * k:
+        raise ValueError("packed weights need MXFP4 activations with the same inner dimension")
+    if len(splits) > 4 or any(s % 256 for s in splits):
+        y = linear_on(qa, None, None, alpha, bias, stream, True, packed=(wp, wsp, n))
+        return list(y.split(splits, dim=1))
+    lib = _engine.lib()
+    pc, ps = qa.packed()
+    outs = [torch.empty(m, s, dtype=torch.bfloat16, device=wp.device) for s in splits]
+    count = len(splits)
+    ys = (ctypes.c_void_p * count)(*[o.data_ptr() for o in outs])
+    ns = (ctypes.c_int64 * count)(*splits)
+    st = lib.fpq_gemm_mxf4_packed_multi(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(), alpha.data_ptr(),
+                                        bias.data_ptr() if bias is not None else None, ys, ns, count, m, k, stream)
+    _engine.check(st, "fpq_gemm_mxf4_packed_multi")
+    return outs
+
+
+def linear_cat(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, group: WeightGroup, alpha: torch.Tensor,
+               shared_source: Optional[torch.Tensor] = None, remember: bool = True) -> List[torch.Tensor]:
+    """The layers of a WeightGroup on `x_flat` (bf16 [m, K], contiguous) from one quantization and ONE
+    GEMM: bf16 [m, n_i] per layer (bias included)."""
+    dev = x_flat.device
+    if torch.cuda.current_device() != dev.index:
+        with torch.cuda.device(dev):
+            return linear_cat(x_flat, hadamard_matrix, group, alpha, shared_source, remember)
+    stream = _current_stream(dev.index)
+    h = as_bf16(hadamard_matrix)
+    kind, norm = classify_rotation(h)
+    qa = key = None
+    if shared_source is not None:
+        key = _sharing_key(x_flat.shape, h, kind, norm, None, stream)
+        if key is not None:
+            qa = _lookup(shared_source, key, True)
+    if qa is None:
+        qa = quantize_activations(x_flat, h, kind, norm, None, False, stream, True, remember)
+        if key is not None:
+            _publish(qa, shared_source, key, h)
+    return linear_on_group(qa, group.wp, group.wsp, group.splits, alpha, group.bias, stream)
+
+
+@torch.library.custom_op("fp_quant::linear_cat_w4a4_op", mutates_args=())
+def linear_cat_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wp: torch.Tensor, wsp: torch.Tensor,
+                       splits: List[int], weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor,
+                       bias: Optional[torch.Tensor]) -> List[torch.Tensor]:
+    """linear_cat for traced callers: the packed weights of a WeightGroup (made when the model was
+    patched, outside any trace) times the activations quantized once; bf16 [m, n_i] per layer."""
+    x = x_flat if x_flat.is_contiguous() else x_flat.contiguous()
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or not x.is_cuda:
+        raise ValueError("x_flat must be a 2-D bfloat16 tensor on a GPU")
+    n = sum(splits)
+    if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_contiguous() or bias.numel() != n):
+        raise ValueError("bias must be a contiguous bfloat16 vector of sum(splits) elements")
+    dev = x.device
+    with torch.cuda.device(dev):
+        stream = _current_stream(dev.index)
+        h = as_bf16(hadamard_matrix)
+        kind, norm = classify_rotation(h)
+        alpha = linear_alpha(weight_global_scale, act_global_scale, remember=False)
+        qa = quantize_activations(x, h, kind, norm, None, False, stream, True, remember=False)
+        outs = linear_on_group(qa, wp, wsp, list(splits), alpha, bias, stream)
+        # operators return tensors that own their memory: column ranges of one matrix are copied out
+        return [o if o.is_contiguous() else o.contiguous() for o in outs]
+
+
+@linear_cat_w4a4_op.register_fake
+def _(x_flat, hadamard_matrix, wp, wsp, splits, weight_global_scale, act_global_scale, bias):
+    return [x_flat.new_empty((x_flat.shape[0], s), dtype=torch.bfloat16) for s in splits]
 
 
 # Traced callers, groups of layers.  A compiler cannot see that q/k/v (or gate/up) quantize the same

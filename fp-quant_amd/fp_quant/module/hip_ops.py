@@ -28,7 +28,7 @@ def _version(t: torch.Tensor):
     return "no-counter" if v is None else v
 
 
-_TENSOR_CACHES = ("_fpq_rotation", "_fpq_bf16", "_fpq_packed", "_fpq_alpha", "_fpq_f32", "_fpq_host")
+_TENSOR_CACHES = ("_fpq_rotation", "_fpq_bf16", "_fpq_packed", "_fpq_group", "_fpq_alpha", "_fpq_f32", "_fpq_host")
 
 
 def drop_tensor_caches(*tensors) -> None:

@@ -87,9 +87,45 @@ def _quantize_alike(layers) -> bool:
     return True
 
 
-def _group_linear(layers, x: torch.Tensor):
-    """The outputs of `layers` on `x` from ONE operator (one quantization, one GEMM each)."""
+def _weight_group(layers, create: bool = False):
+    """The layers' packed weights laid end to end (eager.WeightGroup), if they can be multiplied as one:
+    MXFP4 abs-max layers that quantize alike with equal alpha.  Built when the model is patched
+    (`create`), looked up afterwards (None: the layers were rewritten since, or never qualified)."""
     first = layers[0]
+    if first.config.forward_dtype != FPQuantDtype.MXFP4 or first.config.forward_method != "abs_max":
+        return None
+    if create:
+        if not first.qweight.is_cuda or not _quantize_alike(layers):
+            return None
+        for layer in layers[1:]:
+            if not torch.equal(layer.weight_global_scale.float(), first.weight_global_scale.float()):
+                return None
+    return _eager().weight_group([(l.qweight, l.scales, l.bias) for l in layers], create)
+
+
+def _attach_weight_group(module: nn.Module, names) -> None:
+    """Build the WeightGroup of module.<names> now and keep it in `module._fpq_weight_group`; rebuilt after
+    every load_state_dict into the module (a hook), so that traced code, which cannot check tensor
+    addresses and counters, never multiplies by weights that have been replaced."""
+    def build(*_):
+        layers = [getattr(module, n) for n in names]
+        module._fpq_weight_group = (_weight_group(layers, create=True)
+                                    if all(_is_real_quant_linear(l) for l in layers) else None)
+
+    build()
+    module._fpq_weight_group_hook = module.register_load_state_dict_post_hook(build)
+
+
+def _group_linear(layers, x: torch.Tensor, group=None):
+    """The outputs of `layers` on `x` from ONE operator: one quantization and, where the layers' packed
+    weights lie end to end (`group`, a WeightGroup), one GEMM whose column ranges are the outputs; else
+    one GEMM each."""
+    first = layers[0]
+    if group is not None:
+        outs = _eager().linear_cat_w4a4_op(x.reshape(-1, x.shape[-1]), first.forward_hadamard_matrix, group.wp,
+                                           group.wsp, group.splits, first.weight_global_scale,
+                                           first.act_global_scale, group.bias)
+        return [o.view(*x.shape[:-1], o.shape[-1]) for o in outs]
     outs = _eager().linear_group_w4a4_op(
         x.reshape(-1, x.shape[-1]), first.forward_hadamard_matrix, [l.qweight for l in layers],
         [l.scales for l in layers], [l.weight_global_scale for l in layers], [l.act_global_scale for l in layers],
@@ -159,7 +195,7 @@ def fuse_gated_mlp(mlp: nn.Module) -> bool:
         if traceable and _traceable_call(x):
             # two operators: gate and up from one quantization of x; SiLU*up quantized as it is
             # formed and multiplied by down's weight
-            gate, up = _group_linear((self.gate_proj, self.up_proj), x)
+            gate, up = _group_linear((self.gate_proj, self.up_proj), x, self._fpq_weight_group)
             down = self.down_proj
             y = _eager().silu_mul_linear_w4a4_op(gate, up, down.forward_hadamard_matrix, down.qweight, down.scales,
                                                  down.weight_global_scale, down.act_global_scale, down.bias,
@@ -169,8 +205,12 @@ def fuse_gated_mlp(mlp: nn.Module) -> bool:
         if not _fusable_call(x) or (residual is not None and not _fusable_call(residual)):
             y = unfused(x)
             return y if residual is None else residual + y
-        gate = self.gate_proj(x)
-        up = self.up_proj(x)
+        pair = _eager_group_linear(self, (self.gate_proj, self.up_proj), x) if traceable else None
+        if pair is not None:
+            gate, up = pair            # both from one GEMM
+        else:
+            gate = self.gate_proj(x)
+            up = self.up_proj(x)
         down = self.down_proj
         inter = gate.shape[-1]
         qa = _eager().silu_mul_quantize(gate.reshape(-1, inter), up.reshape(-1, inter),
@@ -181,6 +221,9 @@ def fuse_gated_mlp(mlp: nn.Module) -> bool:
             return y if residual is None else residual + y
         return down.forward_quantized(qa, gate.shape[:-1], residual)
 
+    mlp._fpq_weight_group = None
+    if traceable:
+        _attach_weight_group(mlp, ("gate_proj", "up_proj"))   # gate/up as one GEMM where the format allows
     mlp._fpq_unfused_forward = unfused
     mlp.forward = types.MethodType(forward, mlp)
     return True
@@ -310,12 +353,39 @@ class _ProjectionCalls(ast.NodeTransformer):
         return node
 
 
+def _eager_group_linear(owner: nn.Module, layers, x: torch.Tensor):
+    """Eager counterpart of _group_linear for layers with a WeightGroup: one GEMM (the quantized form of
+    `x` is taken from, or left in, the sharing slot); None if there is no group.  The group kept on
+    `owner` is checked against the layers' tensors as they are now and rebuilt if they were written to."""
+    group = getattr(owner, "_fpq_weight_group", None)
+    if group is None:
+        return None
+    first = layers[0]
+    if group.key != tuple(_eager()._member_key(l.qweight, l.scales, l.bias) for l in layers):
+        group = owner._fpq_weight_group = _weight_group(layers, create=True)
+        if group is None:
+            return None
+    eager = _eager()
+    x_flat = x.reshape(-1, x.shape[-1])
+    if not x_flat.is_contiguous():
+        return None
+    outs = eager.linear_cat(x_flat, first.forward_hadamard_matrix, group,
+                            eager.linear_alpha(first.weight_global_scale, first.act_global_scale), shared_source=x)
+    return [o.unflatten(0, tuple(x.shape[:-1])) for o in outs]
+
+
 def _qkv(attn, hidden_states):
     """q, k and v projections of `hidden_states`: from one operator when a compiler is tracing
-    (which cannot see that the three layers quantize the same tensor), else three ordinary calls
-    (which share the quantization by themselves)."""
+    (which cannot see that the three layers quantize the same tensor); from one GEMM on the layers'
+    concatenated packed weights in eager calls that have them; else three ordinary calls (which
+    share the quantization by themselves)."""
+    layers = (attn.q_proj, attn.k_proj, attn.v_proj)
     if attn._fpq_qkv_alike and _traceable_call(hidden_states):
-        return _group_linear((attn.q_proj, attn.k_proj, attn.v_proj), hidden_states)
+        return _group_linear(layers, hidden_states, attn._fpq_weight_group)
+    if attn._fpq_qkv_alike and _fusable_call(hidden_states):
+        outs = _eager_group_linear(attn, layers, hidden_states)
+        if outs is not None:
+            return outs
     return attn.q_proj(hidden_states), attn.k_proj(hidden_states), attn.v_proj(hidden_states)
 
 
@@ -361,6 +431,9 @@ def fuse_qkv(attn: nn.Module) -> bool:
     except Exception:
         return False
     attn._fpq_qkv_alike = _quantize_alike(layers)
+    attn._fpq_weight_group = None
+    if attn._fpq_qkv_alike:
+        _attach_weight_group(attn, ("q_proj", "k_proj", "v_proj"))   # q/k/v as one GEMM where the format allows
     attn._fpq_qkv = types.MethodType(_qkv, attn)
     attn._fpq_unfused_forward = attn.forward
     attn.forward = types.MethodType(namespace["forward"], attn)
@@ -394,3 +467,9 @@ def unfuse_producers(model: nn.Module) -> None:
             else:
                 module.forward = unfused
             module._fpq_unfused_forward = None
+            hook = getattr(module, "_fpq_weight_group_hook", None)
+            if hook is not None:
+                hook.remove()
+                module._fpq_weight_group_hook = None
+            if hasattr(module, "_fpq_weight_group"):
+                module._fpq_weight_group = None

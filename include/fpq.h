@@ -265,6 +265,25 @@ int fpq_gemm_mxf4_packed_splitk(const void* xq_packed, const void* xs_packed, co
                                 void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * One GEMM for several layers that read the same activations (the q, k and v projections of an
+ * attention block, the gate and up projections of a gated MLP): the layers' packed weights lie end
+ * to end in wq_packed / ws_packed (a packed operand is a sequence of 32-row tiles, so the packed
+ * form of the row-wise concatenation of weights whose row counts are multiples of 32 is the
+ * concatenation of their packed forms), and layer i's result goes to its own dense matrix
+ * ys[i] of shape [M, ns[i]].  The reference launches one GEMM per layer (FPQuantLinear.forward,
+ * linear.py:250-368, once per nn.Linear it replaced); the values are the same, column by column.
+ *   count   1 .. 4 layers
+ *   ns[i]   layer i's output features, a positive multiple of 256
+ *   ys[i]   16-byte aligned device pointers to bf16 [M, ns[i]]
+ *   bias    null or bf16 [sum ns], the layers' biases end to end
+ * Status codes as fpq_gemm_mxf4_packed; FPQ_E_SHAPE also for a count or an ns[i] outside the above.
+ */
+int fpq_gemm_mxf4_packed_multi(const void* xq_packed, const void* xs_packed, const void* wq_packed,
+                               const void* ws_packed, const float* alpha, const void* bias,
+                               void* const* ys, const int64_t* ns, int64_t count, int64_t M, int64_t K,
+                               void* stream);
+
+/*
  * fpq_gemm_mxf4_packed_splitk for callers that cannot allocate or hold a workspace (code recorded
  * into a HIP graph, tight serving loops, harnesses that forbid hipMalloc): the counters and partial
  * tiles of a split K live in a file-scope device array of the library (1 064 960 bytes per GPU, held

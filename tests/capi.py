@@ -1,4 +1,6 @@
 """Thin test helper: call the C ABI of libfpq_hip.so on torch CUDA tensors."""
+import ctypes
+
 import torch
 
 from fp_quant import _engine
@@ -115,6 +117,24 @@ def gemm_packed_splitk(xp, xsp, wp, wsp, m, n, k, alpha, bias=None, residual=Non
         _engine.check(st, "fpq_gemm_mxf4_packed_splitk")
     torch.cuda.synchronize()
     return y.cpu()
+
+
+def gemm_packed_multi(xp, xsp, wp, wsp, m, splits, k, alpha, bias=None):
+    """fpq_gemm_mxf4_packed_multi on packed operands (the weights of len(splits) layers end to end); a list
+    of bf16 [M, splits[i]] on the CPU."""
+    lib = _engine.lib()
+    xp, xsp, wp, wsp = (t.to("cuda").contiguous() for t in (xp, xsp, wp, wsp))
+    outs = [torch.full((m, s), float("nan"), dtype=torch.bfloat16, device="cuda") for s in splits]
+    a = torch.tensor([alpha], dtype=torch.float32, device="cuda")
+    b = bias.to("cuda").contiguous() if bias is not None else None
+    ys = (ctypes.c_void_p * len(splits))(*[o.data_ptr() for o in outs])
+    ns = (ctypes.c_int64 * len(splits))(*splits)
+    st = lib.fpq_gemm_mxf4_packed_multi(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(), a.data_ptr(),
+                                        b.data_ptr() if b is not None else None, ys, ns, len(splits), m, k,
+                                        torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_gemm_mxf4_packed_multi")
+    torch.cuda.synchronize()
+    return [o.cpu() for o in outs]
 
 
 def gemm_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=None, residual=None, in_place=False):

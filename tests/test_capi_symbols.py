@@ -44,5 +44,16 @@ def test_argument_validation_needs_no_device():
     assert lib.fpq_quantize_mx(8, 4, 128, 0, 128, 0.088, None, 16, 16, 4, 4, 0, None) == -4
     assert lib.fpq_quantize_mx(16, 4, 128, 0, 128, 0.088, None, 16, 16, 4, 4, 9, None) == -5
     assert lib.fpq_quantize_nv(16, 4, 128, 0, 16, 0.25, None, None, 16, 16, 4, 8, 0, None) == -1
+    # the multi-output GEMM: 1..4 layers, output features in multiples of 256, aligned outputs
+    ys, ns = (ctypes.c_void_p * 2)(256, 512), (ctypes.c_int64 * 2)(256, 512)
+    args = (16, 16, 16, 16, 16, None)
+    assert lib.fpq_gemm_mxf4_packed_multi(*args, ys, ns, 0, 4, 256, None) == -2
+    assert lib.fpq_gemm_mxf4_packed_multi(*args, ys, ns, 5, 4, 256, None) == -2
+    assert lib.fpq_gemm_mxf4_packed_multi(*args, None, ns, 2, 4, 256, None) == -1
+    assert lib.fpq_gemm_mxf4_packed_multi(*args, ys, (ctypes.c_int64 * 2)(256, 100), 2, 4, 256, None) == -2
+    assert lib.fpq_gemm_mxf4_packed_multi(*args, (ctypes.c_void_p * 2)(256, 8), ns, 2, 4, 256, None) == -4
+    assert lib.fpq_gemm_mxf4_packed_multi(*args, (ctypes.c_void_p * 2)(256, None), ns, 2, 4, 256, None) == -1
+    assert lib.fpq_gemm_mxf4_packed_multi(*args, ys, ns, 2, 4, 100, None) == -2
+    assert lib.fpq_gemm_mxf4_packed_multi(*args, ys, ns, 2, 0, 256, None) == 0
     with pytest.raises(ValueError):
         _engine.check(-2, "x")

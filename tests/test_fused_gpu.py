@@ -488,3 +488,50 @@ def test_compiled_decode_with_grouped_operators_matches_eager(fmt, g, arch):
     torch._dynamo.reset()
     for i, (a, b) in enumerate(zip(got, want)):
         assert torch.equal(a, b), i
+
+
+@pytest.mark.parametrize("tokens", [3, 40, 300])
+def test_grouped_projections_run_as_one_gemm_on_concatenated_packed_weights(tokens):
+    """After fuse_producers q/k/v (and gate/up) of an MXFP4 block are one GEMM on the layers' packed weights
+    laid end to end: same bits as the three (two) layers called one by one, the layers' own packed copies
+    are views into the concatenated buffers, and a load_state_dict is followed."""
+    from fp_quant.module import eager
+    from fp_quant.utils import fuse_producers
+    model = _tiny_llama("mxfp4", 128, seed=3)
+    other = _tiny_llama("mxfp4", 128, seed=4)
+    block, block2 = model.model.layers[0], other.model.layers[0]
+    attn, mlp = block.self_attn, block.mlp
+    x = (torch.randn(1, tokens, 256, device="cuda") * 1.5).to(torch.bfloat16)
+    with torch.no_grad():
+        want = [l(x.clone()) for l in (attn.q_proj, attn.k_proj, attn.v_proj)]
+        want_mlp = [l(x.clone()) for l in (mlp.gate_proj, mlp.up_proj)]
+        want2 = [l(x.clone()) for l in (block2.self_attn.q_proj, block2.self_attn.k_proj, block2.self_attn.v_proj)]
+        assert fuse_producers(model) == 10
+        group = attn._fpq_weight_group
+        assert group is not None and group.n == sum(w.shape[-1] for w in want) and mlp._fpq_weight_group is not None
+        lo, hi = group.wp.data_ptr(), group.wp.data_ptr() + group.wp.numel()
+        for layer in (attn.q_proj, attn.k_proj, attn.v_proj):
+            assert lo <= layer.qweight._fpq_packed[1].data_ptr() < hi        # no further copy of the weights
+        got = attn._fpq_qkv(x)
+        # k and v have 128 output features here: column ranges of one output matrix
+        assert got[0].data_ptr() + 2 * want[0].shape[-1] == got[1].data_ptr()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+        gate, up = want_mlp
+        # gate and up have 512 each (multiples of 256): the one GEMM writes a dense matrix per layer
+        from fp_quant.utils import fuse
+        pair = fuse._eager_group_linear(mlp, (mlp.gate_proj, mlp.up_proj), x)
+        assert all(t.is_contiguous() for t in pair) and torch.equal(pair[0], gate) and torch.equal(pair[1], up)
+        assert torch.equal(block.mlp(x), block.mlp.down_proj(O.silu_mul(
+            gate.cpu().view(-1, gate.shape[-1]), up.cpu().view(-1, up.shape[-1])).view(gate.shape).cuda()))
+        # traced callers: the same through the operator
+        outs = eager.linear_cat_w4a4_op(x.view(-1, 256), attn.q_proj.forward_hadamard_matrix, group.wp, group.wsp,
+                                        group.splits, attn.q_proj.weight_global_scale, attn.q_proj.act_global_scale,
+                                        group.bias)
+        for a, b in zip(outs, want):
+            assert a.is_contiguous() and torch.equal(a.reshape(b.shape), b)
+        # new weights: the hook rebuilds the group
+        attn.load_state_dict(block2.self_attn.state_dict())
+        assert attn._fpq_weight_group is not group
+        for a, b in zip(attn._fpq_qkv(x), want2):
+            assert torch.equal(a, b)

@@ -142,3 +142,29 @@ def test_split_k_rejects_misaligned_workspace():
     wspace = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
     with pytest.raises(ValueError):
         capi.gemm_packed_splitk(xp, xsp, wp, wsp, 4, 64, 1024, ALPHA, workspace=wspace[16:])
+
+
+# rows that take the weight-streaming kernel with one and with two weight tiles per workgroup, the
+# 128 x 128 tile kernel and the 256 x 128 tile kernel; 2 to 4 layers of 256 to 1024 output features
+@pytest.mark.parametrize("m,splits,k", [(1, [512, 256, 256], 512), (16, [1024, 256], 1024), (33, [256, 512], 256),
+                                        (64, [4096, 4096, 256], 256), (128, [256, 256, 256, 256], 768),
+                                        (300, [512, 256, 256], 512), (2048, [2048, 1024, 256, 768], 256),
+                                        (37, [9216], 256)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_layers_end_to_end_get_their_own_outputs(m, splits, k, with_bias):
+    """fpq_gemm_mxf4_packed_multi: every layer's matrix equals its column range of the one-output GEMM
+    on the same operands bit for bit (same kernels, same accumulation order), and that GEMM is checked
+    against the oracle."""
+    n = sum(splits)
+    g, xq, xs, wq, ws = _operands(m, n, k, 4000 + m + n)
+    bias = (torch.randn(n, generator=g) * 2).to(torch.bfloat16) if with_bias else None
+    xp, xsp = pack_by_definition(xq, xs, k)
+    wp, wsp = pack_by_definition(wq, ws, k)
+    whole = capi.gemm_packed(xp, xsp, wp, wsp, m, n, k, ALPHA, bias=bias)
+    _check(whole, xq, xs, wq, ws, bias=bias)
+    outs = capi.gemm_packed_multi(xp, xsp, wp, wsp, m, splits, k, ALPHA, bias=bias)
+    col = 0
+    for o, s in zip(outs, splits):
+        assert o.shape == (m, s)
+        assert torch.equal(o.view(torch.int16), whole[:, col:col + s].contiguous().view(torch.int16))
+        col += s
