@@ -699,6 +699,15 @@ def bench_e2e_llama(torch, layers=32, prefill_batch=4, seq=2048, decode_batches=
     if compiled_decode:   # the traced attention and MLP modules now call the group operators
         fused["decode_compiled"] = compiled_decode_ms(torch, model, cfg, seq, decode_batches, decode_steps, gen)
     out["fused_producers"] = fused
+    if fmt == "mxfp4":
+        # what holding the 4-bit weights once (packed layout only) gives back; nothing is timed on it: the
+        # kernels read the same buffers either way
+        from fp_quant.utils import release_row_major_weights
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        layers = release_row_major_weights(model)
+        torch.cuda.synchronize()
+        out["weights_held_once"] = {"layers": layers, "freed_GB": round((before - torch.cuda.memory_allocated()) / 1e9, 3)}
     if compact:
         del model
         torch.cuda.empty_cache()
@@ -977,6 +986,7 @@ def main():
                 "fused_producers": {"prefill_4x2048_tokens_per_s": e2e["fused_producers"]["prefill"]["tokens_per_s"],
                                     "decode_tokens_per_s": {k: v["tokens_per_s"] for k, v in
                                                             e2e["fused_producers"]["decode"].items()}},
+                "weights_held_once": e2e.get("weights_held_once"),
                 "note": "eager PyTorch model, bf16 KV cache of 2048 tokens, everything outside the linears is stock "
                         "PyTorch-ROCm; python bench.py --only e2e_llama adds the bf16 comparison and the batch sweep",
             }

@@ -67,6 +67,33 @@ __global__ __launch_bounds__(256) void pack_fp4_kernel(const uint8_t* __restrict
   }
 }
 
+// Packed -> row-major (MXFP4), the inverse of pack_fp4_kernel<false> on the rows that exist: what a
+// layer that keeps only its packed weights hands to state_dict().
+__global__ __launch_bounds__(256) void unpack_mxf4_kernel(const uint8_t* __restrict__ pcodes,
+                                                          const uint8_t* __restrict__ pscales, int rows, int K,
+                                                          uint8_t* __restrict__ codes, uint8_t* __restrict__ scales,
+                                                          int64_t scale_stride) {
+  const int kb = blockIdx.x, rt = blockIdx.y;
+  const int t = threadIdx.x;
+  const int r = t >> 3, c = t & 7;
+  const int row = rt * 32 + r;
+  const int ks = kb * 4 + (c >> 1), kh = c & 1;
+  const uint4 v = *(const uint4*)(pcodes + (((size_t)rt * (K >> 6) + ks) * 64 + kh * 32 + r) * 16);
+  if (row < rows) *(uint4*)(codes + (size_t)row * (K >> 1) + kb * 128 + c * 16) = v;
+  if (t < 64) {
+    const int sr = t & 31, skh = t >> 5;
+    const int srow = rt * 32 + sr;
+    const uint32_t in = *(const uint32_t*)(pscales + (((size_t)rt * (K >> 8) + kb) * 64 + t) * 4);
+    if (srow < rows) {
+      uint8_t* sp = scales + (size_t)srow * scale_stride + kb * 8 + skh;
+      sp[0] = (uint8_t)in;
+      sp[2] = (uint8_t)(in >> 8);
+      sp[4] = (uint8_t)(in >> 16);
+      sp[6] = (uint8_t)(in >> 24);
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 constexpr int kRing = 8;                 // 64-K units resident or in flight
 // Scales of a 256-K block: 256 bytes per row tile for MXFP4 (one E8M0 byte per lane and K step), 512
@@ -462,6 +489,22 @@ extern "C" int64_t fpq_packed_scales_bytes_nv(int64_t rows, int64_t K) {
 extern "C" int fpq_pack_mxf4(const void* codes, const void* scales, int64_t scale_stride, int64_t rows,
                              int64_t K, void* packed_codes, void* packed_scales, void* stream) {
   return fpq::pack_operand<false>(codes, scales, scale_stride, rows, K, packed_codes, packed_scales, stream);
+}
+
+extern "C" int fpq_unpack_mxf4(const void* packed_codes, const void* packed_scales, int64_t rows, int64_t K,
+                               void* codes, void* scales, int64_t scale_stride, void* stream) {
+  if (rows < 0 || K < 0) return FPQ_E_SHAPE;
+  if (rows == 0) return FPQ_OK;
+  if (!codes || !scales || !packed_codes || !packed_scales) return FPQ_E_NULL;
+  if (K == 0 || K % 256 != 0 || scale_stride < K / 32) return FPQ_E_SHAPE;
+  if (rows > (1 << 24) || K > (1 << 24)) return FPQ_E_SHAPE;
+  if (((uintptr_t)codes & 15u) || ((uintptr_t)packed_codes & 15u) || ((uintptr_t)packed_scales & 3u))
+    return FPQ_E_ALIGN;
+  const dim3 grid((unsigned)(K / 256), (unsigned)((rows + 31) / 32));
+  hipLaunchKernelGGL(fpq::unpack_mxf4_kernel, grid, dim3(256), 0, (hipStream_t)stream,
+                     (const uint8_t*)packed_codes, (const uint8_t*)packed_scales, (int)rows, (int)K,
+                     (uint8_t*)codes, (uint8_t*)scales, scale_stride);
+  return (int)hipGetLastError();
 }
 
 extern "C" int fpq_pack_nvf4(const void* codes, const void* scales, int64_t scale_stride, int64_t rows,

@@ -22,6 +22,7 @@ from .hip_ops import (
     _version,
     as_bf16,
     classify_rotation,
+    is_packed_only,
     nv_packed_eligible,
     pack_mxf4,
     pack_nvf4,
@@ -30,6 +31,7 @@ from .hip_ops import (
     packed_weight_ready,
     packed_weights_enabled,
     quantize_mx_packed,
+    weight_rows,
 )
 
 
@@ -209,6 +211,11 @@ def wants_packed(m: int, n: int, k: int, nvfp4: bool) -> bool:
     return nv_packed_eligible(m, n, k) if nvfp4 else packed_linear_eligible(m, k, "abs_max")
 
 
+def weight_wants_packed(wq: torch.Tensor, m: int, k: int, nvfp4: bool) -> bool:
+    """wants_packed for the weight `wq`: always for one that is held in the packed layout only."""
+    return True if is_packed_only(wq) else wants_packed(m, wq.shape[0], k, nvfp4)
+
+
 def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alpha: torch.Tensor,
               bias: Optional[torch.Tensor], stream: int, use_packed: Optional[bool] = None,
               residual: Optional[torch.Tensor] = None,
@@ -223,6 +230,12 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
         wp, wsp, n = packed
         if qa.nvfp4 or wp.numel() * 2 != n * k:
             raise ValueError("packed weights need MXFP4 activations with the same inner dimension")
+        use_packed = True
+    elif is_packed_only(wq):   # a layer that holds its weight in the packed layout only
+        if qa.nvfp4:
+            raise ValueError("only MXFP4 weights are held in the packed layout")
+        n = weight_rows(wq, k)
+        wp = wsp = None
         use_packed = True
     else:
         n = wq.shape[0]
@@ -299,7 +312,7 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
     h = as_bf16(hadamard_matrix)
     kind, norm = classify_rotation(h)
     m, k = x_flat.shape
-    want_packed = wants_packed(m, wq.shape[0], k, nvfp4)
+    want_packed = weight_wants_packed(wq, m, k, nvfp4)
     if want_packed and not remember and not packed_weight_ready(wq, ws, nvfp4):
         want_packed = False   # no packed copy of the weight yet and none may be kept: row-major kernels
     qa = key = None
@@ -357,49 +370,67 @@ def _member_key(wq: torch.Tensor, ws: torch.Tensor, bias: Optional[torch.Tensor]
 
 
 def weight_group(members, create: bool = False) -> Optional[WeightGroup]:
-    """The WeightGroup of `members` = [(qweight, scales, bias or None), ...] (MXFP4, row-major, same K, every
-    N a multiple of 32, biases all absent or all contiguous bf16), remembered on the first member's qweight
-    until a member is written to; built now if `create`, else None when there is none."""
+    """The WeightGroup of `members` = [(qweight, scales, bias or None, in_features), ...] (MXFP4, same K, every
+    N a multiple of 32, biases all absent or all contiguous bf16; weights row-major, or all in the packed layout
+    only), remembered on the first member's qweight until a member is written to; built now if `create`,
+    else None when there is none."""
     first = members[0][0]
-    key = tuple(_member_key(*m) for m in members)
+    key = tuple(_member_key(*m[:3]) for m in members)
     hit = getattr(first, "_fpq_group", None)
     if hit is not None and hit.key == key:
         return hit
     if not create or not packed_weights_enabled():
         return None
-    k2 = first.shape[1]
+    k = members[0][3]
     dev = first.device
+    packed_only = is_packed_only(first)
     have_bias = [m[2] is not None for m in members]
-    for wq, ws, bias in members:
-        if (wq.dtype != torch.uint8 or ws.dtype != torch.uint8 or not wq.is_cuda or wq.device != dev
-                or not wq.is_contiguous() or not ws.is_contiguous() or wq.dim() != 2 or wq.shape[1] != k2
-                or wq.shape[0] % 32 != 0 or (k2 * 2) % 256 != 0 or ws.shape != (wq.shape[0], k2 * 2 // 32)):
+    if k < 256 or k % 256 != 0:
+        return None
+    for wq, ws, bias, k_in in members:
+        if (wq.dtype != torch.uint8 or ws.dtype != torch.uint8 or not wq.is_cuda or wq.device != dev or k_in != k
+                or not wq.is_contiguous() or not ws.is_contiguous() or is_packed_only(wq) != packed_only):
+            return None
+        if packed_only:
+            if ws.dim() != 1 or wq.numel() * 2 % (32 * k) != 0 or ws.numel() * 16 != wq.numel():
+                return None
+        elif (wq.dim() != 2 or wq.shape[1] * 2 != k or wq.shape[0] % 32 != 0 or ws.shape != (wq.shape[0], k // 32)):
             return None
         if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_contiguous() or bias.device != dev):
             return None
     if any(have_bias) and not all(have_bias):
         return None
     lib = _engine.lib()
-    k = k2 * 2
-    splits = [m[0].shape[0] for m in members]
+    splits = [weight_rows(m[0], k) for m in members]
     n = sum(splits)
     group = WeightGroup()
-    group.key, group.n, group.splits, group.k = key, n, splits, k
+    group.n, group.splits, group.k = n, splits, k
     with torch.cuda.device(dev):
         stream = _current_stream(dev.index)
-        group.wp = torch.empty(lib.fpq_packed_codes_bytes(n, k), dtype=torch.uint8, device=dev)
-        group.wsp = torch.empty(lib.fpq_packed_scales_bytes(n, k), dtype=torch.uint8, device=dev)
+        if packed_only:
+            # the members' buffers laid end to end; the members then live in the new buffers (views) and
+            # their own are freed, so the weights are still held once
+            group.wp = torch.cat([m[0] for m in members])
+            group.wsp = torch.cat([m[1] for m in members])
+        else:
+            group.wp = torch.empty(lib.fpq_packed_codes_bytes(n, k), dtype=torch.uint8, device=dev)
+            group.wsp = torch.empty(lib.fpq_packed_scales_bytes(n, k), dtype=torch.uint8, device=dev)
         row = 0
-        for wq, ws, _ in members:
-            rows = wq.shape[0]
+        for wq, ws, _, _ in members:
+            rows = weight_rows(wq, k)
             c0, c1 = lib.fpq_packed_codes_bytes(row, k), lib.fpq_packed_codes_bytes(row + rows, k)
             s0, s1 = lib.fpq_packed_scales_bytes(row, k), lib.fpq_packed_scales_bytes(row + rows, k)
             pc, ps = group.wp[c0:c1], group.wsp[s0:s1]
-            st = lib.fpq_pack_mxf4(wq.data_ptr(), ws.data_ptr(), ws.shape[1], rows, k, pc.data_ptr(), ps.data_ptr(), stream)
-            _engine.check(st, "fpq_pack_mxf4")
-            # the member's own packed copy: these views (same key as hip_ops.packed_weight uses)
-            wq._fpq_packed = ((wq.data_ptr(), _version(wq), ws.data_ptr(), _version(ws), tuple(wq.shape), False), pc, ps)
+            if packed_only:
+                wq.data, ws.data = pc, ps
+            else:
+                st = lib.fpq_pack_mxf4(wq.data_ptr(), ws.data_ptr(), ws.shape[1], rows, k, pc.data_ptr(), ps.data_ptr(),
+                                       stream)
+                _engine.check(st, "fpq_pack_mxf4")
+                # the member's own packed copy: these views (same key as hip_ops.packed_weight uses)
+                wq._fpq_packed = ((wq.data_ptr(), _version(wq), ws.data_ptr(), _version(ws), tuple(wq.shape), False), pc, ps)
             row += rows
+    group.key = tuple(_member_key(*m[:3]) for m in members)   # (packed-only members have just moved)
     group.bias = torch.cat([m[2] for m in members]).contiguous() if all(have_bias) else None
     try:
         first._fpq_group = group
@@ -510,7 +541,7 @@ def linear_group_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq
         # already (nothing may be created and kept here); the activations are quantized straight into
         # the packed layout only if every GEMM of the group wants them so (MXFP4), else row-major,
         # from which the packed form is made on demand
-        packed = [wants_packed(m, wq.shape[0], k, nvfp4) and packed_weight_ready(wq, ws, nvfp4)
+        packed = [weight_wants_packed(wq, m, k, nvfp4) and packed_weight_ready(wq, ws, nvfp4)
                   for wq, ws in zip(wqs, wss)]
         qa = quantize_activations(x, h, kind, norm, act_global_scales[0], nvfp4, stream,
                                   all(packed) and not nvfp4, remember=False)
@@ -526,7 +557,7 @@ def linear_group_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq
 
 @linear_group_w4a4_op.register_fake
 def _(x_flat, hadamard_matrix, wqs, wss, weight_global_scales, act_global_scales, biases, nvfp4):
-    return [x_flat.new_empty((x_flat.shape[0], wq.shape[0]), dtype=torch.bfloat16) for wq in wqs]
+    return [x_flat.new_empty((x_flat.shape[0], weight_rows(wq, x_flat.shape[1])), dtype=torch.bfloat16) for wq in wqs]
 
 
 @torch.library.custom_op("fp_quant::silu_mul_linear_w4a4_op", mutates_args=())
@@ -547,14 +578,14 @@ def silu_mul_linear_w4a4_op(gate: torch.Tensor, up: torch.Tensor, hadamard_matri
     dev = gate.device
     with torch.cuda.device(dev):
         alpha = linear_alpha(weight_global_scale, act_global_scale, remember=False)
-        use_packed = ready and wants_packed(qa.m, wq.shape[0], qa.k, nvfp4)
+        use_packed = ready and weight_wants_packed(wq, qa.m, qa.k, nvfp4)
         return linear_on(qa, wq, ws, alpha, bias, _current_stream(dev.index), use_packed)
 
 
 @silu_mul_linear_w4a4_op.register_fake
 def _(gate, up, hadamard_matrix, wq, ws, weight_global_scale, act_global_scale, bias, nvfp4):
     rows = gate.numel() // gate.shape[-1]
-    return gate.new_empty((rows, wq.shape[0]), dtype=torch.bfloat16)
+    return gate.new_empty((rows, weight_rows(wq, gate.shape[-1])), dtype=torch.bfloat16)
 
 
 def prime(hadamard_matrix: torch.Tensor, weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor) -> None:
@@ -588,7 +619,7 @@ def prepare_device(device: torch.device) -> None:
 
 @linear_w4a4_op.register_fake
 def _(x_flat, hadamard_matrix, wq, ws, weight_global_scale, act_global_scale, bias, nvfp4, quest=False):
-    return x_flat.new_empty((x_flat.shape[0], wq.shape[0]), dtype=torch.bfloat16)
+    return x_flat.new_empty((x_flat.shape[0], weight_rows(wq, x_flat.shape[1])), dtype=torch.bfloat16)
 
 
 ### Quantizers fused with the producer of their input

@@ -328,18 +328,54 @@ def nv_packed_eligible(m: int, n: int, k: int) -> bool:
             and ((m + 255) // 256) * ((n + 255) // 256) < 100)
 
 
+def unpack_mxf4(pc: torch.Tensor, ps: torch.Tensor, rows: int, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Packed MXFP4 operand -> row-major codes [rows, k/2] and E8M0 scales [rows, k/32] (the inverse of pack_mxf4)."""
+    lib = _engine.lib()
+    codes = torch.empty(rows, k // 2, dtype=torch.uint8, device=pc.device)
+    scales = torch.empty(rows, k // 32, dtype=torch.uint8, device=pc.device)
+    with torch.cuda.device(pc.device):
+        st = lib.fpq_unpack_mxf4(pc.data_ptr(), ps.data_ptr(), rows, k, codes.data_ptr(), scales.data_ptr(), k // 32,
+                                 _stream(pc))
+    _engine.check(st, "fpq_unpack_mxf4")
+    return codes, scales
+
+
+# A layer may hold its MXFP4 weight in the packed layout ONLY (FPQuantLinear.release_row_major): its
+# `qweight` / `scales` are then the 1-D packed buffers themselves.  The number of dimensions is the marker
+# (it survives every operator boundary); the row count follows from the inner dimension of the activations.
+def is_packed_only(wq: torch.Tensor) -> bool:
+    return wq.dim() == 1
+
+
+def weight_rows(wq: torch.Tensor, k: int) -> int:
+    """Output features of a weight given as row-major codes [n, k/2] or as a 1-D packed buffer (n % 32 == 0)."""
+    if wq.dim() == 2:
+        return wq.shape[0]
+    n = wq.numel() * 2 // max(k, 1)
+    if k < 256 or k % 256 != 0 or n * k != wq.numel() * 2 or n % 32 != 0:
+        raise ValueError(f"a packed weight of {wq.numel()} bytes does not match activations with K={k}")
+    return n
+
+
 def _packed_weight_key(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool):
     return (wq.data_ptr(), _version(wq), ws.data_ptr(), _version(ws), tuple(wq.shape), nvfp4)
 
 
 def packed_weight_ready(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False) -> bool:
     """Whether packed_weight would find its cached copy."""
+    if wq.dim() == 1:
+        return True
     hit = getattr(wq, "_fpq_packed", None)
     return hit is not None and hit[0] == _packed_weight_key(wq, ws, nvfp4)
 
 
 def packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Packed copy of a weight, cached on the code tensor until either tensor is written to."""
+    """Packed copy of a weight, cached on the code tensor until either tensor is written to (a weight
+    held in the packed layout only is its own packed copy)."""
+    if wq.dim() == 1:
+        if nvfp4:
+            raise ValueError("only MXFP4 weights are held in the packed layout")
+        return wq, ws
     key = _packed_weight_key(wq, ws, nvfp4)
     hit = getattr(wq, "_fpq_packed", None)
     if hit is not None and hit[0] == key:

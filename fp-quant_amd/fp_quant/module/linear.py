@@ -6,6 +6,7 @@ inference branch of `forward()` of the reference module
 the reference work unchanged.  Training branches (master weights, quantized backward) and
 pseudo-quantization are not part of this engine and raise.
 """
+import os
 from typing import Optional
 
 import torch
@@ -91,7 +92,9 @@ class FPQuantLinear(nn.Module):
         g = config.hadamard_group_size
         self.register_buffer("forward_hadamard_matrix", torch.empty(g, g, **factory))
         self.register_buffer("backward_hadamard_matrix", torch.empty(g, g, **factory))
+        self._register_load_state_dict_pre_hook(FPQuantLinear._before_load, with_module=True)
         self.register_load_state_dict_post_hook(FPQuantLinear._prime)
+        self._register_state_dict_hook(FPQuantLinear._row_major_state)
 
     @torch.no_grad()
     def pre_forward(self):
@@ -150,6 +153,65 @@ class FPQuantLinear(nn.Module):
         hip_ops.drop_tensor_caches(h, wgs, ags, getattr(self, "qweight", None), getattr(self, "scales", None))
         if all(isinstance(t, torch.Tensor) and t.is_cuda for t in (h, wgs, ags)):
             eager.prime(h, wgs, ags)
+        if self._fpq_single_copy or os.environ.get("FPQ_SINGLE_WEIGHT_COPY", "0") == "1":
+            self.release_row_major()
+
+    # True once release_row_major has been asked for: the layer goes back to the packed layout after
+    # every load_state_dict
+    _fpq_single_copy = False
+
+    @property
+    def weights_packed_only(self) -> bool:
+        q = getattr(self, "qweight", None)
+        return isinstance(q, torch.Tensor) and hip_ops.is_packed_only(q)
+
+    @torch.no_grad()
+    def release_row_major(self) -> bool:
+        """Keep the 4-bit weight once: `qweight` and `scales` become the 1-D buffers of the packed
+        layout the GEMM kernels read (what is otherwise a second copy next to the row-major tensors of
+        the reference, linear.py:87-88), and the row-major tensors are freed.  state_dict() still hands
+        out the reference's row-major tensors (re-tiled on demand) and load_state_dict() accepts them.
+        MXFP4 with in_features % 256 == 0 and out_features % 32 == 0 on a GPU; returns whether the
+        layer is in that state afterwards."""
+        if self.weights_packed_only:
+            return True
+        q, s = getattr(self, "qweight", None), getattr(self, "scales", None)
+        if (self.config.forward_dtype != FPQuantDtype.MXFP4 or q is None or s is None or not q.is_cuda
+                or q.dim() != 2 or q.dtype != torch.uint8 or s.dtype != torch.uint8
+                or self.in_features % 256 != 0 or self.out_features % 32 != 0
+                or tuple(q.shape) != (self.out_features, self.in_features // 2)
+                or tuple(s.shape) != (self.out_features, self.in_features // 32)):
+            return False
+        pc, ps = hip_ops.packed_weight(q.contiguous(), s.contiguous())
+        hip_ops.drop_tensor_caches(q, s)
+        self.qweight = nn.Parameter(pc, requires_grad=False)
+        self.scales = nn.Parameter(ps, requires_grad=False)
+        self._fpq_single_copy = True
+        return True
+
+    @torch.no_grad()
+    def restore_row_major(self) -> None:
+        """Undo release_row_major: `qweight` [out, in/2] and `scales` [out, in/32] as the reference holds them."""
+        if not self.weights_packed_only:
+            return
+        codes, scales = hip_ops.unpack_mxf4(self.qweight, self.scales, self.out_features, self.in_features)
+        self.qweight = nn.Parameter(codes, requires_grad=False)
+        self.scales = nn.Parameter(scales, requires_grad=False)
+        self._fpq_single_copy = False
+
+    def _row_major_state(self, state_dict, prefix, local_metadata):
+        """state_dict() hook: a layer that holds the packed layout only hands out row-major tensors."""
+        if self.weights_packed_only and prefix + "qweight" in state_dict and prefix + "scales" in state_dict:
+            with torch.no_grad():
+                codes, scales = hip_ops.unpack_mxf4(self.qweight.detach(), self.scales.detach(), self.out_features,
+                                                    self.in_features)
+            state_dict[prefix + "qweight"], state_dict[prefix + "scales"] = codes, scales
+
+    def _before_load(self, state_dict, prefix, *_):
+        """load_state_dict() pre-hook: row-major parameters to load into (the post-hook packs them again)."""
+        if self.weights_packed_only and (prefix + "qweight" in state_dict or prefix + "scales" in state_dict):
+            self.restore_row_major()
+            self._fpq_single_copy = True
 
     # A tensor of the output's shape that the next forward adds to its result (inside the GEMM
     # where the kernel can) and then clears; set by a fused decoder block around its attention call.

@@ -2,7 +2,13 @@
 from . import config, export, fuse, replace
 from .config import FPQuantConfig, FPQuantDtype, validate_config
 from .fuse import fuse_producers, unfuse_producers
-from .replace import finalize_master_weights, replace_quantize_with_fp_quant_linear, replace_with_fp_quant_linear
+from .replace import (
+    finalize_master_weights,
+    release_row_major_weights,
+    replace_quantize_with_fp_quant_linear,
+    replace_with_fp_quant_linear,
+    restore_row_major_weights,
+)
 
 __all__ = [
     "FPQuantConfig",
@@ -11,6 +17,8 @@ __all__ = [
     "replace_with_fp_quant_linear",
     "replace_quantize_with_fp_quant_linear",
     "finalize_master_weights",
+    "release_row_major_weights",
+    "restore_row_major_weights",
     "fuse_producers",
     "unfuse_producers",
     "config",

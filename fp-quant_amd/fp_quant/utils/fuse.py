@@ -100,7 +100,7 @@ def _weight_group(layers, create: bool = False):
         for layer in layers[1:]:
             if not torch.equal(layer.weight_global_scale.float(), first.weight_global_scale.float()):
                 return None
-    return _eager().weight_group([(l.qweight, l.scales, l.bias) for l in layers], create)
+    return _eager().weight_group([(l.qweight, l.scales, l.bias, l.in_features) for l in layers], create)
 
 
 def _attach_weight_group(module: nn.Module, names) -> None:
@@ -113,6 +113,7 @@ def _attach_weight_group(module: nn.Module, names) -> None:
                                     if all(_is_real_quant_linear(l) for l in layers) else None)
 
     build()
+    module._fpq_weight_group_build = build   # for whoever rewrites the layers' weights by other means
     module._fpq_weight_group_hook = module.register_load_state_dict_post_hook(build)
 
 
@@ -471,5 +472,6 @@ def unfuse_producers(model: nn.Module) -> None:
             if hook is not None:
                 hook.remove()
                 module._fpq_weight_group_hook = None
+                module._fpq_weight_group_build = None
             if hasattr(module, "_fpq_weight_group"):
                 module._fpq_weight_group = None

@@ -95,3 +95,35 @@ def finalize_master_weights(model, current_key_name=None):
             if module.config.store_master_weights:
                 module.config.store_master_weights = False  # the config object is shared
             module.pre_forward()
+
+
+def release_row_major_weights(model) -> int:
+    """Hold every eligible layer's 4-bit weight once, in the packed layout the GEMM kernels read
+    (FPQuantLinear.release_row_major): frees the row-major `qweight` / `scales` copies, half of the
+    weight memory of a quantized model.  state_dict() and load_state_dict() keep speaking the
+    reference's row-major tensors.  Call it after the linears have been replaced and quantized (before or
+    after fuse_producers).  Returns the number of layers that are in that state afterwards."""
+    from ..module import FPQuantLinear
+
+    count = 0
+    for module in model.modules():
+        if isinstance(module, FPQuantLinear) and module.release_row_major():
+            count += 1
+    for module in model.modules():   # groups of projections built on the old tensors follow their members
+        build = getattr(module, "_fpq_weight_group_build", None)
+        if build is not None:
+            build()
+    return count
+
+
+def restore_row_major_weights(model) -> None:
+    """Undo release_row_major_weights."""
+    from ..module import FPQuantLinear
+
+    for module in model.modules():
+        if isinstance(module, FPQuantLinear):
+            module.restore_row_major()
+    for module in model.modules():
+        build = getattr(module, "_fpq_weight_group_build", None)
+        if build is not None:
+            build()

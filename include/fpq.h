@@ -154,6 +154,14 @@ int64_t fpq_packed_codes_bytes(int64_t rows, int64_t K);
 int64_t fpq_packed_scales_bytes(int64_t rows, int64_t K);
 int fpq_pack_mxf4(const void* codes, const void* scales, int64_t scale_stride, int64_t rows,
                   int64_t K, void* packed_codes, void* packed_scales, void* stream);
+/*
+ * The inverse of fpq_pack_mxf4 for the first `rows` rows: row-major codes [rows, K/2] (16-byte aligned)
+ * and E8M0 scales (entry [row, k/32], row stride scale_stride >= K/32; only those entries are written)
+ * from a packed operand.  A layer that holds its weights in the packed layout only uses it to hand
+ * the reference's `qweight` / `scales` tensors (linear.py:87-88) to state_dict().
+ */
+int fpq_unpack_mxf4(const void* packed_codes, const void* packed_scales, int64_t rows, int64_t K,
+                    void* codes, void* scales, int64_t scale_stride, void* stream);
 
 /*
  * fpq_quantize_mx writing the packed layout directly (same codes and scale bytes; rows past

@@ -81,6 +81,20 @@ def pack(codes, scales, fill=0xCD):
     return pc.cpu(), ps.cpu()
 
 
+def unpack(pc, ps, rows, k, scale_pad=0, fill=0xCD):
+    """fpq_unpack_mxf4: CPU uint8 row-major codes [rows, k/2] and scales [rows, k/32 + scale_pad] (entries past
+    k/32 keep `fill`)."""
+    lib = _engine.lib()
+    pc, ps = pc.to("cuda").contiguous(), ps.to("cuda").contiguous()
+    codes = torch.full((rows, k // 2), fill, dtype=torch.uint8, device="cuda")
+    scales = torch.full((rows, k // 32 + scale_pad), fill, dtype=torch.uint8, device="cuda")
+    st = lib.fpq_unpack_mxf4(pc.data_ptr(), ps.data_ptr(), rows, k, codes.data_ptr(), scales.data_ptr(),
+                             scales.shape[1], torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_unpack_mxf4")
+    torch.cuda.synchronize()
+    return codes.cpu(), scales.cpu()
+
+
 def quantize_packed(x_bf16, rot="hadamard", g=128, norm=None, zero_policy=_engine.ZERO_REFERENCE, fill=0xCD):
     """fpq_quantize_mx_packed; CPU uint8 (packed codes, packed scales)."""
     lib = _engine.lib()

@@ -436,9 +436,10 @@ def test_fused_decoder_block_with_residual_epilogues_is_graph_capturable(tokens)
     assert block.self_attn.o_proj._fpq_residual is None
 
 
-@pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])
-@pytest.mark.parametrize("arch", ["llama", "qwen3"])
-def test_compiled_decode_with_grouped_operators_matches_eager(fmt, g, arch):
+@pytest.mark.parametrize("fmt,g,arch,held_once", [("mxfp4", 128, "llama", False), ("nvfp4", 16, "llama", False),
+                                                  ("mxfp4", 128, "qwen3", False), ("nvfp4", 16, "qwen3", False),
+                                                  ("mxfp4", 128, "llama", True)])
+def test_compiled_decode_with_grouped_operators_matches_eager(fmt, g, arch, held_once):
     """fuse_producers before torch.compile: the traced attention calls one operator for q/k/v and the
     traced MLP two (gate/up; SiLU*up -> down) instead of seven layer operators and an elementwise kernel.
     Reference: the eager model with only its MLPs fused (the fused SiLU*up arithmetic is this library's, the
@@ -480,6 +481,9 @@ def test_compiled_decode_with_grouped_operators_matches_eager(fmt, g, arch):
             assert fuse.fuse_gated_mlp(block.mlp)
         cache = fresh_cache()
         assert fuse.fuse_producers(model) == 10
+        if held_once:    # every operator of the traced model on weights held in the packed layout only
+            from fp_quant.utils import release_row_major_weights
+            assert release_row_major_weights(model) == 14
         torch._dynamo.reset()
         counters.clear()
         with inductor_config.patch(emulate_precision_casts=True):
@@ -535,3 +539,47 @@ def test_grouped_projections_run_as_one_gemm_on_concatenated_packed_weights(toke
         assert attn._fpq_weight_group is not group
         for a, b in zip(attn._fpq_qkv(x), want2):
             assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("order", ["fuse_then_release", "release_then_fuse"])
+def test_model_with_weights_held_once_keeps_its_logits(order):
+    """release_row_major_weights on a whole model, before or after fuse_producers: every layer holds the
+    packed layout only (the groups of projections included: their members are views into the group's
+    buffers), logits keep their bits eagerly and compiled, the state dict is the reference's, and loading
+    another model's state dict is followed."""
+    import fp_quant
+    from fp_quant.utils import fuse_producers, release_row_major_weights, restore_row_major_weights
+    model = _tiny_llama("mxfp4", 128, seed=11)
+    other = _tiny_llama("mxfp4", 128, seed=12)
+    ids = torch.randint(0, 128, (2, 40), generator=torch.Generator().manual_seed(3)).cuda()
+    one = ids[:, :1].contiguous()
+    n_layers = sum(isinstance(m, fp_quant.FPQuantLinear) for m in model.modules())
+    with torch.no_grad():
+        fuse_producers(other)
+        want_other = other(input_ids=ids).logits
+        reference_state = {k: v.clone() for k, v in model.state_dict().items()}
+        if order == "fuse_then_release":
+            assert fuse_producers(model) == 10
+            want, want_one = model(input_ids=ids).logits, model(input_ids=one).logits
+            assert release_row_major_weights(model) == n_layers
+        else:
+            assert release_row_major_weights(model) == n_layers
+            assert fuse_producers(model) == 10
+            restore_row_major_weights(model)
+            want, want_one = model(input_ids=ids).logits, model(input_ids=one).logits
+            assert release_row_major_weights(model) == n_layers
+        for block in model.model.layers:
+            attn, group = block.self_attn, block.self_attn._fpq_weight_group
+            assert group is not None and block.mlp._fpq_weight_group is not None
+            lo, hi = group.wp.data_ptr(), group.wp.data_ptr() + group.wp.numel()
+            for layer in (attn.q_proj, attn.k_proj, attn.v_proj):
+                assert layer.weights_packed_only and lo <= layer.qweight.data_ptr() < hi
+        assert torch.equal(model(input_ids=ids).logits, want)
+        assert torch.equal(model(input_ids=one).logits, want_one)
+        state = model.state_dict()
+        assert list(sorted(state)) == list(sorted(reference_state))
+        for k, v in reference_state.items():
+            assert state[k].shape == v.shape and torch.equal(state[k], v), k
+        model.load_state_dict(other.state_dict())
+        assert all(m.weights_packed_only for m in model.modules() if isinstance(m, fp_quant.FPQuantLinear))
+        assert torch.equal(model(input_ids=ids).logits, want_other)

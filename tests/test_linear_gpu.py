@@ -516,3 +516,72 @@ def test_prepare_device_entry_point():
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g, stream=s):
         assert lib.fpq_prepare_device(s.cuda_stream) == _engine.E_UNSUPPORTED   # must run, not be recorded
+
+
+@pytest.mark.parametrize("bias", [False, True])
+def test_release_row_major_keeps_results_and_the_reference_state_dict(bias):
+    """FPQuantLinear.release_row_major: the packed buffers become the only copy of the weight; outputs keep
+    their bits on every kernel path (1, 40, 300 and 2100 rows), state_dict() still holds the reference's
+    row-major tensors, load_state_dict() accepts them and the layer goes back to the packed layout, and
+    restore_row_major gives the original tensors back."""
+    k, n = 512, 384
+    lin = _quantized_linear("mxfp4", 128, k, n, seed=5, bias=bias)
+    other = _quantized_linear("mxfp4", 128, k, n, seed=6, bias=bias)
+    xs = [torch.randn(m, k, device="cuda", dtype=torch.bfloat16) for m in (1, 40, 300, 2100)]
+    with torch.no_grad():
+        want = [lin(x) for x in xs]
+        want_other = [other(x) for x in xs]
+        q0, s0 = lin.qweight.detach().clone(), lin.scales.detach().clone()
+        keys = list(lin.state_dict().keys())
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        assert lin.release_row_major() and lin.weights_packed_only
+        assert lin.qweight.dim() == 1 and lin.qweight.numel() == n * k // 2 and lin.scales.numel() == n * k // 32
+        torch.cuda.synchronize()
+        assert before - torch.cuda.memory_allocated() >= n * k // 2        # the row-major codes are gone
+        for x, w in zip(xs, want):
+            assert torch.equal(lin(x), w)
+        sd = {key: v.clone() for key, v in lin.state_dict().items()}   # (entries alias the live parameters)
+        assert sorted(sd.keys()) == sorted(keys)
+        assert torch.equal(sd["qweight"], q0) and torch.equal(sd["scales"], s0)
+        # traced callers
+        torch._dynamo.reset()
+        assert torch.equal(torch.compile(lin, fullgraph=True)(xs[1]), want[1])
+        torch._dynamo.reset()
+        # a checkpoint in the reference's layout loads, and the layer is packed-only again afterwards
+        lin.load_state_dict(other.state_dict())
+        assert lin.weights_packed_only
+        for x, w in zip(xs, want_other):
+            assert torch.equal(lin(x), w)
+        lin.load_state_dict(sd)
+        lin.restore_row_major()
+        assert not lin.weights_packed_only
+        assert torch.equal(lin.qweight, q0) and torch.equal(lin.scales, s0)
+        for x, w in zip(xs, want):
+            assert torch.equal(lin(x), w)
+
+
+def test_release_row_major_declines_what_the_packed_layout_cannot_hold():
+    nv = _quantized_linear("nvfp4", 16, 256, 64, seed=1)
+    assert not nv.release_row_major() and nv.qweight.dim() == 2
+    ragged = _quantized_linear("mxfp4", 32, 256, 48, seed=2)        # 48 output features: not whole 32-row tiles
+    assert not ragged.release_row_major() and ragged.qweight.dim() == 2
+    short = _quantized_linear("mxfp4", 32, 128, 64, seed=3)         # K = 128: below one 256-K block
+    assert not short.release_row_major()
+    x = torch.randn(5, 256, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        assert nv(x).shape == (5, 64) and ragged(x).shape == (5, 48)
+
+
+def test_single_weight_copy_by_environment(monkeypatch):
+    """FPQ_SINGLE_WEIGHT_COPY=1: every eligible layer releases its row-major tensors as soon as it is quantized."""
+    monkeypatch.setenv("FPQ_SINGLE_WEIGHT_COPY", "1")
+    lin = _quantized_linear("mxfp4", 128, 256, 64, seed=8)
+    assert lin.weights_packed_only
+    monkeypatch.delenv("FPQ_SINGLE_WEIGHT_COPY")
+    plain = _quantized_linear("mxfp4", 128, 256, 64, seed=8)
+    assert not plain.weights_packed_only
+    x = torch.randn(7, 256, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        assert torch.equal(lin(x), plain(x))
+    assert torch.equal(lin.state_dict()["qweight"], plain.qweight)

@@ -268,3 +268,21 @@ def test_nvfp4_linear_mid_m_runs_packed_and_matches_oracle(monkeypatch):
     monkeypatch.setenv("FPQ_PACKED_WEIGHTS", "0")
     y_rm = lin(x.cuda()).cpu()
     assert ((y.double() - y_rm.double()).abs() <= 2.0 ** -7 * ref.abs() + 1e-5 * mag + 1e-6).all()
+
+
+@pytest.mark.parametrize("rows,k", [(1, 256), (33, 768), (70, 512), (256, 4096), (1000, 1024)])
+def test_unpack_is_the_inverse_of_the_layout_definition(rows, k):
+    """fpq_unpack_mxf4 on a packed operand written by the layout's definition gives back the row-major codes
+    and scales (ragged last row tile; a scale matrix wider than K/32 keeps its other entries)."""
+    g = torch.Generator().manual_seed(rows + k)
+    codes = torch.randint(0, 256, (rows, k // 2), dtype=torch.uint8, generator=g)
+    scales = torch.randint(0, 256, (rows, k // 32), dtype=torch.uint8, generator=g)
+    pc, ps = pack_by_definition(codes, scales, k)
+    got_c, got_s = capi.unpack(pc, ps, rows, k)
+    assert torch.equal(got_c, codes) and torch.equal(got_s, scales)
+    got_c, got_s = capi.unpack(pc, ps, rows, k, scale_pad=4)
+    assert torch.equal(got_c, codes) and torch.equal(got_s[:, : k // 32], scales)
+    assert (got_s[:, k // 32:] == 0xCD).all()
+    # and of fpq_pack_mxf4
+    pc2, ps2 = capi.pack(codes, scales)
+    assert torch.equal(pc2, pc) and torch.equal(ps2, ps)
