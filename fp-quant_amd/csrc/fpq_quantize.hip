@@ -271,6 +271,14 @@ __device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint3
       packed |= e2m1_code<ZERO>(q) << (4 * i);
       mbits |= (uint32_t)(__builtin_fabsf(q) < 6.0f) << i;
     }
+    if (pro.packed_rows != 0u) {   // packed operand layout (no mask there); pad rows get zeros
+      if (chunk < pro.packed_rows * chunks_per_row) {
+        const uint32_t row = chunk / chunks_per_row, cc = chunk - row * chunks_per_row;
+        codes[packed_code_word(row, cc, chunks_per_row)] = active ? packed : 0u;
+        if ((cc & 3u) == 0u) scales[packed_scale_byte<FMT>(row, cc, chunks_per_row)] = active ? (uint8_t)ex : (uint8_t)0;
+      }
+      return;
+    }
     if (active) {
       codes[chunk] = packed;
       if (mask) mask[chunk] = (uint8_t)mbits;
@@ -366,78 +374,6 @@ __global__ __launch_bounds__(256) void quantize_lane8_kernel(
   fill_scale_padding(scales, rows, chunks_per_row / (GROUP / 8), scale_rows, scale_stride);
 }
 
-template <int G, int ROT>
-static int launch_lane8_quest(const void* x, int64_t rows, int64_t cols, float norm, void* codes, void* scales,
-                              int64_t scale_rows, int64_t scale_stride, void* mask, int zero_policy,
-                              hipStream_t stream, const void* h) {
-  const int64_t n_chunks = rows * cols / 8;
-  const dim3 grid((unsigned)((n_chunks + 255) / 256)), block(256);
-  auto args = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint4*)x, (uint32_t*)codes,
-                       (uint8_t*)scales, (uint32_t)n_chunks, (uint32_t)(cols / 8), (uint32_t)rows,
-                       (uint32_t)scale_rows, (uint32_t)scale_stride, norm, (const float*)nullptr,
-                       (const uint16_t*)h, (uint8_t*)mask, Prologue{});
-  };
-  if (zero_policy == FPQ_ZERO_REFERENCE) {
-    args(quantize_lane8_kernel<G, kFmtMx, ROT, kZeroReference, true>);
-  } else {
-    args(quantize_lane8_kernel<G, kFmtMx, ROT, kZeroSigned, true>);
-  }
-  return (int)hipGetLastError();
-}
-
-static int dispatch_quest(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
-                          const void* h, void* codes, void* scales, int64_t scale_rows, int64_t scale_stride,
-                          void* mask, int zero_policy, void* stream_) {
-  hipStream_t stream = (hipStream_t)stream_;
-  if (rows < 0 || cols < 0) return FPQ_E_SHAPE;
-  if (rows == 0 || cols == 0) return FPQ_OK;
-  if (!x || !codes || !scales) return FPQ_E_NULL;
-  if (zero_policy != FPQ_ZERO_REFERENCE && zero_policy != FPQ_ZERO_SIGNED) return FPQ_E_POLICY;
-  if (rot_kind == FPQ_ROT_IDENTITY) g = 32;
-  if (g != 16 && g != 32 && g != 64 && g != 128) return FPQ_E_ROTATION;
-  if (cols % g != 0 || cols % 32 != 0) return FPQ_E_SHAPE;
-  if (scale_rows < rows || scale_stride < cols / 32) return FPQ_E_SHAPE;
-  if (rows * cols >= (int64_t)1 << 34 || scale_rows * scale_stride >= (int64_t)1 << 32) return FPQ_E_SHAPE;
-  if (((uintptr_t)x & 15u) || ((uintptr_t)codes & 3u)) return FPQ_E_ALIGN;
-#define FPQ_LAUNCH_QUEST(GG, RR)                                                                   \
-  return launch_lane8_quest<GG, RR>(x, rows, cols, norm, codes, scales, scale_rows, scale_stride, \
-                                    mask, zero_policy, stream, h)
-  if (rot_kind == FPQ_ROT_GENERAL) {
-    if (!h) return FPQ_E_NULL;
-    if ((uintptr_t)h & 1u) return FPQ_E_ALIGN;
-  }
-  switch (rot_kind) {
-    case FPQ_ROT_IDENTITY: FPQ_LAUNCH_QUEST(32, FPQ_ROT_IDENTITY);
-    case FPQ_ROT_HADAMARD:
-      switch (g) {
-        case 16: FPQ_LAUNCH_QUEST(16, FPQ_ROT_HADAMARD);
-        case 32: FPQ_LAUNCH_QUEST(32, FPQ_ROT_HADAMARD);
-        case 64: FPQ_LAUNCH_QUEST(64, FPQ_ROT_HADAMARD);
-        case 128: FPQ_LAUNCH_QUEST(128, FPQ_ROT_HADAMARD);
-      }
-      break;
-    case FPQ_ROT_GSR:
-      switch (g) {
-        case 16: FPQ_LAUNCH_QUEST(16, FPQ_ROT_GSR);
-        case 32: FPQ_LAUNCH_QUEST(32, FPQ_ROT_GSR);
-        case 64: FPQ_LAUNCH_QUEST(64, FPQ_ROT_GSR);
-        case 128: FPQ_LAUNCH_QUEST(128, FPQ_ROT_GSR);
-      }
-      break;
-    case FPQ_ROT_GENERAL:
-      switch (g) {
-        case 16: FPQ_LAUNCH_QUEST(16, FPQ_ROT_GENERAL);
-        case 32: FPQ_LAUNCH_QUEST(32, FPQ_ROT_GENERAL);
-        case 64: FPQ_LAUNCH_QUEST(64, FPQ_ROT_GENERAL);
-        case 128: FPQ_LAUNCH_QUEST(128, FPQ_ROT_GENERAL);
-      }
-      break;
-  }
-#undef FPQ_LAUNCH_QUEST
-  return FPQ_E_ROTATION;
-}
-
 template <int G, int FMT, int ROT>
 static int launch_lane8(const void* x, int64_t rows, int64_t cols, float norm, const float* gsp,
                         void* codes, void* scales, int64_t scale_rows, int64_t scale_stride,
@@ -508,13 +444,18 @@ __device__ __forceinline__ uint32_t fix_zero_nibbles(uint32_t w) {
 constexpr uint32_t kSiluLdsFirst = 113u << 7;         // bf16 magnitude bits of 2^-14
 constexpr uint32_t kSiluLdsCount = 21u * 128u;        // magnitudes up to (not including) 2^7
 
-template <int EPL, int G, int FMT, int ROT, int ZERO, bool PACKED = false, int PRO = kProNone>
+// QUEST (MXFP4, no prologue): the scale of a group comes from its standard deviation instead of its
+// maximum (the rule and its fixed fp32 summation order are stated at lane8_process); a lane holds whole
+// groups, so the statistic needs no cross-lane step, the scale is a power of two, and the conversion
+// instruction divides by it exactly and saturates at +-6.
+template <int EPL, int G, int FMT, int ROT, int ZERO, bool PACKED = false, int PRO = kProNone, bool QUEST = false>
 __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
     const uint8_t* __restrict__ x, uint8_t* __restrict__ codes, uint8_t* __restrict__ scales,
     uint32_t n_chunks, uint32_t chunks_per_row, uint32_t rows, uint32_t scale_rows,
     uint32_t scale_stride, float norm, const float* __restrict__ global_scale, Prologue pro) {
   static_assert(!PACKED || EPL == 64, "packed output: 64-element chunks");
   static_assert(PRO == kProNone || (PACKED && FMT == kFmtMx), "prologues exist for the packed MXFP4 output only");
+  static_assert(!QUEST || (FMT == kFmtMx && PRO == kProNone), "the quest rule exists for plain MXFP4 only");
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
   constexpr int NG = EPL / GROUP;        // groups (= scale bytes) per chunk
   constexpr int PIECES = EPL / 8;        // 16-byte input pieces per chunk
@@ -739,12 +680,37 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
 #pragma unroll
     for (int gi = 0; gi < NG; ++gi) {
       float a = 0.0f;
+      if (!QUEST) {
 #pragma unroll
-      for (int i = 0; i < GROUP; ++i) a = __builtin_fmaxf(a, __builtin_fabsf(v[gi * GROUP + i]));
+        for (int i = 0; i < GROUP; ++i) a = __builtin_fmaxf(a, __builtin_fabsf(v[gi * GROUP + i]));
+      }
       uint32_t byte;
       bool fast;
       float k1, k2, cvt_scale;
-      if (FMT == kFmtMx) {
+      if (QUEST) {
+        float os[4], oq[4];
+#pragma unroll
+        for (int o = 0; o < 4; ++o) {
+          const float* p = &v[gi * GROUP + 8 * o];
+          float sum = p[0], sq = p[0] * p[0];
+#pragma unroll
+          for (int i = 1; i < 8; ++i) {
+            sum = sum + p[i];
+            sq = sq + p[i] * p[i];
+          }
+          os[o] = sum;
+          oq[o] = sq;
+        }
+        const float sum = (os[0] + os[1]) + (os[2] + os[3]), sq = (oq[0] + oq[1]) + (oq[2] + oq[3]);
+        const float mean = sum * 0.03125f, msq = sq * 0.03125f;
+        float var = msq - mean * mean;
+        var = var > 0.0f ? var : 0.0f;
+        const float sc = __builtin_sqrtf(var) * 0.48707976f + 1e-8f;   // fl32(2.92247856 / 6); >= 1e-8: normal
+        byte = (__float_as_uint(sc) >> 23) & 0xffu;
+        fast = true;
+        k1 = k2 = 0.0f;
+        cvt_scale = __uint_as_float(byte << 23);                         // s = 2^floor(log2(sc))
+      } else if (FMT == kFmtMx) {
         const uint32_t bits = __float_as_uint(a);
         byte = bits >> 23;
         fast = (byte - 29u) <= 198u || bits == 0u;                       // -98 <= e <= 100, or all zero
@@ -772,9 +738,9 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
 #pragma unroll
         for (int h = 0; h < 4; ++h) {
           const float x0 = v[gi * GROUP + d * 8 + 2 * h], x1 = v[gi * GROUP + d * 8 + 2 * h + 1];
-          float q0 = __builtin_fmaf(x0, k1, x0 * k2);
-          float q1 = __builtin_fmaf(x1, k1, x1 * k2);
-          if (ZERO == kZeroSigned) {  // x / s keeps the sign of x, also for -0
+          float q0 = QUEST ? x0 : __builtin_fmaf(x0, k1, x0 * k2);
+          float q1 = QUEST ? x1 : __builtin_fmaf(x1, k1, x1 * k2);
+          if (ZERO == kZeroSigned && !QUEST) {  // x / s keeps the sign of x, also for -0
             q0 = __builtin_copysignf(q0, x0);
             q1 = __builtin_copysignf(q1, x1);
           }
@@ -913,7 +879,7 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
   if (!PACKED) fill_scale_padding(scales, rows, chunks_per_row * NG, scale_rows, scale_stride);
 }
 
-template <int EPL, int G, int FMT, int ROT>
+template <int EPL, int G, int FMT, int ROT, bool QUEST = false>
 static int launch_stream(const void* x, int64_t rows, int64_t cols, float norm, const float* gsp,
                          void* codes, void* scales, int64_t scale_rows, int64_t scale_stride,
                          int zero_policy, hipStream_t stream) {
@@ -928,16 +894,16 @@ static int launch_stream(const void* x, int64_t rows, int64_t cols, float norm, 
                        (uint32_t)scale_rows, (uint32_t)scale_stride, norm, gsp, Prologue{});
   };
   if (zero_policy == FPQ_ZERO_REFERENCE) {
-    go(quantize_stream_kernel<EPL, G, FMT, ROT, kZeroReference>);
+    go(quantize_stream_kernel<EPL, G, FMT, ROT, kZeroReference, false, kProNone, QUEST>);
   } else {
-    go(quantize_stream_kernel<EPL, G, FMT, ROT, kZeroSigned>);
+    go(quantize_stream_kernel<EPL, G, FMT, ROT, kZeroSigned, false, kProNone, QUEST>);
   }
   return (int)hipGetLastError();
 }
 
 constexpr int kSiluDynLds = 4 * 64 * 128 + 2 * (int)kSiluLdsCount * 2;  // second tiles + table copy
 
-template <int G, int ROT, int PRO = kProNone, int FMT = kFmtMx>
+template <int G, int ROT, int PRO = kProNone, int FMT = kFmtMx, bool QUEST = false>
 static int launch_stream_packed(const void* x, int64_t rows, int64_t cols, float norm, void* codes,
                                 void* scales, int zero_policy, hipStream_t stream,
                                 const Prologue& pro = Prologue{}, const float* gsp = nullptr) {
@@ -958,9 +924,9 @@ static int launch_stream_packed(const void* x, int64_t rows, int64_t cols, float
                        (uint32_t)rows, 0u, 0u, norm, gsp, pro);
   };
   if (zero_policy == FPQ_ZERO_REFERENCE) {
-    go(quantize_stream_kernel<64, G, FMT, ROT, kZeroReference, true, PRO>);
+    go(quantize_stream_kernel<64, G, FMT, ROT, kZeroReference, true, PRO, QUEST>);
   } else {
-    go(quantize_stream_kernel<64, G, FMT, ROT, kZeroSigned, true, PRO>);
+    go(quantize_stream_kernel<64, G, FMT, ROT, kZeroSigned, true, PRO, QUEST>);
   }
   if (status) return status;
   return (int)hipGetLastError();
@@ -1014,6 +980,138 @@ static int dispatch_packed(const void* x, int64_t rows, int64_t cols, int rot_ki
     return FPQ_E_UNSUPPORTED;    // arbitrary matrices: quantize row-major, then fpq_pack_mxf4
   }
 #undef FPQ_LAUNCH_PACKED
+  return FPQ_E_ROTATION;
+}
+
+template <int G, int ROT>
+static int launch_lane8_quest(const void* x, int64_t rows, int64_t cols, float norm, void* codes, void* scales,
+                              int64_t scale_rows, int64_t scale_stride, void* mask, int zero_policy,
+                              hipStream_t stream, const void* h, bool packed = false) {
+  const int64_t n_chunks = rows * cols / 8;
+  Prologue pro{};
+  pro.packed_rows = packed ? (uint32_t)((rows + 31) / 32 * 32) : 0u;
+  const int64_t threads = packed ? (int64_t)pro.packed_rows * (cols / 8) : n_chunks;
+  const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+  auto args = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, (const uint4*)x, (uint32_t*)codes,
+                       (uint8_t*)scales, (uint32_t)n_chunks, (uint32_t)(cols / 8), (uint32_t)rows,
+                       (uint32_t)scale_rows, (uint32_t)scale_stride, norm, (const float*)nullptr,
+                       (const uint16_t*)h, (uint8_t*)mask, pro);
+  };
+  if (zero_policy == FPQ_ZERO_REFERENCE) {
+    args(quantize_lane8_kernel<G, kFmtMx, ROT, kZeroReference, true>);
+  } else {
+    args(quantize_lane8_kernel<G, kFmtMx, ROT, kZeroSigned, true>);
+  }
+  return (int)hipGetLastError();
+}
+
+static int dispatch_quest(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                          const void* h, void* codes, void* scales, int64_t scale_rows, int64_t scale_stride,
+                          void* mask, int zero_policy, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (rows < 0 || cols < 0) return FPQ_E_SHAPE;
+  if (rows == 0 || cols == 0) return FPQ_OK;
+  if (!x || !codes || !scales) return FPQ_E_NULL;
+  if (zero_policy != FPQ_ZERO_REFERENCE && zero_policy != FPQ_ZERO_SIGNED) return FPQ_E_POLICY;
+  if (rot_kind == FPQ_ROT_IDENTITY) g = 32;
+  if (g != 16 && g != 32 && g != 64 && g != 128) return FPQ_E_ROTATION;
+  if (cols % g != 0 || cols % 32 != 0) return FPQ_E_SHAPE;
+  if (scale_rows < rows || scale_stride < cols / 32) return FPQ_E_SHAPE;
+  if (rows * cols >= (int64_t)1 << 34 || scale_rows * scale_stride >= (int64_t)1 << 32) return FPQ_E_SHAPE;
+  if (((uintptr_t)x & 15u) || ((uintptr_t)codes & 3u)) return FPQ_E_ALIGN;
+  // big inputs without a clip mask: the streaming kernel, under the conditions of the abs-max dispatch
+  const bool stream_ok = !mask && cols % FPQ_EPL == 0 && rows * cols >= (int64_t)1 << 21 &&
+                         !((uintptr_t)codes & 15u) && !((uintptr_t)scales & 7u);
+#define FPQ_LAUNCH_QUEST(GG, RR)                                                                   \
+  return launch_lane8_quest<GG, RR>(x, rows, cols, norm, codes, scales, scale_rows, scale_stride, \
+                                    mask, zero_policy, stream, h)
+#define FPQ_LAUNCH_QUEST_STREAM(GG, RR)                                                                        \
+  {                                                                                                            \
+    if (stream_ok)                                                                                             \
+      return launch_stream<FPQ_EPL, GG, kFmtMx, RR, true>(x, rows, cols, norm, nullptr, codes, scales,        \
+                                                          scale_rows, scale_stride, zero_policy, stream);     \
+    FPQ_LAUNCH_QUEST(GG, RR);                                                                                  \
+  }
+  if (rot_kind == FPQ_ROT_GENERAL) {
+    if (!h) return FPQ_E_NULL;
+    if ((uintptr_t)h & 1u) return FPQ_E_ALIGN;
+  }
+  switch (rot_kind) {
+    case FPQ_ROT_IDENTITY: FPQ_LAUNCH_QUEST_STREAM(32, FPQ_ROT_IDENTITY);
+    case FPQ_ROT_HADAMARD:
+      switch (g) {
+        case 16: FPQ_LAUNCH_QUEST_STREAM(16, FPQ_ROT_HADAMARD);
+        case 32: FPQ_LAUNCH_QUEST_STREAM(32, FPQ_ROT_HADAMARD);
+        case 64: FPQ_LAUNCH_QUEST_STREAM(64, FPQ_ROT_HADAMARD);
+        case 128: FPQ_LAUNCH_QUEST_STREAM(128, FPQ_ROT_HADAMARD);
+      }
+      break;
+    case FPQ_ROT_GSR:
+      switch (g) {
+        case 16: FPQ_LAUNCH_QUEST_STREAM(16, FPQ_ROT_GSR);
+        case 32: FPQ_LAUNCH_QUEST_STREAM(32, FPQ_ROT_GSR);
+        case 64: FPQ_LAUNCH_QUEST_STREAM(64, FPQ_ROT_GSR);
+        case 128: FPQ_LAUNCH_QUEST(128, FPQ_ROT_GSR);  // a block spans two lanes of the streaming kernel
+      }
+      break;
+    case FPQ_ROT_GENERAL:
+      switch (g) {
+        case 16: FPQ_LAUNCH_QUEST(16, FPQ_ROT_GENERAL);
+        case 32: FPQ_LAUNCH_QUEST(32, FPQ_ROT_GENERAL);
+        case 64: FPQ_LAUNCH_QUEST(64, FPQ_ROT_GENERAL);
+        case 128: FPQ_LAUNCH_QUEST(128, FPQ_ROT_GENERAL);
+      }
+      break;
+  }
+#undef FPQ_LAUNCH_QUEST_STREAM
+#undef FPQ_LAUNCH_QUEST
+  return FPQ_E_ROTATION;
+}
+
+// fpq_quantize_mx_quest writing the packed operand layout (no clip mask): the streaming kernel, or the
+// generic kernel for a few rows, under the conditions of dispatch_packed.
+static int dispatch_quest_packed(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                                 void* codes, void* scales, int zero_policy, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (rows < 0 || cols < 0) return FPQ_E_SHAPE;
+  if (rows == 0 || cols == 0) return FPQ_OK;
+  if (!x || !codes || !scales) return FPQ_E_NULL;
+  if (zero_policy != FPQ_ZERO_REFERENCE && zero_policy != FPQ_ZERO_SIGNED) return FPQ_E_POLICY;
+  if (rot_kind == FPQ_ROT_IDENTITY) g = 32;
+  if (g != 16 && g != 32 && g != 64 && g != 128) return FPQ_E_ROTATION;
+  if (cols % 256 != 0) return FPQ_E_SHAPE;
+  if (rows * cols >= (int64_t)1 << 34) return FPQ_E_SHAPE;
+  if (((uintptr_t)x & 15u) || ((uintptr_t)codes & 15u) || ((uintptr_t)scales & 3u)) return FPQ_E_ALIGN;
+  const bool few = rows <= kPackedFewRows;
+#define FPQ_LAUNCH_QUEST_PACKED(GG, RR)                                                                           \
+  {                                                                                                               \
+    if (few)                                                                                                      \
+      return launch_lane8_quest<GG, RR>(x, rows, cols, norm, codes, scales, rows, cols / 32, nullptr,             \
+                                        zero_policy, stream, nullptr, true);                                      \
+    return launch_stream_packed<GG, RR, kProNone, kFmtMx, true>(x, rows, cols, norm, codes, scales, zero_policy,  \
+                                                                stream);                                          \
+  }
+  if (rot_kind == FPQ_ROT_IDENTITY) {
+    FPQ_LAUNCH_QUEST_PACKED(32, FPQ_ROT_IDENTITY);
+  } else if (rot_kind == FPQ_ROT_HADAMARD) {
+    switch (g) {
+      case 16: FPQ_LAUNCH_QUEST_PACKED(16, FPQ_ROT_HADAMARD);
+      case 32: FPQ_LAUNCH_QUEST_PACKED(32, FPQ_ROT_HADAMARD);
+      case 64: FPQ_LAUNCH_QUEST_PACKED(64, FPQ_ROT_HADAMARD);
+      case 128: FPQ_LAUNCH_QUEST_PACKED(128, FPQ_ROT_HADAMARD);
+    }
+  } else if (rot_kind == FPQ_ROT_GSR) {
+    switch (g) {
+      case 16: FPQ_LAUNCH_QUEST_PACKED(16, FPQ_ROT_GSR);
+      case 32: FPQ_LAUNCH_QUEST_PACKED(32, FPQ_ROT_GSR);
+      case 64: FPQ_LAUNCH_QUEST_PACKED(64, FPQ_ROT_GSR);
+    }
+    return FPQ_E_UNSUPPORTED;  // a 128-wide sequency-ordered block spans two lanes
+  } else if (rot_kind == FPQ_ROT_GENERAL) {
+    return FPQ_E_UNSUPPORTED;    // arbitrary matrices: quantize row-major, then fpq_pack_mxf4
+  }
+#undef FPQ_LAUNCH_QUEST_PACKED
   return FPQ_E_ROTATION;
 }
 
@@ -1357,6 +1455,13 @@ extern "C" int fpq_quantize_mx(const void* x, int64_t rows, int64_t cols, int ro
                                void* stream) {
   return fpq::dispatch<fpq::kFmtMx>(x, rows, cols, rot_kind, g, norm, h, nullptr, codes, scales,
                                     scale_rows, scale_stride, zero_policy, stream);
+}
+
+extern "C" int fpq_quantize_mx_quest_packed(const void* x, int64_t rows, int64_t cols, int rot_kind, int g,
+                                            float norm, void* packed_codes, void* packed_scales, int zero_policy,
+                                            void* stream) {
+  return fpq::dispatch_quest_packed(x, rows, cols, rot_kind, g, norm, packed_codes, packed_scales, zero_policy,
+                                    stream);
 }
 
 extern "C" int fpq_quantize_mx_quest(const void* x, int64_t rows, int64_t cols, int rot_kind, int g,

@@ -34,6 +34,7 @@ _SIGNATURES = {
     "fpq_pack_mxf4": ([_P, _P, _I64, _I64, _I64, _P, _P, _P], _I),
     "fpq_quantize_mx_quest": ([_P, _I64, _I64, _I, _I, _F, _P, _P, _P, _I64, _I64, _P, _I, _P], _I),
     "fpq_quantize_mx_packed": ([_P, _I64, _I64, _I, _I, _F, _P, _P, _I, _P], _I),
+    "fpq_quantize_mx_quest_packed": ([_P, _I64, _I64, _I, _I, _F, _P, _P, _I, _P], _I),
     "fpq_quantize_nv_packed": ([_P, _I64, _I64, _I, _I, _F, _P, _P, _P, _I, _P], _I),
     "fpq_rotated_absmax": ([_P, _I64, _I64, _I, _I, _F, _P, _P, _P], _I),
     "fpq_row_inv_rms": ([_P, _I64, _I64, _I64, _F, _P, _P], _I),

@@ -160,8 +160,17 @@ def quantize_activations(x_flat: torch.Tensor, h: torch.Tensor, kind: int, norm:
     dev = x_flat.device
     g = h.shape[0]
     qa = QuantizedActivations(m, k, nvfp4)
+    if quest and want_packed:
+        pc = torch.empty(lib.fpq_packed_codes_bytes(m, k), dtype=torch.uint8, device=dev)
+        ps = torch.empty(lib.fpq_packed_scales_bytes(m, k), dtype=torch.uint8, device=dev)
+        st = lib.fpq_quantize_mx_quest_packed(x_flat.data_ptr(), m, k, kind, g, norm, pc.data_ptr(), ps.data_ptr(),
+                                              ZERO_NIBBLE_POLICY, stream)
+        if st != _engine.E_UNSUPPORTED:
+            _engine.check(st, "fpq_quantize_mx_quest_packed")
+            qa.mx_packed = (pc, ps)
+            return qa
     if quest:
-        # the quest rule (MXFP4) has a row-major kernel only; the packed form is made from it on demand
+        # rotations the packed kernel does not take: row-major, the packed form is made from it on demand
         codes = torch.empty(m, k // 2, dtype=torch.uint8, device=dev)
         scales = torch.empty(m, k // 32, dtype=torch.uint8, device=dev)
         st = lib.fpq_quantize_mx_quest(x_flat.data_ptr(), m, k, kind, g, norm, h.data_ptr(), codes.data_ptr(),

@@ -104,6 +104,14 @@ int fpq_quantize_mx(const void* x, int64_t rows, int64_t cols, int rot_kind, int
 int fpq_quantize_mx_quest(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
                           const void* h, void* codes, void* scales, int64_t scale_rows,
                           int64_t scale_stride, void* mask, int zero_policy, void* stream);
+/*
+ * fpq_quantize_mx_quest (without a mask) writing the packed operand layout directly, as
+ * fpq_quantize_mx_packed does for the abs-max rule: same codes and scale bytes, re-tiled; same
+ * conditions (cols % 256 == 0; Hadamard 16..128, identity, sequency-ordered Hadamard up to 64 wide;
+ * other rotations return FPQ_E_UNSUPPORTED).
+ */
+int fpq_quantize_mx_quest_packed(const void* x, int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                                 void* packed_codes, void* packed_scales, int zero_policy, void* stream);
 
 /*
  * Fused rotate + NVFP4 quantize (group 16, E4M3 scales, fp32 per-tensor multiplier).

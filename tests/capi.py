@@ -197,6 +197,23 @@ def quantize_quest(x_bf16, rot="hadamard", g=128, norm=None, h=None, zero_policy
     return codes.cpu(), scales.cpu(), (mask.cpu() if want_mask else None)
 
 
+def quantize_quest_packed(x_bf16, rot="hadamard", g=128, norm=None, zero_policy=_engine.ZERO_REFERENCE, fill=0xCD):
+    """fpq_quantize_mx_quest_packed; CPU uint8 (packed codes, packed scales)."""
+    lib = _engine.lib()
+    x = x_bf16.to("cuda").contiguous()
+    rows, cols = x.shape
+    nc, ns = packed_sizes(rows, cols)
+    pc = torch.full((nc,), fill, dtype=torch.uint8, device="cuda")
+    ps = torch.full((ns,), fill, dtype=torch.uint8, device="cuda")
+    if norm is None:
+        norm = float(torch.tensor(g ** -0.5, dtype=torch.bfloat16))
+    st = lib.fpq_quantize_mx_quest_packed(x.data_ptr(), rows, cols, ROT[rot], g, norm, pc.data_ptr(), ps.data_ptr(),
+                                          zero_policy, torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_quantize_mx_quest_packed")
+    torch.cuda.synchronize()
+    return pc.cpu(), ps.cpu()
+
+
 def pack_nv(codes, scales, fill=0xCD):
     """fpq_pack_nvf4 on row-major codes [R, K/2] and E4M3 scales [>=R, >=K/16]; CPU uint8 results."""
     lib = _engine.lib()

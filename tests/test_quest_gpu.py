@@ -119,3 +119,65 @@ def test_quest_module_equals_the_operator_chain(m):
     xg = x.clone().requires_grad_(True)
     with pytest.raises(NotImplementedError):
         layers[0](xg).sum().backward()
+
+
+def _quest_input(rows, cols, seed):
+    x = make_outlier_normal(rows, cols, seed, frac=0.02, mult=40.0)
+    x[0, 64:96] = 0.0
+    x[0, 32:64] = 1.5            # a constant group: variance rounds to ~0
+    if rows > 8:
+        x[6] *= 2.0 ** -60
+        x[8] *= 2.0 ** 40
+        x[5, :128] = -x[5, :128].abs() * 2.0 ** -120     # negative values far below every scale
+    return x
+
+
+STREAM_CASES = [("hadamard", 128), ("hadamard", 64), ("hadamard", 32), ("hadamard", 16), ("identity", 32),
+                ("gsr", 64), ("gsr", 16)]
+
+
+@pytest.mark.parametrize("rot,g", STREAM_CASES)
+@pytest.mark.parametrize("policy", [_engine.ZERO_REFERENCE, _engine.ZERO_SIGNED])
+def test_quest_streaming_kernel_bit_exact(rot, g, policy):
+    """Inputs of 2^21 elements and more without a clip mask take the streaming kernel: same codes and scale
+    bytes as the oracle (the last tile is ragged: 1030 rows of 2048)."""
+    rows, cols = 1030, 2048
+    x = _quest_input(rows, cols, 7 * g + len(rot))
+    norm = float(O.hadamard_matrix(g)[0, 0])
+    wc, ws, _, _ = O.quantize_mx_quest(x, OK[rot], g, norm, zero_nibble=policy)
+    codes, scales, none = capi.quantize_quest(x, rot=rot, g=g, norm=norm, zero_policy=policy, want_mask=False)
+    assert none is None
+    assert torch.equal(scales, ws)
+    assert torch.equal(codes, wc)
+    # with a mask the generic kernel runs: same codes
+    codes2, scales2, _ = capi.quantize_quest(x, rot=rot, g=g, norm=norm, zero_policy=policy)
+    assert torch.equal(codes2, wc) and torch.equal(scales2, ws)
+
+
+@pytest.mark.parametrize("rot,g", STREAM_CASES)
+@pytest.mark.parametrize("rows,cols", [(1, 256), (20, 768), (64, 512), (70, 512), (300, 1024), (2100, 256)])
+def test_quest_packed_bit_exact(rot, g, rows, cols):
+    """fpq_quantize_mx_quest_packed (generic kernel up to 64 rows, streaming kernel beyond): the oracle's
+    codes and scales in the packed layout, zero padding rows."""
+    from test_packed_gpu import pack_by_definition
+    x = _quest_input(rows, cols, rows + g)
+    norm = float(O.hadamard_matrix(g)[0, 0])
+    wc, ws, _, _ = O.quantize_mx_quest(x, OK[rot], g, norm)
+    want_c, want_s = pack_by_definition(wc, ws, cols)
+    pc, ps = capi.quantize_quest_packed(x, rot=rot, g=g, norm=norm)
+    assert torch.equal(ps, want_s)
+    assert torch.equal(pc, want_c)
+
+
+def test_quest_packed_declines_rotations_it_cannot_take():
+    lib = _engine.lib()
+    x = torch.zeros(64, 256, dtype=torch.bfloat16, device="cuda")
+    pc = torch.zeros(64 * 128, dtype=torch.uint8, device="cuda")
+    ps = torch.zeros(64 * 8, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    assert lib.fpq_quantize_mx_quest_packed(x.data_ptr(), 64, 256, _engine.ROT_GSR, 128, 0.088, pc.data_ptr(),
+                                            ps.data_ptr(), 0, st) == _engine.E_UNSUPPORTED
+    assert lib.fpq_quantize_mx_quest_packed(x.data_ptr(), 64, 256, _engine.ROT_GENERAL, 32, 0.088, pc.data_ptr(),
+                                            ps.data_ptr(), 0, st) == _engine.E_UNSUPPORTED
+    assert lib.fpq_quantize_mx_quest_packed(x.data_ptr(), 64, 200, 0, 32, 0.088, pc.data_ptr(), ps.data_ptr(), 0,
+                                            st) == -2
