@@ -35,8 +35,8 @@ constexpr int64_t kStreamCounterBytes = kStreamCounters * 4;  // they open the w
 constexpr int kStreamMaxRows = 128;
 
 // NT weight row tiles per workgroup, MT activation row tiles (exactly ceil(M / 32)), DB 256-K blocks
-// of loads in flight per wave, NW waves.  Every workgroup re-reads all activations, so with more
-// than 32 activation rows two weight tiles per workgroup halve what the L2 has to deliver.
+// of loads in flight per wave, NW waves.  Every workgroup re-reads all activations (NT = 2 halves
+// that, at a register cost that stream_plan explains; only NT = 1 is instantiated).
 template <int NT, int MT, int DB, int NW>
 __global__ __launch_bounds__(64 * NW) void gemm_mxf4_stream_kernel(
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
@@ -273,9 +273,11 @@ struct StreamPlan {
 };
 
 // Which shapes run here and how (all thresholds are measured break-even points on Llama-3-8B and
-// Qwen3-8B layer shapes).  Up to 32 activation rows: always, one weight tile per workgroup.  More
-// rows: one weight tile per workgroup while those fit one round of the 256 CUs; two per workgroup
-// for up to 64 rows; beyond that the 128x128 tile kernel, which shares activations through LDS.
+// Qwen3-8B layer shapes).  Up to 64 activation rows: always, one weight tile per workgroup.  More
+// rows: while the weight tiles fit one round of the 256 CUs; beyond that the 128x128 tile kernel,
+// which shares activations through LDS.  (Two weight tiles per workgroup halve what the L2 has to
+// deliver for 33-64 rows, but need so many registers that one workgroup fills a CU; one tile per
+// workgroup with two blocks in flight, two workgroups per CU, measured 5-13 % faster.)
 // K is split across workgroups only for at most 32 rows, when the weight tiles leave at least half
 // of the CUs idle and every part keeps at least 4096 of K (the exchange of partial tiles through
 // the workspace costs about as much as streaming 16 blocks); fewer parts if the workspace is small.
@@ -283,9 +285,7 @@ static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace
   StreamPlan plan{false, 1, 1, 0};
   if (M < 1 || M > kStreamMaxRows || N < 1 || K < 256 || K % 256 != 0) return plan;
   const int64_t rt_m = (M + 31) / 32, tiles = (N + 31) / 32, nkb = K / 256;
-  if (rt_m == 1 || tiles <= 256) plan.nt = 1;
-  else if (rt_m == 2) plan.nt = 2;
-  else return plan;
+  if (rt_m > 2 && tiles > 256) return plan;
   plan.use = true;
   const int64_t groups = (tiles + plan.nt - 1) / plan.nt;
   int64_t ksplit = 1;
@@ -328,12 +328,12 @@ int gemm_mxf4_stream(const void* xq, const void* xs, const void* wq, const void*
   if (plan.nt == 1) {
     switch (mt) {
       case 1: FPQ_STREAM(1, 1, 4); break;
-      case 2: FPQ_STREAM(1, 2, 3); break;
+      case 2: FPQ_STREAM(1, 2, 2); break;
       case 3: FPQ_STREAM(1, 3, 2); break;
       default: FPQ_STREAM(1, 4, 2); break;
     }
   } else {
-    FPQ_STREAM(2, 2, 2);
+    return FPQ_E_UNSUPPORTED;   // no plan asks for more than one weight tile per workgroup
   }
 #undef FPQ_STREAM
   return (int)hipGetLastError();

@@ -49,8 +49,8 @@ def _workspace(m, n, k, cap=None):
     return need, torch.zeros(max(size, 256), dtype=torch.uint8, device="cuda")
 
 
-# one weight tile per workgroup (up to 32 rows, or at most 256 weight tiles), two per workgroup (33-64 rows,
-# more tiles; 8200 columns make the tile count odd), ragged rows and columns, one to 56 blocks of K
+# one to four activation row tiles (more than 64 rows only with at most 256 weight tiles), odd tile counts,
+# ragged rows and columns, one to 56 blocks of K
 SHAPES = [(1, 32, 256), (1, 100, 512), (5, 257, 768), (16, 1024, 1024), (31, 64, 1280), (32, 4096, 4096),
           (33, 130, 2048), (64, 96, 3072), (70, 515, 1024), (96, 2048, 4096), (100, 36, 256), (128, 1000, 2304),
           (127, 4099, 1536), (8, 1024, 14336), (64, 8200, 512), (40, 8290, 768), (33, 16384, 256)]
@@ -144,7 +144,7 @@ def test_split_k_rejects_misaligned_workspace():
         capi.gemm_packed_splitk(xp, xsp, wp, wsp, 4, 64, 1024, ALPHA, workspace=wspace[16:])
 
 
-# rows that take the weight-streaming kernel with one and with two weight tiles per workgroup, the
+# rows that take the weight-streaming kernel with one and with two activation row tiles, the
 # 128 x 128 tile kernel and the 256 x 128 tile kernel; 2 to 4 layers of 256 to 1024 output features
 @pytest.mark.parametrize("m,splits,k", [(1, [512, 256, 256], 512), (16, [1024, 256], 1024), (33, [256, 512], 256),
                                         (64, [4096, 4096, 256], 256), (128, [256, 256, 256, 256], 768),

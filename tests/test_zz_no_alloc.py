@@ -45,7 +45,7 @@ def _with_workspace(ops, m, n, k, bias, res):
 
 
 # K split in two and in three, then smaller inputs on the same array: a split over fewer weight tiles,
-# K whole (no scratch use), two weight tiles per workgroup, and the 128x128 tile kernel
+# K whole (no scratch use), two activation row tiles, and the 128x128 tile kernel
 SEQUENCE = [(16, 4096, 14336), (8, 1024, 14336), (5, 257, 12288), (1, 32, 8192), (32, 2048, 4096),
             (64, 8200, 512), (128, 8320, 256), (17, 515, 9216)]
 
