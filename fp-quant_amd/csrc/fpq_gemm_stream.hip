@@ -327,7 +327,13 @@ int gemm_mxf4_stream(const void* xq, const void* xs, const void* wq, const void*
   const int mt = (int)((M + 31) / 32);
   if (plan.nt == 1) {
     switch (mt) {
-      case 1: FPQ_STREAM(1, 1, 4); break;
+      case 1:
+        // enough workgroups for three per CU: two blocks in flight per wave (98 registers, three
+        // workgroups per CU) beat four (200 registers, two per CU) by 4-5 %; with fewer workgroups the
+        // deeper ring of each wave is what keeps the memory system busy
+        if ((int64_t)grid.x * grid.y >= 384) FPQ_STREAM(1, 1, 2);
+        else FPQ_STREAM(1, 1, 4);
+        break;
       case 2: FPQ_STREAM(1, 2, 2); break;
       case 3: FPQ_STREAM(1, 3, 2); break;
       default: FPQ_STREAM(1, 4, 2); break;
