@@ -585,3 +585,16 @@ def test_single_weight_copy_by_environment(monkeypatch):
     with torch.no_grad():
         assert torch.equal(lin(x), plain(x))
     assert torch.equal(lin.state_dict()["qweight"], plain.qweight)
+
+
+@pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])
+def test_empty_batch(fmt, g):
+    """No rows: every path returns an empty tensor of the right shape (the C entry points accept zero rows)."""
+    lin = _quantized_linear(fmt, g, 256, 96, seed=3, bias=True)
+    with torch.no_grad():
+        for shape in ((0, 256), (2, 0, 256), (0, 5, 256)):
+            y = lin(torch.empty(*shape, device="cuda", dtype=torch.bfloat16))
+            assert y.shape == (*shape[:-1], 96) and y.dtype == torch.bfloat16
+        if fmt == "mxfp4":
+            assert lin.release_row_major()
+            assert lin(torch.empty(0, 256, device="cuda", dtype=torch.bfloat16)).shape == (0, 96)
