@@ -997,7 +997,7 @@ def main():
         "kernels": kernels,
     }
     if not args.no_e2e:
-        # BASELINE config 5 in compact form: the whole-model forward (see bench_e2e_llama); an error here
+        # the end-to-end configuration in compact form: the whole-model forward (see bench_e2e_llama); an error here
         # (e.g. a transformers version without the model class) is recorded, the kernel figures stand
         try:
             e2e = bench_e2e_llama(torch, compact=True)

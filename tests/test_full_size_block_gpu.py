@@ -1,4 +1,4 @@
-"""One decoder layer at the sizes of BASELINE config 5 (Llama-3.1-8B: hidden 4096, 32 query / 8 key-value
+"""One decoder layer at the sizes of the end-to-end benchmark configuration (Llama-3.1-8B: hidden 4096, 32 query / 8 key-value
 heads, intermediate 14336) on 4 x 2048 = 8192 tokens, every linear an MXFP4 FPQuantLinear with Hadamard 128.
 Drives the kernels FPQuantLinear dispatches at prefill size (packed quantizer, 256 x 128 tile GEMM, fused
 producers, residual epilogues) through the module surface."""

@@ -117,7 +117,7 @@ def test_split_k_is_taken_for_few_weight_rows_and_long_k():
 
 @pytest.mark.parametrize("m", [1, 16, 128])
 def test_config3_small_m_on_packed_operands(m):
-    """BASELINE config 3 at M = 1, 16, 128 on the kernel FPQuantLinear runs for those rows."""
+    """The benchmark linear (weight [14336, 4096], Hadamard 128) at M = 1, 16, 128 on the kernel FPQuantLinear runs for those rows."""
     gen = torch.Generator().manual_seed(50 + m)
     n, k = 14336, 4096
     x = torch.randn(m, k, generator=gen).to(torch.bfloat16)
