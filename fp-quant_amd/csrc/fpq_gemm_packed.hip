@@ -406,9 +406,9 @@ static int launch_packed(const void* xq, const void* xs, const void* wq, const v
 // fpq_gemm_stream.hip: the weight-streaming kernel for at most 128 activation rows
 bool stream_eligible(int64_t M, int64_t N, int64_t K);
 int64_t gemm_mxf4_stream_workspace_bytes(int64_t M, int64_t N, int64_t K);
-int gemm_mxf4_stream(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
-                     const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
-                     void* workspace, int64_t workspace_bytes, const OutSegments& seg, hipStream_t stream);
+int gemm_fp4_stream(bool nv, const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
+                    const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                    void* workspace, int64_t workspace_bytes, const OutSegments& seg, hipStream_t stream);
 
 template <bool NV>
 static int gemm_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
@@ -435,6 +435,9 @@ static int pack_operand(const void* codes, const void* scales, int64_t scale_str
 }
 }  // namespace fpq
 
+#ifndef FPQ_NV_STREAM_ROWS
+#define FPQ_NV_STREAM_ROWS 96   // NVFP4: up to this many rows the weight-streaming kernel (where its plan applies)
+#endif
 #ifndef FPQ_PACKED_HALF_TILES
 #define FPQ_PACKED_HALF_TILES 1  // large M: 1 = 256x128 tiles for MXFP4, 2 = for NVFP4 too, 0 = 256x256
 #endif
@@ -460,9 +463,9 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
       ((uintptr_t)y & 15u) || ((uintptr_t)residual & 15u))
     return FPQ_E_ALIGN;
   if ((uintptr_t)workspace & 255u) return FPQ_E_ALIGN;
-  if (!NV && stream_eligible(M, N, K))
-    return gemm_mxf4_stream(xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, workspace, workspace_bytes,
-                            seg, (hipStream_t)stream);
+  if (stream_eligible(M, N, K) && (!NV || M <= FPQ_NV_STREAM_ROWS))
+    return gemm_fp4_stream(NV, xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, workspace, workspace_bytes,
+                           seg, (hipStream_t)stream);
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
   if (big_tiles < FPQ_PACKED_SMALL_BELOW)
     return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);

@@ -1,4 +1,5 @@
-// Weight-streaming MXFP4 GEMM on packed operands for at most 128 activation rows.
+// Weight-streaming FP4 GEMM on packed operands for at most 128 activation rows (MXFP4; NVFP4 with the
+// operands dequantized in registers to exact fp16, as in the NVFP4 tile kernel).
 //
 // With so few rows the time is the one pass over the weights (31 MB for the Llama-3-8B up/gate
 // projection: 3.9 us at 8 TB/s), so the kernel is built around bytes in flight, not around tiles:
@@ -37,14 +38,18 @@ constexpr int kStreamMaxRows = 128;
 // NT weight row tiles per workgroup, MT activation row tiles (exactly ceil(M / 32)), DB 256-K blocks
 // of loads in flight per wave, NW waves.  Every workgroup re-reads all activations (NT = 2 halves
 // that, at a register cost that stream_plan explains; only NT = 1 is instantiated).
-template <int NT, int MT, int DB, int NW>
-__global__ __launch_bounds__(64 * NW) void gemm_mxf4_stream_kernel(
+// NV: NVFP4 operands (two E4M3 scale bytes per lane and K step, 512-byte scale blocks): a lane's dword s
+// of a 64-K unit, times its group's scale, is its fp16 operand of the s-th 32x32x16 matrix instruction
+// of the unit on both sides, so the K order is permuted consistently and the sum is complete.
+template <int NT, int MT, int DB, int NW, bool NV = false>
+__global__ __launch_bounds__(64 * NW) void gemm_fp4_stream_kernel(
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias,
     const uint16_t* residual, uint16_t* y, int M, int N, int K, int bps, int ksplit,
     float* partial, unsigned* counters, const OutSegments seg) {
   static_assert(NW == 4, "the partial sums meet in two rounds of two");
   __shared__ v4f part[2][NT * MT][4][64];
+  constexpr int kSB = NV ? 512 : 256;    // scale bytes per row tile and 256-K block
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int nu = K >> 6, nkb = K >> 8;
   const int rtg = blockIdx.x, split = blockIdx.y;
@@ -60,7 +65,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_mxf4_stream_kernel(
   for (int i = 0; i < NT; ++i) {
     const int rt = min(rtg * NT + i, rt_n - 1);
     wcode[i] = wq + (size_t)rt * nu * 1024 + lane * 16;
-    wscale[i] = ws + (size_t)rt * nkb * 256 + lane * 4;
+    wscale[i] = ws + (size_t)rt * nkb * kSB + lane * (kSB / 64);
   }
   // Lanes whose activation row lies past M (last row tile only) read what the lane of row 0 in
   // their K half reads: no further cache line is touched for rows that are never stored.
@@ -72,7 +77,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_mxf4_stream_kernel(
   for (int j = 0; j < MT; ++j) {
     const int l = j == MT - 1 ? xl : lane;
     xcode[j] = xq + (size_t)j * nu * 1024 + l * 16;
-    xscale[j] = xs + (size_t)j * nkb * 256 + l * 4;
+    xscale[j] = xs + (size_t)j * nkb * kSB + l * (kSB / 64);
   }
 
   v16f acc[NT * MT];
@@ -85,7 +90,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_mxf4_stream_kernel(
   // last one is clamped to it and its matrix instructions are skipped): with loads under branches
   // the compiler can no longer count which of them are still in flight and waits for all.
   uint4 a[DB][4][NT], b[DB][4][MT];
-  uint32_t sa[DB][NT], sb[DB][MT];
+  uint2 sa[DB][NT], sb[DB][MT];   // MXFP4 uses .x only
   const int t_last = nblk > 0 ? nblk - 1 : 0;
   auto load_block = [&](auto slot, int t) {
     constexpr int s = decltype(slot)::value;
@@ -97,26 +102,49 @@ __global__ __launch_bounds__(64 * NW) void gemm_mxf4_stream_kernel(
         const v4u_s ld = __builtin_nontemporal_load((const v4u_s*)(wcode[i] + (size_t)(kb * 4 + u) * 1024));
         a[s][u][i] = make_uint4(ld.x, ld.y, ld.z, ld.w);
       }
-      sa[s][i] = *(const uint32_t*)(wscale[i] + (size_t)kb * 256);
+      if constexpr (NV) sa[s][i] = *(const uint2*)(wscale[i] + (size_t)kb * kSB);
+      else sa[s][i].x = *(const uint32_t*)(wscale[i] + (size_t)kb * kSB);
     }
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
 #pragma unroll
       for (int u = 0; u < 4; ++u) b[s][u][j] = *(const uint4*)(xcode[j] + (size_t)(kb * 4 + u) * 1024);
-      sb[s][j] = *(const uint32_t*)(xscale[j] + (size_t)kb * 256);
+      if constexpr (NV) sb[s][j] = *(const uint2*)(xscale[j] + (size_t)kb * kSB);
+      else sb[s][j].x = *(const uint32_t*)(xscale[j] + (size_t)kb * kSB);
     }
   };
   auto compute_block = [&](auto slot) {
     constexpr int s = decltype(slot)::value;
 #define FPQ_STREAM_STEP(U)                                                                              \
-  _Pragma("unroll") for (int i = 0; i < NT; ++i) {                                                      \
-    const uint4 aq = a[s][U][i];                                                                        \
-    const v8i av = v8i{(int)aq.x, (int)aq.y, (int)aq.z, (int)aq.w, 0, 0, 0, 0};                         \
+  if constexpr (NV) {                                                                                   \
+    v8h bh[MT][4];                                                                                      \
     _Pragma("unroll") for (int j = 0; j < MT; ++j) {                                                    \
       const uint4 bq = b[s][U][j];                                                                      \
-      const v8i bv = v8i{(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w, 0, 0, 0, 0};                       \
-      acc[i * MT + j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(                                \
-          av, bv, acc[i * MT + j], 4, 4, U, (int)sa[s][i], U, (int)sb[s][j]);                           \
+      const uint32_t bw[4] = {bq.x, bq.y, bq.z, bq.w};                                                  \
+      const uint32_t bsc = ((U) < 2 ? sb[s][j].x : sb[s][j].y) >> (16 * ((U) & 1));                     \
+      _Pragma("unroll") for (int s4 = 0; s4 < 4; ++s4)                                                  \
+        bh[j][s4] = dequant8_f16_s(bw[s4], e4m3_pair_f16(bsc >> (8 * (s4 >> 1))));                      \
+    }                                                                                                   \
+    _Pragma("unroll") for (int i = 0; i < NT; ++i) {                                                    \
+      const uint4 aq = a[s][U][i];                                                                      \
+      const uint32_t aw[4] = {aq.x, aq.y, aq.z, aq.w};                                                  \
+      const uint32_t asc = ((U) < 2 ? sa[s][i].x : sa[s][i].y) >> (16 * ((U) & 1));                     \
+      _Pragma("unroll") for (int s4 = 0; s4 < 4; ++s4) {                                                \
+        const v8h ah = dequant8_f16_s(aw[s4], e4m3_pair_f16(asc >> (8 * (s4 >> 1))));                   \
+        _Pragma("unroll") for (int j = 0; j < MT; ++j)                                                  \
+          acc[i * MT + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[j][s4], acc[i * MT + j], 0, 0, 0); \
+      }                                                                                                 \
+    }                                                                                                   \
+  } else {                                                                                              \
+    _Pragma("unroll") for (int i = 0; i < NT; ++i) {                                                    \
+      const uint4 aq = a[s][U][i];                                                                      \
+      const v8i av = v8i{(int)aq.x, (int)aq.y, (int)aq.z, (int)aq.w, 0, 0, 0, 0};                       \
+      _Pragma("unroll") for (int j = 0; j < MT; ++j) {                                                  \
+        const uint4 bq = b[s][U][j];                                                                    \
+        const v8i bv = v8i{(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w, 0, 0, 0, 0};                     \
+        acc[i * MT + j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(                              \
+            av, bv, acc[i * MT + j], 4, 4, U, (int)sa[s][i].x, U, (int)sb[s][j].x);                     \
+      }                                                                                                 \
     }                                                                                                   \
   }
     FPQ_STREAM_STEP(0)
@@ -311,38 +339,50 @@ int64_t gemm_mxf4_stream_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 }
 
 // Arguments are validated by the caller (gemm_packed); `workspace` is null or 256-byte aligned with
-// its first kStreamCounterBytes zero.
-int gemm_mxf4_stream(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
-                     const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
-                     void* workspace, int64_t workspace_bytes, const OutSegments& seg, hipStream_t stream) {
+// its first kStreamCounterBytes zero.  NV: NVFP4 operands.
+template <bool NV>
+static int launch_stream(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
+                         const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                         void* workspace, int64_t workspace_bytes, const OutSegments& seg, hipStream_t stream) {
   const StreamPlan plan = stream_plan(M, N, K, workspace ? workspace_bytes : 0);
   const dim3 grid((unsigned)(((N + 31) / 32 + plan.nt - 1) / plan.nt), (unsigned)plan.ksplit);
   unsigned* counters = (unsigned*)workspace;
   float* partial = workspace ? (float*)((uint8_t*)workspace + kStreamCounterBytes) : nullptr;
 #define FPQ_STREAM(NTT, MTT, DBB)                                                                       \
-  hipLaunchKernelGGL((gemm_mxf4_stream_kernel<NTT, MTT, DBB, 4>), grid, dim3(256), 0, stream, (const uint8_t*)xq, \
-                     (const uint8_t*)xs, (const uint8_t*)wq, (const uint8_t*)ws, alpha,                 \
+  hipLaunchKernelGGL((gemm_fp4_stream_kernel<NTT, MTT, DBB, 4, NV>), grid, dim3(256), 0, stream,        \
+                     (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq, (const uint8_t*)ws, alpha, \
                      (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, (int)M, (int)N,    \
                      (int)K, plan.bps, plan.ksplit, partial, counters, seg)
   const int mt = (int)((M + 31) / 32);
-  if (plan.nt == 1) {
-    switch (mt) {
-      case 1:
-        // enough workgroups for three per CU: two blocks in flight per wave (98 registers, three
-        // workgroups per CU) beat four (200 registers, two per CU) by 4-5 %; with fewer workgroups the
-        // deeper ring of each wave is what keeps the memory system busy
-        if ((int64_t)grid.x * grid.y >= 384) FPQ_STREAM(1, 1, 2);
-        else FPQ_STREAM(1, 1, 4);
-        break;
-      case 2: FPQ_STREAM(1, 2, 2); break;
-      case 3: FPQ_STREAM(1, 3, 2); break;
-      default: FPQ_STREAM(1, 4, 2); break;
-    }
-  } else {
-    return FPQ_E_UNSUPPORTED;   // no plan asks for more than one weight tile per workgroup
+  if (plan.nt != 1) return FPQ_E_UNSUPPORTED;   // no plan asks for more than one weight tile per workgroup
+  switch (mt) {
+    case 1:
+      // enough workgroups for three per CU: two blocks in flight per wave (98 registers, three
+      // workgroups per CU) beat four (200 registers, two per CU) by 4-5 %; with fewer workgroups the
+      // deeper ring of each wave is what keeps the memory system busy
+      if ((int64_t)grid.x * grid.y >= 384) FPQ_STREAM(1, 1, 2);
+      else FPQ_STREAM(1, 1, 4);
+      break;
+    case 2: FPQ_STREAM(1, 2, 2); break;
+    case 3: FPQ_STREAM(1, 3, 2); break;
+    default:
+      // NVFP4 with four activation row tiles does not fit the register file (dequantized fp16 operands
+      // of four tiles next to 64 accumulators): the caller keeps those shapes on the tile kernel
+      if constexpr (NV) return FPQ_E_UNSUPPORTED;
+      else FPQ_STREAM(1, 4, 2);
+      break;
   }
 #undef FPQ_STREAM
   return (int)hipGetLastError();
+}
+
+int gemm_fp4_stream(bool nv, const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
+                    const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                    void* workspace, int64_t workspace_bytes, const OutSegments& seg, hipStream_t stream) {
+  return nv ? launch_stream<true>(xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, workspace, workspace_bytes, seg,
+                                  stream)
+            : launch_stream<false>(xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, workspace, workspace_bytes, seg,
+                                   stream);
 }
 
 

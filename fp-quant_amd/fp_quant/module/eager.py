@@ -217,7 +217,7 @@ def quantize_activations(x_flat: torch.Tensor, h: torch.Tensor, kind: int, norm:
 
 def wants_packed(m: int, n: int, k: int, nvfp4: bool) -> bool:
     """Whether the GEMM of an [m, k] x [n, k] linear runs on packed operands."""
-    return nv_packed_eligible(m, n, k) if nvfp4 else packed_linear_eligible(m, k, "abs_max")
+    return nv_packed_eligible(m, n, k, fused_linear=True) if nvfp4 else packed_linear_eligible(m, k, "abs_max")
 
 
 def weight_wants_packed(wq: torch.Tensor, m: int, k: int, nvfp4: bool) -> bool:

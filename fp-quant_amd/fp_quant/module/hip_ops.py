@@ -286,8 +286,10 @@ def rotated_absmax(x: torch.Tensor, hadamard_matrix: torch.Tensor, amax: Optiona
 # re-tiled weights are made once per weight tensor and kept next to it, which doubles the memory
 # held by 4-bit weights; FPQ_PACKED_WEIGHTS=0 keeps every call on the row-major kernels.
 PACKED_MIN_M = 48          # GEMM operator on row-major operands (pays for re-tiling the activations)
-NV_PACKED_MIN_M = 65       # NVFP4 fused linear: from here on (and while the 128x128 tiles apply) packed;
-#                            below, the split-K weight-streaming kernel on row-major operands is faster
+NV_PACKED_MIN_M = 65       # NVFP4 GEMM operator on row-major operands: from here on (and while the 128x128
+#                            tiles apply) packed; below, re-tiling the activations costs more than it saves
+NV_PACKED_LINEAR_MIN_M = 2 # NVFP4 fused linear (activations quantized straight into the packed layout): the
+#                            weight-streaming kernel up to 96 rows; one row is as fast on the row-major split-K kernel
 # fused linear: activations are quantized straight into the packed layout; the weight-streaming
 # kernel on packed operands serves the few-row (decode) calls; FPQ_PACKED_MIN_ROWS raises the bar
 PACKED_LINEAR_MIN_M = int(os.environ.get("FPQ_PACKED_MIN_ROWS", "1"))
@@ -321,11 +323,11 @@ def pack_nvf4(codes: torch.Tensor, scales: torch.Tensor, rows: int, k: int) -> T
     return pc, ps
 
 
-def nv_packed_eligible(m: int, n: int, k: int) -> bool:
-    """NVFP4: the packed kernel wins where its 128x128 tiles apply (mid-sized M); large M runs at
-    the same speed on row-major operands, tiny M is faster on the direct kernel."""
-    return (NV_PACKED_MIN_M <= m and k % 256 == 0 and packed_weights_enabled()
-            and ((m + 255) // 256) * ((n + 255) // 256) < 100)
+def nv_packed_eligible(m: int, n: int, k: int, fused_linear: bool = False) -> bool:
+    """NVFP4: the packed kernels win for few and mid-sized M (weight-streaming kernel, 128x128 tiles);
+    large M runs at the same speed on row-major operands."""
+    return ((NV_PACKED_LINEAR_MIN_M if fused_linear else NV_PACKED_MIN_M) <= m and k % 256 == 0
+            and packed_weights_enabled() and ((m + 255) // 256) * ((n + 255) // 256) < 100)
 
 
 def unpack_mxf4(pc: torch.Tensor, ps: torch.Tensor, rows: int, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
