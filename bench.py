@@ -546,7 +546,18 @@ def bench_power(torch, seconds=3.0):
     clocks = torch.empty(blocks * 2, dtype=torch.int64, device=dev)
     src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 256)
     dst = torch.empty_like(src)
+    # the NVFP4 large-M GEMM (row-major operands, fp16 matrix path after in-register dequantization)
+    nm, nn = 4096, 24576
+    gen_d = torch.Generator(device=dev).manual_seed(3)
+    nxq = torch.randint(0, 256, (nm, k // 2), dtype=torch.uint8, device=dev, generator=gen_d)
+    nwq = torch.randint(0, 256, (nn, k // 2), dtype=torch.uint8, device=dev, generator=gen_d)
+    nxs = torch.randint(40, 72, (nm, k // 16), dtype=torch.uint8, device=dev, generator=gen_d)
+    nws = torch.randint(40, 72, (nn, k // 16), dtype=torch.uint8, device=dev, generator=gen_d)
+    ny = torch.empty(nm, nn, dtype=torch.bfloat16, device=dev)
     legs = {
+        "nvfp4_gemm_M4096_gate_up": lambda: lib.fpq_gemm_nvf4(nxq.data_ptr(), nxs.data_ptr(), k // 16, nwq.data_ptr(),
+                                                              nws.data_ptr(), k // 16, alpha.data_ptr(), None,
+                                                              ny.data_ptr(), nm, nn, k, st),
         "mxfp4_gemm_M2048": lambda: lib.fpq_gemm_mxf4_packed(xp.data_ptr(), xs.data_ptr(), wp.data_ptr(), ws.data_ptr(),
                                                              alpha.data_ptr(), None, y.data_ptr(), m, n, k, st),
         "mfma_only_quantized_bits": lambda: lib.fpq_test_mfma_rate(words.data_ptr(), blocks, 192, sink.data_ptr(),
