@@ -67,12 +67,13 @@ __global__ __launch_bounds__(256) void pack_fp4_kernel(const uint8_t* __restrict
   }
 }
 
-// Packed -> row-major (MXFP4), the inverse of pack_fp4_kernel<false> on the rows that exist: what a
-// layer that keeps only its packed weights hands to state_dict().
-__global__ __launch_bounds__(256) void unpack_mxf4_kernel(const uint8_t* __restrict__ pcodes,
-                                                          const uint8_t* __restrict__ pscales, int rows, int K,
-                                                          uint8_t* __restrict__ codes, uint8_t* __restrict__ scales,
-                                                          int64_t scale_stride) {
+// Packed -> row-major, the inverse of pack_fp4_kernel on the rows that exist: what a layer that keeps
+// only its packed weights hands to state_dict().
+template <bool NV>
+__global__ __launch_bounds__(256) void unpack_fp4_kernel(const uint8_t* __restrict__ pcodes,
+                                                         const uint8_t* __restrict__ pscales, int rows, int K,
+                                                         uint8_t* __restrict__ codes, uint8_t* __restrict__ scales,
+                                                         int64_t scale_stride) {
   const int kb = blockIdx.x, rt = blockIdx.y;
   const int t = threadIdx.x;
   const int r = t >> 3, c = t & 7;
@@ -83,13 +84,28 @@ __global__ __launch_bounds__(256) void unpack_mxf4_kernel(const uint8_t* __restr
   if (t < 64) {
     const int sr = t & 31, skh = t >> 5;
     const int srow = rt * 32 + sr;
-    const uint32_t in = *(const uint32_t*)(pscales + (((size_t)rt * (K >> 8) + kb) * 64 + t) * 4);
-    if (srow < rows) {
-      uint8_t* sp = scales + (size_t)srow * scale_stride + kb * 8 + skh;
-      sp[0] = (uint8_t)in;
-      sp[2] = (uint8_t)(in >> 8);
-      sp[4] = (uint8_t)(in >> 16);
-      sp[6] = (uint8_t)(in >> 24);
+    if (NV) {
+      const uint2 in = *(const uint2*)(pscales + (((size_t)rt * (K >> 8) + kb) * 64 + t) * 8);
+      if (srow < rows) {
+        uint8_t* sp = scales + (size_t)srow * scale_stride + kb * 16 + 2 * skh;
+        sp[0] = (uint8_t)in.x;
+        sp[1] = (uint8_t)(in.x >> 8);
+        sp[4] = (uint8_t)(in.x >> 16);
+        sp[5] = (uint8_t)(in.x >> 24);
+        sp[8] = (uint8_t)in.y;
+        sp[9] = (uint8_t)(in.y >> 8);
+        sp[12] = (uint8_t)(in.y >> 16);
+        sp[13] = (uint8_t)(in.y >> 24);
+      }
+    } else {
+      const uint32_t in = *(const uint32_t*)(pscales + (((size_t)rt * (K >> 8) + kb) * 64 + t) * 4);
+      if (srow < rows) {
+        uint8_t* sp = scales + (size_t)srow * scale_stride + kb * 8 + skh;
+        sp[0] = (uint8_t)in;
+        sp[2] = (uint8_t)(in >> 8);
+        sp[4] = (uint8_t)(in >> 16);
+        sp[6] = (uint8_t)(in >> 24);
+      }
     }
   }
 }
@@ -494,20 +510,34 @@ extern "C" int fpq_pack_mxf4(const void* codes, const void* scales, int64_t scal
   return fpq::pack_operand<false>(codes, scales, scale_stride, rows, K, packed_codes, packed_scales, stream);
 }
 
-extern "C" int fpq_unpack_mxf4(const void* packed_codes, const void* packed_scales, int64_t rows, int64_t K,
-                               void* codes, void* scales, int64_t scale_stride, void* stream) {
+namespace fpq {
+template <bool NV>
+static int unpack_operand(const void* packed_codes, const void* packed_scales, int64_t rows, int64_t K, void* codes,
+                          void* scales, int64_t scale_stride, void* stream) {
+  constexpr int GROUP = NV ? 16 : 32;
   if (rows < 0 || K < 0) return FPQ_E_SHAPE;
   if (rows == 0) return FPQ_OK;
   if (!codes || !scales || !packed_codes || !packed_scales) return FPQ_E_NULL;
-  if (K == 0 || K % 256 != 0 || scale_stride < K / 32) return FPQ_E_SHAPE;
+  if (K == 0 || K % 256 != 0 || scale_stride < K / GROUP) return FPQ_E_SHAPE;
   if (rows > (1 << 24) || K > (1 << 24)) return FPQ_E_SHAPE;
-  if (((uintptr_t)codes & 15u) || ((uintptr_t)packed_codes & 15u) || ((uintptr_t)packed_scales & 3u))
+  if (((uintptr_t)codes & 15u) || ((uintptr_t)packed_codes & 15u) || ((uintptr_t)packed_scales & (NV ? 7u : 3u)))
     return FPQ_E_ALIGN;
   const dim3 grid((unsigned)(K / 256), (unsigned)((rows + 31) / 32));
-  hipLaunchKernelGGL(fpq::unpack_mxf4_kernel, grid, dim3(256), 0, (hipStream_t)stream,
-                     (const uint8_t*)packed_codes, (const uint8_t*)packed_scales, (int)rows, (int)K,
-                     (uint8_t*)codes, (uint8_t*)scales, scale_stride);
+  hipLaunchKernelGGL(unpack_fp4_kernel<NV>, grid, dim3(256), 0, (hipStream_t)stream, (const uint8_t*)packed_codes,
+                     (const uint8_t*)packed_scales, (int)rows, (int)K, (uint8_t*)codes, (uint8_t*)scales,
+                     scale_stride);
   return (int)hipGetLastError();
+}
+}  // namespace fpq
+
+extern "C" int fpq_unpack_mxf4(const void* packed_codes, const void* packed_scales, int64_t rows, int64_t K,
+                               void* codes, void* scales, int64_t scale_stride, void* stream) {
+  return fpq::unpack_operand<false>(packed_codes, packed_scales, rows, K, codes, scales, scale_stride, stream);
+}
+
+extern "C" int fpq_unpack_nvf4(const void* packed_codes, const void* packed_scales, int64_t rows, int64_t K,
+                               void* codes, void* scales, int64_t scale_stride, void* stream) {
+  return fpq::unpack_operand<true>(packed_codes, packed_scales, rows, K, codes, scales, scale_stride, stream);
 }
 
 extern "C" int fpq_pack_nvf4(const void* codes, const void* scales, int64_t scale_stride, int64_t rows,

@@ -53,6 +53,7 @@ _SIGNATURES = {
     "fpq_gemm_mxf4_packed_residual": ([_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _I),
     "fpq_gemm_mxf4_packed_multi": ([_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _I),
     "fpq_unpack_mxf4": ([_P, _P, _I64, _I64, _P, _P, _I64, _P], _I),
+    "fpq_unpack_nvf4": ([_P, _P, _I64, _I64, _P, _P, _I64, _P], _I),
     "fpq_prepare_device": ([_P], _I),
     "fpq_gemm_mxf4_packed_noalloc_max_rows": ([], _I64),
     "fpq_gemm_mxf4_packed_noalloc": ([_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _I),

@@ -241,8 +241,6 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
             raise ValueError("packed weights need MXFP4 activations with the same inner dimension")
         use_packed = True
     elif is_packed_only(wq):   # a layer that holds its weight in the packed layout only
-        if qa.nvfp4:
-            raise ValueError("only MXFP4 weights are held in the packed layout")
         n = weight_rows(wq, k)
         wp = wsp = None
         use_packed = True

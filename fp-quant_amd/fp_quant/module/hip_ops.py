@@ -330,19 +330,21 @@ def nv_packed_eligible(m: int, n: int, k: int, fused_linear: bool = False) -> bo
             and packed_weights_enabled() and ((m + 255) // 256) * ((n + 255) // 256) < 100)
 
 
-def unpack_mxf4(pc: torch.Tensor, ps: torch.Tensor, rows: int, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Packed MXFP4 operand -> row-major codes [rows, k/2] and E8M0 scales [rows, k/32] (the inverse of pack_mxf4)."""
+def unpack_fp4(pc: torch.Tensor, ps: torch.Tensor, rows: int, k: int, nvfp4: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Packed operand -> row-major codes [rows, k/2] and scales [rows, k/32] (MXFP4, E8M0) or [rows, k/16]
+    (NVFP4, E4M3): the inverse of pack_mxf4 / pack_nvf4."""
     lib = _engine.lib()
+    group = 16 if nvfp4 else 32
     codes = torch.empty(rows, k // 2, dtype=torch.uint8, device=pc.device)
-    scales = torch.empty(rows, k // 32, dtype=torch.uint8, device=pc.device)
+    scales = torch.empty(rows, k // group, dtype=torch.uint8, device=pc.device)
+    entry = lib.fpq_unpack_nvf4 if nvfp4 else lib.fpq_unpack_mxf4
     with torch.cuda.device(pc.device):
-        st = lib.fpq_unpack_mxf4(pc.data_ptr(), ps.data_ptr(), rows, k, codes.data_ptr(), scales.data_ptr(), k // 32,
-                                 _stream(pc))
-    _engine.check(st, "fpq_unpack_mxf4")
+        st = entry(pc.data_ptr(), ps.data_ptr(), rows, k, codes.data_ptr(), scales.data_ptr(), k // group, _stream(pc))
+    _engine.check(st, "fpq_unpack_nvf4" if nvfp4 else "fpq_unpack_mxf4")
     return codes, scales
 
 
-# A layer may hold its MXFP4 weight in the packed layout ONLY (FPQuantLinear.release_row_major): its
+# A layer may hold its weight in the packed layout ONLY (FPQuantLinear.release_row_major): its
 # `qweight` / `scales` are then the 1-D packed buffers themselves.  The number of dimensions is the marker
 # (it survives every operator boundary); the row count follows from the inner dimension of the activations.
 def is_packed_only(wq: torch.Tensor) -> bool:
@@ -375,8 +377,6 @@ def packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False) -> Tu
     """Packed copy of a weight, cached on the code tensor until either tensor is written to (a weight
     held in the packed layout only is its own packed copy)."""
     if wq.dim() == 1:
-        if nvfp4:
-            raise ValueError("only MXFP4 weights are held in the packed layout")
         return wq, ws
     key = _packed_weight_key(wq, ws, nvfp4)
     hit = getattr(wq, "_fpq_packed", None)

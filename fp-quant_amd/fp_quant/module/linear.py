@@ -171,18 +171,19 @@ class FPQuantLinear(nn.Module):
         layout the GEMM kernels read (what is otherwise a second copy next to the row-major tensors of
         the reference, linear.py:87-88), and the row-major tensors are freed.  state_dict() still hands
         out the reference's row-major tensors (re-tiled on demand) and load_state_dict() accepts them.
-        MXFP4 with in_features % 256 == 0 and out_features % 32 == 0 on a GPU; returns whether the
-        layer is in that state afterwards."""
+        MXFP4 or NVFP4 with in_features % 256 == 0 and out_features % 32 == 0 on a GPU; returns whether
+        the layer is in that state afterwards."""
         if self.weights_packed_only:
             return True
         q, s = getattr(self, "qweight", None), getattr(self, "scales", None)
-        if (self.config.forward_dtype != FPQuantDtype.MXFP4 or q is None or s is None or not q.is_cuda
-                or q.dim() != 2 or q.dtype != torch.uint8 or s.dtype != torch.uint8
+        nvfp4 = self.config.forward_dtype == FPQuantDtype.NVFP4
+        if (self.config.forward_dtype not in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4) or q is None or s is None
+                or not q.is_cuda or q.dim() != 2 or q.dtype != torch.uint8 or s.dtype != torch.uint8
                 or self.in_features % 256 != 0 or self.out_features % 32 != 0
                 or tuple(q.shape) != (self.out_features, self.in_features // 2)
-                or tuple(s.shape) != (self.out_features, self.in_features // 32)):
+                or tuple(s.shape) != (self.out_features, self.in_features // self.config.forward_dtype.scale_group)):
             return False
-        pc, ps = hip_ops.packed_weight(q.contiguous(), s.contiguous())
+        pc, ps = hip_ops.packed_weight(q.contiguous(), s.contiguous(), nvfp4)
         hip_ops.drop_tensor_caches(q, s)
         self.qweight = nn.Parameter(pc, requires_grad=False)
         self.scales = nn.Parameter(ps, requires_grad=False)
@@ -194,7 +195,8 @@ class FPQuantLinear(nn.Module):
         """Undo release_row_major: `qweight` [out, in/2] and `scales` [out, in/32] as the reference holds them."""
         if not self.weights_packed_only:
             return
-        codes, scales = hip_ops.unpack_mxf4(self.qweight, self.scales, self.out_features, self.in_features)
+        codes, scales = hip_ops.unpack_fp4(self.qweight, self.scales, self.out_features, self.in_features,
+                                           self.config.forward_dtype == FPQuantDtype.NVFP4)
         self.qweight = nn.Parameter(codes, requires_grad=False)
         self.scales = nn.Parameter(scales, requires_grad=False)
         self._fpq_single_copy = False
@@ -203,8 +205,8 @@ class FPQuantLinear(nn.Module):
         """state_dict() hook: a layer that holds the packed layout only hands out row-major tensors."""
         if self.weights_packed_only and prefix + "qweight" in state_dict and prefix + "scales" in state_dict:
             with torch.no_grad():
-                codes, scales = hip_ops.unpack_mxf4(self.qweight.detach(), self.scales.detach(), self.out_features,
-                                                    self.in_features)
+                codes, scales = hip_ops.unpack_fp4(self.qweight.detach(), self.scales.detach(), self.out_features,
+                                                   self.in_features, self.config.forward_dtype == FPQuantDtype.NVFP4)
             state_dict[prefix + "qweight"], state_dict[prefix + "scales"] = codes, scales
 
     def _before_load(self, state_dict, prefix, *_):

@@ -337,6 +337,9 @@ int fpq_test_e2m1(const float* in, uint8_t* out, int64_t n, int zero_policy, voi
 int64_t fpq_packed_scales_bytes_nv(int64_t rows, int64_t K);
 int fpq_pack_nvf4(const void* codes, const void* scales, int64_t scale_stride, int64_t rows,
                   int64_t K, void* packed_codes, void* packed_scales, void* stream);
+/* The inverse of fpq_pack_nvf4 for the first `rows` rows (E4M3 scales, entry [row, k/16], scale_stride >= K/16). */
+int fpq_unpack_nvf4(const void* packed_codes, const void* packed_scales, int64_t rows, int64_t K,
+                    void* codes, void* scales, int64_t scale_stride, void* stream);
 int fpq_gemm_nvf4_packed(const void* xq_packed, const void* xs_packed, const void* wq_packed,
                          const void* ws_packed, const float* alpha, const void* bias, void* y,
                          int64_t M, int64_t N, int64_t K, void* stream);

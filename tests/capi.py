@@ -81,16 +81,18 @@ def pack(codes, scales, fill=0xCD):
     return pc.cpu(), ps.cpu()
 
 
-def unpack(pc, ps, rows, k, scale_pad=0, fill=0xCD):
-    """fpq_unpack_mxf4: CPU uint8 row-major codes [rows, k/2] and scales [rows, k/32 + scale_pad] (entries past
-    k/32 keep `fill`)."""
+def unpack(pc, ps, rows, k, scale_pad=0, fill=0xCD, nv=False):
+    """fpq_unpack_mxf4 (nv: fpq_unpack_nvf4): CPU uint8 row-major codes [rows, k/2] and scales
+    [rows, k/group + scale_pad] (entries past k/group keep `fill`)."""
     lib = _engine.lib()
     pc, ps = pc.to("cuda").contiguous(), ps.to("cuda").contiguous()
+    group = 16 if nv else 32
     codes = torch.full((rows, k // 2), fill, dtype=torch.uint8, device="cuda")
-    scales = torch.full((rows, k // 32 + scale_pad), fill, dtype=torch.uint8, device="cuda")
-    st = lib.fpq_unpack_mxf4(pc.data_ptr(), ps.data_ptr(), rows, k, codes.data_ptr(), scales.data_ptr(),
-                             scales.shape[1], torch.cuda.current_stream().cuda_stream)
-    _engine.check(st, "fpq_unpack_mxf4")
+    scales = torch.full((rows, k // group + scale_pad), fill, dtype=torch.uint8, device="cuda")
+    entry = lib.fpq_unpack_nvf4 if nv else lib.fpq_unpack_mxf4
+    st = entry(pc.data_ptr(), ps.data_ptr(), rows, k, codes.data_ptr(), scales.data_ptr(),
+               scales.shape[1], torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_unpack")
     torch.cuda.synchronize()
     return codes.cpu(), scales.cpu()
 

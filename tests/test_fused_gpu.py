@@ -541,16 +541,17 @@ def test_grouped_projections_run_as_one_gemm_on_concatenated_packed_weights(toke
             assert torch.equal(a, b)
 
 
-@pytest.mark.parametrize("order", ["fuse_then_release", "release_then_fuse"])
-def test_model_with_weights_held_once_keeps_its_logits(order):
+@pytest.mark.parametrize("order,fmt,g", [("fuse_then_release", "mxfp4", 128), ("release_then_fuse", "mxfp4", 128),
+                                         ("fuse_then_release", "nvfp4", 16)])
+def test_model_with_weights_held_once_keeps_its_logits(order, fmt, g):
     """release_row_major_weights on a whole model, before or after fuse_producers: every layer holds the
     packed layout only (the groups of projections included: their members are views into the group's
     buffers), logits keep their bits eagerly and compiled, the state dict is the reference's, and loading
     another model's state dict is followed."""
     import fp_quant
     from fp_quant.utils import fuse_producers, release_row_major_weights, restore_row_major_weights
-    model = _tiny_llama("mxfp4", 128, seed=11)
-    other = _tiny_llama("mxfp4", 128, seed=12)
+    model = _tiny_llama(fmt, g, seed=11)
+    other = _tiny_llama(fmt, g, seed=12)
     ids = torch.randint(0, 128, (2, 40), generator=torch.Generator().manual_seed(3)).cuda()
     one = ids[:, :1].contiguous()
     n_layers = sum(isinstance(m, fp_quant.FPQuantLinear) for m in model.modules())
@@ -570,6 +571,9 @@ def test_model_with_weights_held_once_keeps_its_logits(order):
             assert release_row_major_weights(model) == n_layers
         for block in model.model.layers:
             attn, group = block.self_attn, block.self_attn._fpq_weight_group
+            if fmt != "mxfp4":      # groups of projections exist for MXFP4 only
+                assert group is None and all(l.weights_packed_only for l in (attn.q_proj, attn.k_proj, attn.v_proj))
+                continue
             assert group is not None and block.mlp._fpq_weight_group is not None
             lo, hi = group.wp.data_ptr(), group.wp.data_ptr() + group.wp.numel()
             for layer in (attn.q_proj, attn.k_proj, attn.v_proj):

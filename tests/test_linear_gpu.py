@@ -518,15 +518,17 @@ def test_prepare_device_entry_point():
         assert lib.fpq_prepare_device(s.cuda_stream) == _engine.E_UNSUPPORTED   # must run, not be recorded
 
 
+@pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])
 @pytest.mark.parametrize("bias", [False, True])
-def test_release_row_major_keeps_results_and_the_reference_state_dict(bias):
+def test_release_row_major_keeps_results_and_the_reference_state_dict(bias, fmt, g):
     """FPQuantLinear.release_row_major: the packed buffers become the only copy of the weight; outputs keep
     their bits on every kernel path (1, 40, 300 and 2100 rows), state_dict() still holds the reference's
     row-major tensors, load_state_dict() accepts them and the layer goes back to the packed layout, and
     restore_row_major gives the original tensors back."""
     k, n = 512, 384
-    lin = _quantized_linear("mxfp4", 128, k, n, seed=5, bias=bias)
-    other = _quantized_linear("mxfp4", 128, k, n, seed=6, bias=bias)
+    group = 32 if fmt == "mxfp4" else 16
+    lin = _quantized_linear(fmt, g, k, n, seed=5, bias=bias)
+    other = _quantized_linear(fmt, g, k, n, seed=6, bias=bias)
     xs = [torch.randn(m, k, device="cuda", dtype=torch.bfloat16) for m in (1, 40, 300, 2100)]
     with torch.no_grad():
         want = [lin(x) for x in xs]
@@ -536,7 +538,7 @@ def test_release_row_major_keeps_results_and_the_reference_state_dict(bias):
         torch.cuda.synchronize()
         before = torch.cuda.memory_allocated()
         assert lin.release_row_major() and lin.weights_packed_only
-        assert lin.qweight.dim() == 1 and lin.qweight.numel() == n * k // 2 and lin.scales.numel() == n * k // 32
+        assert lin.qweight.dim() == 1 and lin.qweight.numel() == n * k // 2 and lin.scales.numel() == n * k // group
         torch.cuda.synchronize()
         assert before - torch.cuda.memory_allocated() >= n * k // 2        # the row-major codes are gone
         for x, w in zip(xs, want):
@@ -562,7 +564,7 @@ def test_release_row_major_keeps_results_and_the_reference_state_dict(bias):
 
 
 def test_release_row_major_declines_what_the_packed_layout_cannot_hold():
-    nv = _quantized_linear("nvfp4", 16, 256, 64, seed=1)
+    nv = _quantized_linear("nvfp4", 16, 256, 48, seed=1)
     assert not nv.release_row_major() and nv.qweight.dim() == 2
     ragged = _quantized_linear("mxfp4", 32, 256, 48, seed=2)        # 48 output features: not whole 32-row tiles
     assert not ragged.release_row_major() and ragged.qweight.dim() == 2
@@ -570,7 +572,7 @@ def test_release_row_major_declines_what_the_packed_layout_cannot_hold():
     assert not short.release_row_major()
     x = torch.randn(5, 256, device="cuda", dtype=torch.bfloat16)
     with torch.no_grad():
-        assert nv(x).shape == (5, 64) and ragged(x).shape == (5, 48)
+        assert nv(x).shape == (5, 48) and ragged(x).shape == (5, 48)
 
 
 def test_single_weight_copy_by_environment(monkeypatch):

@@ -289,3 +289,16 @@ def test_unpack_is_the_inverse_of_the_layout_definition(rows, k):
     # and of fpq_pack_mxf4
     pc2, ps2 = capi.pack(codes, scales)
     assert torch.equal(pc2, pc) and torch.equal(ps2, ps)
+
+
+@pytest.mark.parametrize("rows,k", [(1, 256), (33, 768), (70, 512), (1000, 1024)])
+def test_unpack_nv_is_the_inverse_of_the_layout_definition(rows, k):
+    g = torch.Generator().manual_seed(rows + k)
+    codes = torch.randint(0, 256, (rows, k // 2), dtype=torch.uint8, generator=g)
+    scales = torch.randint(0, 256, (rows, k // 16), dtype=torch.uint8, generator=g)
+    pc, ps = pack_nv_by_definition(codes, scales, k)
+    got_c, got_s = capi.unpack(pc, ps, rows, k, nv=True)
+    assert torch.equal(got_c, codes) and torch.equal(got_s, scales)
+    got_c, got_s = capi.unpack(pc, ps, rows, k, scale_pad=8, nv=True)
+    assert torch.equal(got_c, codes) and torch.equal(got_s[:, : k // 16], scales)
+    assert (got_s[:, k // 16:] == 0xCD).all()
