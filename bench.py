@@ -294,10 +294,19 @@ def bench_linear(torch, fmt, m, n, k, g, steps, warmup, seed, check=False):
     p = [(xs_[i].data_ptr(), xq[i].data_ptr(), xsc[i].data_ptr(), ys[i].data_ptr()) for i in range(n_buf)]
 
     from fp_quant.module import hip_ops
-    if fmt == "mxfp4" and hip_ops.packed_linear_eligible(m, k, "abs_max"):
+    nv_packed = fmt == "nvfp4" and hip_ops.nv_packed_eligible(m, n, k, fused_linear=True)
+    if (fmt == "mxfp4" and hip_ops.packed_linear_eligible(m, k, "abs_max")) or nv_packed:
         # what FPQuantLinear.forward runs for this many rows: activations quantized straight into the
         # packed operand layout, weights re-tiled once (outside the timed region, like their quantization)
-        wp, wsp = hip_ops.pack_mxf4(wq, ws, n, k)
+        wp, wsp = (hip_ops.pack_nvf4 if nv_packed else hip_ops.pack_mxf4)(wq, ws, n, k)
+        scales_bytes = lib.fpq_packed_scales_bytes_nv if nv_packed else lib.fpq_packed_scales_bytes
+        gemm_packed = lib.fpq_gemm_nvf4_packed if nv_packed else lib.fpq_gemm_mxf4_packed
+
+        def quant_packed(src, codes, scales):
+            if nv_packed:
+                return lib.fpq_quantize_nv_packed(src, m, k, 0, g, norm, gs.data_ptr(), codes, scales, 0, stream)
+            return lib.fpq_quantize_mx_packed(src, m, k, 0, g, norm, codes, scales, 0, stream)
+
         # Up to 128 rows the GEMM streams the weights (HBM-bound): they rotate through enough copies to
         # exceed the 256 MB last-level cache, so that every launch reads them from HBM as a decode step
         # does; the figure with one resident copy is reported beside it.
@@ -305,34 +314,34 @@ def bench_linear(torch, fmt, m, n, k, g, steps, warmup, seed, check=False):
         wps = [(wp, wsp)] + [(wp.clone(), wsp.clone()) for _ in range(n_w - 1)]
         wptr = [(a.data_ptr(), b.data_ptr()) for a, b in wps]
         xp = [torch.empty(lib.fpq_packed_codes_bytes(m, k), dtype=torch.uint8, device=dev) for _ in range(n_buf)]
-        xsp = [torch.empty(lib.fpq_packed_scales_bytes(m, k), dtype=torch.uint8, device=dev) for _ in range(n_buf)]
+        xsp = [torch.empty(scales_bytes(m, k), dtype=torch.uint8, device=dev) for _ in range(n_buf)]
         pp = [(xs_[i].data_ptr(), xp[i].data_ptr(), xsp[i].data_ptr(), ys[i].data_ptr()) for i in range(n_buf)]
 
         def run_linear(i):
             a, b, c, d = pp[i]
             wc, wsc = wptr[i % n_w]
-            st = lib.fpq_quantize_mx_packed(a, m, k, 0, g, norm, b, c, 0, stream)
-            st = st or lib.fpq_gemm_mxf4_packed(b, c, wc, wsc, alpha.data_ptr(), None, d, m, n, k, stream)
+            st = quant_packed(a, b, c)
+            st = st or gemm_packed(b, c, wc, wsc, alpha.data_ptr(), None, d, m, n, k, stream)
             if st != 0:
                 _engine.check(st, "bench packed linear")
 
         def run_gemm(i):
             a, b, c, d = pp[i]
             wc, wsc = wptr[i % n_w]
-            st = lib.fpq_gemm_mxf4_packed(b, c, wc, wsc, alpha.data_ptr(), None, d, m, n, k, stream)
+            st = gemm_packed(b, c, wc, wsc, alpha.data_ptr(), None, d, m, n, k, stream)
             if st != 0:
                 _engine.check(st, "bench packed gemm")
 
         def run_gemm_resident(i):
             a, b, c, d = pp[i]
-            st = lib.fpq_gemm_mxf4_packed(b, c, wptr[0][0], wptr[0][1], alpha.data_ptr(), None, d, m, n, k, stream)
+            st = gemm_packed(b, c, wptr[0][0], wptr[0][1], alpha.data_ptr(), None, d, m, n, k, stream)
             if st != 0:
                 _engine.check(st, "bench packed gemm")
 
         res = _time_linear(torch, run_linear, run_gemm, fmt, m, n, k, g, group, n_buf, steps, warmup, "packed",
                            run_gemm_resident if n_w > 1 else None)
         res["weight_copies"] = n_w
-        if check:
+        if check and fmt == "mxfp4":
             run_linear(0)
             res["output_check"] = check_linear_output(torch, xs_[0], ys[0], w, wq, ws, m, n, k, g, float(alpha))
         return res
@@ -922,6 +931,8 @@ def main():
         linears[m] = bench_linear(torch, "mxfp4", m, 14336, 4096, 128, args.steps, args.warmup, seed=2, check=True)
     nv = bench_linear(torch, "nvfp4", 4096, 24576, 4096, 16, max(10, args.steps // 10), max(2, args.warmup // 10), seed=3)
 
+    nv64 = bench_linear(torch, "nvfp4", 64, 24576, 4096, 16, args.steps, args.warmup, seed=3)
+
     ceiling = bench_mfma_ceiling(torch)
     quant = results["nvfp4_quantize"]
     head = linears[2048]
@@ -946,6 +957,13 @@ def main():
         "workload": nv["workload"], "gemm_us": round(nv["gemm_ms"] * 1e3, 3),
         "gemm_TFLOP/s": round(nv["gemm_tflops"], 2),
         "mfma_frac_of_f16_peak": round(nv["gemm_tflops"] / BF16_PEAK_TFLOPS, 4)}
+    kernels["nvfp4_gemm_M64_gate_up"] = {
+        "workload": nv64["workload"], "gemm_us": round(nv64["gemm_ms"] * 1e3, 3),
+        "linear_us": round(nv64["linear_ms"] * 1e3, 3), "gemm_GB/s": round(nv64["gemm_gbps"], 2),
+        "hbm_frac": round(nv64["gemm_gbps"] / HBM_PEAK_GBS, 4), "operand_layout": nv64["operand_layout"],
+        "gemm_us_cache_resident": round(nv64["gemm_ms_cache_resident"] * 1e3, 3)
+        if nv64.get("gemm_ms_cache_resident") is not None else None,
+        "weight_copies": nv64.get("weight_copies")}
     traffic = {}
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
