@@ -579,15 +579,17 @@ extern "C" int fpq_gemm_mxf4_packed_splitk(const void* xq, const void* xs, const
                                    stream);
 }
 
-extern "C" int fpq_gemm_mxf4_packed_multi(const void* xq, const void* xs, const void* wq, const void* ws,
-                                          const float* alpha, const void* bias, void* const* ys,
-                                          const int64_t* ns, int64_t count, int64_t M, int64_t K, void* stream) {
-  if (count < 1 || count > fpq::kMaxSegments) return FPQ_E_SHAPE;
+namespace fpq {
+template <bool NV>
+static int gemm_packed_multi(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
+                             const void* bias, void* const* ys, const int64_t* ns, int64_t count, int64_t M,
+                             int64_t K, void* stream) {
+  if (count < 1 || count > kMaxSegments) return FPQ_E_SHAPE;
   if (!ys || !ns) return FPQ_E_NULL;
-  fpq::OutSegments seg{};
+  OutSegments seg{};
   int64_t N = 0;
   for (int64_t i = 0; i < count; ++i) {
-    if (ns[i] < 1 || ns[i] % fpq::kSegmentAlign != 0 || N + ns[i] > (1 << 24)) return FPQ_E_SHAPE;
+    if (ns[i] < 1 || ns[i] % kSegmentAlign != 0 || N + ns[i] > (1 << 24)) return FPQ_E_SHAPE;
     if (M > 0 && !ys[i]) return FPQ_E_NULL;
     if ((uintptr_t)ys[i] & 15u) return FPQ_E_ALIGN;
     N += ns[i];
@@ -595,7 +597,20 @@ extern "C" int fpq_gemm_mxf4_packed_multi(const void* xq, const void* xs, const 
     seg.y[i] = (uint16_t*)ys[i];
   }
   seg.count = (int)count;
-  return fpq::gemm_packed<false>(xq, xs, wq, ws, alpha, bias, ys[0], M, N, K, stream, nullptr, nullptr, 0, seg);
+  return gemm_packed<NV>(xq, xs, wq, ws, alpha, bias, ys[0], M, N, K, stream, nullptr, nullptr, 0, seg);
+}
+}  // namespace fpq
+
+extern "C" int fpq_gemm_mxf4_packed_multi(const void* xq, const void* xs, const void* wq, const void* ws,
+                                          const float* alpha, const void* bias, void* const* ys,
+                                          const int64_t* ns, int64_t count, int64_t M, int64_t K, void* stream) {
+  return fpq::gemm_packed_multi<false>(xq, xs, wq, ws, alpha, bias, ys, ns, count, M, K, stream);
+}
+
+extern "C" int fpq_gemm_nvf4_packed_multi(const void* xq, const void* xs, const void* wq, const void* ws,
+                                          const float* alpha, const void* bias, void* const* ys,
+                                          const int64_t* ns, int64_t count, int64_t M, int64_t K, void* stream) {
+  return fpq::gemm_packed_multi<true>(xq, xs, wq, ws, alpha, bias, ys, ns, count, M, K, stream);
 }
 
 extern "C" int fpq_gemm_nvf4_packed(const void* xq, const void* xs, const void* wq, const void* ws,

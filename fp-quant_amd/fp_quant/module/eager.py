@@ -237,8 +237,8 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
     m, k = qa.m, qa.k
     if packed is not None:   # packed MXFP4 weights of `n` rows handed in directly (a WeightGroup): wq, ws unused
         wp, wsp, n = packed
-        if qa.nvfp4 or wp.numel() * 2 != n * k:
-            raise ValueError("packed weights need MXFP4 activations with the same inner dimension")
+        if wp.numel() * 2 != n * k:
+            raise ValueError("packed weights need activations with the same inner dimension")
         use_packed = True
     elif is_packed_only(wq):   # a layer that holds its weight in the packed layout only
         n = weight_rows(wq, k)
@@ -264,7 +264,8 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
     if qa.nvfp4:
         if use_packed:
             xp, xsp = qa.packed()
-            wp, wsp = packed_weight(wq, ws, True)
+            if packed is None:
+                wp, wsp = packed_weight(wq, ws, True)
             st = lib.fpq_gemm_nvf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
                                           alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
             _engine.check(st, "fpq_gemm_nvf4_packed")
@@ -368,7 +369,7 @@ def linear_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torc
 # are column slices of it.  The layers' own packed copies become views into the concatenated buffers, so
 # no 4-bit weight is held a further time.  MXFP4 only (the NVFP4 packed kernel serves mid-sized batches only).
 class WeightGroup:
-    __slots__ = ("key", "wp", "wsp", "bias", "n", "splits", "k")
+    __slots__ = ("key", "wp", "wsp", "bias", "n", "splits", "k", "nvfp4")
 
 
 def _member_key(wq: torch.Tensor, ws: torch.Tensor, bias: Optional[torch.Tensor]):
@@ -376,19 +377,20 @@ def _member_key(wq: torch.Tensor, ws: torch.Tensor, bias: Optional[torch.Tensor]
             None if bias is None else (bias.data_ptr(), _version(bias)))
 
 
-def weight_group(members, create: bool = False) -> Optional[WeightGroup]:
-    """The WeightGroup of `members` = [(qweight, scales, bias or None, in_features), ...] (MXFP4, same K, every
-    N a multiple of 32, biases all absent or all contiguous bf16; weights row-major, or all in the packed layout
-    only), remembered on the first member's qweight until a member is written to; built now if `create`,
-    else None when there is none."""
+def weight_group(members, create: bool = False, nvfp4: bool = False) -> Optional[WeightGroup]:
+    """The WeightGroup of `members` = [(qweight, scales, bias or None, in_features), ...] (one format, same K,
+    every N a multiple of 32, biases all absent or all contiguous bf16; weights row-major, or all in the packed
+    layout only), remembered on the first member's qweight until a member is written to; built now if
+    `create`, else None when there is none."""
     first = members[0][0]
     key = tuple(_member_key(*m[:3]) for m in members)
     hit = getattr(first, "_fpq_group", None)
-    if hit is not None and hit.key == key:
+    if hit is not None and hit.key == key and hit.nvfp4 == nvfp4:
         return hit
     if not create or not packed_weights_enabled():
         return None
     k = members[0][3]
+    sgroup = 16 if nvfp4 else 32
     dev = first.device
     packed_only = is_packed_only(first)
     have_bias = [m[2] is not None for m in members]
@@ -399,9 +401,10 @@ def weight_group(members, create: bool = False) -> Optional[WeightGroup]:
                 or not wq.is_contiguous() or not ws.is_contiguous() or is_packed_only(wq) != packed_only):
             return None
         if packed_only:
-            if ws.dim() != 1 or wq.numel() * 2 % (32 * k) != 0 or ws.numel() * 16 != wq.numel():
+            if ws.dim() != 1 or wq.numel() * 2 % (32 * k) != 0 or ws.numel() * (sgroup // 2) != wq.numel():
                 return None
-        elif (wq.dim() != 2 or wq.shape[1] * 2 != k or wq.shape[0] % 32 != 0 or ws.shape != (wq.shape[0], k // 32)):
+        elif (wq.dim() != 2 or wq.shape[1] * 2 != k or wq.shape[0] % 32 != 0
+                or ws.shape != (wq.shape[0], k // sgroup)):
             return None
         if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_contiguous() or bias.device != dev):
             return None
@@ -411,7 +414,9 @@ def weight_group(members, create: bool = False) -> Optional[WeightGroup]:
     splits = [weight_rows(m[0], k) for m in members]
     n = sum(splits)
     group = WeightGroup()
-    group.n, group.splits, group.k = n, splits, k
+    group.n, group.splits, group.k, group.nvfp4 = n, splits, k, nvfp4
+    scales_bytes = lib.fpq_packed_scales_bytes_nv if nvfp4 else lib.fpq_packed_scales_bytes
+    pack = lib.fpq_pack_nvf4 if nvfp4 else lib.fpq_pack_mxf4
     with torch.cuda.device(dev):
         stream = _current_stream(dev.index)
         if packed_only:
@@ -421,21 +426,20 @@ def weight_group(members, create: bool = False) -> Optional[WeightGroup]:
             group.wsp = torch.cat([m[1] for m in members])
         else:
             group.wp = torch.empty(lib.fpq_packed_codes_bytes(n, k), dtype=torch.uint8, device=dev)
-            group.wsp = torch.empty(lib.fpq_packed_scales_bytes(n, k), dtype=torch.uint8, device=dev)
+            group.wsp = torch.empty(scales_bytes(n, k), dtype=torch.uint8, device=dev)
         row = 0
         for wq, ws, _, _ in members:
             rows = weight_rows(wq, k)
             c0, c1 = lib.fpq_packed_codes_bytes(row, k), lib.fpq_packed_codes_bytes(row + rows, k)
-            s0, s1 = lib.fpq_packed_scales_bytes(row, k), lib.fpq_packed_scales_bytes(row + rows, k)
+            s0, s1 = scales_bytes(row, k), scales_bytes(row + rows, k)
             pc, ps = group.wp[c0:c1], group.wsp[s0:s1]
             if packed_only:
                 wq.data, ws.data = pc, ps
             else:
-                st = lib.fpq_pack_mxf4(wq.data_ptr(), ws.data_ptr(), ws.shape[1], rows, k, pc.data_ptr(), ps.data_ptr(),
-                                       stream)
-                _engine.check(st, "fpq_pack_mxf4")
+                st = pack(wq.data_ptr(), ws.data_ptr(), ws.shape[1], rows, k, pc.data_ptr(), ps.data_ptr(), stream)
+                _engine.check(st, "fpq_pack")
                 # the member's own packed copy: these views (same key as hip_ops.packed_weight uses)
-                wq._fpq_packed = ((wq.data_ptr(), _version(wq), ws.data_ptr(), _version(ws), tuple(wq.shape), False), pc, ps)
+                wq._fpq_packed = ((wq.data_ptr(), _version(wq), ws.data_ptr(), _version(ws), tuple(wq.shape), nvfp4), pc, ps)
             row += rows
     group.key = tuple(_member_key(*m[:3]) for m in members)   # (packed-only members have just moved)
     group.bias = torch.cat([m[2] for m in members]).contiguous() if all(have_bias) else None
@@ -453,8 +457,8 @@ def linear_on_group(qa: QuantizedActivations, wp: torch.Tensor, wsp: torch.Tenso
     layer gets a dense matrix of its own from the kernel when all n_i are multiples of 256; else the
     outputs are column ranges of one [m, sum n_i] matrix (rows keep the full stride)."""
     m, k, n = qa.m, qa.k, sum(splits)
-    if qa.nvfp4 or wp.numel() * 2 != n * k:
-        raise ValueError("packed weights need MXFP4 activations with the same inner dimension")
+    if wp.numel() * 2 != n * k:
+        raise ValueError("packed weights need activations with the same inner dimension")
     if len(splits) > 4 or any(s % 256 for s in splits):
         y = linear_on(qa, None, None, alpha, bias, stream, True, packed=(wp, wsp, n))
         return list(y.split(splits, dim=1))
@@ -464,30 +468,36 @@ def linear_on_group(qa: QuantizedActivations, wp: torch.Tensor, wsp: torch.Tenso
     count = len(splits)
     ys = (ctypes.c_void_p * count)(*[o.data_ptr() for o in outs])
     ns = (ctypes.c_int64 * count)(*splits)
-    st = lib.fpq_gemm_mxf4_packed_multi(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(), alpha.data_ptr(),
-                                        bias.data_ptr() if bias is not None else None, ys, ns, count, m, k, stream)
-    _engine.check(st, "fpq_gemm_mxf4_packed_multi")
+    entry = lib.fpq_gemm_nvf4_packed_multi if qa.nvfp4 else lib.fpq_gemm_mxf4_packed_multi
+    st = entry(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(), alpha.data_ptr(),
+               bias.data_ptr() if bias is not None else None, ys, ns, count, m, k, stream)
+    _engine.check(st, "fpq_gemm_packed_multi")
     return outs
 
 
 def linear_cat(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, group: WeightGroup, alpha: torch.Tensor,
-               shared_source: Optional[torch.Tensor] = None, remember: bool = True) -> List[torch.Tensor]:
+               shared_source: Optional[torch.Tensor] = None, remember: bool = True,
+               act_global_scale: Optional[torch.Tensor] = None) -> List[torch.Tensor]:
     """The layers of a WeightGroup on `x_flat` (bf16 [m, K], contiguous) from one quantization and ONE
-    GEMM: bf16 [m, n_i] per layer (bias included)."""
+    GEMM: bf16 [m, n_i] per layer (bias included).  `act_global_scale`: the layers' common activation
+    scale (NVFP4 groups)."""
     dev = x_flat.device
     if torch.cuda.current_device() != dev.index:
         with torch.cuda.device(dev):
-            return linear_cat(x_flat, hadamard_matrix, group, alpha, shared_source, remember)
+            return linear_cat(x_flat, hadamard_matrix, group, alpha, shared_source, remember, act_global_scale)
     stream = _current_stream(dev.index)
     h = as_bf16(hadamard_matrix)
     kind, norm = classify_rotation(h)
+    ags = act_global_scale if group.nvfp4 else None
+    if group.nvfp4 and ags is None:
+        raise ValueError("an NVFP4 group needs the activation global scale")
     qa = key = None
     if shared_source is not None:
-        key = _sharing_key(x_flat.shape, h, kind, norm, None, stream)
+        key = _sharing_key(x_flat.shape, h, kind, norm, ags, stream)
         if key is not None:
             qa = _lookup(shared_source, key, True)
     if qa is None:
-        qa = quantize_activations(x_flat, h, kind, norm, None, False, stream, True, remember)
+        qa = quantize_activations(x_flat, h, kind, norm, ags, group.nvfp4, stream, True, remember)
         if key is not None:
             _publish(qa, shared_source, key, h)
     return linear_on_group(qa, group.wp, group.wsp, group.splits, alpha, group.bias, stream)
@@ -496,7 +506,7 @@ def linear_cat(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, group: Weigh
 @torch.library.custom_op("fp_quant::linear_cat_w4a4_op", mutates_args=())
 def linear_cat_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wp: torch.Tensor, wsp: torch.Tensor,
                        splits: List[int], weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor,
-                       bias: Optional[torch.Tensor]) -> List[torch.Tensor]:
+                       bias: Optional[torch.Tensor], nvfp4: bool = False) -> List[torch.Tensor]:
     """linear_cat for traced callers: the packed weights of a WeightGroup (made when the model was
     patched, outside any trace) times the activations quantized once; bf16 [m, n_i] per layer."""
     x = x_flat if x_flat.is_contiguous() else x_flat.contiguous()
@@ -511,14 +521,15 @@ def linear_cat_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wp: 
         h = as_bf16(hadamard_matrix)
         kind, norm = classify_rotation(h)
         alpha = linear_alpha(weight_global_scale, act_global_scale, remember=False)
-        qa = quantize_activations(x, h, kind, norm, None, False, stream, True, remember=False)
+        qa = quantize_activations(x, h, kind, norm, act_global_scale if nvfp4 else None, nvfp4, stream, True,
+                                  remember=False)
         outs = linear_on_group(qa, wp, wsp, list(splits), alpha, bias, stream)
         # operators return tensors that own their memory: column ranges of one matrix are copied out
-        return [o if o.is_contiguous() else o.contiguous() for o in outs]
+        return [o.clone() if o._is_view() else o for o in outs]
 
 
 @linear_cat_w4a4_op.register_fake
-def _(x_flat, hadamard_matrix, wp, wsp, splits, weight_global_scale, act_global_scale, bias):
+def _(x_flat, hadamard_matrix, wp, wsp, splits, weight_global_scale, act_global_scale, bias, nvfp4=False):
     return [x_flat.new_empty((x_flat.shape[0], s), dtype=torch.bfloat16) for s in splits]
 
 

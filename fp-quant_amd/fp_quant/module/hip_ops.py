@@ -288,8 +288,9 @@ def rotated_absmax(x: torch.Tensor, hadamard_matrix: torch.Tensor, amax: Optiona
 PACKED_MIN_M = 48          # GEMM operator on row-major operands (pays for re-tiling the activations)
 NV_PACKED_MIN_M = 65       # NVFP4 GEMM operator on row-major operands: from here on (and while the 128x128
 #                            tiles apply) packed; below, re-tiling the activations costs more than it saves
-NV_PACKED_LINEAR_MIN_M = 2 # NVFP4 fused linear (activations quantized straight into the packed layout): the
-#                            weight-streaming kernel up to 96 rows; one row is as fast on the row-major split-K kernel
+NV_PACKED_LINEAR_MIN_M = 1 # NVFP4 fused linear (activations quantized straight into the packed layout): the
+#                            weight-streaming kernel up to 96 rows (one row is as fast on the row-major split-K
+#                            kernel; it stays here so that a layer gives the same bits alone and in a group)
 # fused linear: activations are quantized straight into the packed layout; the weight-streaming
 # kernel on packed operands serves the few-row (decode) calls; FPQ_PACKED_MIN_ROWS raises the bar
 PACKED_LINEAR_MIN_M = int(os.environ.get("FPQ_PACKED_MIN_ROWS", "1"))

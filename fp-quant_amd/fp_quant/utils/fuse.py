@@ -89,10 +89,11 @@ def _quantize_alike(layers) -> bool:
 
 def _weight_group(layers, create: bool = False):
     """The layers' packed weights laid end to end (eager.WeightGroup), if they can be multiplied as one:
-    MXFP4 abs-max layers that quantize alike with equal alpha.  Built when the model is patched
+    abs-max layers (MXFP4 or NVFP4) that quantize alike with equal alpha.  Built when the model is patched
     (`create`), looked up afterwards (None: the layers were rewritten since, or never qualified)."""
     first = layers[0]
-    if first.config.forward_dtype != FPQuantDtype.MXFP4 or first.config.forward_method != "abs_max":
+    if (first.config.forward_dtype not in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4)
+            or first.config.forward_method != "abs_max"):
         return None
     if create:
         if not first.qweight.is_cuda or not _quantize_alike(layers):
@@ -100,7 +101,8 @@ def _weight_group(layers, create: bool = False):
         for layer in layers[1:]:
             if not torch.equal(layer.weight_global_scale.float(), first.weight_global_scale.float()):
                 return None
-    return _eager().weight_group([(l.qweight, l.scales, l.bias, l.in_features) for l in layers], create)
+    return _eager().weight_group([(l.qweight, l.scales, l.bias, l.in_features) for l in layers], create,
+                                 first.config.forward_dtype == FPQuantDtype.NVFP4)
 
 
 def _attach_weight_group(module: nn.Module, names) -> None:
@@ -117,15 +119,25 @@ def _attach_weight_group(module: nn.Module, names) -> None:
     module._fpq_weight_group_hook = module.register_load_state_dict_post_hook(build)
 
 
+# NVFP4: the one GEMM pays for decode-sized batches (weight-streaming and 128x128-tile kernels on packed
+# operands, the same kernels the layers run one by one there); large batches are faster on the row-major
+# kernel, layer by layer.
+_NV_GROUP_MAX_ROWS = 128
+
+
+def _group_serves(group, x: torch.Tensor) -> bool:
+    return not group.nvfp4 or x.numel() // x.shape[-1] <= _NV_GROUP_MAX_ROWS
+
+
 def _group_linear(layers, x: torch.Tensor, group=None):
     """The outputs of `layers` on `x` from ONE operator: one quantization and, where the layers' packed
     weights lie end to end (`group`, a WeightGroup), one GEMM whose column ranges are the outputs; else
     one GEMM each."""
     first = layers[0]
-    if group is not None:
+    if group is not None and _group_serves(group, x):
         outs = _eager().linear_cat_w4a4_op(x.reshape(-1, x.shape[-1]), first.forward_hadamard_matrix, group.wp,
                                            group.wsp, group.splits, first.weight_global_scale,
-                                           first.act_global_scale, group.bias)
+                                           first.act_global_scale, group.bias, group.nvfp4)
         return [o.view(*x.shape[:-1], o.shape[-1]) for o in outs]
     outs = _eager().linear_group_w4a4_op(
         x.reshape(-1, x.shape[-1]), first.forward_hadamard_matrix, [l.qweight for l in layers],
@@ -359,7 +371,7 @@ def _eager_group_linear(owner: nn.Module, layers, x: torch.Tensor):
     `x` is taken from, or left in, the sharing slot); None if there is no group.  The group kept on
     `owner` is checked against the layers' tensors as they are now and rebuilt if they were written to."""
     group = getattr(owner, "_fpq_weight_group", None)
-    if group is None:
+    if group is None or not _group_serves(group, x):
         return None
     first = layers[0]
     if group.key != tuple(_eager()._member_key(l.qweight, l.scales, l.bias) for l in layers):
@@ -371,7 +383,8 @@ def _eager_group_linear(owner: nn.Module, layers, x: torch.Tensor):
     if not x_flat.is_contiguous():
         return None
     outs = eager.linear_cat(x_flat, first.forward_hadamard_matrix, group,
-                            eager.linear_alpha(first.weight_global_scale, first.act_global_scale), shared_source=x)
+                            eager.linear_alpha(first.weight_global_scale, first.act_global_scale), shared_source=x,
+                            act_global_scale=first.act_global_scale)
     return [o.unflatten(0, tuple(x.shape[:-1])) for o in outs]
 
 

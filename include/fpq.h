@@ -298,6 +298,11 @@ int fpq_gemm_mxf4_packed_multi(const void* xq_packed, const void* xs_packed, con
                                const void* ws_packed, const float* alpha, const void* bias,
                                void* const* ys, const int64_t* ns, int64_t count, int64_t M, int64_t K,
                                void* stream);
+/* The same for packed NVFP4 operands (fpq_gemm_nvf4_packed). */
+int fpq_gemm_nvf4_packed_multi(const void* xq_packed, const void* xs_packed, const void* wq_packed,
+                               const void* ws_packed, const float* alpha, const void* bias,
+                               void* const* ys, const int64_t* ns, int64_t count, int64_t M, int64_t K,
+                               void* stream);
 
 /*
  * fpq_gemm_mxf4_packed_splitk for callers that cannot allocate or hold a workspace (code recorded

@@ -135,9 +135,9 @@ def gemm_packed_splitk(xp, xsp, wp, wsp, m, n, k, alpha, bias=None, residual=Non
     return y.cpu()
 
 
-def gemm_packed_multi(xp, xsp, wp, wsp, m, splits, k, alpha, bias=None):
-    """fpq_gemm_mxf4_packed_multi on packed operands (the weights of len(splits) layers end to end); a list
-    of bf16 [M, splits[i]] on the CPU."""
+def gemm_packed_multi(xp, xsp, wp, wsp, m, splits, k, alpha, bias=None, nv=False):
+    """fpq_gemm_mxf4_packed_multi (nv: fpq_gemm_nvf4_packed_multi) on packed operands (the weights of
+    len(splits) layers end to end); a list of bf16 [M, splits[i]] on the CPU."""
     lib = _engine.lib()
     xp, xsp, wp, wsp = (t.to("cuda").contiguous() for t in (xp, xsp, wp, wsp))
     outs = [torch.full((m, s), float("nan"), dtype=torch.bfloat16, device="cuda") for s in splits]
@@ -145,10 +145,11 @@ def gemm_packed_multi(xp, xsp, wp, wsp, m, splits, k, alpha, bias=None):
     b = bias.to("cuda").contiguous() if bias is not None else None
     ys = (ctypes.c_void_p * len(splits))(*[o.data_ptr() for o in outs])
     ns = (ctypes.c_int64 * len(splits))(*splits)
-    st = lib.fpq_gemm_mxf4_packed_multi(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(), a.data_ptr(),
-                                        b.data_ptr() if b is not None else None, ys, ns, len(splits), m, k,
-                                        torch.cuda.current_stream().cuda_stream)
-    _engine.check(st, "fpq_gemm_mxf4_packed_multi")
+    entry = lib.fpq_gemm_nvf4_packed_multi if nv else lib.fpq_gemm_mxf4_packed_multi
+    st = entry(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(), a.data_ptr(),
+               b.data_ptr() if b is not None else None, ys, ns, len(splits), m, k,
+               torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_gemm_packed_multi")
     torch.cuda.synchronize()
     return [o.cpu() for o in outs]
 

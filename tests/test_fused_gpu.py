@@ -494,15 +494,17 @@ def test_compiled_decode_with_grouped_operators_matches_eager(fmt, g, arch, held
         assert torch.equal(a, b), i
 
 
-@pytest.mark.parametrize("tokens", [3, 40, 300])
-def test_grouped_projections_run_as_one_gemm_on_concatenated_packed_weights(tokens):
+@pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])
+@pytest.mark.parametrize("tokens", [1, 3, 40, 300])
+def test_grouped_projections_run_as_one_gemm_on_concatenated_packed_weights(tokens, fmt, g):
     """After fuse_producers q/k/v (and gate/up) of an MXFP4 block are one GEMM on the layers' packed weights
     laid end to end: same bits as the three (two) layers called one by one, the layers' own packed copies
     are views into the concatenated buffers, and a load_state_dict is followed."""
     from fp_quant.module import eager
     from fp_quant.utils import fuse_producers
-    model = _tiny_llama("mxfp4", 128, seed=3)
-    other = _tiny_llama("mxfp4", 128, seed=4)
+    model = _tiny_llama(fmt, g, seed=3)
+    other = _tiny_llama(fmt, g, seed=4)
+    grouped = fmt == "mxfp4" or tokens <= 128      # NVFP4: one GEMM for decode-sized batches only
     block, block2 = model.model.layers[0], other.model.layers[0]
     attn, mlp = block.self_attn, block.mlp
     x = (torch.randn(1, tokens, 256, device="cuda") * 1.5).to(torch.bfloat16)
@@ -518,20 +520,22 @@ def test_grouped_projections_run_as_one_gemm_on_concatenated_packed_weights(toke
             assert lo <= layer.qweight._fpq_packed[1].data_ptr() < hi        # no further copy of the weights
         got = attn._fpq_qkv(x)
         # k and v have 128 output features here: column ranges of one output matrix
-        assert got[0].data_ptr() + 2 * want[0].shape[-1] == got[1].data_ptr()
+        assert (got[0].data_ptr() + 2 * want[0].shape[-1] == got[1].data_ptr()) == grouped
         for a, b in zip(got, want):
             assert torch.equal(a, b)
         gate, up = want_mlp
         # gate and up have 512 each (multiples of 256): the one GEMM writes a dense matrix per layer
         from fp_quant.utils import fuse
         pair = fuse._eager_group_linear(mlp, (mlp.gate_proj, mlp.up_proj), x)
-        assert all(t.is_contiguous() for t in pair) and torch.equal(pair[0], gate) and torch.equal(pair[1], up)
+        assert (pair is not None) == grouped
+        if grouped:
+            assert all(t.is_contiguous() for t in pair) and torch.equal(pair[0], gate) and torch.equal(pair[1], up)
         assert torch.equal(block.mlp(x), block.mlp.down_proj(O.silu_mul(
             gate.cpu().view(-1, gate.shape[-1]), up.cpu().view(-1, up.shape[-1])).view(gate.shape).cuda()))
         # traced callers: the same through the operator
         outs = eager.linear_cat_w4a4_op(x.view(-1, 256), attn.q_proj.forward_hadamard_matrix, group.wp, group.wsp,
                                         group.splits, attn.q_proj.weight_global_scale, attn.q_proj.act_global_scale,
-                                        group.bias)
+                                        group.bias, fmt == "nvfp4")
         for a, b in zip(outs, want):
             assert a.is_contiguous() and torch.equal(a.reshape(b.shape), b)
         # new weights: the hook rebuilds the group
@@ -542,7 +546,7 @@ def test_grouped_projections_run_as_one_gemm_on_concatenated_packed_weights(toke
 
 
 @pytest.mark.parametrize("order,fmt,g", [("fuse_then_release", "mxfp4", 128), ("release_then_fuse", "mxfp4", 128),
-                                         ("fuse_then_release", "nvfp4", 16)])
+                                         ("fuse_then_release", "nvfp4", 16), ("release_then_fuse", "nvfp4", 16)])
 def test_model_with_weights_held_once_keeps_its_logits(order, fmt, g):
     """release_row_major_weights on a whole model, before or after fuse_producers: every layer holds the
     packed layout only (the groups of projections included: their members are views into the group's
@@ -571,9 +575,6 @@ def test_model_with_weights_held_once_keeps_its_logits(order, fmt, g):
             assert release_row_major_weights(model) == n_layers
         for block in model.model.layers:
             attn, group = block.self_attn, block.self_attn._fpq_weight_group
-            if fmt != "mxfp4":      # groups of projections exist for MXFP4 only
-                assert group is None and all(l.weights_packed_only for l in (attn.q_proj, attn.k_proj, attn.v_proj))
-                continue
             assert group is not None and block.mlp._fpq_weight_group is not None
             lo, hi = group.wp.data_ptr(), group.wp.data_ptr() + group.wp.numel()
             for layer in (attn.q_proj, attn.k_proj, attn.v_proj):

@@ -302,3 +302,28 @@ def test_unpack_nv_is_the_inverse_of_the_layout_definition(rows, k):
     got_c, got_s = capi.unpack(pc, ps, rows, k, scale_pad=8, nv=True)
     assert torch.equal(got_c, codes) and torch.equal(got_s[:, : k // 16], scales)
     assert (got_s[:, k // 16:] == 0xCD).all()
+
+
+@pytest.mark.parametrize("m,splits,k", [(1, [512, 256, 256], 512), (48, [1024, 256], 1024), (96, [256, 512], 256),
+                                        (128, [256, 256, 256, 256], 768), (300, [512, 256, 256], 512),
+                                        (2048, [2048, 1024, 256, 768], 256)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_nv_layers_end_to_end_get_their_own_outputs(m, splits, k, with_bias):
+    """fpq_gemm_nvf4_packed_multi: every layer's matrix equals its column range of fpq_gemm_nvf4_packed on the
+    same operands bit for bit (weight-streaming kernel, 128x128 tiles, 256x256 tiles)."""
+    n = sum(splits)
+    g = torch.Generator().manual_seed(900 + m + n)
+    xq = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=g)
+    wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=g)
+    xs = torch.randint(24, 72, (m, k // 16), dtype=torch.uint8, generator=g)
+    ws = torch.randint(24, 72, (n, k // 16), dtype=torch.uint8, generator=g)
+    bias = torch.randn(n, generator=g).to(torch.bfloat16) if with_bias else None
+    xp, xsp = pack_nv_by_definition(xq, xs, k)
+    wp, wsp = pack_nv_by_definition(wq, ws, k)
+    whole = capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, 2.0 ** -6, bias=bias)
+    outs = capi.gemm_packed_multi(xp, xsp, wp, wsp, m, splits, k, 2.0 ** -6, bias=bias, nv=True)
+    col = 0
+    for o, s_ in zip(outs, splits):
+        assert o.shape == (m, s_)
+        assert torch.equal(o.view(torch.int16), whole[:, col:col + s_].contiguous().view(torch.int16))
+        col += s_
