@@ -177,6 +177,8 @@ class FPQuantLinear(nn.Module):
             return True
         q, s = getattr(self, "qweight", None), getattr(self, "scales", None)
         nvfp4 = self.config.forward_dtype == FPQuantDtype.NVFP4
+        if not hip_ops.packed_weights_enabled():   # FPQ_PACKED_WEIGHTS=0: every call stays on the row-major kernels
+            return False
         if (self.config.forward_dtype not in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4) or q is None or s is None
                 or not q.is_cuda or q.dim() != 2 or q.dtype != torch.uint8 or s.dtype != torch.uint8
                 or self.in_features % 256 != 0 or self.out_features % 32 != 0
