@@ -452,7 +452,7 @@ static int pack_operand(const void* codes, const void* scales, int64_t scale_str
 }  // namespace fpq
 
 #ifndef FPQ_NV_STREAM_ROWS
-#define FPQ_NV_STREAM_ROWS 96   // NVFP4: up to this many rows the weight-streaming kernel (where its plan applies)
+#define FPQ_NV_STREAM_ROWS 128  // NVFP4: up to this many rows the weight-streaming kernel (where its plan applies)
 #endif
 #ifndef FPQ_PACKED_HALF_TILES
 #define FPQ_PACKED_HALF_TILES 1  // large M: 1 = 256x128 tiles for MXFP4, 2 = for NVFP4 too, 0 = 256x256

@@ -92,7 +92,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_fp4_stream_kernel(
   uint4 a[DB][4][NT], b[DB][4][MT];
   uint2 sa[DB][NT], sb[DB][MT];   // MXFP4 uses .x only
   const int t_last = nblk > 0 ? nblk - 1 : 0;
-  auto load_block = [&](auto slot, int t) {
+  // (the lambdas must be inlined whatever their size: a call would pin the register arrays they capture
+  // to memory)
+  auto load_block = [&](auto slot, int t) __attribute__((always_inline)) {
     constexpr int s = decltype(slot)::value;
     const int kb = min(first + NW * min(t, t_last), nkb - 1);
 #pragma unroll
@@ -113,26 +115,32 @@ __global__ __launch_bounds__(64 * NW) void gemm_fp4_stream_kernel(
       else sb[s][j].x = *(const uint32_t*)(xscale[j] + (size_t)kb * kSB);
     }
   };
-  auto compute_block = [&](auto slot) {
+  // NVFP4: activation row tiles whose fp16 operands are held at a time (four tiles: two and two, the
+  // weight operand is converted once more; all four at once left the register file)
+  constexpr int kJB = (MT == 4) ? 2 : MT;
+  auto compute_block = [&](auto slot) __attribute__((always_inline)) {
     constexpr int s = decltype(slot)::value;
 #define FPQ_STREAM_STEP(U)                                                                              \
   if constexpr (NV) {                                                                                   \
-    v8h bh[MT][4];                                                                                      \
-    _Pragma("unroll") for (int j = 0; j < MT; ++j) {                                                    \
-      const uint4 bq = b[s][U][j];                                                                      \
-      const uint32_t bw[4] = {bq.x, bq.y, bq.z, bq.w};                                                  \
-      const uint32_t bsc = ((U) < 2 ? sb[s][j].x : sb[s][j].y) >> (16 * ((U) & 1));                     \
-      _Pragma("unroll") for (int s4 = 0; s4 < 4; ++s4)                                                  \
-        bh[j][s4] = dequant8_f16_s(bw[s4], e4m3_pair_f16(bsc >> (8 * (s4 >> 1))));                      \
-    }                                                                                                   \
-    _Pragma("unroll") for (int i = 0; i < NT; ++i) {                                                    \
-      const uint4 aq = a[s][U][i];                                                                      \
-      const uint32_t aw[4] = {aq.x, aq.y, aq.z, aq.w};                                                  \
-      const uint32_t asc = ((U) < 2 ? sa[s][i].x : sa[s][i].y) >> (16 * ((U) & 1));                     \
-      _Pragma("unroll") for (int s4 = 0; s4 < 4; ++s4) {                                                \
-        const v8h ah = dequant8_f16_s(aw[s4], e4m3_pair_f16(asc >> (8 * (s4 >> 1))));                   \
-        _Pragma("unroll") for (int j = 0; j < MT; ++j)                                                  \
-          acc[i * MT + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[j][s4], acc[i * MT + j], 0, 0, 0); \
+    _Pragma("unroll") for (int j0 = 0; j0 < MT; j0 += kJB) {                                            \
+      v8h bh[kJB][4];                                                                                   \
+      _Pragma("unroll") for (int j = 0; j < kJB; ++j) {                                                 \
+        const uint4 bq = b[s][U][j0 + j];                                                               \
+        const uint32_t bw[4] = {bq.x, bq.y, bq.z, bq.w};                                                \
+        const uint32_t bsc = ((U) < 2 ? sb[s][j0 + j].x : sb[s][j0 + j].y) >> (16 * ((U) & 1));         \
+        _Pragma("unroll") for (int s4 = 0; s4 < 4; ++s4)                                                \
+          bh[j][s4] = dequant8_f16_s(bw[s4], e4m3_pair_f16(bsc >> (8 * (s4 >> 1))));                    \
+      }                                                                                                 \
+      _Pragma("unroll") for (int i = 0; i < NT; ++i) {                                                  \
+        const uint4 aq = a[s][U][i];                                                                    \
+        const uint32_t aw[4] = {aq.x, aq.y, aq.z, aq.w};                                                \
+        const uint32_t asc = ((U) < 2 ? sa[s][i].x : sa[s][i].y) >> (16 * ((U) & 1));                   \
+        _Pragma("unroll") for (int s4 = 0; s4 < 4; ++s4) {                                              \
+          const v8h ah = dequant8_f16_s(aw[s4], e4m3_pair_f16(asc >> (8 * (s4 >> 1))));                 \
+          _Pragma("unroll") for (int j = 0; j < kJB; ++j)                                               \
+            acc[i * MT + j0 + j] =                                                                      \
+                __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[j][s4], acc[i * MT + j0 + j], 0, 0, 0);   \
+        }                                                                                               \
       }                                                                                                 \
     }                                                                                                   \
   } else {                                                                                              \
@@ -153,7 +161,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fp4_stream_kernel(
     FPQ_STREAM_STEP(3)
 #undef FPQ_STREAM_STEP
   };
-  auto for_slots = [&](auto&& f) {
+  auto for_slots = [&](auto&& f) __attribute__((always_inline)) {
     f(std::integral_constant<int, 0>{});
     if constexpr (DB > 1) f(std::integral_constant<int, 1>{});
     if constexpr (DB > 2) f(std::integral_constant<int, 2>{});
@@ -180,14 +188,14 @@ __global__ __launch_bounds__(64 * NW) void gemm_fp4_stream_kernel(
   }
 
   // ---- the four K parts of the workgroup, summed in the fixed order (w0 + w2) + (w1 + w3)
-  auto put = [&](int slot) {
+  auto put = [&](int slot) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < NT * MT; ++j)
 #pragma unroll
       for (int g = 0; g < 4; ++g)
         part[slot][j][g][lane] = v4f{acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]};
   };
-  auto take = [&](int slot) {
+  auto take = [&](int slot) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < NT * MT; ++j)
 #pragma unroll
@@ -366,10 +374,7 @@ static int launch_stream(const void* xq, const void* xs, const void* wq, const v
     case 2: FPQ_STREAM(1, 2, 2); break;
     case 3: FPQ_STREAM(1, 3, 2); break;
     default:
-      // NVFP4 with four activation row tiles does not fit the register file (dequantized fp16 operands
-      // of four tiles next to 64 accumulators): the caller keeps those shapes on the tile kernel
-      if constexpr (NV) return FPQ_E_UNSUPPORTED;
-      else FPQ_STREAM(1, 4, 2);
+      FPQ_STREAM(1, 4, 2);
       break;
   }
 #undef FPQ_STREAM
