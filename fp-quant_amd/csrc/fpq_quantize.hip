@@ -123,7 +123,8 @@ template <int G, int ROT, int PRO = kProNone>
 __device__ __forceinline__ void lane8_load_rotate(const uint4* __restrict__ x, uint32_t chunk, bool active,
                                                   uint32_t lane, float norm, float* __restrict__ stage,
                                                   const uint16_t* __restrict__ hmat, float (&p)[8],
-                                                  const Prologue& pro = Prologue{}) {
+                                                  const Prologue& pro = Prologue{}, float row_scale = -1.0f) {
+  // row_scale >= 0: the row's 1 / rms, computed by the caller in this launch (else pro.row_scale[row])
   uint4 raw = make_uint4(0u, 0u, 0u, 0u);
   if (PRO == kProNone) {
     if (active) raw = x[chunk];
@@ -136,7 +137,7 @@ __device__ __forceinline__ void lane8_load_rotate(const uint4* __restrict__ x, u
       raw = x[(size_t)row * pro.ld_first + cc];
       if (PRO == kProRmsNorm) {
         aux = pro.col_scale[cc];
-        rs = pro.row_scale[row];
+        rs = row_scale >= 0.0f ? row_scale : pro.row_scale[row];
       } else {
         aux = pro.second[(size_t)row * pro.ld_second + cc];
       }
@@ -240,11 +241,11 @@ __device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint3
                                               uint32_t scale_stride, float norm, float gscale, float rg,
                                               float* __restrict__ stage, const uint16_t* __restrict__ hmat,
                                               uint8_t* __restrict__ mask = nullptr,
-                                              const Prologue& pro = Prologue{}) {
+                                              const Prologue& pro = Prologue{}, float row_scale = -1.0f) {
   static_assert(!QUEST || FMT == kFmtMx, "the quest rule exists for MXFP4 only");
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
   float p[8];
-  lane8_load_rotate<G, ROT, PRO>(x, chunk, active, lane, norm, stage, hmat, p, pro);
+  lane8_load_rotate<G, ROT, PRO>(x, chunk, active, lane, norm, stage, hmat, p, pro, row_scale);
 
   if (QUEST) {
     float sum = p[0], sq = p[0] * p[0];
@@ -1377,6 +1378,56 @@ __global__ __launch_bounds__(256) void row_inv_rms_kernel(const uint4* __restric
   if (lane == 0u) out[row] = 1.0f / __builtin_sqrtf(a / cols_f + eps);
 }
 
+// RMSNorm + rotate + quantize of a few rows in ONE launch (decode): a workgroup per row computes the
+// row's 1 / rms exactly as row_inv_rms_kernel does (the octet sums go through LDS, then one wave adds
+// them in that kernel's order) and quantizes the row with the generic kernel's arithmetic into the
+// packed operand layout.  Workgroups past `rows` (the padding of the last 32-row tile) write zeros.
+constexpr uint32_t kRowsKernelMaxChunks = 2048;   // cols <= 16384
+template <int G, int ROT, int ZERO>
+__global__ __launch_bounds__(256) void rmsnorm_rows_quantize_kernel(const uint4* __restrict__ x,
+                                                                    uint32_t* __restrict__ codes,
+                                                                    uint8_t* __restrict__ scales, uint32_t rows,
+                                                                    float norm, float cols_f, float eps,
+                                                                    float* __restrict__ inv_rms_out, Prologue pro) {
+  __shared__ float oct[kRowsKernelMaxChunks];
+  __shared__ float inv_shared;
+  const uint32_t row = blockIdx.x, cpr = pro.chunks_per_row, lane = threadIdx.x & 63u;
+  const bool real = row < rows;
+  if (real) {
+    const uint4* src = x + (size_t)row * pro.ld_first;
+    for (uint32_t c = threadIdx.x; c < cpr; c += 256u) {
+      float p[8];
+      unpack8(src[c], p);
+      float s = p[0] * p[0];
+#pragma unroll
+      for (int i = 1; i < 8; ++i) s = s + p[i] * p[i];
+      oct[c] = s;
+    }
+  }
+  __syncthreads();
+  if (real && threadIdx.x < 64u) {
+    float a = 0.0f;
+    for (uint32_t c = lane; c < cpr; c += 64u) a = a + oct[c];
+#pragma unroll
+    for (int lm = 1; lm < 64; lm *= 2) a = a + __shfl_xor(a, lm, 64);
+    if (lane == 0u) {
+      const float inv = 1.0f / __builtin_sqrtf(a / cols_f + eps);
+      inv_shared = inv;
+      if (inv_rms_out) inv_rms_out[row] = inv;
+    }
+  }
+  __syncthreads();
+  const float rs = real ? inv_shared : 0.0f;
+  for (uint32_t c0 = 0; c0 < cpr; c0 += 256u) {   // the same trip count for every thread: lanes exchange values
+    const uint32_t cc = c0 + threadIdx.x;
+    const bool in = cc < cpr;
+    // a chunk index past the packed output makes the generic kernel skip the store
+    const uint32_t chunk = in ? row * cpr + cc : 0xffffffffu;
+    lane8_process<G, kFmtMx, ROT, ZERO, false, kProRmsNorm>(x, codes, scales, chunk, real && in, lane, cpr, 0u, norm,
+                                                            1.0f, 1.0f, nullptr, nullptr, nullptr, pro, rs);
+  }
+}
+
 // ------------------------------------------------------------------------------------------
 // max |rotate(x)| over a whole tensor, folded into *amax with an atomic maximum on the bit
 // pattern (non-negative floats order like unsigned integers).  The rotation is the quantizers'
@@ -1566,6 +1617,67 @@ extern "C" int fpq_rmsnorm_quantize_mx_packed(const void* x, int64_t ld, const f
   return fpq::dispatch_prologue_packed<fpq::kProRmsNorm>(x, ld, nullptr, 0, inv_rms, weight, normed, rows, cols,
                                                          rot_kind, g, norm, packed_codes, packed_scales,
                                                          zero_policy, stream);
+}
+
+namespace fpq {
+static int dispatch_rmsnorm_rows(const void* x, int64_t ld, const void* weight, int64_t rows, int64_t cols, float eps,
+                                 int rot_kind, int g, float norm, float* inv_rms, void* normed, void* codes,
+                                 void* scales, int zero_policy, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (rows < 0 || cols < 0) return FPQ_E_SHAPE;
+  if (rows == 0 || cols == 0) return FPQ_OK;
+  if (!x || !weight || !codes || !scales) return FPQ_E_NULL;
+  if (zero_policy != FPQ_ZERO_REFERENCE && zero_policy != FPQ_ZERO_SIGNED) return FPQ_E_POLICY;
+  if (rot_kind == FPQ_ROT_IDENTITY) g = 32;
+  if (rot_kind != FPQ_ROT_IDENTITY && rot_kind != FPQ_ROT_HADAMARD) {
+    return (rot_kind == FPQ_ROT_GSR || rot_kind == FPQ_ROT_GENERAL) ? FPQ_E_UNSUPPORTED : FPQ_E_ROTATION;
+  }
+  if (g != 16 && g != 32 && g != 64 && g != 128) return FPQ_E_ROTATION;
+  if (cols % 256 != 0 || ld < cols || ld % 8 != 0 || ld >= (int64_t)1 << 24) return FPQ_E_SHAPE;
+  if (rows > kPackedFewRows || cols / 8 > (int64_t)kRowsKernelMaxChunks) return FPQ_E_LIMIT;
+  if (((uintptr_t)x & 15u) || ((uintptr_t)weight & 15u) || ((uintptr_t)normed & 15u) || ((uintptr_t)inv_rms & 3u) ||
+      ((uintptr_t)codes & 15u) || ((uintptr_t)scales & 3u)) {
+    return FPQ_E_ALIGN;
+  }
+  Prologue pro{};
+  pro.col_scale = (const uint4*)weight;
+  pro.out = (uint4*)normed;
+  pro.chunks_per_row = (uint32_t)(cols / 8);
+  pro.ld_first = (uint32_t)(ld / 8);
+  pro.packed_rows = (uint32_t)((rows + 31) / 32 * 32);
+  const dim3 grid(pro.packed_rows), block(256);
+#define FPQ_LAUNCH_ROWS(GG, RR)                                                                                 \
+  {                                                                                                             \
+    if (zero_policy == FPQ_ZERO_REFERENCE)                                                                      \
+      hipLaunchKernelGGL((rmsnorm_rows_quantize_kernel<GG, RR, kZeroReference>), grid, block, 0, stream,        \
+                         (const uint4*)x, (uint32_t*)codes, (uint8_t*)scales, (uint32_t)rows, norm, (float)cols, \
+                         eps, inv_rms, pro);                                                                    \
+    else                                                                                                        \
+      hipLaunchKernelGGL((rmsnorm_rows_quantize_kernel<GG, RR, kZeroSigned>), grid, block, 0, stream,           \
+                         (const uint4*)x, (uint32_t*)codes, (uint8_t*)scales, (uint32_t)rows, norm, (float)cols, \
+                         eps, inv_rms, pro);                                                                    \
+    return (int)hipGetLastError();                                                                              \
+  }
+  if (rot_kind == FPQ_ROT_IDENTITY) FPQ_LAUNCH_ROWS(32, FPQ_ROT_IDENTITY);
+  switch (g) {
+    case 16: FPQ_LAUNCH_ROWS(16, FPQ_ROT_HADAMARD);
+    case 32: FPQ_LAUNCH_ROWS(32, FPQ_ROT_HADAMARD);
+    case 64: FPQ_LAUNCH_ROWS(64, FPQ_ROT_HADAMARD);
+    case 128: FPQ_LAUNCH_ROWS(128, FPQ_ROT_HADAMARD);
+  }
+#undef FPQ_LAUNCH_ROWS
+  return FPQ_E_ROTATION;
+}
+}  // namespace fpq
+
+extern "C" int64_t fpq_rmsnorm_rows_max_rows(void) { return fpq::kPackedFewRows; }
+
+extern "C" int fpq_rmsnorm_rows_quantize_mx_packed(const void* x, int64_t ld, const void* weight, int64_t rows,
+                                                   int64_t cols, float eps, int rot_kind, int g, float norm,
+                                                   float* inv_rms, void* normed, void* packed_codes,
+                                                   void* packed_scales, int zero_policy, void* stream) {
+  return fpq::dispatch_rmsnorm_rows(x, ld, weight, rows, cols, eps, rot_kind, g, norm, inv_rms, normed, packed_codes,
+                                    packed_scales, zero_policy, stream);
 }
 
 extern "C" int fpq_silu_mul_quantize_mx_packed(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,

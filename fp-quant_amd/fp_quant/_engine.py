@@ -15,6 +15,7 @@ _lib = None
 ROT_HADAMARD, ROT_IDENTITY, ROT_GSR, ROT_GENERAL = 0, 1, 2, 3
 ZERO_REFERENCE, ZERO_SIGNED = 0, 1
 E_UNSUPPORTED = -6
+E_LIMIT = -7
 
 _P, _I64, _I, _F = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
 
@@ -55,6 +56,8 @@ _SIGNATURES = {
     "fpq_gemm_nvf4_packed_multi": ([_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _I),
     "fpq_unpack_mxf4": ([_P, _P, _I64, _I64, _P, _P, _I64, _P], _I),
     "fpq_unpack_nvf4": ([_P, _P, _I64, _I64, _P, _P, _I64, _P], _I),
+    "fpq_rmsnorm_rows_max_rows": ([], _I64),
+    "fpq_rmsnorm_rows_quantize_mx_packed": ([_P, _I64, _P, _I64, _I64, _F, _I, _I, _F, _P, _P, _P, _P, _I, _P], _I),
     "fpq_prepare_device": ([_P], _I),
     "fpq_gemm_mxf4_packed_noalloc_max_rows": ([], _I64),
     "fpq_gemm_mxf4_packed_noalloc": ([_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _I),

@@ -681,6 +681,9 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
     return qa
 
 
+_ROWS_KERNEL_MAX_ROWS = 64   # fpq_rmsnorm_rows_max_rows()
+
+
 def rmsnorm_quantize(x: torch.Tensor, weight: torch.Tensor, eps: float, hadamard_matrix: torch.Tensor,
                      act_global_scale: Optional[torch.Tensor], nvfp4: bool) -> Optional[torch.Tensor]:
     """RMSNorm of bf16 `x` over its last dimension, y = bf16(weight * bf16(x / rms)), in one pass
@@ -701,13 +704,26 @@ def rmsnorm_quantize(x: torch.Tensor, weight: torch.Tensor, eps: float, hadamard
         if kind not in (_engine.ROT_HADAMARD, _engine.ROT_IDENTITY) or cols % max(h.shape[0], 32) != 0:
             return None
         lib = _engine.lib()
-        inv = torch.empty(rows, dtype=torch.float32, device=dev)
-        _engine.check(lib.fpq_row_inv_rms(x_flat.data_ptr(), cols, rows, cols, eps, inv.data_ptr(), stream),
-                      "fpq_row_inv_rms")
         y = torch.empty_like(x_flat)
         w = weight.contiguous()
-        qa = _fused_quantize("rmsnorm", (x_flat.data_ptr(), cols, inv.data_ptr(), w.data_ptr()), rows, cols, h, kind,
-                             norm, act_global_scale, nvfp4, y, stream, dev)
+        qa = None
+        if (not nvfp4 and rows <= _ROWS_KERNEL_MAX_ROWS and cols % 256 == 0 and cols <= 16384
+                and packed_linear_eligible(rows, cols, "abs_max")):
+            # a decode step's few rows: statistic, normalisation and quantization in one launch
+            pc = torch.empty(lib.fpq_packed_codes_bytes(rows, cols), dtype=torch.uint8, device=dev)
+            ps = torch.empty(lib.fpq_packed_scales_bytes(rows, cols), dtype=torch.uint8, device=dev)
+            st = lib.fpq_rmsnorm_rows_quantize_mx_packed(x_flat.data_ptr(), cols, w.data_ptr(), rows, cols, eps, kind,
+                                                         h.shape[0], norm, None, y.data_ptr(), pc.data_ptr(),
+                                                         ps.data_ptr(), ZERO_NIBBLE_POLICY, stream)
+            _engine.check(st, "fpq_rmsnorm_rows_quantize_mx_packed")
+            qa = QuantizedActivations(rows, cols, nvfp4)
+            qa.mx_packed = (pc, ps)
+        if qa is None:
+            inv = torch.empty(rows, dtype=torch.float32, device=dev)
+            _engine.check(lib.fpq_row_inv_rms(x_flat.data_ptr(), cols, rows, cols, eps, inv.data_ptr(), stream),
+                          "fpq_row_inv_rms")
+            qa = _fused_quantize("rmsnorm", (x_flat.data_ptr(), cols, inv.data_ptr(), w.data_ptr()), rows, cols, h, kind,
+                                 norm, act_global_scale, nvfp4, y, stream, dev)
         if qa is None:
             return None
         y = y.view(x.shape)

@@ -232,6 +232,20 @@ int fpq_rmsnorm_quantize_mx_packed(const void* x, int64_t ld, const float* inv_r
                                    int64_t rows, int64_t cols, int rot_kind, int g, float norm,
                                    void* normed, void* packed_codes, void* packed_scales, int zero_policy,
                                    void* stream);
+/*
+ * fpq_row_inv_rms followed by fpq_rmsnorm_quantize_mx_packed in ONE launch, for the few rows of a decode
+ * step: same bits (the row statistic keeps its summation order), one kernel instead of two.
+ *   rows      at most fpq_rmsnorm_rows_max_rows() (64); cols % 256 == 0, cols <= 16384; FPQ_E_LIMIT beyond
+ *   inv_rms   null, or fp32 [rows] that receives the row statistic
+ *   normed    null, or bf16 [rows, cols] that receives weight * (x / rms)
+ * Hadamard 16..128 and identity rotations; others return FPQ_E_UNSUPPORTED.  No counterpart in the reference,
+ * which normalises with PyTorch's RMSNorm module and then quantizes (llama_utils.py:132-160).
+ */
+int64_t fpq_rmsnorm_rows_max_rows(void);
+int fpq_rmsnorm_rows_quantize_mx_packed(const void* x, int64_t ld, const void* weight, int64_t rows,
+                                        int64_t cols, float eps, int rot_kind, int g, float norm,
+                                        float* inv_rms, void* normed, void* packed_codes,
+                                        void* packed_scales, int zero_policy, void* stream);
 int fpq_silu_mul_quantize_mx_packed(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
                                     int64_t rows, int64_t cols, int rot_kind, int g, float norm,
                                     void* product, void* packed_codes, void* packed_scales, int zero_policy,

@@ -356,6 +356,31 @@ def fused_quantize_packed(kind, a, b, g=128, rot="hadamard", norm=None, eps=1e-5
     return pc.cpu(), ps.cpu(), (out.cpu() if out is not None else None)
 
 
+def rmsnorm_rows_quantize_packed(x, w, g=128, rot="hadamard", norm=None, eps=1e-5, want_out=True, want_inv=True,
+                                 ld=None, zero_policy=_engine.ZERO_REFERENCE, fill=0xCD):
+    """fpq_rmsnorm_rows_quantize_mx_packed (row statistic + RMSNorm + rotate + quantize of a few rows in one
+    launch).  Returns CPU (packed codes, packed scales, normed or None, inv_rms or None)."""
+    lib = _engine.lib()
+    rows, cols = x.shape
+    ld = cols if ld is None else ld
+    x_dev = _strided(x, ld)
+    cb, sb = packed_sizes(rows, cols)
+    pc = torch.full((cb,), fill, dtype=torch.uint8, device="cuda")
+    ps = torch.full((sb,), fill, dtype=torch.uint8, device="cuda")
+    out = torch.full((rows, cols), float("nan"), dtype=torch.bfloat16, device="cuda") if want_out else None
+    inv = torch.full((rows,), float("nan"), dtype=torch.float32, device="cuda") if want_inv else None
+    if norm is None:
+        norm = float(torch.tensor(g ** -0.5, dtype=torch.bfloat16))
+    wd = w.to("cuda").contiguous()
+    st = lib.fpq_rmsnorm_rows_quantize_mx_packed(x_dev.data_ptr(), ld, wd.data_ptr(), rows, cols, eps, ROT[rot], g, norm,
+                                                 inv.data_ptr() if inv is not None else None,
+                                                 out.data_ptr() if out is not None else None, pc.data_ptr(),
+                                                 ps.data_ptr(), zero_policy, torch.cuda.current_stream().cuda_stream)
+    _engine.check(st, "fpq_rmsnorm_rows_quantize_mx_packed")
+    torch.cuda.synchronize()
+    return pc.cpu(), ps.cpu(), (out.cpu() if out is not None else None), (inv.cpu() if inv is not None else None)
+
+
 def quantize_nv_packed(x_bf16, global_scale, rot="hadamard", g=16, norm=None, zero_policy=_engine.ZERO_REFERENCE,
                        fill=0xCD):
     """Run fpq_quantize_nv_packed; returns CPU uint8 (packed codes, packed scales)."""

@@ -113,6 +113,51 @@ def test_fused_quantize_packed_bit_exact(kind, rot, g, rows, cols):
     assert none is None and torch.equal(pc2, want_c) and torch.equal(ps2, want_s)
 
 
+@pytest.mark.parametrize("rot,g", PACKED_CASES)
+@pytest.mark.parametrize("rows,cols", [(1, 256), (1, 4096), (5, 768), (33, 4096), (64, 1024), (20, 16384)])
+def test_rmsnorm_rows_in_one_launch_bit_exact(rot, g, rows, cols):
+    """fpq_rmsnorm_rows_quantize_mx_packed: the row statistic, the normalised bf16 tensor and the packed codes
+    and scales of the oracle (and so of fpq_row_inv_rms + fpq_rmsnorm_quantize_mx_packed), zero padding rows,
+    a strided input, both optional outputs absent."""
+    from tests.test_packed_gpu import pack_by_definition
+    x = make_student_t(rows, cols, seed=rows + g) * 2
+    gen = torch.Generator().manual_seed(cols)
+    w = (1 + 0.3 * torch.randn(cols, generator=gen)).to(torch.bfloat16)
+    if rows > 4:
+        w[64:96] = 0.0
+        x[3] *= 2.0 ** -60
+        x[4] = 0.0                                    # an all-zero row: 1 / sqrt(eps)
+    want_v = O.rmsnorm(x, w, 1e-5)
+    okind = O.ROT_HADAMARD if rot == "hadamard" else O.ROT_IDENTITY
+    wc, ws, _ = O.quantize_mx(want_v, okind, g, float(O.hadamard_matrix(g)[0, 0]))
+    want_c, want_s = pack_by_definition(wc, ws, cols)
+    ld = cols + 64 if rows in (5, 33) else None
+    pc, ps, out, inv = capi.rmsnorm_rows_quantize_packed(x, w, g=g, rot=rot, ld=ld)
+    assert torch.equal(inv, O.row_inv_rms(x, 1e-5))
+    assert torch.equal(out.view(torch.int16), want_v.view(torch.int16))
+    assert torch.equal(pc, want_c) and torch.equal(ps, want_s)
+    pc2, ps2, none, none2 = capi.rmsnorm_rows_quantize_packed(x, w, g=g, rot=rot, want_out=False, want_inv=False)
+    assert none is None and none2 is None and torch.equal(pc2, want_c) and torch.equal(ps2, want_s)
+
+
+def test_rmsnorm_rows_limits():
+    from fp_quant import _engine
+    lib = _engine.lib()
+    assert lib.fpq_rmsnorm_rows_max_rows() == 64
+    x = torch.zeros(65, 256, dtype=torch.bfloat16, device="cuda")
+    w = torch.ones(256, dtype=torch.bfloat16, device="cuda")
+    pc = torch.zeros(96 * 128, dtype=torch.uint8, device="cuda")
+    ps = torch.zeros(96 * 8, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    args = (x.data_ptr(), 256, w.data_ptr())
+    tail = (1e-5, 1, 32, 0.177, None, None, pc.data_ptr(), ps.data_ptr(), 0, st)
+    assert lib.fpq_rmsnorm_rows_quantize_mx_packed(*args, 65, 256, *tail) == _engine.E_LIMIT
+    assert lib.fpq_rmsnorm_rows_quantize_mx_packed(*args, 4, 200, *tail) == -2
+    assert lib.fpq_rmsnorm_rows_quantize_mx_packed(*args, 4, 256, 1e-5, _engine.ROT_GSR, 32, 0.177, None, None,
+                                                   pc.data_ptr(), ps.data_ptr(), 0, st) == _engine.E_UNSUPPORTED
+    assert lib.fpq_rmsnorm_rows_quantize_mx_packed(*args, 0, 256, *tail) == 0
+
+
 def test_fused_quantize_packed_full_size_matches_generic_kernel():
     """A down_proj-sized input: the streaming fused kernel equals the generic fused kernel re-tiled."""
     from tests.test_packed_gpu import pack_by_definition
