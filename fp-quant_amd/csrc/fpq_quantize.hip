@@ -1294,15 +1294,19 @@ static int dispatch_prologue(const void* x, int64_t ld_first, const void* second
 }
 
 // The same with the packed operand layout as output (streaming kernel; cols % 256 == 0).
-template <int PRO>
+// FMT = kFmtNv: the generic kernel only, i.e. at most kPackedFewRows rows (FPQ_E_UNSUPPORTED beyond: the
+// caller quantizes row-major and re-tiles)
+template <int PRO, int FMT = kFmtMx>
 static int dispatch_prologue_packed(const void* x, int64_t ld_first, const void* second, int64_t ld_second,
                                     const float* row_scale, const void* col_scale, void* out, int64_t rows,
                                     int64_t cols, int rot_kind, int g, float norm, void* codes, void* scales,
-                                    int zero_policy, void* stream_) {
+                                    int zero_policy, void* stream_, const float* gsp = nullptr) {
   hipStream_t stream = (hipStream_t)stream_;
   if (rows < 0 || cols < 0) return FPQ_E_SHAPE;
   if (rows == 0 || cols == 0) return FPQ_OK;
   if (!x || !codes || !scales) return FPQ_E_NULL;
+  if (FMT == kFmtNv && !gsp) return FPQ_E_NULL;
+  if (FMT == kFmtNv && rows > kPackedFewRows) return FPQ_E_UNSUPPORTED;
   if (PRO == kProRmsNorm && (!row_scale || !col_scale)) return FPQ_E_NULL;
   if (PRO == kProSiluMul && !second) return FPQ_E_NULL;
   if (zero_policy != FPQ_ZERO_REFERENCE && zero_policy != FPQ_ZERO_SIGNED) return FPQ_E_POLICY;
@@ -1320,7 +1324,7 @@ static int dispatch_prologue_packed(const void* x, int64_t ld_first, const void*
   }
   if (((uintptr_t)x & 15u) || ((uintptr_t)second & 15u) || ((uintptr_t)col_scale & 15u) ||
       ((uintptr_t)out & 15u) || ((uintptr_t)row_scale & 3u) || ((uintptr_t)codes & 15u) ||
-      ((uintptr_t)scales & 3u)) {
+      ((uintptr_t)scales & (FMT == kFmtNv ? 7u : 3u)) || ((uintptr_t)gsp & 3u)) {
     return FPQ_E_ALIGN;
   }
   if (PRO == kProSiluMul) {
@@ -1340,9 +1344,11 @@ static int dispatch_prologue_packed(const void* x, int64_t ld_first, const void*
 #define FPQ_LAUNCH_PRO_PACKED(GG, RR)                                                                          \
   {                                                                                                            \
     if (few)                                                                                                   \
-      return launch_lane8_prologue<GG, kFmtMx, RR, PRO>(x, rows, cols, norm, nullptr, codes, scales, rows,     \
-                                                        cols / 32, zero_policy, stream, pro);                  \
-    return launch_stream_packed<GG, RR, PRO>(x, rows, cols, norm, codes, scales, zero_policy, stream, pro);    \
+      return launch_lane8_prologue<GG, FMT, RR, PRO>(x, rows, cols, norm, gsp, codes, scales, rows,            \
+                                                     cols / (FMT == kFmtNv ? 16 : 32), zero_policy, stream, pro); \
+    if constexpr (FMT == kFmtMx)                                                                               \
+      return launch_stream_packed<GG, RR, PRO>(x, rows, cols, norm, codes, scales, zero_policy, stream, pro);  \
+    return FPQ_E_UNSUPPORTED;                                                                                  \
   }
   if (rot_kind == FPQ_ROT_IDENTITY) FPQ_LAUNCH_PRO_PACKED(32, FPQ_ROT_IDENTITY);
   switch (g) {
@@ -1383,19 +1389,21 @@ __global__ __launch_bounds__(256) void row_inv_rms_kernel(const uint4* __restric
 // them in that kernel's order) and quantizes the row with the generic kernel's arithmetic into the
 // packed operand layout.  Workgroups past `rows` (the padding of the last 32-row tile) write zeros.
 constexpr uint32_t kRowsKernelMaxChunks = 2048;   // cols <= 16384
-template <int G, int ROT, int ZERO>
-__global__ __launch_bounds__(256) void rmsnorm_rows_quantize_kernel(const uint4* __restrict__ x,
+template <int G, int FMT, int ROT, int ZERO>
+__global__ __launch_bounds__(1024) void rmsnorm_rows_quantize_kernel(const uint4* __restrict__ x,
                                                                     uint32_t* __restrict__ codes,
                                                                     uint8_t* __restrict__ scales, uint32_t rows,
                                                                     float norm, float cols_f, float eps,
-                                                                    float* __restrict__ inv_rms_out, Prologue pro) {
+                                                                    float* __restrict__ inv_rms_out,
+                                                                    const float* __restrict__ global_scale,
+                                                                    Prologue pro) {
   __shared__ float oct[kRowsKernelMaxChunks];
   __shared__ float inv_shared;
-  const uint32_t row = blockIdx.x, cpr = pro.chunks_per_row, lane = threadIdx.x & 63u;
+  const uint32_t row = blockIdx.x, cpr = pro.chunks_per_row, lane = threadIdx.x & 63u, nthr = blockDim.x;
   const bool real = row < rows;
   if (real) {
     const uint4* src = x + (size_t)row * pro.ld_first;
-    for (uint32_t c = threadIdx.x; c < cpr; c += 256u) {
+    for (uint32_t c = threadIdx.x; c < cpr; c += nthr) {
       float p[8];
       unpack8(src[c], p);
       float s = p[0] * p[0];
@@ -1418,13 +1426,18 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_quantize_kernel(const uint4*
   }
   __syncthreads();
   const float rs = real ? inv_shared : 0.0f;
-  for (uint32_t c0 = 0; c0 < cpr; c0 += 256u) {   // the same trip count for every thread: lanes exchange values
+  float gs = 1.0f, rg = 1.0f;
+  if (FMT == kFmtNv) {
+    gs = *global_scale;
+    rg = gs == 0.0f ? 0.0f : 1.0f / gs;
+  }
+  for (uint32_t c0 = 0; c0 < cpr; c0 += nthr) {   // the same trip count for every thread: lanes exchange values
     const uint32_t cc = c0 + threadIdx.x;
     const bool in = cc < cpr;
     // a chunk index past the packed output makes the generic kernel skip the store
     const uint32_t chunk = in ? row * cpr + cc : 0xffffffffu;
-    lane8_process<G, kFmtMx, ROT, ZERO, false, kProRmsNorm>(x, codes, scales, chunk, real && in, lane, cpr, 0u, norm,
-                                                            1.0f, 1.0f, nullptr, nullptr, nullptr, pro, rs);
+    lane8_process<G, FMT, ROT, ZERO, false, kProRmsNorm>(x, codes, scales, chunk, real && in, lane, cpr, 0u, norm, gs,
+                                                         rg, nullptr, nullptr, nullptr, pro, rs);
   }
 }
 
@@ -1620,13 +1633,15 @@ extern "C" int fpq_rmsnorm_quantize_mx_packed(const void* x, int64_t ld, const f
 }
 
 namespace fpq {
+template <int FMT>
 static int dispatch_rmsnorm_rows(const void* x, int64_t ld, const void* weight, int64_t rows, int64_t cols, float eps,
                                  int rot_kind, int g, float norm, float* inv_rms, void* normed, void* codes,
-                                 void* scales, int zero_policy, void* stream_) {
+                                 void* scales, int zero_policy, void* stream_, const float* gsp = nullptr) {
   hipStream_t stream = (hipStream_t)stream_;
   if (rows < 0 || cols < 0) return FPQ_E_SHAPE;
   if (rows == 0 || cols == 0) return FPQ_OK;
   if (!x || !weight || !codes || !scales) return FPQ_E_NULL;
+  if (FMT == kFmtNv && !gsp) return FPQ_E_NULL;
   if (zero_policy != FPQ_ZERO_REFERENCE && zero_policy != FPQ_ZERO_SIGNED) return FPQ_E_POLICY;
   if (rot_kind == FPQ_ROT_IDENTITY) g = 32;
   if (rot_kind != FPQ_ROT_IDENTITY && rot_kind != FPQ_ROT_HADAMARD) {
@@ -1636,7 +1651,7 @@ static int dispatch_rmsnorm_rows(const void* x, int64_t ld, const void* weight, 
   if (cols % 256 != 0 || ld < cols || ld % 8 != 0 || ld >= (int64_t)1 << 24) return FPQ_E_SHAPE;
   if (rows > kPackedFewRows || cols / 8 > (int64_t)kRowsKernelMaxChunks) return FPQ_E_LIMIT;
   if (((uintptr_t)x & 15u) || ((uintptr_t)weight & 15u) || ((uintptr_t)normed & 15u) || ((uintptr_t)inv_rms & 3u) ||
-      ((uintptr_t)codes & 15u) || ((uintptr_t)scales & 3u)) {
+      ((uintptr_t)codes & 15u) || ((uintptr_t)scales & (FMT == kFmtNv ? 7u : 3u)) || ((uintptr_t)gsp & 3u)) {
     return FPQ_E_ALIGN;
   }
   Prologue pro{};
@@ -1645,17 +1660,18 @@ static int dispatch_rmsnorm_rows(const void* x, int64_t ld, const void* weight, 
   pro.chunks_per_row = (uint32_t)(cols / 8);
   pro.ld_first = (uint32_t)(ld / 8);
   pro.packed_rows = (uint32_t)((rows + 31) / 32 * 32);
-  const dim3 grid(pro.packed_rows), block(256);
+  // a row is one workgroup's work: wider rows get more waves (the row statistic does not depend on the count)
+  const dim3 grid(pro.packed_rows), block(pro.chunks_per_row >= 1024u ? 1024 : pro.chunks_per_row >= 512u ? 512 : 256);
 #define FPQ_LAUNCH_ROWS(GG, RR)                                                                                 \
   {                                                                                                             \
     if (zero_policy == FPQ_ZERO_REFERENCE)                                                                      \
-      hipLaunchKernelGGL((rmsnorm_rows_quantize_kernel<GG, RR, kZeroReference>), grid, block, 0, stream,        \
+      hipLaunchKernelGGL((rmsnorm_rows_quantize_kernel<GG, FMT, RR, kZeroReference>), grid, block, 0, stream,   \
                          (const uint4*)x, (uint32_t*)codes, (uint8_t*)scales, (uint32_t)rows, norm, (float)cols, \
-                         eps, inv_rms, pro);                                                                    \
+                         eps, inv_rms, gsp, pro);                                                               \
     else                                                                                                        \
-      hipLaunchKernelGGL((rmsnorm_rows_quantize_kernel<GG, RR, kZeroSigned>), grid, block, 0, stream,           \
+      hipLaunchKernelGGL((rmsnorm_rows_quantize_kernel<GG, FMT, RR, kZeroSigned>), grid, block, 0, stream,      \
                          (const uint4*)x, (uint32_t*)codes, (uint8_t*)scales, (uint32_t)rows, norm, (float)cols, \
-                         eps, inv_rms, pro);                                                                    \
+                         eps, inv_rms, gsp, pro);                                                               \
     return (int)hipGetLastError();                                                                              \
   }
   if (rot_kind == FPQ_ROT_IDENTITY) FPQ_LAUNCH_ROWS(32, FPQ_ROT_IDENTITY);
@@ -1676,8 +1692,36 @@ extern "C" int fpq_rmsnorm_rows_quantize_mx_packed(const void* x, int64_t ld, co
                                                    int64_t cols, float eps, int rot_kind, int g, float norm,
                                                    float* inv_rms, void* normed, void* packed_codes,
                                                    void* packed_scales, int zero_policy, void* stream) {
-  return fpq::dispatch_rmsnorm_rows(x, ld, weight, rows, cols, eps, rot_kind, g, norm, inv_rms, normed, packed_codes,
-                                    packed_scales, zero_policy, stream);
+  return fpq::dispatch_rmsnorm_rows<fpq::kFmtMx>(x, ld, weight, rows, cols, eps, rot_kind, g, norm, inv_rms, normed,
+                                                 packed_codes, packed_scales, zero_policy, stream);
+}
+
+extern "C" int fpq_rmsnorm_rows_quantize_nv_packed(const void* x, int64_t ld, const void* weight, int64_t rows,
+                                                   int64_t cols, float eps, int rot_kind, int g, float norm,
+                                                   const float* global_scale, float* inv_rms, void* normed,
+                                                   void* packed_codes, void* packed_scales, int zero_policy,
+                                                   void* stream) {
+  return fpq::dispatch_rmsnorm_rows<fpq::kFmtNv>(x, ld, weight, rows, cols, eps, rot_kind, g, norm, inv_rms, normed,
+                                                 packed_codes, packed_scales, zero_policy, stream, global_scale);
+}
+
+extern "C" int fpq_rmsnorm_quantize_nv_packed(const void* x, int64_t ld, const float* inv_rms, const void* weight,
+                                              int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                                              const float* global_scale, void* normed, void* packed_codes,
+                                              void* packed_scales, int zero_policy, void* stream) {
+  return fpq::dispatch_prologue_packed<fpq::kProRmsNorm, fpq::kFmtNv>(x, ld, nullptr, 0, inv_rms, weight, normed, rows,
+                                                                      cols, rot_kind, g, norm, packed_codes,
+                                                                      packed_scales, zero_policy, stream, global_scale);
+}
+
+extern "C" int fpq_silu_mul_quantize_nv_packed(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                                               int64_t rows, int64_t cols, int rot_kind, int g, float norm,
+                                               const float* global_scale, void* product, void* packed_codes,
+                                               void* packed_scales, int zero_policy, void* stream) {
+  return fpq::dispatch_prologue_packed<fpq::kProSiluMul, fpq::kFmtNv>(gate, ld_gate, up, ld_up, nullptr, nullptr,
+                                                                      product, rows, cols, rot_kind, g, norm,
+                                                                      packed_codes, packed_scales, zero_policy,
+                                                                      stream, global_scale);
 }
 
 extern "C" int fpq_silu_mul_quantize_mx_packed(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,

@@ -31,6 +31,7 @@ from .hip_ops import (
     packed_weight_ready,
     packed_weights_enabled,
     quantize_mx_packed,
+    unpack_fp4,
     weight_rows,
 )
 
@@ -93,9 +94,16 @@ class QuantizedActivations:
         self.mx_packed = self.row_major = self.nv_packed = None
 
     def serves(self, want_packed: bool) -> bool:
-        """Whether a GEMM on packed (or on row-major) operands can run from what is held: the packed
-        form can be made from the row-major one, not the other way round."""
-        return want_packed or self.row_major is not None
+        """Whether a GEMM on packed (or on row-major) operands can run from what is held: either form
+        is made from the other on demand (a re-tiling pass over the 4-bit codes, exact both ways)."""
+        return self.row_major is not None or self.mx_packed is not None or self.nv_packed is not None
+
+    def rows(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Row-major codes [m, k/2] and scales (unpacked from the packed form if that is all there is)."""
+        if self.row_major is None:
+            pc, ps = self.nv_packed if self.nvfp4 else self.mx_packed
+            self.row_major = unpack_fp4(pc, ps, self.m, self.k, self.nvfp4)
+        return self.row_major
 
     def packed(self) -> Tuple[torch.Tensor, torch.Tensor]:
         """Codes and scales in the packed GEMM layout (re-tiled from the row-major ones if need be)."""
@@ -259,8 +267,6 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
         raise ValueError("residual must be on the weights' device")
     if use_packed is None:
         use_packed = wants_packed(m, n, k, qa.nvfp4)
-    if not qa.serves(use_packed):
-        raise ValueError("these activations were quantized into the packed layout only")
     if qa.nvfp4:
         if use_packed:
             xp, xsp = qa.packed()
@@ -270,7 +276,7 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
                                           alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
             _engine.check(st, "fpq_gemm_nvf4_packed")
         else:
-            codes, scales = qa.row_major
+            codes, scales = qa.rows()
             st = lib.fpq_gemm_nvf4(codes.data_ptr(), scales.data_ptr(), scales.shape[-1], wq.data_ptr(),
                                    ws.data_ptr(), ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
             _engine.check(st, "fpq_gemm_nvf4")
@@ -290,7 +296,7 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
                                           alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
         _engine.check(st, "fpq_gemm_mxf4_packed")
         return y
-    codes, scales = qa.row_major
+    codes, scales = qa.rows()
     st = lib.fpq_gemm_mxf4(codes.data_ptr(), scales.data_ptr(), scales.shape[-1], wq.data_ptr(), ws.data_ptr(),
                            ws.shape[-1], alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
     _engine.check(st, "fpq_gemm_mxf4")
@@ -665,6 +671,20 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
         qa = QuantizedActivations(rows, cols, nvfp4)
         qa.mx_packed = (pc, ps)
         return qa
+    if (allow_packed and nvfp4 and rows <= _ROWS_KERNEL_MAX_ROWS and cols % 256 == 0
+            and nv_packed_eligible(rows, 32, cols, fused_linear=True)):
+        # a decode step's few rows straight into the packed NVFP4 layout (generic kernel)
+        gs = as_f32_scalar(act_global_scale, remember)
+        pc = torch.empty(lib.fpq_packed_codes_bytes(rows, cols), dtype=torch.uint8, device=dev)
+        ps = torch.empty(lib.fpq_packed_scales_bytes_nv(rows, cols), dtype=torch.uint8, device=dev)
+        st = getattr(lib, f"fpq_{entry}_quantize_nv_packed")(*head, rows, cols, kind, h.shape[0], norm, gs.data_ptr(),
+                                                             optr, pc.data_ptr(), ps.data_ptr(), ZERO_NIBBLE_POLICY,
+                                                             stream)
+        if st != _engine.E_UNSUPPORTED:
+            _engine.check(st, f"fpq_{entry}_quantize_nv_packed")
+            qa = QuantizedActivations(rows, cols, nvfp4)
+            qa.nv_packed = (pc, ps)
+            return qa
     codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=dev)
     scales = torch.empty(rows, cols // group, dtype=torch.uint8, device=dev)
     tail = (optr, codes.data_ptr(), scales.data_ptr(), rows, cols // group, ZERO_NIBBLE_POLICY, stream)
@@ -707,17 +727,26 @@ def rmsnorm_quantize(x: torch.Tensor, weight: torch.Tensor, eps: float, hadamard
         y = torch.empty_like(x_flat)
         w = weight.contiguous()
         qa = None
-        if (not nvfp4 and rows <= _ROWS_KERNEL_MAX_ROWS and cols % 256 == 0 and cols <= 16384
-                and packed_linear_eligible(rows, cols, "abs_max")):
+        if (rows <= _ROWS_KERNEL_MAX_ROWS and cols % 256 == 0 and cols <= 16384
+                and (nv_packed_eligible(rows, 32, cols, fused_linear=True) if nvfp4
+                     else packed_linear_eligible(rows, cols, "abs_max"))):
             # a decode step's few rows: statistic, normalisation and quantization in one launch
             pc = torch.empty(lib.fpq_packed_codes_bytes(rows, cols), dtype=torch.uint8, device=dev)
-            ps = torch.empty(lib.fpq_packed_scales_bytes(rows, cols), dtype=torch.uint8, device=dev)
-            st = lib.fpq_rmsnorm_rows_quantize_mx_packed(x_flat.data_ptr(), cols, w.data_ptr(), rows, cols, eps, kind,
-                                                         h.shape[0], norm, None, y.data_ptr(), pc.data_ptr(),
-                                                         ps.data_ptr(), ZERO_NIBBLE_POLICY, stream)
-            _engine.check(st, "fpq_rmsnorm_rows_quantize_mx_packed")
             qa = QuantizedActivations(rows, cols, nvfp4)
-            qa.mx_packed = (pc, ps)
+            if nvfp4:
+                ps = torch.empty(lib.fpq_packed_scales_bytes_nv(rows, cols), dtype=torch.uint8, device=dev)
+                gs = as_f32_scalar(act_global_scale)
+                st = lib.fpq_rmsnorm_rows_quantize_nv_packed(x_flat.data_ptr(), cols, w.data_ptr(), rows, cols, eps,
+                                                             kind, h.shape[0], norm, gs.data_ptr(), None, y.data_ptr(),
+                                                             pc.data_ptr(), ps.data_ptr(), ZERO_NIBBLE_POLICY, stream)
+                qa.nv_packed = (pc, ps)
+            else:
+                ps = torch.empty(lib.fpq_packed_scales_bytes(rows, cols), dtype=torch.uint8, device=dev)
+                st = lib.fpq_rmsnorm_rows_quantize_mx_packed(x_flat.data_ptr(), cols, w.data_ptr(), rows, cols, eps,
+                                                             kind, h.shape[0], norm, None, y.data_ptr(), pc.data_ptr(),
+                                                             ps.data_ptr(), ZERO_NIBBLE_POLICY, stream)
+                qa.mx_packed = (pc, ps)
+            _engine.check(st, "fpq_rmsnorm_rows_quantize_packed")
         if qa is None:
             inv = torch.empty(rows, dtype=torch.float32, device=dev)
             _engine.check(lib.fpq_row_inv_rms(x_flat.data_ptr(), cols, rows, cols, eps, inv.data_ptr(), stream),

@@ -325,15 +325,18 @@ def fused_quantize(kind, fmt, a, b, g=128, rot="hadamard", norm=None, global_sca
 
 
 def fused_quantize_packed(kind, a, b, g=128, rot="hadamard", norm=None, eps=1e-5, want_out=True, ld_a=None,
-                          ld_b=None, zero_policy=_engine.ZERO_REFERENCE, fill=0xCD):
-    """fused_quantize for MXFP4 with the packed operand layout as output.  Returns CPU
-    (packed codes, packed scales, out or None)."""
+                          ld_b=None, zero_policy=_engine.ZERO_REFERENCE, fill=0xCD, global_scale=None):
+    """fused_quantize with the packed operand layout as output (NVFP4 when `global_scale` is given: a few
+    rows only).  Returns CPU (packed codes, packed scales, out or None)."""
     lib = _engine.lib()
     rows, cols = a.shape
     ld_a = cols if ld_a is None else ld_a
     ld_b = cols if ld_b is None else ld_b
     a_dev = _strided(a, ld_a)
     cb, sb = packed_sizes(rows, cols)
+    if global_scale is not None:
+        sb = lib.fpq_packed_scales_bytes_nv(rows, cols)
+        gs = torch.tensor([global_scale], dtype=torch.float32, device="cuda")
     pc = torch.full((cb,), fill, dtype=torch.uint8, device="cuda")
     ps = torch.full((sb,), fill, dtype=torch.uint8, device="cuda")
     out = torch.full((rows, cols), float("nan"), dtype=torch.bfloat16, device="cuda") if want_out else None
@@ -345,26 +348,33 @@ def fused_quantize_packed(kind, a, b, g=128, rot="hadamard", norm=None, eps=1e-5
         w = b.to("cuda").contiguous()
         inv = torch.empty(rows, dtype=torch.float32, device="cuda")
         _engine.check(lib.fpq_row_inv_rms(a_dev.data_ptr(), ld_a, rows, cols, eps, inv.data_ptr(), stream), "fpq_row_inv_rms")
-        st = lib.fpq_rmsnorm_quantize_mx_packed(a_dev.data_ptr(), ld_a, inv.data_ptr(), w.data_ptr(), rows, cols,
-                                                ROT[rot], g, norm, optr, pc.data_ptr(), ps.data_ptr(), zero_policy, stream)
+        head = (a_dev.data_ptr(), ld_a, inv.data_ptr(), w.data_ptr(), rows, cols, ROT[rot], g, norm)
     else:
         b_dev = _strided(b, ld_b)
-        st = lib.fpq_silu_mul_quantize_mx_packed(a_dev.data_ptr(), ld_a, b_dev.data_ptr(), ld_b, rows, cols, ROT[rot],
-                                                 g, norm, optr, pc.data_ptr(), ps.data_ptr(), zero_policy, stream)
-    _engine.check(st, f"fpq_{kind}_quantize_mx_packed")
+        head = (a_dev.data_ptr(), ld_a, b_dev.data_ptr(), ld_b, rows, cols, ROT[rot], g, norm)
+    tail = (optr, pc.data_ptr(), ps.data_ptr(), zero_policy, stream)
+    if global_scale is not None:
+        st = getattr(lib, f"fpq_{kind}_quantize_nv_packed")(*head, gs.data_ptr(), *tail)
+    else:
+        st = getattr(lib, f"fpq_{kind}_quantize_mx_packed")(*head, *tail)
+    _engine.check(st, f"fpq_{kind}_quantize_packed")
     torch.cuda.synchronize()
     return pc.cpu(), ps.cpu(), (out.cpu() if out is not None else None)
 
 
 def rmsnorm_rows_quantize_packed(x, w, g=128, rot="hadamard", norm=None, eps=1e-5, want_out=True, want_inv=True,
-                                 ld=None, zero_policy=_engine.ZERO_REFERENCE, fill=0xCD):
-    """fpq_rmsnorm_rows_quantize_mx_packed (row statistic + RMSNorm + rotate + quantize of a few rows in one
-    launch).  Returns CPU (packed codes, packed scales, normed or None, inv_rms or None)."""
+                                 ld=None, zero_policy=_engine.ZERO_REFERENCE, fill=0xCD, global_scale=None):
+    """fpq_rmsnorm_rows_quantize_{mx,nv}_packed (row statistic + RMSNorm + rotate + quantize of a few rows in
+    one launch; NVFP4 when `global_scale` is given).  Returns CPU (packed codes, packed scales, normed or None,
+    inv_rms or None)."""
     lib = _engine.lib()
     rows, cols = x.shape
     ld = cols if ld is None else ld
     x_dev = _strided(x, ld)
     cb, sb = packed_sizes(rows, cols)
+    if global_scale is not None:
+        sb = lib.fpq_packed_scales_bytes_nv(rows, cols)
+        gs = torch.tensor([global_scale], dtype=torch.float32, device="cuda")
     pc = torch.full((cb,), fill, dtype=torch.uint8, device="cuda")
     ps = torch.full((sb,), fill, dtype=torch.uint8, device="cuda")
     out = torch.full((rows, cols), float("nan"), dtype=torch.bfloat16, device="cuda") if want_out else None
@@ -372,11 +382,14 @@ def rmsnorm_rows_quantize_packed(x, w, g=128, rot="hadamard", norm=None, eps=1e-
     if norm is None:
         norm = float(torch.tensor(g ** -0.5, dtype=torch.bfloat16))
     wd = w.to("cuda").contiguous()
-    st = lib.fpq_rmsnorm_rows_quantize_mx_packed(x_dev.data_ptr(), ld, wd.data_ptr(), rows, cols, eps, ROT[rot], g, norm,
-                                                 inv.data_ptr() if inv is not None else None,
-                                                 out.data_ptr() if out is not None else None, pc.data_ptr(),
-                                                 ps.data_ptr(), zero_policy, torch.cuda.current_stream().cuda_stream)
-    _engine.check(st, "fpq_rmsnorm_rows_quantize_mx_packed")
+    head = (x_dev.data_ptr(), ld, wd.data_ptr(), rows, cols, eps, ROT[rot], g, norm)
+    tail = (inv.data_ptr() if inv is not None else None, out.data_ptr() if out is not None else None, pc.data_ptr(),
+            ps.data_ptr(), zero_policy, torch.cuda.current_stream().cuda_stream)
+    if global_scale is not None:
+        st = lib.fpq_rmsnorm_rows_quantize_nv_packed(*head, gs.data_ptr(), *tail)
+    else:
+        st = lib.fpq_rmsnorm_rows_quantize_mx_packed(*head, *tail)
+    _engine.check(st, "fpq_rmsnorm_rows_quantize_packed")
     torch.cuda.synchronize()
     return pc.cpu(), ps.cpu(), (out.cpu() if out is not None else None), (inv.cpu() if inv is not None else None)
 

@@ -140,6 +140,85 @@ def test_rmsnorm_rows_in_one_launch_bit_exact(rot, g, rows, cols):
     assert none is None and none2 is None and torch.equal(pc2, want_c) and torch.equal(ps2, want_s)
 
 
+NV_PACKED_CASES = [("hadamard", 16), ("hadamard", 32), ("hadamard", 128), ("identity", 16)]
+
+
+@pytest.mark.parametrize("rot,g", NV_PACKED_CASES)
+@pytest.mark.parametrize("rows,cols", [(1, 256), (1, 4096), (5, 768), (33, 4096), (64, 1024)])
+def test_rmsnorm_rows_in_one_launch_nvfp4_bit_exact(rot, g, rows, cols):
+    """fpq_rmsnorm_rows_quantize_nv_packed: as the MXFP4 entry, with E4M3 scales under a global scale."""
+    from tests.test_packed_gpu import pack_nv_by_definition
+    x = make_student_t(rows, cols, seed=rows + g) * 2
+    gen = torch.Generator().manual_seed(cols)
+    w = (1 + 0.3 * torch.randn(cols, generator=gen)).to(torch.bfloat16)
+    if rows > 4:
+        w[64:96] = 0.0
+        x[3] *= 2.0 ** -60
+        x[4] = 0.0
+    want_v = O.rmsnorm(x, w, 1e-5)
+    wc, ws = _oracle_quantize(want_v, "nvfp4", rot, g, 777.0)
+    want_c, want_s = pack_nv_by_definition(wc, ws, cols)
+    ld = cols + 64 if rows in (5, 33) else None
+    pc, ps, out, inv = capi.rmsnorm_rows_quantize_packed(x, w, g=g, rot=rot, ld=ld, global_scale=777.0)
+    assert torch.equal(inv, O.row_inv_rms(x, 1e-5))
+    assert torch.equal(out.view(torch.int16), want_v.view(torch.int16))
+    assert torch.equal(pc, want_c) and torch.equal(ps, want_s)
+    pc2, ps2, none, none2 = capi.rmsnorm_rows_quantize_packed(x, w, g=g, rot=rot, want_out=False, want_inv=False,
+                                                              global_scale=777.0)
+    assert none is None and none2 is None and torch.equal(pc2, want_c) and torch.equal(ps2, want_s)
+
+
+@pytest.mark.parametrize("rot,g", NV_PACKED_CASES)
+@pytest.mark.parametrize("kind", ["rmsnorm", "silu_mul"])
+@pytest.mark.parametrize("rows,cols", [(1, 256), (20, 768), (64, 512)])
+def test_fused_quantize_packed_nvfp4_bit_exact(kind, rot, g, rows, cols):
+    """The NVFP4 fused producers writing the packed layout (a few rows): codes, E4M3 scales and the bf16
+    by-product of the oracle; more rows than the entry serves are refused, not mis-served."""
+    from fp_quant import _engine
+    from tests.test_packed_gpu import pack_nv_by_definition
+    a = make_student_t(rows, cols, seed=rows + g) * 2
+    if kind == "rmsnorm":
+        gen = torch.Generator().manual_seed(cols)
+        b = (1 + 0.3 * torch.randn(cols, generator=gen)).to(torch.bfloat16)
+        if rows > 8:
+            b[64:96] = 0.0
+            a[5] *= 2.0 ** -60
+        want_v = O.rmsnorm(a, b, 1e-5)
+    else:
+        b = make_outlier_normal(rows, cols, seed=cols + g)
+        a[0, :8] = torch.tensor([-300.0, 300.0, 0.0, -0.0, -88.5, 88.5, -20.0, 1e-30]).to(torch.bfloat16)
+        if rows > 8:
+            b[3, 64:96] = 0.0
+            b[7] *= 2.0 ** -110
+            b[9] *= 2.0 ** 100
+        want_v = O.silu_mul(a, b)
+    wc, ws = _oracle_quantize(want_v, "nvfp4", rot, g, 777.0)
+    want_c, want_s = pack_nv_by_definition(wc, ws, cols)
+    lds = dict(ld_a=cols + 64, ld_b=2 * cols) if rows == 20 else {}
+    pc, ps, out = capi.fused_quantize_packed(kind, a, b, g=g, rot=rot, global_scale=777.0, **lds)
+    assert torch.equal(out.view(torch.int16), want_v.view(torch.int16))
+    assert torch.equal(pc, want_c) and torch.equal(ps, want_s)
+    pc2, ps2, none = capi.fused_quantize_packed(kind, a, b, g=g, rot=rot, want_out=False, global_scale=777.0)
+    assert none is None and torch.equal(pc2, want_c) and torch.equal(ps2, want_s)
+
+
+def test_fused_quantize_packed_nvfp4_refuses_many_rows():
+    from fp_quant import _engine
+    lib = _engine.lib()
+    rows, cols = 300, 256
+    x = torch.zeros(rows, cols, dtype=torch.bfloat16, device="cuda")
+    gs = torch.ones(1, dtype=torch.float32, device="cuda")
+    pc = torch.zeros(lib.fpq_packed_codes_bytes(rows, cols), dtype=torch.uint8, device="cuda")
+    ps = torch.zeros(lib.fpq_packed_scales_bytes_nv(rows, cols), dtype=torch.uint8, device="cuda")
+    st = lib.fpq_silu_mul_quantize_nv_packed(x.data_ptr(), cols, x.data_ptr(), cols, rows, cols, 1, 16, 0.25,
+                                             gs.data_ptr(), None, pc.data_ptr(), ps.data_ptr(), 0,
+                                             torch.cuda.current_stream().cuda_stream)
+    assert st == _engine.E_UNSUPPORTED
+    assert lib.fpq_silu_mul_quantize_nv_packed(x.data_ptr(), cols, x.data_ptr(), cols, 4, cols, 1, 16, 0.25, None,
+                                               None, pc.data_ptr(), ps.data_ptr(), 0,
+                                               torch.cuda.current_stream().cuda_stream) == -1   # no global scale
+
+
 def test_rmsnorm_rows_limits():
     from fp_quant import _engine
     lib = _engine.lib()
@@ -243,7 +322,7 @@ def test_fused_norm_and_mlp_match_the_oracle_composition(fmt, g, tokens):
         y = block.input_layernorm(x)
         assert torch.equal(y, want_y)
         slot = eager._shared_activations[0]
-        assert slot.ref() is y and (slot.row_major is not None or slot.mx_packed is not None)
+        assert slot.ref() is y and slot.serves(True)
         assert torch.equal(block.self_attn.q_proj(y), want_q)
         assert torch.equal(block.self_attn.k_proj(y), want_k)
         assert eager._shared_activations[0] is slot         # both projections used the norm's quantization
