@@ -37,12 +37,14 @@ constexpr int kStreamMaxRows = 128;
 
 // NT weight row tiles per workgroup, MT activation row tiles (exactly ceil(M / 32)), DB 256-K blocks
 // of loads in flight per wave, NW waves.  Every workgroup re-reads all activations (NT = 2 halves
-// that, at a register cost that stream_plan explains; only NT = 1 is instantiated).
+// that, at a register cost that stream_plan explains).  Two weight tiles per workgroup, and three or
+// four activation row tiles with one block in flight, are compiled for two workgroups per CU (at most
+// 256 registers): left alone the compiler takes more and one workgroup fills the CU.
 // NV: NVFP4 operands (two E4M3 scale bytes per lane and K step, 512-byte scale blocks): a lane's dword s
 // of a 64-K unit, times its group's scale, is its fp16 operand of the s-th 32x32x16 matrix instruction
 // of the unit on both sides, so the K order is permuted consistently and the sum is complete.
 template <int NT, int MT, int DB, int NW, bool NV = false>
-__global__ __launch_bounds__(64 * NW) void gemm_fp4_stream_kernel(
+__global__ __launch_bounds__(64 * NW, (NT == 2 || (MT >= 3 && DB == 1)) ? 2 : 1) void gemm_fp4_stream_kernel(
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias,
     const uint16_t* residual, uint16_t* y, int M, int N, int K, int bps, int ksplit,
@@ -313,16 +315,19 @@ struct StreamPlan {
 // rows: while the weight tiles fit one round of the 256 CUs; beyond that the 128x128 tile kernel,
 // which shares activations through LDS.  (Two weight tiles per workgroup halve what the L2 has to
 // deliver for 33-64 rows, but need so many registers that one workgroup fills a CU; one tile per
-// workgroup with two blocks in flight, two workgroups per CU, measured 5-13 % faster.)
+// workgroup with two blocks in flight, two workgroups per CU, measured 5-13 % faster -- except from
+// 768 weight tiles on, where two tiles per workgroup with ONE block in flight, held to 256 registers,
+// are 12-16 % faster: MXFP4, N = 28672 at 64 rows 20.1 -> 17.0 us, N = 128256 73.5 -> 61.6 us.)
 // K is split across workgroups only for at most 32 rows, when the weight tiles leave at least half
 // of the CUs idle and every part keeps at least 4096 of K (the exchange of partial tiles through
 // the workspace costs about as much as streaming 16 blocks); fewer parts if the workspace is small.
-static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_bytes) {
+static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_bytes, bool nv = false) {
   StreamPlan plan{false, 1, 1, 0};
   if (M < 1 || M > kStreamMaxRows || N < 1 || K < 256 || K % 256 != 0) return plan;
   const int64_t rt_m = (M + 31) / 32, tiles = (N + 31) / 32, nkb = K / 256;
   if (rt_m > 2 && tiles > 256) return plan;
   plan.use = true;
+  if (rt_m == 2 && tiles >= 768 && !nv) plan.nt = 2;
   const int64_t groups = (tiles + plan.nt - 1) / plan.nt;
   int64_t ksplit = 1;
   if (rt_m == 1 && workspace_bytes > kStreamCounterBytes && groups <= kStreamCounters) {
@@ -352,7 +357,7 @@ template <bool NV>
 static int launch_stream(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                          const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
                          void* workspace, int64_t workspace_bytes, const OutSegments& seg, hipStream_t stream) {
-  const StreamPlan plan = stream_plan(M, N, K, workspace ? workspace_bytes : 0);
+  const StreamPlan plan = stream_plan(M, N, K, workspace ? workspace_bytes : 0, NV);
   const dim3 grid((unsigned)(((N + 31) / 32 + plan.nt - 1) / plan.nt), (unsigned)plan.ksplit);
   unsigned* counters = (unsigned*)workspace;
   float* partial = workspace ? (float*)((uint8_t*)workspace + kStreamCounterBytes) : nullptr;
@@ -362,7 +367,18 @@ static int launch_stream(const void* xq, const void* xs, const void* wq, const v
                      (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, (int)M, (int)N,    \
                      (int)K, plan.bps, plan.ksplit, partial, counters, seg)
   const int mt = (int)((M + 31) / 32);
-  if (plan.nt != 1) return FPQ_E_UNSUPPORTED;   // no plan asks for more than one weight tile per workgroup
+  if (plan.nt == 2) {   // MXFP4, 33-64 rows only
+    if constexpr (!NV) {
+      if (mt != 2) return FPQ_E_UNSUPPORTED;
+      FPQ_STREAM(2, 2, 1);
+      return (int)hipGetLastError();
+    }
+    return FPQ_E_UNSUPPORTED;
+  }
+  // 65-128 rows of MXFP4 at K up to 4096: one block in flight per wave and two workgroups per CU beat two
+  // blocks and one workgroup (128 rows, N = 4096 / 8192: 9.7 -> 8.9 / 10.6 -> 9.8 us); a longer K prefers
+  // the deeper ring (N = 4096, K = 14336, 96 rows: 18.4 against 19.0 us)
+  const bool shallow = !NV && K <= 4096;
   switch (mt) {
     case 1:
       // enough workgroups for three per CU: two blocks in flight per wave (98 registers, three
@@ -372,8 +388,22 @@ static int launch_stream(const void* xq, const void* xs, const void* wq, const v
       else FPQ_STREAM(1, 1, 4);
       break;
     case 2: FPQ_STREAM(1, 2, 2); break;
-    case 3: FPQ_STREAM(1, 3, 2); break;
+    case 3:
+      if constexpr (!NV) {
+        if (shallow) {
+          FPQ_STREAM(1, 3, 1);
+          break;
+        }
+      }
+      FPQ_STREAM(1, 3, 2);
+      break;
     default:
+      if constexpr (!NV) {
+        if (shallow) {
+          FPQ_STREAM(1, 4, 1);
+          break;
+        }
+      }
       FPQ_STREAM(1, 4, 2);
       break;
   }

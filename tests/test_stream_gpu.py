@@ -53,7 +53,9 @@ def _workspace(m, n, k, cap=None):
 # ragged rows and columns, one to 56 blocks of K
 SHAPES = [(1, 32, 256), (1, 100, 512), (5, 257, 768), (16, 1024, 1024), (31, 64, 1280), (32, 4096, 4096),
           (33, 130, 2048), (64, 96, 3072), (70, 515, 1024), (96, 2048, 4096), (100, 36, 256), (128, 1000, 2304),
-          (127, 4099, 1536), (8, 1024, 14336), (64, 8200, 512), (40, 8290, 768), (33, 16384, 256)]
+          (127, 4099, 1536), (8, 1024, 14336), (64, 8200, 512), (40, 8290, 768), (33, 16384, 256),
+          # 768 weight tiles or more at 33-64 rows: two weight tiles per workgroup (an odd tile count, a ragged N)
+          (64, 24600, 512), (45, 28672, 256), (33, 24577, 256)]
 # shapes whose K is split when a workspace is given (few weight tiles, K of 8192 or more)
 SPLIT_SHAPES = [(1, 32, 8192), (5, 257, 12288), (16, 1024, 8192), (31, 64, 16384), (32, 4096, 8192),
                 (8, 1024, 14336), (17, 515, 9216)]
@@ -149,7 +151,7 @@ def test_split_k_rejects_misaligned_workspace():
 @pytest.mark.parametrize("m,splits,k", [(1, [512, 256, 256], 512), (16, [1024, 256], 1024), (33, [256, 512], 256),
                                         (64, [4096, 4096, 256], 256), (128, [256, 256, 256, 256], 768),
                                         (300, [512, 256, 256], 512), (2048, [2048, 1024, 256, 768], 256),
-                                        (37, [9216], 256)])
+                                        (37, [9216], 256), (64, [14336, 14336], 256), (40, [12288, 256, 12288], 256)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_layers_end_to_end_get_their_own_outputs(m, splits, k, with_bias):
     """fpq_gemm_mxf4_packed_multi: every layer's matrix equals its column range of the one-output GEMM
