@@ -462,7 +462,7 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
     uint32_t n_chunks, uint32_t chunks_per_row, uint32_t rows, uint32_t scale_rows,
     uint32_t scale_stride, float norm, const float* __restrict__ global_scale, Prologue pro) {
   static_assert(!PACKED || EPL == 64, "packed output: 64-element chunks");
-  static_assert(PRO == kProNone || (PACKED && FMT == kFmtMx), "prologues exist for the packed MXFP4 output only");
+  static_assert(PRO == kProNone || PACKED, "prologues exist for the packed output only");
   static_assert(!QUEST || (FMT == kFmtMx && PRO == kProNone), "the quest rule exists for plain MXFP4 only");
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
   constexpr int NG = EPL / GROUP;        // groups (= scale bytes) per chunk
@@ -1294,8 +1294,6 @@ static int dispatch_prologue(const void* x, int64_t ld_first, const void* second
 }
 
 // The same with the packed operand layout as output (streaming kernel; cols % 256 == 0).
-// FMT = kFmtNv: the generic kernel only, i.e. at most kPackedFewRows rows (FPQ_E_UNSUPPORTED beyond: the
-// caller quantizes row-major and re-tiles)
 template <int PRO, int FMT = kFmtMx>
 static int dispatch_prologue_packed(const void* x, int64_t ld_first, const void* second, int64_t ld_second,
                                     const float* row_scale, const void* col_scale, void* out, int64_t rows,
@@ -1306,7 +1304,6 @@ static int dispatch_prologue_packed(const void* x, int64_t ld_first, const void*
   if (rows == 0 || cols == 0) return FPQ_OK;
   if (!x || !codes || !scales) return FPQ_E_NULL;
   if (FMT == kFmtNv && !gsp) return FPQ_E_NULL;
-  if (FMT == kFmtNv && rows > kPackedFewRows) return FPQ_E_UNSUPPORTED;
   if (PRO == kProRmsNorm && (!row_scale || !col_scale)) return FPQ_E_NULL;
   if (PRO == kProSiluMul && !second) return FPQ_E_NULL;
   if (zero_policy != FPQ_ZERO_REFERENCE && zero_policy != FPQ_ZERO_SIGNED) return FPQ_E_POLICY;
@@ -1346,9 +1343,8 @@ static int dispatch_prologue_packed(const void* x, int64_t ld_first, const void*
     if (few)                                                                                                   \
       return launch_lane8_prologue<GG, FMT, RR, PRO>(x, rows, cols, norm, gsp, codes, scales, rows,            \
                                                      cols / (FMT == kFmtNv ? 16 : 32), zero_policy, stream, pro); \
-    if constexpr (FMT == kFmtMx)                                                                               \
-      return launch_stream_packed<GG, RR, PRO>(x, rows, cols, norm, codes, scales, zero_policy, stream, pro);  \
-    return FPQ_E_UNSUPPORTED;                                                                                  \
+    return launch_stream_packed<GG, RR, PRO, FMT>(x, rows, cols, norm, codes, scales, zero_policy, stream,    \
+                                                  pro, gsp);                                                  \
   }
   if (rot_kind == FPQ_ROT_IDENTITY) FPQ_LAUNCH_PRO_PACKED(32, FPQ_ROT_IDENTITY);
   switch (g) {

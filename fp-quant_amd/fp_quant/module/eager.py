@@ -161,8 +161,9 @@ def _lookup(src: torch.Tensor, key, want_packed: bool) -> Optional[QuantizedActi
 def quantize_activations(x_flat: torch.Tensor, h: torch.Tensor, kind: int, norm: float,
                          act_global_scale: Optional[torch.Tensor], nvfp4: bool, stream: int,
                          want_packed: bool, remember: bool = True, quest: bool = False) -> QuantizedActivations:
-    """Rotate and quantize bf16 [m, k]: MXFP4 straight into the packed layout when the packed GEMM will
-    run, row-major otherwise (NVFP4 always; its packed form is made on demand)."""
+    """Rotate and quantize bf16 [m, k]: straight into the packed layout when the packed GEMM will run
+    (row-major first, re-tiled on demand, for the rotations the packed quantizers do not take), row-major
+    otherwise."""
     lib = _engine.lib()
     m, k = x_flat.shape
     dev = x_flat.device
@@ -373,7 +374,7 @@ def linear_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torc
 # 32-row tiles, so the packed weights of several layers with the same K, laid end to end, are the packed
 # weight of their concatenation along N: one launch computes [m, n_1 + n_2 + ...] and the layers' outputs
 # are column slices of it.  The layers' own packed copies become views into the concatenated buffers, so
-# no 4-bit weight is held a further time.  MXFP4 only (the NVFP4 packed kernel serves mid-sized batches only).
+# no 4-bit weight is held a further time.  MXFP4 and NVFP4 (one format per group).
 class WeightGroup:
     __slots__ = ("key", "wp", "wsp", "bias", "n", "splits", "k", "nvfp4")
 
@@ -671,9 +672,9 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
         qa = QuantizedActivations(rows, cols, nvfp4)
         qa.mx_packed = (pc, ps)
         return qa
-    if (allow_packed and nvfp4 and rows <= _ROWS_KERNEL_MAX_ROWS and cols % 256 == 0
+    if (allow_packed and nvfp4 and rows <= _NV_PACKED_PRODUCER_MAX_ROWS and cols % 256 == 0
             and nv_packed_eligible(rows, 32, cols, fused_linear=True)):
-        # a decode step's few rows straight into the packed NVFP4 layout (generic kernel)
+        # the row counts whose consumers run the packed NVFP4 GEMM: straight into its layout
         gs = as_f32_scalar(act_global_scale, remember)
         pc = torch.empty(lib.fpq_packed_codes_bytes(rows, cols), dtype=torch.uint8, device=dev)
         ps = torch.empty(lib.fpq_packed_scales_bytes_nv(rows, cols), dtype=torch.uint8, device=dev)
@@ -702,6 +703,10 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
 
 
 _ROWS_KERNEL_MAX_ROWS = 64   # fpq_rmsnorm_rows_max_rows()
+# NVFP4 layers take the packed GEMM up to mid-sized batches (nv_packed_eligible: fewer than 100 tiles of
+# 256 x 256) and the row-major one beyond; a fused producer does not know its consumers' widths, so it
+# writes the packed layout up to this many rows (a consumer that wants the other layout re-tiles, exactly).
+_NV_PACKED_PRODUCER_MAX_ROWS = 512
 
 
 def rmsnorm_quantize(x: torch.Tensor, weight: torch.Tensor, eps: float, hadamard_matrix: torch.Tensor,

@@ -251,9 +251,8 @@ int fpq_rmsnorm_rows_quantize_nv_packed(const void* x, int64_t ld, const void* w
                                         const float* global_scale, float* inv_rms, void* normed,
                                         void* packed_codes, void* packed_scales, int zero_policy, void* stream);
 /*
- * The NVFP4 fused producers writing the packed operand layout of fpq_gemm_nvf4_packed: at most 64 rows (what a
- * decode step quantizes; FPQ_E_UNSUPPORTED beyond: quantize row-major with fpq_*_quantize_nv, then
- * fpq_pack_nvf4).  Arguments as fpq_rmsnorm_quantize_nv / fpq_silu_mul_quantize_nv.
+ * The NVFP4 fused producers writing the packed operand layout of fpq_gemm_nvf4_packed (cols % 256 == 0, as for
+ * fpq_quantize_nv_packed).  Arguments as fpq_rmsnorm_quantize_nv / fpq_silu_mul_quantize_nv.
  */
 int fpq_rmsnorm_quantize_nv_packed(const void* x, int64_t ld, const float* inv_rms, const void* weight,
                                    int64_t rows, int64_t cols, int rot_kind, int g, float norm,

@@ -170,10 +170,10 @@ def test_rmsnorm_rows_in_one_launch_nvfp4_bit_exact(rot, g, rows, cols):
 
 @pytest.mark.parametrize("rot,g", NV_PACKED_CASES)
 @pytest.mark.parametrize("kind", ["rmsnorm", "silu_mul"])
-@pytest.mark.parametrize("rows,cols", [(1, 256), (20, 768), (64, 512)])
+@pytest.mark.parametrize("rows,cols", [(1, 256), (20, 768), (64, 512), (70, 512), (300, 1024)])
 def test_fused_quantize_packed_nvfp4_bit_exact(kind, rot, g, rows, cols):
-    """The NVFP4 fused producers writing the packed layout (a few rows): codes, E4M3 scales and the bf16
-    by-product of the oracle; more rows than the entry serves are refused, not mis-served."""
+    """The NVFP4 fused producers writing the packed layout (generic kernel up to 64 rows, streaming kernel
+    beyond): codes, E4M3 scales and the bf16 by-product of the oracle."""
     from fp_quant import _engine
     from tests.test_packed_gpu import pack_nv_by_definition
     a = make_student_t(rows, cols, seed=rows + g) * 2
@@ -194,7 +194,7 @@ def test_fused_quantize_packed_nvfp4_bit_exact(kind, rot, g, rows, cols):
         want_v = O.silu_mul(a, b)
     wc, ws = _oracle_quantize(want_v, "nvfp4", rot, g, 777.0)
     want_c, want_s = pack_nv_by_definition(wc, ws, cols)
-    lds = dict(ld_a=cols + 64, ld_b=2 * cols) if rows == 20 else {}
+    lds = dict(ld_a=cols + 64, ld_b=2 * cols) if rows in (20, 70) else {}
     pc, ps, out = capi.fused_quantize_packed(kind, a, b, g=g, rot=rot, global_scale=777.0, **lds)
     assert torch.equal(out.view(torch.int16), want_v.view(torch.int16))
     assert torch.equal(pc, want_c) and torch.equal(ps, want_s)
@@ -202,21 +202,16 @@ def test_fused_quantize_packed_nvfp4_bit_exact(kind, rot, g, rows, cols):
     assert none is None and torch.equal(pc2, want_c) and torch.equal(ps2, want_s)
 
 
-def test_fused_quantize_packed_nvfp4_refuses_many_rows():
+def test_fused_quantize_packed_nvfp4_needs_a_global_scale():
     from fp_quant import _engine
     lib = _engine.lib()
-    rows, cols = 300, 256
+    rows, cols = 4, 256
     x = torch.zeros(rows, cols, dtype=torch.bfloat16, device="cuda")
-    gs = torch.ones(1, dtype=torch.float32, device="cuda")
     pc = torch.zeros(lib.fpq_packed_codes_bytes(rows, cols), dtype=torch.uint8, device="cuda")
     ps = torch.zeros(lib.fpq_packed_scales_bytes_nv(rows, cols), dtype=torch.uint8, device="cuda")
-    st = lib.fpq_silu_mul_quantize_nv_packed(x.data_ptr(), cols, x.data_ptr(), cols, rows, cols, 1, 16, 0.25,
-                                             gs.data_ptr(), None, pc.data_ptr(), ps.data_ptr(), 0,
-                                             torch.cuda.current_stream().cuda_stream)
-    assert st == _engine.E_UNSUPPORTED
-    assert lib.fpq_silu_mul_quantize_nv_packed(x.data_ptr(), cols, x.data_ptr(), cols, 4, cols, 1, 16, 0.25, None,
+    assert lib.fpq_silu_mul_quantize_nv_packed(x.data_ptr(), cols, x.data_ptr(), cols, rows, cols, 1, 16, 0.25, None,
                                                None, pc.data_ptr(), ps.data_ptr(), 0,
-                                               torch.cuda.current_stream().cuda_stream) == -1   # no global scale
+                                               torch.cuda.current_stream().cuda_stream) == -1
 
 
 def test_rmsnorm_rows_limits():
