@@ -399,10 +399,13 @@ static int launch_lane8(const void* x, int64_t rows, int64_t cols, float norm, c
 }
 
 // -------------------------------------------------------------------------------------------
-// Streaming kernel for cols % EPL == 0 (EPL = 64 or 128): one lane owns EPL consecutive elements
+// Streaming kernel for cols % 64 == 0 (EPL = 32, 64 or 128): one lane owns EPL consecutive elements
 // (2*EPL bytes in, EPL/2 bytes of codes and EPL/32 or EPL/16 scale bytes out), so the butterfly
 // stages with stride < EPL, every group maximum and the packing stay inside the lane's registers;
-// a 128-wide rotation with EPL = 64 adds one exchange between neighbouring lanes.  A wave moves
+// a rotation wider than EPL adds one or two exchanges between neighbouring lanes.  Inputs below 2^24
+// elements run with EPL = 32: every wave then owns at most a tile or two, all loads are issued at once
+// and the arithmetic of the wave whose data arrive last is exposed -- half the tile, half that tail
+// (2048 x 4096, Hadamard 128: 7.4 -> 6.5 us; from 2^24 elements on the two sizes measure alike).  A wave moves
 // 64 such chunks per tile: direct global -> LDS loads in full contiguous runs, then each lane
 // reads its own chunk back with 16-byte LDS reads.  The 16-byte pieces of a chunk are
 // XOR-swizzled by the lane number (through the choice of the piece each DMA lane fetches) so
@@ -520,9 +523,11 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
   // DMA lane map: instruction i fills LDS pieces [64 i, 64 i + 64); piece p = PIECES * b + j
   // belongs to chunk b and holds that chunk's 16-byte piece j ^ sw(b).  sw(b) is chosen so that
   // the 16-byte reads "piece k of my own chunk" of all lanes hit every LDS bank group once per
-  // pass (checked with the bank-conflict counter): b % 16 for 256-byte chunks, and
-  // (b % 8) ^ ((b / 8) & 1) for 128-byte chunks.
-  auto sw = [](uint32_t b) -> uint32_t { return PIECES == 8 ? ((b & 7u) ^ ((b >> 3) & 1u)) : (b % PIECES); };
+  // pass (checked with the bank-conflict counter): b % 16 for 256-byte chunks,
+  // (b % 8) ^ ((b / 8) & 1) for 128-byte chunks and (b / 4) % 4 for 64-byte chunks.
+  auto sw = [](uint32_t b) -> uint32_t {
+    return PIECES == 8 ? ((b & 7u) ^ ((b >> 3) & 1u)) : PIECES == 4 ? ((b >> 2) & 3u) : (b % PIECES);
+  };
   const uint32_t b_lo = lane / PIECES, j_lo = lane % PIECES;
   constexpr int NV_OFF = PIECES == 8 ? 2 : 4;  // distinct swizzle phases over the instruction index
   // bytes from one row to the next (a prologue's inputs may sit in wider buffers)
@@ -666,6 +671,19 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
           const float other = __uint_as_float((uint32_t)__builtin_amdgcn_mov_dpp(
               (int)__float_as_uint(v[i]), 0xB1 /* quad_perm [1,0,3,2] */, 0xF, 0xF, true));
           v[i] = other + __uint_as_float(__float_as_uint(v[i]) ^ flip);
+        }
+        if (G > 2 * EPL) {
+          // stride 2 EPL (a 128-wide rotation with EPL = 32): the quarters of a block sit in lanes
+          // 4u .. 4u + 3 and the partner is lane ^ 2
+          static_assert(G <= 4 * EPL, "at most two exchanges between lanes");
+          __builtin_amdgcn_sched_barrier(0);
+          const uint32_t flip2 = (lane & 2u) << 30;
+#pragma unroll
+          for (int i = 0; i < EPL; ++i) {
+            const float other = __uint_as_float((uint32_t)__builtin_amdgcn_mov_dpp(
+                (int)__float_as_uint(v[i]), 0x4E /* quad_perm [2,3,0,1] */, 0xF, 0xF, true));
+            v[i] = other + __uint_as_float(__float_as_uint(v[i]) ^ flip2);
+          }
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -835,7 +853,7 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
     // different bank groups) -> contiguous rows
 #pragma unroll
     for (int k4 = 0; k4 < CQ; ++k4) {
-      const uint32_t sw = CQ == 4 ? ((lane >> 1) & 3u) : ((lane >> 2) & 1u);
+      const uint32_t sw = CQ == 4 ? ((lane >> 1) & 3u) : CQ == 2 ? ((lane >> 2) & 1u) : 0u;
       *(uint4*)(my + (lane * CQ + (k4 ^ sw)) * 16u) =
           make_uint4(cw[4 * k4], cw[4 * k4 + 1], cw[4 * k4 + 2], cw[4 * k4 + 3]);
     }
@@ -843,14 +861,14 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
 #pragma unroll
     for (int i = 0; i < CQ; ++i) {
       const uint32_t g = 64u * i + lane, l = g / CQ, k4 = g % CQ;
-      const uint32_t sw = CQ == 4 ? ((l >> 1) & 3u) : ((l >> 2) & 1u);
+      const uint32_t sw = CQ == 4 ? ((l >> 1) & 3u) : CQ == 2 ? ((l >> 2) & 1u) : 0u;
       const uint4 o = *(const uint4*)(my + (l * CQ + (k4 ^ sw)) * 16u);
       if (l < valid) store16_nt(dst + g * 16u, o);
     }
 
     if (lane < valid) {
       const uint32_t chunk = tile * 64u + lane;
-      constexpr uint32_t SB = NG;  // scale bytes per chunk: 2, 4 or 8
+      constexpr uint32_t SB = NG;  // scale bytes per chunk: 1, 2, 4 or 8
       size_t so;
       if (scale_stride == chunks_per_row * SB) {
         so = (size_t)chunk * SB;
@@ -859,7 +877,8 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
         so = (size_t)row * scale_stride + (chunk - row * chunks_per_row) * SB;
       }
       if ((scale_stride & (SB - 1u)) == 0u) {
-        if (SB == 2) *(uint16_t*)(scales + so) = (uint16_t)sbytes;
+        if (SB == 1) scales[so] = (uint8_t)sbytes;
+        else if (SB == 2) *(uint16_t*)(scales + so) = (uint16_t)sbytes;
         else if (SB == 4) *(uint32_t*)(scales + so) = sbytes;
         else *(uint2*)(scales + so) = make_uint2(sb_lo, sbytes);
       } else {
@@ -908,6 +927,22 @@ static int launch_stream(const void* x, int64_t rows, int64_t cols, float norm, 
     go(quantize_stream_kernel<EPL, G, FMT, ROT, kZeroSigned, false, kProNone, QUEST>);
   }
   return (int)hipGetLastError();
+}
+
+// The streaming kernel with the chunk size that suits the input (see the kernel's head); a sequency-ordered
+// block has to fit in one lane.
+constexpr int64_t kHalfTileElements = (int64_t)1 << 24;
+template <int G, int FMT, int ROT, bool QUEST = false>
+static int launch_stream_sized(const void* x, int64_t rows, int64_t cols, float norm, const float* gsp,
+                               void* codes, void* scales, int64_t scale_rows, int64_t scale_stride,
+                               int zero_policy, hipStream_t stream) {
+  if constexpr (ROT != FPQ_ROT_GSR || G <= 32) {
+    if (rows * cols < kHalfTileElements)
+      return launch_stream<32, G, FMT, ROT, QUEST>(x, rows, cols, norm, gsp, codes, scales, scale_rows,
+                                                   scale_stride, zero_policy, stream);
+  }
+  return launch_stream<FPQ_EPL, G, FMT, ROT, QUEST>(x, rows, cols, norm, gsp, codes, scales, scale_rows,
+                                                    scale_stride, zero_policy, stream);
 }
 
 constexpr int kSiluDynLds = 4 * 64 * 128 + 2 * (int)kSiluLdsCount * 2;  // second tiles + table copy
@@ -1042,8 +1077,8 @@ static int dispatch_quest(const void* x, int64_t rows, int64_t cols, int rot_kin
 #define FPQ_LAUNCH_QUEST_STREAM(GG, RR)                                                                        \
   {                                                                                                            \
     if (stream_ok)                                                                                             \
-      return launch_stream<FPQ_EPL, GG, kFmtMx, RR, true>(x, rows, cols, norm, nullptr, codes, scales,        \
-                                                          scale_rows, scale_stride, zero_policy, stream);     \
+      return launch_stream_sized<GG, kFmtMx, RR, true>(x, rows, cols, norm, nullptr, codes, scales,           \
+                                                       scale_rows, scale_stride, zero_policy, stream);        \
     FPQ_LAUNCH_QUEST(GG, RR);                                                                                  \
   }
   if (rot_kind == FPQ_ROT_GENERAL) {
@@ -1150,7 +1185,7 @@ static int dispatch(const void* x, int64_t rows, int64_t cols, int rot_kind, int
   const bool stream_ok = cols % FPQ_EPL == 0 && rows * cols >= (int64_t)1 << 21 &&
                          !((uintptr_t)codes & 15u) && !((uintptr_t)scales & 7u);
 #define FPQ_LAUNCH(GG, RR)                                                                       \
-  return stream_ok ? launch_stream<FPQ_EPL, GG, FMT, RR>(x, rows, cols, norm, gsp, codes, scales,\
+  return stream_ok ? launch_stream_sized<GG, FMT, RR>(x, rows, cols, norm, gsp, codes, scales,   \
                                                   scale_rows, scale_stride, zero_policy, stream) \
                    : launch_lane8<GG, FMT, RR>(x, rows, cols, norm, gsp, codes, scales,          \
                                                scale_rows, scale_stride, zero_policy, stream)

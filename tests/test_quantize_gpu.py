@@ -179,6 +179,26 @@ def test_streaming_kernel_adversarial_and_ragged(cols):
     _check(x, "nvfp4", "hadamard", 16, 0, gs=2688.0 / 7.0)
 
 
+def test_streaming_kernel_from_two_to_the_24_elements():
+    """From 2^24 elements on a lane of the streaming kernel owns 64 elements instead of 32 (below, the test
+    above): the same adversarial rows in a ragged input of that size."""
+    cols = 4096
+    adv = _adversarial_rows(cols)
+    n_rows = (1 << 24) // cols + 37
+    x = make_outlier_normal(n_rows, cols, seed=24).float()
+    pos = torch.randperm(n_rows, generator=torch.Generator().manual_seed(5))[: adv.shape[0] * 3]
+    for i, p in enumerate(pos.tolist()):
+        x[p] = adv[i % adv.shape[0]]
+    x[-1] = adv[2]
+    x = x.to(torch.bfloat16)
+    _check(x, "mxfp4", "hadamard", 128, 0)
+    _check(x, "mxfp4", "hadamard", 32, 1, pad=True)
+    _check(x, "mxfp4", "identity", 32, 0)
+    _check(x, "nvfp4", "hadamard", 64, 0, gs=10.0)
+    _check(x, "nvfp4", "identity", 16, 1, gs=3.0)
+    _check(x, "nvfp4", "hadamard", 16, 0, gs=1e-25)   # global scale outside the fast range
+
+
 def test_negative_zero_inputs_keep_their_sign_under_signed_policy():
     x = torch.zeros(64, 128)
     x[::2] = -0.0

@@ -154,6 +154,17 @@ def test_quest_streaming_kernel_bit_exact(rot, g, policy):
     assert torch.equal(codes2, wc) and torch.equal(scales2, ws)
 
 
+@pytest.mark.parametrize("rot,g", [("hadamard", 128), ("hadamard", 32), ("gsr", 64)])
+def test_quest_streaming_kernel_from_two_to_the_24_elements(rot, g):
+    """From 2^24 elements on a lane of the streaming kernel owns 64 elements instead of 32."""
+    rows, cols = 4100, 4096
+    x = _quest_input(rows, cols, 11 * g + len(rot))
+    norm = float(O.hadamard_matrix(g)[0, 0])
+    wc, ws, _, _ = O.quantize_mx_quest(x, OK[rot], g, norm)
+    codes, scales, _ = capi.quantize_quest(x, rot=rot, g=g, norm=norm, want_mask=False)
+    assert torch.equal(scales, ws) and torch.equal(codes, wc)
+
+
 @pytest.mark.parametrize("rot,g", STREAM_CASES)
 @pytest.mark.parametrize("rows,cols", [(1, 256), (20, 768), (64, 512), (70, 512), (300, 1024), (2100, 256)])
 def test_quest_packed_bit_exact(rot, g, rows, cols):
