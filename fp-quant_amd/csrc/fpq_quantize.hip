@@ -440,11 +440,12 @@ __device__ __forceinline__ uint32_t fix_zero_nibbles(uint32_t w) {
 }
 
 //
-// PACKED (EPL = 64 only) writes the operand layout of fpq_gemm_mxf4_packed / fpq_gemm_nvf4_packed instead of
-// row-major codes and scales.  A wave tile is then 32 rows x two neighbouring chunks (lane =
-// 2 * row + chunk, so the lane pairing of a 128-wide rotation is unchanged): the loads are 256-byte
-// row segments, and every 16-byte half of a lane's codes is exactly one lane slot of a packed
-// kilobyte block, so codes are stored straight from registers in two 512-byte runs per store.
+// PACKED (EPL = 64, or 32 without a prologue) writes the operand layout of fpq_gemm_mxf4_packed /
+// fpq_gemm_nvf4_packed instead of row-major codes and scales.  A wave tile is then 32 rows x two
+// neighbouring chunks (lane = 2 * row + chunk, so the lane pairing of a rotation wider than a chunk is
+// unchanged): the loads are 256-byte (128-byte) row segments, and every 16 bytes of a lane's codes are
+// exactly one lane slot of a packed kilobyte block, so codes are stored straight from registers in two
+// 512-byte runs per store.
 //
 // PRO != kProNone (PACKED only) applies a producer's arithmetic to the values as they leave LDS (see
 // Prologue): kProRmsNorm scales by the row's 1/rms and the column's weight (16-byte loads that hit
@@ -464,7 +465,8 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
     const uint8_t* __restrict__ x, uint8_t* __restrict__ codes, uint8_t* __restrict__ scales,
     uint32_t n_chunks, uint32_t chunks_per_row, uint32_t rows, uint32_t scale_rows,
     uint32_t scale_stride, float norm, const float* __restrict__ global_scale, Prologue pro) {
-  static_assert(!PACKED || EPL == 64, "packed output: 64-element chunks");
+  static_assert(!PACKED || EPL == 64 || (EPL == 32 && PRO == kProNone),
+                "packed output: 64-element chunks; 32-element chunks without a prologue");
   static_assert(PRO == kProNone || PACKED, "prologues exist for the packed output only");
   static_assert(!QUEST || (FMT == kFmtMx && PRO == kProNone), "the quest rule exists for plain MXFP4 only");
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
@@ -533,8 +535,13 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
   // bytes from one row to the next (a prologue's inputs may sit in wider buffers)
   const uint32_t row_bytes = PRO == kProNone ? chunks_per_row * CB : pro.ld_first * 16u;
   const uint32_t row_bytes2 = PRO == kProSiluMul ? pro.ld_second * 16u : 0u;
-  // PACKED: chunk b of the tile is row b / 2 of the row tile, chunk b % 2 of the pair
-  const uint32_t b_off = PACKED ? (b_lo >> 1) * row_bytes + (b_lo & 1u) * CB : b_lo * CB;
+  // PACKED: chunk b of the tile is row b / CPR of the tile, chunk b % CPR of its columns.  With 64-element
+  // chunks a tile is the 32 rows of a row tile x 2 chunks; with 32-element chunks it is 16 rows (half a row
+  // tile) x 4 chunks, so that the 128 columns of the widest rotation still sit in neighbouring lanes.
+  constexpr bool P32 = PACKED && EPL == 32;
+  constexpr uint32_t CPR = P32 ? 4u : 2u;     // chunks per row of a packed tile
+  constexpr uint32_t RPI = CPI / CPR;         // rows filled by one DMA instruction
+  const uint32_t b_off = PACKED ? (b_lo / CPR) * row_bytes + (b_lo % CPR) * CB : b_lo * CB;
   uint32_t voff[NV_OFF], voff2[PRO == kProSiluMul ? NV_OFF : 1];
 #pragma unroll
   for (int m = 0; m < NV_OFF; ++m) {
@@ -543,14 +550,30 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
   }
   const uint32_t rd_base = lane * CB, l_sw = sw(lane);
 
-  const uint32_t pairs = chunks_per_row / 2u;  // PACKED: tiles per row tile
-  const uint32_t n_tiles = PACKED ? ((rows + 31u) / 32u) * pairs : (n_chunks + 63u) / 64u;
+  const uint32_t pairs = chunks_per_row / CPR;  // PACKED: tiles side by side in a row (half) tile
+  const uint32_t n_tiles = PACKED ? ((rows + 31u) / 32u) * pairs * (P32 ? 2u : 1u) : (n_chunks + 63u) / 64u;
   const uint32_t total_waves = gridDim.x * 4u;
   for (uint32_t tile = blockIdx.x * 4u + wave; tile < n_tiles; tile += total_waves) {
-    const uint32_t rt = PACKED ? tile / pairs : 0u, pr = PACKED ? tile - rt * pairs : 0u;
+    const uint32_t per_rt = pairs * (P32 ? 2u : 1u);
+    const uint32_t rt = PACKED ? tile / per_rt : 0u;
+    const uint32_t hh = P32 ? (tile - rt * per_rt) / pairs : 0u;             // which 16 rows of the row tile
+    const uint32_t pr = PACKED ? tile - rt * per_rt - hh * pairs : 0u;
     // chunks (row-major) or rows (PACKED) of this tile that exist
-    const uint32_t valid = PACKED ? min(32u, rows - rt * 32u) : min(64u, n_chunks - tile * 64u);
-    const uint8_t* src = PACKED ? x + (size_t)rt * 32u * row_bytes + (size_t)(2u * pr) * CB
+    const uint32_t rows_rt = PACKED ? min(32u, rows - rt * 32u) : 0u;
+    const uint32_t valid = P32      ? (rows_rt > 16u * hh ? min(16u, rows_rt - 16u * hh) : 0u)
+                           : PACKED ? rows_rt
+                                    : min(64u, n_chunks - tile * 64u);
+    if (P32 && valid == 0u) {
+      // sixteen padding rows of the last row tile: zero codes and scale bytes, nothing to read
+      const uint32_t units = chunks_per_row / 2u, unit = 2u * pr + ((lane >> 1) & 1u);
+      const uint32_t slot = (lane & 1u) * 32u + 16u * hh + (lane >> 2);
+      store16_nt(codes + (((size_t)rt * units + unit) * 64u + slot) * 16u, make_uint4(0u, 0u, 0u, 0u));
+      uint8_t* sblk = scales + ((size_t)rt * (units / 4u) + (unit >> 2)) * (FMT == kFmtMx ? 256u : 512u);
+      if (FMT == kFmtMx) sblk[slot * 4u + (unit & 3u)] = 0;
+      else *(uint16_t*)(sblk + slot * 8u + 2u * (unit & 3u)) = 0;
+      continue;
+    }
+    const uint8_t* src = PACKED ? x + ((size_t)rt * 32u + 16u * hh) * row_bytes + (size_t)(CPR * pr) * CB
                                 : x + (size_t)tile * TILE;
     const uint8_t* src2 = PRO == kProSiluMul
                               ? (const uint8_t*)pro.second + (size_t)rt * 32u * row_bytes2 + (size_t)(2u * pr) * CB
@@ -562,13 +585,13 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
       // chunk of this instruction if that one is valid, else the first chunk of the tile.
       uint32_t off = voff[i % NV_OFF];
       if (PACKED) {
-        const bool instr_valid = (uint32_t)(CPI / 2 * i) < valid;          // wave-uniform
-        const uint8_t* base_i = instr_valid ? src + (size_t)(CPI / 2 * i) * row_bytes : src;
-        const bool past = CPI / 2 * i + (b_lo >> 1) >= valid;
-        if (past) off = (b_lo & 1u) * CB + j_lo * 16u;
+        const bool instr_valid = (uint32_t)(RPI * i) < valid;              // wave-uniform
+        const uint8_t* base_i = instr_valid ? src + (size_t)(RPI * i) * row_bytes : src;
+        const bool past = RPI * i + b_lo / CPR >= valid;
+        if (past) off = (b_lo % CPR) * CB + j_lo * 16u;
         lds_dma16_nt(base_i, off, my_base + i * 1024u);
         if (PRO == kProSiluMul) {
-          const uint8_t* base2_i = instr_valid ? src2 + (size_t)(CPI / 2 * i) * row_bytes2 : src2;
+          const uint8_t* base2_i = instr_valid ? src2 + (size_t)(RPI * i) * row_bytes2 : src2;
           lds_dma16_nt(base2_i, past ? off : voff2[i % NV_OFF], my2_base + i * 1024u);
         }
       } else {
@@ -816,17 +839,36 @@ __global__ __launch_bounds__(256, 2) void quantize_stream_kernel(
           sbytes |= (g.byte & 0xffu) << (8 * gi);
         }
       }
-      const uint32_t r = lane >> 1, ksl = lane & 1u;
+      const uint32_t r = P32 ? lane >> 2 : lane >> 1, ksl = lane & 1u;
       const bool row_ok = r < valid;
       if (!row_ok) {  // padding rows of the last row tile: zero codes, zero scale bytes
 #pragma unroll
         for (int k = 0; k < CW; ++k) cw[k] = 0u;
         sbytes = 0u;
       }
+      if constexpr (EPL == 32) {
+        // The lane (row 16 hh + r, chunk c = lane % 4 of the tile's 128 columns) holds K half c % 2 of
+        // the 64-K unit 2 pr + c / 2, i.e. lane slot (c % 2) * 32 + row of that packed kilobyte block, and
+        // one (MXFP4) or two (NVFP4) scale bytes: byte unit % 4 (bytes 2 (unit % 4), + 1) of that slot's
+        // entry in scale block (rt, unit / 4).
+        const uint32_t units = chunks_per_row / 2u, unit = 2u * pr + ((lane >> 1) & 1u);
+        const uint32_t slot = ksl * 32u + 16u * hh + r;
+        store16_nt(codes + (((size_t)rt * units + unit) * 64u + slot) * 16u, make_uint4(cw[0], cw[1], cw[2], cw[3]));
+        if (FMT == kFmtMx) {
+          uint8_t* sblk = scales + ((size_t)rt * (units / 4u) + (unit >> 2)) * 256u;
+          sblk[slot * 4u + (unit & 3u)] = (uint8_t)sbytes;
+        } else {
+          uint8_t* sblk = scales + ((size_t)rt * (units / 4u) + (unit >> 2)) * 512u;
+          *(uint16_t*)(sblk + slot * 8u + 2u * (unit & 3u)) = (uint16_t)sbytes;
+        }
+        asm volatile("" ::: "memory");
+        continue;
+      }
       const uint32_t ks = 2u * pr + ksl;
       uint8_t* blk = codes + (((size_t)rt * chunks_per_row + ks) * 64u + r) * 16u;
       store16_nt(blk, make_uint4(cw[0], cw[1], cw[2], cw[3]));              // K half 0
-      store16_nt(blk + 512, make_uint4(cw[4], cw[5], cw[6], cw[7]));        // K half 1
+      store16_nt(blk + 512, make_uint4(cw[CW > 4 ? 4 : 0], cw[CW > 4 ? 5 : 1], cw[CW > 4 ? 6 : 2],
+                                       cw[CW > 4 ? 7 : 3]));                // K half 1
       // scale bytes: byte (ks % 4) of dword (kh, r) in block (rt, ks / 4).  The pair of lanes
       // of a row holds bytes q and q + 1 of both dwords: the even lane stores the half-word of
       // K half 0, the odd lane that of K half 1.
@@ -947,11 +989,11 @@ static int launch_stream_sized(const void* x, int64_t rows, int64_t cols, float 
 
 constexpr int kSiluDynLds = 4 * 64 * 128 + 2 * (int)kSiluLdsCount * 2;  // second tiles + table copy
 
-template <int G, int ROT, int PRO = kProNone, int FMT = kFmtMx, bool QUEST = false>
+template <int G, int ROT, int PRO = kProNone, int FMT = kFmtMx, bool QUEST = false, int EPL = 64>
 static int launch_stream_packed(const void* x, int64_t rows, int64_t cols, float norm, void* codes,
                                 void* scales, int zero_policy, hipStream_t stream,
                                 const Prologue& pro = Prologue{}, const float* gsp = nullptr) {
-  const int64_t n_tiles = ((rows + 31) / 32) * (cols / 128);
+  const int64_t n_tiles = ((rows + 31) / 32) * (cols / 128) * (EPL == 32 ? 2 : 1);
   int64_t blocks = (n_tiles + 3) / 4;
   // Waves stride over the tiles of a capped grid.  The SiLU*up prologue (two workgroups fit a CU, each
   // copies the table's busy part into LDS first) is best with one resident round; the RMSNorm prologue
@@ -968,16 +1010,29 @@ static int launch_stream_packed(const void* x, int64_t rows, int64_t cols, float
       if ((status = limit.ensure((const void*)kernel, kDyn)) != 0) return;
     }
     hipLaunchKernelGGL(kernel, grid, block, kDyn, stream, (const uint8_t*)x, (uint8_t*)codes,
-                       (uint8_t*)scales, (uint32_t)(rows * cols / 64), (uint32_t)(cols / 64),
+                       (uint8_t*)scales, (uint32_t)(rows * cols / EPL), (uint32_t)(cols / EPL),
                        (uint32_t)rows, 0u, 0u, norm, gsp, pro);
   };
   if (zero_policy == FPQ_ZERO_REFERENCE) {
-    go(quantize_stream_kernel<64, G, FMT, ROT, kZeroReference, true, PRO, QUEST>);
+    go(quantize_stream_kernel<EPL, G, FMT, ROT, kZeroReference, true, PRO, QUEST>);
   } else {
-    go(quantize_stream_kernel<64, G, FMT, ROT, kZeroSigned, true, PRO, QUEST>);
+    go(quantize_stream_kernel<EPL, G, FMT, ROT, kZeroSigned, true, PRO, QUEST>);
   }
   if (status) return status;
   return (int)hipGetLastError();
+}
+
+// The packed streaming kernel (no prologue) with the chunk size that suits the input, as launch_stream_sized.
+template <int G, int ROT, int FMT, bool QUEST = false>
+static int launch_stream_packed_sized(const void* x, int64_t rows, int64_t cols, float norm, void* codes,
+                                      void* scales, int zero_policy, hipStream_t stream, const float* gsp) {
+  if constexpr (ROT != FPQ_ROT_GSR || G <= 32) {
+    if (rows * cols < kHalfTileElements)
+      return launch_stream_packed<G, ROT, kProNone, FMT, QUEST, 32>(x, rows, cols, norm, codes, scales, zero_policy,
+                                                                    stream, Prologue{}, gsp);
+  }
+  return launch_stream_packed<G, ROT, kProNone, FMT, QUEST>(x, rows, cols, norm, codes, scales, zero_policy, stream,
+                                                            Prologue{}, gsp);
 }
 
 constexpr int64_t kPackedFewRows = 64;
@@ -1005,8 +1060,7 @@ static int dispatch_packed(const void* x, int64_t rows, int64_t cols, int rot_ki
     if (few)                                                                                                      \
       return launch_lane8<GG, FMT, RR>(x, rows, cols, norm, gsp, codes, scales, rows, cols / kGroupCols,          \
                                        zero_policy, stream, nullptr, true);                                       \
-    return launch_stream_packed<GG, RR, kProNone, FMT>(x, rows, cols, norm, codes, scales, zero_policy, stream,   \
-                                                       Prologue{}, gsp);                                          \
+    return launch_stream_packed_sized<GG, RR, FMT>(x, rows, cols, norm, codes, scales, zero_policy, stream, gsp); \
   }
   if (rot_kind == FPQ_ROT_IDENTITY) {
     FPQ_LAUNCH_PACKED(32, FPQ_ROT_IDENTITY);
@@ -1137,8 +1191,8 @@ static int dispatch_quest_packed(const void* x, int64_t rows, int64_t cols, int 
     if (few)                                                                                                      \
       return launch_lane8_quest<GG, RR>(x, rows, cols, norm, codes, scales, rows, cols / 32, nullptr,             \
                                         zero_policy, stream, nullptr, true);                                      \
-    return launch_stream_packed<GG, RR, kProNone, kFmtMx, true>(x, rows, cols, norm, codes, scales, zero_policy,  \
-                                                                stream);                                          \
+    return launch_stream_packed_sized<GG, RR, kFmtMx, true>(x, rows, cols, norm, codes, scales, zero_policy,      \
+                                                            stream, nullptr);                                     \
   }
   if (rot_kind == FPQ_ROT_IDENTITY) {
     FPQ_LAUNCH_QUEST_PACKED(32, FPQ_ROT_IDENTITY);

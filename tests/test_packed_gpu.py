@@ -235,6 +235,29 @@ def test_quantize_nv_packed_bit_exact(rot, g, policy, rows):
         assert torch.equal(ps, want_s)
 
 
+@pytest.mark.parametrize("fmt,rot,g", [("mxfp4", "hadamard", 128), ("mxfp4", "gsr", 64), ("mxfp4", "identity", 32),
+                                       ("nvfp4", "hadamard", 16), ("nvfp4", "hadamard", 128)])
+def test_quantize_packed_from_two_to_the_24_elements(fmt, rot, g):
+    """From 2^24 elements on a lane of the packed streaming quantizer owns 64 elements instead of 32: equal to
+    re-tiling the row-major quantizer's result (itself checked against the oracle at this size), ragged last
+    row tile, rows with exponents outside the fast range."""
+    rows, cols = 4100, 4096
+    gen = torch.Generator().manual_seed(g + len(rot))
+    x = (torch.randn(rows, cols, generator=gen) * 3).to(torch.bfloat16)
+    x[7] *= 2.0 ** -110
+    x[9] *= 2.0 ** 105
+    x[11, 64:96] = 0.0
+    if fmt == "mxfp4":
+        rc, rs = capi.quantize(x, fmt, rot=rot, g=g)
+        want_c, want_s = pack_by_definition(rc, rs, cols)
+        pc, ps = capi.quantize_packed(x, rot=rot, g=g)
+    else:
+        rc, rs = capi.quantize(x, fmt, rot=rot, g=g, global_scale=25.0)
+        want_c, want_s = pack_nv_by_definition(rc, rs, cols)
+        pc, ps = capi.quantize_nv_packed(x, 25.0, rot=rot, g=g)
+    assert torch.equal(pc, want_c) and torch.equal(ps, want_s)
+
+
 def test_quantize_nv_packed_large_matches_row_major_path():
     gen = torch.Generator().manual_seed(6)
     x = (torch.randn(1000, 4096, generator=gen) * 3).to(torch.bfloat16)

@@ -163,6 +163,10 @@ def test_quest_streaming_kernel_from_two_to_the_24_elements(rot, g):
     wc, ws, _, _ = O.quantize_mx_quest(x, OK[rot], g, norm)
     codes, scales, _ = capi.quantize_quest(x, rot=rot, g=g, norm=norm, want_mask=False)
     assert torch.equal(scales, ws) and torch.equal(codes, wc)
+    from test_packed_gpu import pack_by_definition
+    want_c, want_s = pack_by_definition(wc, ws, cols)
+    pc, ps = capi.quantize_quest_packed(x, rot=rot, g=g, norm=norm)
+    assert torch.equal(pc, want_c) and torch.equal(ps, want_s)
 
 
 @pytest.mark.parametrize("rot,g", STREAM_CASES)
