@@ -618,3 +618,10 @@ extern "C" int fpq_gemm_nvf4_packed(const void* xq, const void* xs, const void* 
                                     int64_t N, int64_t K, void* stream) {
   return fpq::gemm_packed<true>(xq, xs, wq, ws, alpha, bias, y, M, N, K, stream);
 }
+
+extern "C" int fpq_gemm_nvf4_packed_residual(const void* xq, const void* xs, const void* wq, const void* ws,
+                                             const float* alpha, const void* bias, const void* residual, void* y,
+                                             int64_t M, int64_t N, int64_t K, void* stream) {
+  if (!residual) return FPQ_E_NULL;
+  return fpq::gemm_packed<true>(xq, xs, wq, ws, alpha, bias, y, M, N, K, stream, residual);
+}

@@ -273,6 +273,12 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
             xp, xsp = qa.packed()
             if packed is None:
                 wp, wsp = packed_weight(wq, ws, True)
+            if residual is not None:
+                st = lib.fpq_gemm_nvf4_packed_residual(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
+                                                       alpha.data_ptr(), b_ptr, residual.data_ptr(), y.data_ptr(),
+                                                       m, n, k, stream)
+                _engine.check(st, "fpq_gemm_nvf4_packed_residual")
+                return y
             st = lib.fpq_gemm_nvf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
                                           alpha.data_ptr(), b_ptr, y.data_ptr(), m, n, k, stream)
             _engine.check(st, "fpq_gemm_nvf4_packed")

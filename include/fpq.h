@@ -378,6 +378,11 @@ int fpq_unpack_nvf4(const void* packed_codes, const void* packed_scales, int64_t
 int fpq_gemm_nvf4_packed(const void* xq_packed, const void* xs_packed, const void* wq_packed,
                          const void* ws_packed, const float* alpha, const void* bias, void* y,
                          int64_t M, int64_t N, int64_t K, void* stream);
+/* fpq_gemm_nvf4_packed with the residual addition of fpq_gemm_mxf4_packed_residual (same rounding, `residual` may be `y`). */
+int fpq_gemm_nvf4_packed_residual(const void* xq_packed, const void* xs_packed, const void* wq_packed,
+                                  const void* ws_packed, const float* alpha, const void* bias,
+                                  const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                                  void* stream);
 /*
  * fpq_quantize_nv writing the packed layout directly (same codes and scale bytes; rows past `rows`
  * in the last 32-row tile get zero codes and zero scale bytes).  cols % 256 == 0; rotations as for

@@ -231,16 +231,25 @@ def pack_nv(codes, scales, fill=0xCD):
     return pc.cpu(), ps.cpu()
 
 
-def gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=None):
-    """fpq_gemm_nvf4_packed on packed operands; bf16 [M, N] on the CPU."""
+def gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=None, residual=None, in_place=False):
+    """fpq_gemm_nvf4_packed (with `residual`: fpq_gemm_nvf4_packed_residual, `in_place`: writing over the
+    residual tensor) on packed operands; bf16 [M, N] on the CPU."""
     lib = _engine.lib()
     xp, xsp, wp, wsp = (t.to("cuda").contiguous() for t in (xp, xsp, wp, wsp))
     y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     a = torch.tensor([alpha], dtype=torch.float32, device="cuda")
     b = bias.to("cuda").contiguous() if bias is not None else None
-    st = lib.fpq_gemm_nvf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(), a.data_ptr(),
-                                  b.data_ptr() if b is not None else None, y.data_ptr(), m, n, k,
-                                  torch.cuda.current_stream().cuda_stream)
+    bp = b.data_ptr() if b is not None else None
+    stream = torch.cuda.current_stream().cuda_stream
+    if residual is not None:
+        r = residual.to("cuda").contiguous().clone()
+        if in_place:
+            y = r
+        st = lib.fpq_gemm_nvf4_packed_residual(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
+                                               a.data_ptr(), bp, r.data_ptr(), y.data_ptr(), m, n, k, stream)
+    else:
+        st = lib.fpq_gemm_nvf4_packed(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(), a.data_ptr(),
+                                      bp, y.data_ptr(), m, n, k, stream)
     _engine.check(st, "fpq_gemm_nvf4_packed")
     torch.cuda.synchronize()
     return y.cpu()

@@ -190,6 +190,11 @@ def test_gemm_nv_packed_matches_oracle(m, n, k, bias):
     assert ((y.double() - want.double()).abs() <= tol).all()
     exact = (y.view(torch.int16) == want.view(torch.int16)).double().mean()
     assert exact > 0.97
+    # the residual epilogue is the separate bf16 addition, bit for bit, also written in place
+    res = (torch.randn(m, n, generator=g) * 4).to(torch.bfloat16)
+    yr = capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=b, residual=res)
+    assert torch.equal(yr, y + res)
+    assert torch.equal(capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=b, residual=res, in_place=True), yr)
 
 
 @pytest.mark.parametrize("m,n,k", [(32, 32, 256), (65, 100, 256), (300, 520, 768), (256, 4096, 512), (2048, 1024, 512)])
