@@ -295,6 +295,33 @@ def _quantized_linear(fmt, g, k, n, seed, bias=False):
     return lin
 
 
+@pytest.mark.parametrize("fmt,g,m", [("mxfp4", 128, 5), ("mxfp4", 32, 200), ("nvfp4", 16, 8), ("nvfp4", 16, 300)])
+def test_activations_quantized_into_one_layout_serve_the_other(fmt, g, m):
+    """Quantized activations held in the packed layout only feed a GEMM on row-major operands (they are
+    re-tiled back, exactly) and the other way round: same output bits as quantizing for that layout."""
+    from fp_quant import _engine
+    from fp_quant.module import eager, hip_ops
+    k, n = 512, 384
+    lin = _quantized_linear(fmt, g, k, n, seed=11, bias=True)
+    nv = fmt == "nvfp4"
+    x = torch.randn(m, k, device="cuda", dtype=torch.bfloat16)
+    stream = torch.cuda.current_stream().cuda_stream
+    h = hip_ops.as_bf16(lin.forward_hadamard_matrix)
+    kind, norm = _engine.classify_rotation(h)
+    alpha = eager.linear_alpha(lin.weight_global_scale, lin.act_global_scale)
+    ags = lin.act_global_scale if nv else None
+    with torch.no_grad():
+        packed = eager.quantize_activations(x, h, kind, norm, ags, nv, stream, True)
+        rows = eager.quantize_activations(x, h, kind, norm, ags, nv, stream, False)
+        assert packed.row_major is None and rows.row_major is not None
+        assert rows.mx_packed is None and rows.nv_packed is None
+        want_rows = eager.linear_on(rows, lin.qweight, lin.scales, alpha, lin.bias, stream, False)
+        want_packed = eager.linear_on(packed, lin.qweight, lin.scales, alpha, lin.bias, stream, True)
+        assert torch.equal(eager.linear_on(packed, lin.qweight, lin.scales, alpha, lin.bias, stream, False), want_rows)
+        assert torch.equal(eager.linear_on(rows, lin.qweight, lin.scales, alpha, lin.bias, stream, True), want_packed)
+        assert torch.equal(packed.rows()[0], rows.row_major[0]) and torch.equal(packed.rows()[1], rows.row_major[1])
+
+
 @pytest.mark.parametrize("fmt,g,m", [("mxfp4", 128, 1), ("mxfp4", 32, 200), ("nvfp4", 16, 8), ("nvfp4", 16, 100),
                                      ("nvfp4", 64, 700)])
 def test_layers_sharing_an_input_share_its_quantization(fmt, g, m):
