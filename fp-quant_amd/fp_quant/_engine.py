@@ -2,6 +2,7 @@
 
 There is no fallback: if the library is missing or fails to load, every call raises.
 """
+import contextlib
 import ctypes
 import os
 import threading
@@ -119,6 +120,16 @@ def check(status: int, what: str) -> None:
 
 
 # ---- rotation matrices: shared by the fp_quant operators and the qutlass stand-in -------------------------
+_SAME_DEVICE = contextlib.nullcontext()
+
+
+def on_device(dev):
+    """`with on_device(dev):` -- torch.cuda.device(dev) when another GPU is current, else a context that does
+    nothing (entering the real one costs several microseconds of host time per call)."""
+    import torch
+    return _SAME_DEVICE if torch.cuda.current_device() == dev.index else torch.cuda.device(dev)
+
+
 def tensor_version(t):
     """The tensor's in-place modification counter, or None for tensors created under
     torch.inference_mode(), which have none."""

@@ -24,6 +24,7 @@ from .hip_ops import (
     classify_rotation,
     is_packed_only,
     nv_packed_eligible,
+    on_device,
     pack_mxf4,
     pack_nvf4,
     packed_linear_eligible,
@@ -326,7 +327,7 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
         raise ValueError("fp_quant HIP operators need tensors on a GPU; there is no CPU path")
     dev = x_flat.device
     if torch.cuda.current_device() != dev.index:
-        with torch.cuda.device(dev):
+        with on_device(dev):
             return linear_w4a4(x_flat, hadamard_matrix, wq, ws, alpha, act_global_scale, bias, nvfp4, shared_source,
                                residual, remember, quest)
     stream = _current_stream(dev.index)
@@ -430,7 +431,7 @@ def weight_group(members, create: bool = False, nvfp4: bool = False) -> Optional
     group.n, group.splits, group.k, group.nvfp4 = n, splits, k, nvfp4
     scales_bytes = lib.fpq_packed_scales_bytes_nv if nvfp4 else lib.fpq_packed_scales_bytes
     pack = lib.fpq_pack_nvf4 if nvfp4 else lib.fpq_pack_mxf4
-    with torch.cuda.device(dev):
+    with on_device(dev):
         stream = _current_stream(dev.index)
         if packed_only:
             # the members' buffers laid end to end; the members then live in the new buffers (views) and
@@ -496,7 +497,7 @@ def linear_cat(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, group: Weigh
     scale (NVFP4 groups)."""
     dev = x_flat.device
     if torch.cuda.current_device() != dev.index:
-        with torch.cuda.device(dev):
+        with on_device(dev):
             return linear_cat(x_flat, hadamard_matrix, group, alpha, shared_source, remember, act_global_scale)
     stream = _current_stream(dev.index)
     h = as_bf16(hadamard_matrix)
@@ -529,7 +530,7 @@ def linear_cat_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wp: 
     if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_contiguous() or bias.numel() != n):
         raise ValueError("bias must be a contiguous bfloat16 vector of sum(splits) elements")
     dev = x.device
-    with torch.cuda.device(dev):
+    with on_device(dev):
         stream = _current_stream(dev.index)
         h = as_bf16(hadamard_matrix)
         kind, norm = classify_rotation(h)
@@ -563,7 +564,7 @@ def linear_group_w4a4_op(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq
     if not (len(wss) == len(weight_global_scales) == len(act_global_scales) == len(biases) == n_layers) or not n_layers:
         raise ValueError("one entry per layer is needed in every list")
     dev = x.device
-    with torch.cuda.device(dev):
+    with on_device(dev):
         stream = _current_stream(dev.index)
         h = as_bf16(hadamard_matrix)
         kind, norm = classify_rotation(h)
@@ -607,7 +608,7 @@ def silu_mul_linear_w4a4_op(gate: torch.Tensor, up: torch.Tensor, hadamard_matri
     if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_contiguous()):
         raise ValueError("bias must be a contiguous bfloat16 vector")
     dev = gate.device
-    with torch.cuda.device(dev):
+    with on_device(dev):
         alpha = linear_alpha(weight_global_scale, act_global_scale, remember=False)
         use_packed = ready and weight_wants_packed(wq, qa.m, qa.k, nvfp4)
         return linear_on(qa, wq, ws, alpha, bias, _current_stream(dev.index), use_packed)
@@ -728,7 +729,7 @@ def rmsnorm_quantize(x: torch.Tensor, weight: torch.Tensor, eps: float, hadamard
     if rows == 0 or weight.numel() != cols:
         return None
     dev = x.device
-    with torch.cuda.device(dev):
+    with on_device(dev):
         stream = _current_stream(dev.index)
         h = as_bf16(hadamard_matrix)
         kind, norm = classify_rotation(h)
@@ -785,7 +786,7 @@ def silu_mul_quantize(gate: torch.Tensor, up: torch.Tensor, hadamard_matrix: tor
     if rows == 0:
         return None
     dev = gate.device
-    with torch.cuda.device(dev):
+    with on_device(dev):
         stream = _current_stream(dev.index)
         h = as_bf16(hadamard_matrix)
         kind, norm = classify_rotation(h)

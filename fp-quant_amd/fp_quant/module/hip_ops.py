@@ -20,6 +20,9 @@ HAS_HIP_ENGINE = _engine.available()
 # zero-nibble policy used by the operators (see include/fpq.h)
 ZERO_NIBBLE_POLICY = _engine.ZERO_REFERENCE
 
+on_device = _engine.on_device
+
+
 def _version(t: torch.Tensor):
     """Cache key part for everything remembered per tensor: the in-place modification counter, or for
     tensors created under torch.inference_mode() (which have none) a marker -- what is remembered for
@@ -154,7 +157,7 @@ def linear_mxf4_packed_op(
         b_ptr = bias.data_ptr()
     y = torch.empty(m, n, dtype=torch.bfloat16, device=x.device)
     a = alpha.contiguous()
-    with torch.cuda.device(x.device):
+    with on_device(x.device):
         xp, xsp = quantize_mx_packed(x, hadamard_matrix)
         wp, wsp = packed_weight(wq, ws_b)
         st = _engine.lib().fpq_gemm_mxf4_packed(
@@ -194,13 +197,13 @@ def fused_quantize_mx_op(
     h = hadamard_matrix.contiguous()
     if forward_method == "quest":
         mask = torch.empty(rows, cols // 8, dtype=torch.uint8, device=x.device) if return_mask else None
-        with torch.cuda.device(x.device):
+        with on_device(x.device):
             st = _engine.lib().fpq_quantize_mx_quest(
                 x.data_ptr(), rows, cols, kind, g, norm, h.data_ptr(), codes.data_ptr(), scales.data_ptr(),
                 prow, pcol, mask.data_ptr() if mask is not None else None, ZERO_NIBBLE_POLICY, _stream(x))
         _engine.check(st, "fused_quantize_mx_op")
         return codes, scales.view(torch.float8_e8m0fnu), mask
-    with torch.cuda.device(x.device):
+    with on_device(x.device):
         st = _engine.lib().fpq_quantize_mx(
             x.data_ptr(), rows, cols, kind, g, norm, h.data_ptr(), codes.data_ptr(),
             scales.data_ptr(), prow, pcol, ZERO_NIBBLE_POLICY, _stream(x))
@@ -239,7 +242,7 @@ def fused_quantize_nv_op(
     scales = torch.empty(prow, pcol, dtype=torch.uint8, device=x.device)
     h = hadamard_matrix.contiguous()
     gs = global_scale.contiguous()
-    with torch.cuda.device(x.device):
+    with on_device(x.device):
         st = _engine.lib().fpq_quantize_nv(
             x.data_ptr(), rows, cols, kind, g, norm, h.data_ptr(), gs.data_ptr(), codes.data_ptr(),
             scales.data_ptr(), prow, pcol, ZERO_NIBBLE_POLICY, _stream(x))
@@ -272,7 +275,7 @@ def rotated_absmax(x: torch.Tensor, hadamard_matrix: torch.Tensor, amax: Optiona
         raise ValueError("amax must be a one-element float32 tensor on the device of x")
     kind, norm = classify_rotation(hadamard_matrix)
     h = as_bf16(hadamard_matrix)
-    with torch.cuda.device(x.device):
+    with on_device(x.device):
         st = _engine.lib().fpq_rotated_absmax(x.data_ptr(), rows, cols, kind, hadamard_matrix.shape[0], norm,
                                               h.data_ptr(), amax.data_ptr(), _stream(x))
     _engine.check(st, "fpq_rotated_absmax")
@@ -339,7 +342,7 @@ def unpack_fp4(pc: torch.Tensor, ps: torch.Tensor, rows: int, k: int, nvfp4: boo
     codes = torch.empty(rows, k // 2, dtype=torch.uint8, device=pc.device)
     scales = torch.empty(rows, k // group, dtype=torch.uint8, device=pc.device)
     entry = lib.fpq_unpack_nvf4 if nvfp4 else lib.fpq_unpack_mxf4
-    with torch.cuda.device(pc.device):
+    with on_device(pc.device):
         st = entry(pc.data_ptr(), ps.data_ptr(), rows, k, codes.data_ptr(), scales.data_ptr(), k // group, _stream(pc))
     _engine.check(st, "fpq_unpack_nvf4" if nvfp4 else "fpq_unpack_mxf4")
     return codes, scales
@@ -420,7 +423,7 @@ def _gemm(entry: str, x, w, xs, ws, alpha, bias: Optional[torch.Tensor], group: 
         b_ptr = bias.data_ptr()
     a = alpha.contiguous()
     if entry == "fpq_gemm_mxf4" and m >= PACKED_MIN_M and k % 256 == 0 and packed_weights_enabled():
-        with torch.cuda.device(x.device):
+        with on_device(x.device):
             wp, wsp = packed_weight(wq, ws_b)
             xp, xsp = pack_mxf4(xq, xs_b, m, k)
             st = _engine.lib().fpq_gemm_mxf4_packed(
@@ -429,7 +432,7 @@ def _gemm(entry: str, x, w, xs, ws, alpha, bias: Optional[torch.Tensor], group: 
         _engine.check(st, "fpq_gemm_mxf4_packed")
         return y
     if entry == "fpq_gemm_nvf4" and nv_packed_eligible(m, n, k):
-        with torch.cuda.device(x.device):
+        with on_device(x.device):
             wp, wsp = packed_weight(wq, ws_b, True)
             xp, xsp = pack_nvf4(xq, xs_b, m, k)
             st = _engine.lib().fpq_gemm_nvf4_packed(
@@ -437,7 +440,7 @@ def _gemm(entry: str, x, w, xs, ws, alpha, bias: Optional[torch.Tensor], group: 
                 y.data_ptr(), m, n, k, _stream(x))
         _engine.check(st, "fpq_gemm_nvf4_packed")
         return y
-    with torch.cuda.device(x.device):
+    with on_device(x.device):
         st = getattr(_engine.lib(), entry)(
             xq.data_ptr(), xs_b.data_ptr(), xs_b.shape[1], wq.data_ptr(), ws_b.data_ptr(),
             ws_b.shape[1], a.data_ptr(), b_ptr, y.data_ptr(), m, n, k, _stream(x))

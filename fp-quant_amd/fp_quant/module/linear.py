@@ -267,7 +267,7 @@ class FPQuantLinear(nn.Module):
         bias = self.bias
         fused_bias = bias if (bias is not None and bias.dtype == torch.bfloat16 and bias.is_contiguous()) else None
         in_gemm = residual is not None and (bias is None or fused_bias is not None)
-        with torch.cuda.device(self.qweight.device):
+        with hip_ops.on_device(self.qweight.device):
             y = eager.linear_on(activations, self.qweight, self.scales, alpha, fused_bias,
                                   hip_ops._current_stream(self.qweight.device.index),
                                   residual=residual.contiguous().flatten(end_dim=-2) if in_gemm else None)

@@ -75,7 +75,7 @@ def fusedQuantizeMx(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, method:
     codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=x.device)
     scales = torch.empty(prow, pcol, dtype=torch.uint8, device=x.device)
     lib = _engine.lib()
-    with torch.cuda.device(x.device):
+    with _engine.on_device(x.device):
         if method == "quest":
             mask = torch.empty(rows, cols // 8, dtype=torch.uint8, device=x.device) if return_mask else None
             st = lib.fpq_quantize_mx_quest(x.data_ptr(), rows, cols, kind, h.shape[0], norm, h.data_ptr(),
@@ -107,7 +107,7 @@ def fusedQuantizeNv(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, global_
     codes = torch.empty(*x.shape[:-1], cols // 2, dtype=torch.uint8, device=x.device)
     scales = torch.empty(prow, pcol, dtype=torch.uint8, device=x.device)
     gs = global_scale.contiguous()
-    with torch.cuda.device(x.device):
+    with _engine.on_device(x.device):
         st = _engine.lib().fpq_quantize_nv(x.data_ptr(), rows, cols, kind, h.shape[0], norm, h.data_ptr(),
                                            gs.data_ptr(), codes.data_ptr(), scales.data_ptr(), prow, pcol,
                                            _ZERO_POLICY, _stream(x))
@@ -152,7 +152,7 @@ def _matmul(entry: str, group: int, x, w, xs, ws, alpha) -> torch.Tensor:
     y = torch.empty(*x.shape[:-1], n, dtype=torch.bfloat16, device=x.device)
     a = alpha.contiguous()
     lib = _engine.lib()
-    with torch.cuda.device(x.device):
+    with _engine.on_device(x.device):
         if entry == "fpq_gemm_mxf4" and m >= _PACKED_MIN_M and k % 256 == 0 \
                 and os.environ.get("FPQ_PACKED_WEIGHTS", "1") != "0":
             wp, wsp = _packed_weight(lib, wq, ws_b, n, k)
