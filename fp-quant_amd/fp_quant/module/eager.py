@@ -127,14 +127,17 @@ def _sharing_key(x_shape, h, kind: int, norm: float, act_global_scale, stream: i
     copy of the scale (read once per buffer); an unrecognised rotation matrix only matches itself."""
     if not SHARE_ACT_QUANT or torch.is_inference_mode_enabled():
         return None   # in inference mode in-place writes to the source could not be noticed
-    capture_id = ctypes.c_ulonglong()   # per call: host threads may run layers concurrently
-    _engine.check(_engine.lib().fpq_stream_capture_id(stream, ctypes.byref(capture_id)), "fpq_stream_capture_id")
+    capture = 0
+    if torch.cuda.is_current_stream_capturing():   # (`stream` is the current stream; the cheap test first)
+        capture_id = ctypes.c_ulonglong()   # per call: host threads may run layers concurrently
+        _engine.check(_engine.lib().fpq_stream_capture_id(stream, ctypes.byref(capture_id)), "fpq_stream_capture_id")
+        capture = capture_id.value
     rot = (kind, norm, h.shape[0]) if kind != _engine.ROT_GENERAL else (kind, id(h), _version(h))
     gs = None
     if act_global_scale is not None:
         gs = cached_on(act_global_scale, "_fpq_host", (_version(act_global_scale), act_global_scale.data_ptr()),
                        lambda: float(act_global_scale))
-    return (rot, gs, stream, capture_id.value, tuple(x_shape), quest)
+    return (rot, gs, stream, capture, tuple(x_shape), quest)
 
 
 def _publish(qa: QuantizedActivations, src: torch.Tensor, key, keep) -> None:
