@@ -188,3 +188,24 @@ def test_nv_packed_large_llama_shape():
     ri, ci = _sample(gen, m, n, rows=32, cols=256)
     ref, mag = O.gemm_ref(xq[ri], xs[ri], wq[ci], ws[ci], alpha, "nvfp4")
     _assert_close(y[ri][:, ci], ref, mag, "nv packed 2048x14336x4096")
+
+
+@pytest.mark.parametrize("m", [16, 64, 128])
+def test_vocabulary_sized_output(m):
+    """A vocabulary-sized N (4008 weight tiles; an `lm_head` if someone quantizes it) on the weight-streaming
+    kernel with one and with two weight tiles per workgroup, and on the tile kernel: a sample of columns that
+    includes the last ones, against the oracle."""
+    n, k = 128256, 512
+    g = torch.Generator().manual_seed(m)
+    xq = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=g)
+    wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=g)
+    xs = torch.randint(118, 134, (m, k // 32), dtype=torch.uint8, generator=g)
+    ws = torch.randint(118, 134, (n, k // 32), dtype=torch.uint8, generator=g)
+    xp, xsp = pack_by_definition(xq, xs, k)
+    wp, wsp = capi.pack(wq, ws)
+    y = capi.gemm_packed(xp, xsp, wp, wsp, m, n, k, ALPHA_MX)
+    assert not torch.isnan(y.float()).any()
+    ci = torch.cat([torch.tensor([0, 31, 32, 63, 64, n - 65, n - 64, n - 33, n - 32, n - 1]),
+                    torch.randperm(n, generator=g)[:1024]]).unique()
+    ref, mag = O.gemm_ref(xq, xs, wq[ci], ws[ci], ALPHA_MX, "mxfp4")
+    _assert_close(y[:, ci], ref, mag, f"N = {n}, M = {m}")
