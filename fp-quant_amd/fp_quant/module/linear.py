@@ -271,7 +271,7 @@ class FPQuantLinear(nn.Module):
             y = eager.linear_on(activations, self.qweight, self.scales, alpha, fused_bias,
                                   hip_ops._current_stream(self.qweight.device.index),
                                   residual=residual.contiguous().flatten(end_dim=-2) if in_gemm else None)
-        y = y.unflatten(dim=0, sizes=tuple(leading_shape))
+        y = y.view(*leading_shape, y.shape[-1])
         if bias is not None and fused_bias is None:
             y += bias
         if residual is not None and not in_gemm:

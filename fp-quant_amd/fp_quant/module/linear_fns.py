@@ -108,7 +108,7 @@ class FPQuant4x16NoMasterFn(Function):
             # alpha is evaluated in the buffers' dtype, as the reference does (bf16 buffers round 1/9)
             y = forward_gemm(x_q, weight_q, x_scales, weight_scales,
                              linear_alpha_op(weight_global_scale, act_global_scale), dtype, fused_bias)
-        y = y.unflatten(dim=0, sizes=x.shape[:-1])
+        y = y.view(*x.shape[:-1], y.shape[-1])
         if bias is not None and fused_bias is None:
             y += bias
         if residual is not None and not residual_done:

@@ -385,7 +385,8 @@ def _eager_group_linear(owner: nn.Module, layers, x: torch.Tensor):
     outs = eager.linear_cat(x_flat, first.forward_hadamard_matrix, group,
                             eager.linear_alpha(first.weight_global_scale, first.act_global_scale), shared_source=x,
                             act_global_scale=first.act_global_scale)
-    return [o.unflatten(0, tuple(x.shape[:-1])) for o in outs]
+    lead = x.shape[:-1]
+    return [o.view(*lead, o.shape[-1]) for o in outs]
 
 
 def _qkv(attn, hidden_states):
