@@ -390,7 +390,8 @@ class WeightGroup:
 
 
 def _member_key(wq: torch.Tensor, ws: torch.Tensor, bias: Optional[torch.Tensor]):
-    return (wq.data_ptr(), _version(wq), ws.data_ptr(), _version(ws), tuple(wq.shape),
+    # (a tensor of another shape has another address or another counter: the shape itself need not be compared)
+    return (wq.data_ptr(), _version(wq), ws.data_ptr(), _version(ws),
             None if bias is None else (bias.data_ptr(), _version(bias)))
 
 
@@ -727,7 +728,7 @@ def rmsnorm_quantize(x: torch.Tensor, weight: torch.Tensor, eps: float, hadamard
     fused kernel; the caller then normalises as usual."""
     if not x.is_cuda or x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
         return None
-    x_flat = x.contiguous().view(-1, x.shape[-1])
+    x_flat = (x if x.is_contiguous() else x.contiguous()).view(-1, x.shape[-1])
     rows, cols = x_flat.shape
     if rows == 0 or weight.numel() != cols:
         return None

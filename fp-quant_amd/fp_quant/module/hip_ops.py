@@ -27,8 +27,10 @@ def _version(t: torch.Tensor):
     """Cache key part for everything remembered per tensor: the in-place modification counter, or for
     tensors created under torch.inference_mode() (which have none) a marker -- what is remembered for
     those is only dropped by drop_tensor_caches, which FPQuantLinear runs after load_state_dict."""
-    v = _engine.tensor_version(t)
-    return "no-counter" if v is None else v
+    try:
+        return t._version
+    except RuntimeError:
+        return "no-counter"
 
 
 _TENSOR_CACHES = ("_fpq_rotation", "_fpq_bf16", "_fpq_packed", "_fpq_group", "_fpq_alpha", "_fpq_f32", "_fpq_host")

@@ -39,10 +39,18 @@ from torch import nn
 from .config import FPQuantDtype
 
 
-def _eager():
-    from ..module import eager
+_eager_module = None
 
-    return eager
+
+def _eager():
+    """fp_quant.module.eager, imported on first use (it needs the built library) and remembered: the import
+    statement alone costs most of a microsecond per call."""
+    global _eager_module
+    if _eager_module is None:
+        from ..module import eager
+
+        _eager_module = eager
+    return _eager_module
 
 
 def _is_real_quant_linear(layer) -> bool:
