@@ -171,16 +171,29 @@ __global__ __launch_bounds__(64 * NW, (NT == 2 || (MT >= 3 && DB == 1)) ? 2 : 1)
   };
   static_assert(DB >= 1 && DB <= 4, "at most four blocks in flight");
 
-  for_slots([&](auto slot) { load_block(slot, decltype(slot)::value); });
+  // With a ring of two or more blocks the loads of a slot and the matrix instructions of the next must stay
+  // in program order: left alone, the instruction scheduler groups the loads of all slots (weights first,
+  // then scales and activations), and since loads complete in order the wait for one slot's last operand
+  // then covers the other slots' weights as well -- the ring degenerates into load everything, wait for
+  // everything, compute everything (M = 1, N = 14336: 8.4 against 7.8 us from HBM; it also takes 40 registers
+  // more).  The variants with one block in flight rely on that freedom and are left to the scheduler.
+  constexpr bool kOrdered = NT == 1 && MT <= 2 && DB >= 2;
+  for_slots([&](auto slot) {
+    load_block(slot, decltype(slot)::value);
+    if constexpr (kOrdered) __builtin_amdgcn_sched_barrier(0);
+  });
   int t0 = 0;
   for (; t0 + 2 * DB <= nblk; t0 += DB) {   // steady state: the block DB ahead exists
     for_slots([&](auto slot) {
       compute_block(slot);
+      if constexpr (kOrdered) __builtin_amdgcn_sched_barrier(0);
       load_block(slot, t0 + DB + decltype(slot)::value);
+      if constexpr (kOrdered) __builtin_amdgcn_sched_barrier(0);
     });
   }
   for_slots([&](auto slot) {                // the ring's last full or partial content
     if (t0 + decltype(slot)::value < nblk) compute_block(slot);
+    if constexpr (kOrdered) __builtin_amdgcn_sched_barrier(0);
   });
   if (nblk - t0 > DB) {                     // up to DB - 1 blocks more
     for_slots([&](auto slot) { load_block(slot, t0 + DB + decltype(slot)::value); });
@@ -381,9 +394,8 @@ static int launch_stream(const void* xq, const void* xs, const void* wq, const v
   const bool shallow = !NV && K <= 4096;
   switch (mt) {
     case 1:
-      // enough workgroups for three per CU: two blocks in flight per wave (98 registers, three
-      // workgroups per CU) beat four (200 registers, two per CU) by 4-5 %; with fewer workgroups the
-      // deeper ring of each wave is what keeps the memory system busy
+      // enough workgroups for three per CU: two blocks in flight per wave beat four by 3-5 %; with fewer
+      // workgroups the deeper ring of each wave is what keeps the memory system busy
       if ((int64_t)grid.x * grid.y >= 384) FPQ_STREAM(1, 1, 2);
       else FPQ_STREAM(1, 1, 4);
       break;
