@@ -32,6 +32,7 @@ from .hip_ops import (
     packed_weight_ready,
     packed_weights_enabled,
     quantize_mx_packed,
+    splitk_workspace,
     unpack_fp4,
     weight_rows,
 )
@@ -241,11 +242,13 @@ def weight_wants_packed(wq: torch.Tensor, m: int, k: int, nvfp4: bool) -> bool:
 def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alpha: torch.Tensor,
               bias: Optional[torch.Tensor], stream: int, use_packed: Optional[bool] = None,
               residual: Optional[torch.Tensor] = None,
-              packed: Optional[Tuple[torch.Tensor, torch.Tensor, int]] = None) -> torch.Tensor:
+              packed: Optional[Tuple[torch.Tensor, torch.Tensor, int]] = None,
+              remember: bool = False) -> torch.Tensor:
     """bf16 [m, n] = alpha * dq(activations) @ dq(w).T (+ bias) on quantized activations, with the
     kernel and operand layout the shape calls for (`use_packed`: the caller's decision, if it has
     made it already).  `residual` (bf16 [m, n]) is added as a separate bf16 addition would add it:
-    inside the packed MXFP4 kernel's epilogue, by a PyTorch addition after the other kernels."""
+    inside the packed kernels' epilogue, by a PyTorch addition after the other kernels.  `remember`: the
+    call may create and keep what the layer lacks (its split-K workspace)."""
     lib = _engine.lib()
     m, k = qa.m, qa.k
     if packed is not None:   # packed MXFP4 weights of `n` rows handed in directly (a WeightGroup): wq, ws unused
@@ -298,7 +301,14 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
         pc, ps = qa.packed()
         if packed is None:
             wp, wsp = packed_weight(wq, ws)
-        if residual is not None:
+        workspace = splitk_workspace(wq, n, k, remember) if (m <= 32 and packed is None) else None
+        if workspace is not None:
+            # few weight rows and a long K at decode sizes: K split across workgroups (deterministic sum)
+            st = lib.fpq_gemm_mxf4_packed_splitk(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
+                                                 alpha.data_ptr(), b_ptr,
+                                                 residual.data_ptr() if residual is not None else None, y.data_ptr(),
+                                                 m, n, k, workspace.data_ptr(), workspace.numel(), stream)
+        elif residual is not None:
             st = lib.fpq_gemm_mxf4_packed_residual(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
                                                    alpha.data_ptr(), b_ptr, residual.data_ptr(), y.data_ptr(),
                                                    m, n, k, stream)
@@ -353,7 +363,7 @@ def linear_w4a4(x_flat: torch.Tensor, hadamard_matrix: torch.Tensor, wq: torch.T
                                   quest)
         if key is not None:
             _publish(qa, shared_source, key, h)
-    return linear_on(qa, wq, ws, alpha, bias, stream, want_packed, residual)
+    return linear_on(qa, wq, ws, alpha, bias, stream, want_packed, residual, remember=remember)
 
 
 @torch.library.custom_op("fp_quant::linear_w4a4_op", mutates_args=())

@@ -33,7 +33,8 @@ def _version(t: torch.Tensor):
         return "no-counter"
 
 
-_TENSOR_CACHES = ("_fpq_rotation", "_fpq_bf16", "_fpq_packed", "_fpq_group", "_fpq_alpha", "_fpq_f32", "_fpq_host")
+_TENSOR_CACHES = ("_fpq_rotation", "_fpq_bf16", "_fpq_packed", "_fpq_group", "_fpq_alpha", "_fpq_f32", "_fpq_host",
+                  "_fpq_splitk")
 
 
 def drop_tensor_caches(*tensors) -> None:
@@ -395,6 +396,34 @@ def packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False) -> Tu
         pass
     return pc, ps
 
+
+
+_splitk_need = {}   # (n, k) -> workspace bytes with which fpq_gemm_mxf4_packed_splitk splits K at up to 32 rows
+
+
+def splitk_workspace(wq: torch.Tensor, n: int, k: int, create: bool) -> Optional[torch.Tensor]:
+    """The workspace with which the MXFP4 GEMM of a layer [n, k] splits K across workgroups at up to 32
+    activation rows (few weight rows and a long K: a Llama down-projection), or None where it would not
+    split.  It belongs to the layer -- kept on its code tensor `wq`, zeroed once, left zeroed by every call --
+    so that the layer takes the same kernel, and gives the same bits, on every stream, eagerly, traced or
+    under a graph capture; `create`: make it now if it does not exist (never during a capture, where the
+    memory would belong to the graph).  Two calls of the SAME layer must not overlap in time on the GPU."""
+    need = _splitk_need.get((n, k))
+    if need is None:
+        need = _splitk_need[(n, k)] = int(_engine.lib().fpq_gemm_mxf4_packed_workspace_bytes(32, n, k))
+    if need == 0:
+        return None
+    hit = getattr(wq, "_fpq_splitk", None)
+    if hit is not None and hit.numel() >= need and hit.device == wq.device:
+        return hit
+    if not create or torch.cuda.is_current_stream_capturing():
+        return None
+    workspace = torch.zeros(need, dtype=torch.uint8, device=wq.device)
+    try:
+        wq._fpq_splitk = workspace
+    except (AttributeError, RuntimeError):
+        return None   # cannot be kept: a workspace per call would cost more than the split gains
+    return workspace
 
 
 def _gemm(entry: str, x, w, xs, ws, alpha, bias: Optional[torch.Tensor], group: int) -> torch.Tensor:

@@ -155,6 +155,15 @@ class FPQuantLinear(nn.Module):
             eager.prime(h, wgs, ags)
         if self._fpq_single_copy or os.environ.get("FPQ_SINGLE_WEIGHT_COPY", "0") == "1":
             self.release_row_major()
+        self._ensure_splitk_workspace()
+
+    def _ensure_splitk_workspace(self) -> None:
+        """The layer's split-K workspace (hip_ops.splitk_workspace) made now, outside any trace or capture,
+        so that every later call -- eager, traced, captured -- takes the same kernel."""
+        qweight = getattr(self, "qweight", None)
+        if (isinstance(qweight, torch.Tensor) and qweight.is_cuda and hip_ops.packed_weights_enabled()
+                and self.config.forward_dtype == FPQuantDtype.MXFP4 and self.in_features % 256 == 0):
+            hip_ops.splitk_workspace(qweight, self.out_features, self.in_features, True)
 
     # True once release_row_major has been asked for: the layer goes back to the packed layout after
     # every load_state_dict
@@ -190,6 +199,7 @@ class FPQuantLinear(nn.Module):
         self.qweight = nn.Parameter(pc, requires_grad=False)
         self.scales = nn.Parameter(ps, requires_grad=False)
         self._fpq_single_copy = True
+        self._ensure_splitk_workspace()
         return True
 
     @torch.no_grad()
@@ -202,6 +212,7 @@ class FPQuantLinear(nn.Module):
         self.qweight = nn.Parameter(codes, requires_grad=False)
         self.scales = nn.Parameter(scales, requires_grad=False)
         self._fpq_single_copy = False
+        self._ensure_splitk_workspace()
 
     def _row_major_state(self, state_dict, prefix, local_metadata):
         """state_dict() hook: a layer that holds the packed layout only hands out row-major tensors."""
@@ -270,7 +281,8 @@ class FPQuantLinear(nn.Module):
         with hip_ops.on_device(self.qweight.device):
             y = eager.linear_on(activations, self.qweight, self.scales, alpha, fused_bias,
                                   hip_ops._current_stream(self.qweight.device.index),
-                                  residual=residual.contiguous().flatten(end_dim=-2) if in_gemm else None)
+                                  residual=residual.contiguous().flatten(end_dim=-2) if in_gemm else None,
+                                  remember=True)
         y = y.view(*leading_shape, y.shape[-1])
         if bias is not None and fused_bias is None:
             y += bias

@@ -65,6 +65,69 @@ def test_linear_matches_oracle_pipeline(fmt, g, bias):
     assert rel < 0.25, rel
 
 
+@pytest.mark.parametrize("bias", [False, True])
+def test_decode_rows_on_a_long_k_split_k_across_workgroups(bias):
+    """A layer with few output features and a long K (a down-projection) owns a workspace with which its GEMM
+    splits K at up to 32 rows: oracle values, the same bits as the C entry point with a workspace of its own,
+    the same bits eagerly, under a graph capture on another stream and through the traced operator, the
+    residual taken inside the kernel, counters left at zero; more rows run the kernel that does not split."""
+    import capi
+    from fp_quant import _engine
+    from fp_quant.module import eager, hip_ops
+    from test_packed_gpu import pack_by_definition
+    k, n = 8192, 256
+    lin = _quantized_linear("mxfp4", 128, k, n, seed=21, bias=bias)
+    wsk = getattr(lin.qweight, "_fpq_splitk", None)
+    assert wsk is not None and wsk.numel() == _engine.lib().fpq_gemm_mxf4_packed_workspace_bytes(32, n, k) > 16384
+    norm = float(O.hadamard_matrix(128)[0, 0])
+    alpha = O.alpha_from_global_scales(lin.weight_global_scale.cpu(), lin.act_global_scale.cpu())
+    wq, ws = lin.qweight.cpu(), lin.scales.cpu()
+    wp, wsp = pack_by_definition(wq, ws, k)
+    b = lin.bias.detach().cpu() if bias else None
+    for m in (1, 20, 32):
+        x = torch.randn(m, k, generator=torch.Generator().manual_seed(m)).to(torch.bfloat16)
+        xq, xs, _ = O.quantize_mx(x, O.ROT_HADAMARD, 128, norm)
+        ref, mag = O.gemm_ref(xq, xs, wq, ws, alpha, "mxfp4")
+        want = ref.to(torch.bfloat16) + b if bias else ref.to(torch.bfloat16)
+        with torch.no_grad():
+            y = lin(x.cuda())
+        close = (y.cpu().double() - want.double()).abs() <= 2.0 ** -7 * want.double().abs() + 1e-5 * mag + 1e-6
+        assert close.all()
+        xp, xsp = pack_by_definition(xq, xs, k)
+        own = torch.zeros(wsk.numel(), dtype=torch.uint8, device="cuda")
+        direct = capi.gemm_packed_splitk(xp, xsp, wp, wsp, m, n, k, alpha, bias=b, workspace=own)
+        assert torch.equal(y.cpu(), direct)
+        assert not wsk[:16384].any()
+        # the traced operator and a capture on a side stream take the same kernel
+        xd = x.cuda()
+        with torch.no_grad():
+            op = eager.linear_w4a4_op(xd, lin.forward_hadamard_matrix, lin.qweight, lin.scales, lin.weight_global_scale,
+                                      lin.act_global_scale, lin.bias, False)
+            assert torch.equal(op, y)
+            graph = torch.cuda.CUDAGraph()
+            static_x = xd.clone()
+            with torch.cuda.graph(graph):
+                static_y = lin(static_x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_y, y)
+            res = torch.randn(m, n, device="cuda").to(torch.bfloat16)
+            lin._fpq_residual = res
+            assert torch.equal(lin(xd), y + res) and lin._fpq_residual is None
+    with torch.no_grad():
+        x = torch.randn(33, k, generator=torch.Generator().manual_seed(33)).to(torch.bfloat16)
+        xq, xs, _ = O.quantize_mx(x, O.ROT_HADAMARD, 128, norm)
+        xp, xsp = pack_by_definition(xq, xs, k)
+        assert torch.equal(lin(x.cuda()).cpu(), capi.gemm_packed(xp, xsp, wp, wsp, 33, n, k, alpha, bias=b))
+        # the layer keeps a workspace when its weight changes hands (packed layout only and back)
+        x = torch.randn(7, k, generator=torch.Generator().manual_seed(7)).to(torch.bfloat16).cuda()
+        want = lin(x)
+        assert lin.release_row_major() and getattr(lin.qweight, "_fpq_splitk", None) is not None
+        assert torch.equal(lin(x), want)
+        lin.restore_row_major()
+        assert getattr(lin.qweight, "_fpq_splitk", None) is not None and torch.equal(lin(x), want)
+
+
 @pytest.mark.parametrize("init", ["identity", "gsr"])
 def test_other_transform_inits(init):
     """transform_init identity / gsr go through the same operators (matrix recognised on the host)."""
