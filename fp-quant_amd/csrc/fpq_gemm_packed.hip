@@ -579,6 +579,14 @@ extern "C" int fpq_gemm_mxf4_packed_splitk(const void* xq, const void* xs, const
                                    stream);
 }
 
+extern "C" int fpq_gemm_nvf4_packed_splitk(const void* xq, const void* xs, const void* wq, const void* ws,
+                                           const float* alpha, const void* bias, const void* residual, void* y,
+                                           int64_t M, int64_t N, int64_t K, void* workspace,
+                                           int64_t workspace_bytes, void* stream) {
+  return fpq::gemm_packed<true>(xq, xs, wq, ws, alpha, bias, y, M, N, K, stream, residual, workspace,
+                                workspace ? workspace_bytes : 0);
+}
+
 namespace fpq {
 template <bool NV>
 static int gemm_packed_multi(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,

@@ -280,6 +280,15 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
             xp, xsp = qa.packed()
             if packed is None:
                 wp, wsp = packed_weight(wq, ws, True)
+            workspace = splitk_workspace(wq, n, k, remember) if (m <= 32 and packed is None) else None
+            if workspace is not None:
+                st = lib.fpq_gemm_nvf4_packed_splitk(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
+                                                     alpha.data_ptr(), b_ptr,
+                                                     residual.data_ptr() if residual is not None else None,
+                                                     y.data_ptr(), m, n, k, workspace.data_ptr(), workspace.numel(),
+                                                     stream)
+                _engine.check(st, "fpq_gemm_nvf4_packed_splitk")
+                return y
             if residual is not None:
                 st = lib.fpq_gemm_nvf4_packed_residual(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
                                                        alpha.data_ptr(), b_ptr, residual.data_ptr(), y.data_ptr(),

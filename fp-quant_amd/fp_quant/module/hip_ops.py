@@ -402,7 +402,7 @@ _splitk_need = {}   # (n, k) -> workspace bytes with which fpq_gemm_mxf4_packed_
 
 
 def splitk_workspace(wq: torch.Tensor, n: int, k: int, create: bool) -> Optional[torch.Tensor]:
-    """The workspace with which the MXFP4 GEMM of a layer [n, k] splits K across workgroups at up to 32
+    """The workspace with which the packed GEMM of a layer [n, k] (either format) splits K across workgroups at up to 32
     activation rows (few weight rows and a long K: a Llama down-projection), or None where it would not
     split.  It belongs to the layer -- kept on its code tensor `wq`, zeroed once, left zeroed by every call --
     so that the layer takes the same kernel, and gives the same bits, on every stream, eagerly, traced or

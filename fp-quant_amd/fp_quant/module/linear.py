@@ -162,7 +162,8 @@ class FPQuantLinear(nn.Module):
         so that every later call -- eager, traced, captured -- takes the same kernel."""
         qweight = getattr(self, "qweight", None)
         if (isinstance(qweight, torch.Tensor) and qweight.is_cuda and hip_ops.packed_weights_enabled()
-                and self.config.forward_dtype == FPQuantDtype.MXFP4 and self.in_features % 256 == 0):
+                and self.config.forward_dtype in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4)
+                and self.in_features % 256 == 0):
             hip_ops.splitk_workspace(qweight, self.out_features, self.in_features, True)
 
     # True once release_row_major has been asked for: the layer goes back to the packed layout after

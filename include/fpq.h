@@ -309,6 +309,12 @@ int fpq_gemm_mxf4_packed_splitk(const void* xq_packed, const void* xs_packed, co
                                 const void* ws_packed, const float* alpha, const void* bias,
                                 const void* residual, void* y, int64_t M, int64_t N, int64_t K,
                                 void* workspace, int64_t workspace_bytes, void* stream);
+/* The same for packed NVFP4 operands (fpq_gemm_nvf4_packed, with `residual` non-null fpq_gemm_nvf4_packed_residual);
+ * workspace as above, sized by fpq_gemm_mxf4_packed_workspace_bytes (the split is the same for both formats). */
+int fpq_gemm_nvf4_packed_splitk(const void* xq_packed, const void* xs_packed, const void* wq_packed,
+                                const void* ws_packed, const float* alpha, const void* bias,
+                                const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                                void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
  * One GEMM for several layers that read the same activations (the q, k and v projections of an

@@ -114,10 +114,12 @@ def quantize_packed(x_bf16, rot="hadamard", g=128, norm=None, zero_policy=_engin
     return pc.cpu(), ps.cpu()
 
 
-def gemm_packed_splitk(xp, xsp, wp, wsp, m, n, k, alpha, bias=None, residual=None, workspace=None, calls=1):
-    """fpq_gemm_mxf4_packed_splitk on packed operands with `workspace` (a CUDA uint8 tensor whose first
-    16 KB are zero, or None), `calls` times in a row on the same buffers; bf16 [M, N] on the CPU."""
+def gemm_packed_splitk(xp, xsp, wp, wsp, m, n, k, alpha, bias=None, residual=None, workspace=None, calls=1, nv=False):
+    """fpq_gemm_mxf4_packed_splitk (nv: fpq_gemm_nvf4_packed_splitk) on packed operands with `workspace` (a CUDA
+    uint8 tensor whose first 16 KB are zero, or None), `calls` times in a row on the same buffers; bf16 [M, N]
+    on the CPU."""
     lib = _engine.lib()
+    entry = lib.fpq_gemm_nvf4_packed_splitk if nv else lib.fpq_gemm_mxf4_packed_splitk
     xp, xsp, wp, wsp = (t.to("cuda").contiguous() for t in (xp, xsp, wp, wsp))
     a = torch.tensor([alpha], dtype=torch.float32, device="cuda")
     b = bias.to("cuda").contiguous() if bias is not None else None
@@ -125,12 +127,12 @@ def gemm_packed_splitk(xp, xsp, wp, wsp, m, n, k, alpha, bias=None, residual=Non
     stream = torch.cuda.current_stream().cuda_stream
     for _ in range(calls):
         y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
-        st = lib.fpq_gemm_mxf4_packed_splitk(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
-                                             a.data_ptr(), b.data_ptr() if b is not None else None,
-                                             r.data_ptr() if r is not None else None, y.data_ptr(), m, n, k,
-                                             workspace.data_ptr() if workspace is not None else None,
-                                             workspace.numel() if workspace is not None else 0, stream)
-        _engine.check(st, "fpq_gemm_mxf4_packed_splitk")
+        st = entry(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
+                   a.data_ptr(), b.data_ptr() if b is not None else None,
+                   r.data_ptr() if r is not None else None, y.data_ptr(), m, n, k,
+                   workspace.data_ptr() if workspace is not None else None,
+                   workspace.numel() if workspace is not None else 0, stream)
+        _engine.check(st, "fpq_gemm_packed_splitk")
     torch.cuda.synchronize()
     return y.cpu()
 

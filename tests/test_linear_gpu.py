@@ -65,6 +65,37 @@ def test_linear_matches_oracle_pipeline(fmt, g, bias):
     assert rel < 0.25, rel
 
 
+def test_nvfp4_layer_with_a_long_k_owns_a_split_k_workspace():
+    """The NVFP4 counterpart of the test below, in short: workspace made at priming, oracle values, eager ==
+    traced operator == C entry point with a workspace of its own."""
+    import capi
+    from fp_quant.module import eager
+    from test_packed_gpu import pack_nv_by_definition
+    k, n, m = 8192, 256, 9
+    lin = _quantized_linear("nvfp4", 16, k, n, seed=22, bias=True)
+    wsk = getattr(lin.qweight, "_fpq_splitk", None)
+    assert wsk is not None and wsk.numel() > 16384
+    norm = float(O.hadamard_matrix(16)[0, 0])
+    alpha = O.alpha_from_global_scales(lin.weight_global_scale.cpu(), lin.act_global_scale.cpu())
+    x = torch.randn(m, k, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16)
+    xq, xs, _ = O.quantize_nv(x, float(lin.act_global_scale), O.ROT_HADAMARD, 16, norm)
+    wq, ws = lin.qweight.cpu(), lin.scales.cpu()
+    ref, mag = O.gemm_ref(xq, xs, wq, ws, alpha, "nvfp4")
+    want = ref.to(torch.bfloat16) + lin.bias.detach().cpu()
+    with torch.no_grad():
+        y = lin(x.cuda())
+        op = eager.linear_w4a4_op(x.cuda(), lin.forward_hadamard_matrix, lin.qweight, lin.scales,
+                                  lin.weight_global_scale, lin.act_global_scale, lin.bias, True)
+    assert torch.equal(op, y)
+    assert ((y.cpu().double() - want.double()).abs() <= 2.0 ** -6 * want.double().abs() + 1e-5 * mag + 1e-6).all()
+    xp, xsp = pack_nv_by_definition(xq, xs, k)
+    wp, wsp = pack_nv_by_definition(wq, ws, k)
+    own = torch.zeros(wsk.numel(), dtype=torch.uint8, device="cuda")
+    direct = capi.gemm_packed_splitk(xp, xsp, wp, wsp, m, n, k, alpha, bias=lin.bias.detach().cpu(), workspace=own,
+                                     nv=True)
+    assert torch.equal(y.cpu(), direct) and not wsk[:16384].any()
+
+
 @pytest.mark.parametrize("bias", [False, True])
 def test_decode_rows_on_a_long_k_split_k_across_workgroups(bias):
     """A layer with few output features and a long K (a down-projection) owns a workspace with which its GEMM

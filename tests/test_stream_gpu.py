@@ -106,6 +106,34 @@ def test_stream_split_k_matches_oracle_and_is_deterministic(m, n, k):
     assert torch.equal(y0, capi.gemm_packed(xp, xsp, wp, wsp, m, n, k, ALPHA))
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 32, 8192), (16, 1024, 8192), (31, 64, 16384), (17, 515, 9216), (16, 1024, 1024)])
+def test_nvfp4_split_k_matches_oracle_and_is_deterministic(m, n, k):
+    """fpq_gemm_nvf4_packed_splitk: the same split, exchange and fixed summation order on NVFP4 operands."""
+    from test_packed_gpu import pack_nv_by_definition
+    g = torch.Generator().manual_seed(m + n + k)
+    xq = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=g)
+    wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=g)
+    xs = torch.randint(0x20, 0x50, (m, k // 16), dtype=torch.uint8, generator=g)
+    ws = torch.randint(0x20, 0x50, (n, k // 16), dtype=torch.uint8, generator=g)
+    alpha = 2.0 ** -6
+    xp, xsp = pack_nv_by_definition(xq, xs, k)
+    wp, wsp = pack_nv_by_definition(wq, ws, k)
+    need, wspace = _workspace(m, n, k)
+    y = capi.gemm_packed_splitk(xp, xsp, wp, wsp, m, n, k, alpha, workspace=wspace, nv=True)
+    ref, mag = O.gemm_ref(xq, xs, wq, ws, alpha, "nvfp4")
+    assert not torch.isnan(y.float()).any()
+    assert ((y.double() - ref).abs() <= 2.0 ** -8 * ref.abs() + 1e-5 * mag + 1e-6).all()
+    assert int(wspace[:16384].max()) == 0
+    again = capi.gemm_packed_splitk(xp, xsp, wp, wsp, m, n, k, alpha, workspace=wspace, calls=4, nv=True)
+    assert torch.equal(again.view(torch.int16), y.view(torch.int16)) and int(wspace[:16384].max()) == 0
+    b = torch.randn(n, generator=g).to(torch.bfloat16)
+    res = (torch.randn(m, n, generator=g) * 8).to(torch.bfloat16)
+    yr = capi.gemm_packed_splitk(xp, xsp, wp, wsp, m, n, k, alpha, bias=b, residual=res, workspace=wspace, nv=True)
+    assert torch.equal(yr, (y + b) + res)
+    y0 = capi.gemm_packed_splitk(xp, xsp, wp, wsp, m, n, k, alpha, nv=True)     # no workspace: the plain entry
+    assert torch.equal(y0, capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha))
+
+
 def test_split_k_is_taken_for_few_weight_rows_and_long_k():
     need = _engine.lib().fpq_gemm_mxf4_packed_workspace_bytes
     assert need(16, 4096, 14336) == 16384 + 2 * 128 * 4096   # 128 weight tiles, 56 blocks: two parts
