@@ -399,6 +399,9 @@ def packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False) -> Tu
 
 
 _splitk_need = {}   # (n, k) -> workspace bytes with which fpq_gemm_mxf4_packed_splitk splits K at up to 32 rows
+# FPQ_SPLIT_K=0: no layer keeps a split-K workspace (for callers that run ONE layer object on several streams at
+# the same time, whose kernels would share it)
+SPLIT_K = os.environ.get("FPQ_SPLIT_K", "1") != "0"
 
 
 def splitk_workspace(wq: torch.Tensor, n: int, k: int, create: bool) -> Optional[torch.Tensor]:
@@ -408,6 +411,8 @@ def splitk_workspace(wq: torch.Tensor, n: int, k: int, create: bool) -> Optional
     so that the layer takes the same kernel, and gives the same bits, on every stream, eagerly, traced or
     under a graph capture; `create`: make it now if it does not exist (never during a capture, where the
     memory would belong to the graph).  Two calls of the SAME layer must not overlap in time on the GPU."""
+    if not SPLIT_K:
+        return None
     need = _splitk_need.get((n, k))
     if need is None:
         need = _splitk_need[(n, k)] = int(_engine.lib().fpq_gemm_mxf4_packed_workspace_bytes(32, n, k))
