@@ -49,8 +49,8 @@ __global__ __launch_bounds__(64 * NW, (NT == 2 || (MT >= 3 && DB == 1)) ? 2 : 1)
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias,
     const uint16_t* residual, uint16_t* y, int M, int N, int K, int bps, int ksplit,
     float* partial, unsigned* counters, const OutSegments seg) {
-  static_assert(NW == 4, "the partial sums meet in two rounds of two");
-  __shared__ v4f part[2][NT * MT][4][64];
+  static_assert(NW == 4, "three waves hand their partial sums to the first");
+  __shared__ v4f part[3][NT * MT][4][64];
   constexpr int kSB = NV ? 512 : 256;    // scale bytes per row tile and 256-K block
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int nu = K >> 6, nkb = K >> 8;
@@ -210,24 +210,18 @@ __global__ __launch_bounds__(64 * NW, (NT == 2 || (MT >= 3 && DB == 1)) ? 2 : 1)
       for (int g = 0; g < 4; ++g)
         part[slot][j][g][lane] = v4f{acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]};
   };
-  auto take = [&](int slot) __attribute__((always_inline)) {
-#pragma unroll
-    for (int j = 0; j < NT * MT; ++j)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const v4f p = part[slot][j][g][lane];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) acc[j][4 * g + q] += p[q];
-      }
-  };
-  if (wave >= 2) put(wave - 2);
-  __syncthreads();
-  if (wave < 2) take(wave);
-  __syncthreads();
-  if (wave == 1) put(0);
+  // waves 1-3 hand their partial tiles to wave 0 through LDS (one barrier); wave 0 adds them as stated
+  if (wave != 0) put(wave - 1);
   __syncthreads();
   if (wave != 0) return;
-  take(0);
+#pragma unroll
+  for (int j = 0; j < NT * MT; ++j)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const v4f p1 = part[0][j][g][lane], p2 = part[1][j][g][lane], p3 = part[2][j][g][lane];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) acc[j][4 * g + q] = (acc[j][4 * g + q] + p2[q]) + (p1[q] + p3[q]);
+    }
 
   // ---- K split across workgroups: partial tiles through the workspace, last arrival finishes
   if (ksplit > 1) {
