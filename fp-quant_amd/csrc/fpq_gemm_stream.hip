@@ -55,6 +55,7 @@ __global__ __launch_bounds__(64 * NW, (NT == 2 || (MT >= 3 && DB == 1)) ? 2 : 1)
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int nu = K >> 6, nkb = K >> 8;
   const int rtg = blockIdx.x, split = blockIdx.y;
+  const float alpha = *alpha_p;   // asked for now: the epilogue, on the critical path of every workgroup, finds it there
   const int rt_n = (N + 31) >> 5;
   const int kb_begin = split * bps, kb_end = min(nkb, kb_begin + bps);
   const int first = kb_begin + wave;                                   // this wave: first, first + NW, ...
@@ -258,7 +259,6 @@ __global__ __launch_bounds__(64 * NW, (NT == 2 || (MT >= 3 && DB == 1)) ? 2 : 1)
 
   // ---- y[m][n] = bf16(alpha * acc) (+ bias) (+ residual, a further bf16 add): register 4g + q of
   // tile (i, j) is m = 32 j + lane % 32, n = 32 (NT rtg + i) + 8 g + 4 (lane / 32) + q
-  const float alpha = *alpha_p;
   const int r32 = lane & 31, kh = lane >> 5;
 #pragma unroll
   for (int ig = 0; ig < NT * 4; ++ig) {
