@@ -37,14 +37,13 @@ constexpr int kStreamMaxRows = 128;
 
 // NT weight row tiles per workgroup, MT activation row tiles (exactly ceil(M / 32)), DB 256-K blocks
 // of loads in flight per wave, NW waves.  Every workgroup re-reads all activations (NT = 2 halves
-// that, at a register cost that stream_plan explains).  Two weight tiles per workgroup, and three or
-// four activation row tiles with one block in flight, are compiled for two workgroups per CU (at most
-// 256 registers): left alone the compiler takes more and one workgroup fills the CU.
+// that, at a register cost that stream_plan explains).  Two weight tiles per workgroup are compiled for
+// two workgroups per CU (at most 256 registers).
 // NV: NVFP4 operands (two E4M3 scale bytes per lane and K step, 512-byte scale blocks): a lane's dword s
 // of a 64-K unit, times its group's scale, is its fp16 operand of the s-th 32x32x16 matrix instruction
 // of the unit on both sides, so the K order is permuted consistently and the sum is complete.
 template <int NT, int MT, int DB, int NW, bool NV = false>
-__global__ __launch_bounds__(64 * NW, (NT == 2 || (MT >= 3 && DB == 1)) ? 2 : 1) void gemm_fp4_stream_kernel(
+__global__ __launch_bounds__(64 * NW, NT == 2 ? 2 : 1) void gemm_fp4_stream_kernel(
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias,
     const uint16_t* residual, uint16_t* y, int M, int N, int K, int bps, int ksplit,
@@ -177,12 +176,35 @@ __global__ __launch_bounds__(64 * NW, (NT == 2 || (MT >= 3 && DB == 1)) ? 2 : 1)
   // then scales and activations), and since loads complete in order the wait for one slot's last operand
   // then covers the other slots' weights as well -- the ring degenerates into load everything, wait for
   // everything, compute everything (M = 1, N = 14336: 8.4 against 7.8 us from HBM; it also takes 40 registers
-  // more).  The variants with one block in flight rely on that freedom and are left to the scheduler.
-  constexpr bool kOrdered = NT == 1 && MT <= 2 && DB >= 2;
+  // more).  With three or four activation row tiles the effect is within +-4 % either way; only four tiles
+  // of NVFP4 gain throughout (128 rows, N = 4096: 15.1 -> 14.6 us).  One block in flight has nothing to order.
+  constexpr bool kOrdered = NT == 1 && DB >= 2 && (MT <= 2 || (NV && MT == 4));
   for_slots([&](auto slot) {
     load_block(slot, decltype(slot)::value);
     if constexpr (kOrdered) __builtin_amdgcn_sched_barrier(0);
   });
+  // Where the epilogue will store, worked out while the first loads are in flight (after the reduction
+  // every instruction delays the workgroup's end).  The epilogue's lane layout: 8 consecutive columns
+  // (16 bytes) of row lane / 4 and of that row + 16.  16-byte accesses need the whole tile inside N and
+  // aligned rows and bases (a residual never comes with segments: one output, its rows N long).
+  const int row16 = lane >> 2, c = lane & 3;
+  int res_rows = __builtin_amdgcn_readfirstlane(residual && (N & 7) == 0 && ((uintptr_t)residual & 15) == 0);
+  const uint16_t* res_src = residual + (size_t)row16 * N + rtg * NT * 32 + 8 * c;
+  uint16_t* out_dst[NT];
+  int out_ld[NT], out_whole[NT];
+#pragma unroll
+  for (int i = 0; i < NT; ++i) {
+    const int tn0 = (rtg * NT + i) * 32;
+    const OutView out = out_view(seg, y, nullptr, tn0, N);   // the matrix this tile's columns go to (unused past N)
+    out_ld[i] = __builtin_amdgcn_readfirstlane(out.N);
+    out_dst[i] = out.y + (size_t)row16 * out.N + out.n0 + 8 * c;
+    out_whole[i] = __builtin_amdgcn_readfirstlane(tn0 + 32 <= N && (out.N & 7) == 0 && ((uintptr_t)out.y & 15) == 0 &&
+                                                  (!residual || res_rows));
+    // (values the compiler may not look through: it would otherwise move their computation, kernel
+    // argument loads included, to their first use behind the reduction)
+    if constexpr (NT == 1) asm volatile("" : "+s"(out_ld[i]), "+s"(out_whole[i]), "+v"(out_dst[i]));
+  }
+  if constexpr (NT == 1) asm volatile("" : "+s"(res_rows), "+v"(res_src));
   int t0 = 0;
   for (; t0 + 2 * DB <= nblk; t0 += DB) {   // steady state: the block DB ahead exists
     for_slots([&](auto slot) {
@@ -215,6 +237,20 @@ __global__ __launch_bounds__(64 * NW, (NT == 2 || (MT >= 3 && DB == 1)) ? 2 : 1)
   if (wave != 0) put(wave - 1);
   __syncthreads();
   if (wave != 0) return;
+  // The rows of the residual this wave will add are asked for now: they arrive during the reduction.
+  uint4 rv[NT][MT][2];
+  if (res_rows) {
+#pragma unroll
+    for (int i = 0; i < NT; ++i)
+#pragma unroll
+      for (int j = 0; j < MT; ++j)
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          const int m = j * 32 + 16 * p + row16, n = (rtg * NT + i) * 32 + 8 * c;
+          rv[i][j][p] = m < M && n < N ? *(const uint4*)(res_src + (size_t)(j * 32 + 16 * p) * N + 32 * i)
+                                       : make_uint4(0, 0, 0, 0);
+        }
+  }
 #pragma unroll
   for (int j = 0; j < NT * MT; ++j)
 #pragma unroll
@@ -258,53 +294,98 @@ __global__ __launch_bounds__(64 * NW, (NT == 2 || (MT >= 3 && DB == 1)) ? 2 : 1)
   }
 
   // ---- y[m][n] = bf16(alpha * acc) (+ bias) (+ residual, a further bf16 add): register 4g + q of
-  // tile (i, j) is m = 32 j + lane % 32, n = 32 (NT rtg + i) + 8 g + 4 (lane / 32) + q
+  // tile (i, j) is m = 32 j + lane % 32, n = 32 (NT rtg + i) + 8 g + 4 (lane / 32) + q.  Stored from
+  // there, an instruction would write 16 bytes into each of 32 rows; so many small pieces cost 5-8 %
+  // of the whole kernel (M = 16, N = 14336: 8.0 -> 7.6 us; M = 64: 11.3 -> 10.4 us).  The rounded tile
+  // goes through LDS instead -- the buffer of the partial sums, which only this wave still uses --
+  // and comes back with a lane holding 8 consecutive columns: 64 contiguous bytes per row and store.
   const int r32 = lane & 31, kh = lane >> 5;
+  constexpr int kStageRow = 20;   // dwords: 16 of a row's 32 bf16 + 4, rows stay 16-byte aligned
+  uint32_t* stage = (uint32_t*)&part[0][0][0][0];
+  static_assert(sizeof(part[0][0]) >= 32 * kStageRow * 4, "a staged tile fits a partial tile's place");
+  constexpr int kStageTile = sizeof(part[0][0]) / 4;
+  // (this wave alone is what the workgroup still waits for, so every instruction here is on the critical
+  // path: the case without a bias is a code path of its own rather than a select after the additions)
+  uint32_t* lane_stage = stage + r32 * kStageRow + 2 * kh;
+  if (!bias) {
 #pragma unroll
-  for (int ig = 0; ig < NT * 4; ++ig) {
-    const int i = ig >> 2, g = ig & 3;
-    const int n = (rtg * NT + i) * 32 + 8 * g + 4 * kh;
-    // the matrix this weight tile's columns are stored to (bias is indexed by the product's column n)
-    const OutView out = out_view(seg, y, nullptr, (rtg * NT + i) * 32, N);
-    const int ldy = out.N, nl = out.n0 + 8 * g + 4 * kh;
-    const bool vec_ok = (ldy & 3) == 0;
-    float bv[4] = {0.f, 0.f, 0.f, 0.f};
-    if (bias) {
+    for (int t = 0; t < NT * MT; ++t)
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        if (n + q < N) bv[q] = __uint_as_float((uint32_t)bias[n + q] << 16);
-    }
+      for (int g = 0; g < 4; ++g)
+        *(uint2*)(lane_stage + t * kStageTile + 4 * g) =
+            make_uint2(pack_bf16x2(acc[t][4 * g + 0] * alpha, acc[t][4 * g + 1] * alpha),
+                       pack_bf16x2(acc[t][4 * g + 2] * alpha, acc[t][4 * g + 3] * alpha));
+  } else {
 #pragma unroll
-    for (int j = 0; j < MT; ++j) {
-      const int m = j * 32 + r32;
-      if (m >= M || n >= N) continue;
-      const v16f& t = acc[i * MT + j];
-      uint32_t lo = pack_bf16x2(t[4 * g + 0] * alpha, t[4 * g + 1] * alpha);
-      uint32_t hi = pack_bf16x2(t[4 * g + 2] * alpha, t[4 * g + 3] * alpha);
-      if (bias) {
-        lo = pack_bf16x2(__uint_as_float(lo << 16) + bv[0], __uint_as_float(lo & 0xffff0000u) + bv[1]);
-        hi = pack_bf16x2(__uint_as_float(hi << 16) + bv[2], __uint_as_float(hi & 0xffff0000u) + bv[3]);
+    for (int ig = 0; ig < NT * 4; ++ig) {
+      const int i = ig >> 2, g = ig & 3;
+      const int n = (rtg * NT + i) * 32 + 8 * g + 4 * kh;   // bias is indexed by the product's column
+      float bv[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) bv[q] = n + q < N ? __uint_as_float((uint32_t)bias[n + q] << 16) : 0.f;
+#pragma unroll
+      for (int j = 0; j < MT; ++j) {
+        const v16f& t = acc[i * MT + j];
+        const uint32_t lo = pack_bf16x2(t[4 * g + 0] * alpha, t[4 * g + 1] * alpha);
+        const uint32_t hi = pack_bf16x2(t[4 * g + 2] * alpha, t[4 * g + 3] * alpha);
+        *(uint2*)(lane_stage + (i * MT + j) * kStageTile + 4 * g) =
+            make_uint2(pack_bf16x2(__uint_as_float(lo << 16) + bv[0], __uint_as_float(lo & 0xffff0000u) + bv[1]),
+                       pack_bf16x2(__uint_as_float(hi << 16) + bv[2], __uint_as_float(hi & 0xffff0000u) + bv[3]));
       }
-      uint16_t* dst = out.y + (size_t)m * ldy + nl;
-      if (vec_ok && n + 3 < N) {
-        if (residual) {   // never together with segments: one output, ldy == N and nl == n
-          const uint2 rv = *(const uint2*)(residual + (size_t)m * N + n);
-          lo = pack_bf16x2(__uint_as_float(lo << 16) + __uint_as_float(rv.x << 16),
-                           __uint_as_float(lo & 0xffff0000u) + __uint_as_float(rv.x & 0xffff0000u));
-          hi = pack_bf16x2(__uint_as_float(hi << 16) + __uint_as_float(rv.y << 16),
-                           __uint_as_float(hi & 0xffff0000u) + __uint_as_float(rv.y & 0xffff0000u));
-        }
-        *(uint2*)dst = make_uint2(lo, hi);
-      } else {
-        const uint32_t w[2] = {lo, hi};
+    }
+  }
+  // (the wave reads back what other lanes of it wrote: LDS serves one wave's accesses in order)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          if (n + q >= N) continue;
-          uint32_t h = (w[q >> 1] >> (16 * (q & 1))) & 0xffffu;
-          if (residual)
-            h = pack_bf16x2(__uint_as_float(h << 16) + __uint_as_float((uint32_t)residual[(size_t)m * N + n + q] << 16), 0.0f) & 0xffffu;
-          dst[q] = (uint16_t)h;
-        }
+  for (int i = 0; i < NT; ++i) {
+    const int tn0 = (rtg * NT + i) * 32, n = tn0 + 8 * c;
+    if (tn0 >= N) continue;
+    const int ldy = out_ld[i];
+    const uint32_t* tile = stage + i * MT * kStageTile + row16 * kStageRow + 4 * c;
+    uint16_t* dst = out_dst[i];
+    // The same for every lane, so the common case is branch-free: all staged rows are asked for at once
+    // and the stores follow.
+    const bool whole = out_whole[i];
+    if (whole) {
+      uint4 v[MT][2];
+#pragma unroll
+      for (int j = 0; j < MT; ++j)
+#pragma unroll
+        for (int p = 0; p < 2; ++p) v[j][p] = *(const uint4*)(tile + j * kStageTile + 16 * p * kStageRow);
+      if (residual) {
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+#pragma unroll
+          for (int p = 0; p < 2; ++p) {
+            const uint32_t w[4] = {v[j][p].x, v[j][p].y, v[j][p].z, v[j][p].w};
+            const uint32_t r[4] = {rv[i][j][p].x, rv[i][j][p].y, rv[i][j][p].z, rv[i][j][p].w};
+            uint32_t o[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              o[q] = pack_bf16x2(__uint_as_float(w[q] << 16) + __uint_as_float(r[q] << 16),
+                                 __uint_as_float(w[q] & 0xffff0000u) + __uint_as_float(r[q] & 0xffff0000u));
+            v[j][p] = make_uint4(o[0], o[1], o[2], o[3]);
+          }
+      }
+#pragma unroll
+      for (int j = 0; j < MT; ++j)
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+          if (j * 32 + 16 * p + row16 < M) *(uint4*)(dst + (size_t)(j * 32 + 16 * p) * ldy) = v[j][p];
+      continue;
+    }
+    if (n >= N) continue;
+    for (int jp = 0; jp < 2 * MT; ++jp) {   // N's last tile, or an unaligned output: element by element
+      const int m = 16 * jp + row16;
+      if (m >= M) continue;
+      const uint4 v = *(const uint4*)(tile + (jp >> 1) * kStageTile + 16 * (jp & 1) * kStageRow);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        if (n + q >= N) continue;
+        uint32_t h = (w[q >> 1] >> (16 * (q & 1))) & 0xffffu;
+        if (residual)
+          h = pack_bf16x2(__uint_as_float(h << 16) + __uint_as_float((uint32_t)residual[(size_t)m * N + n + q] << 16), 0.0f) & 0xffffu;
+        dst[(size_t)16 * jp * ldy + q] = (uint16_t)h;
       }
     }
   }
@@ -382,10 +463,6 @@ static int launch_stream(const void* xq, const void* xs, const void* wq, const v
     }
     return FPQ_E_UNSUPPORTED;
   }
-  // 65-128 rows of MXFP4 at K up to 4096: one block in flight per wave and two workgroups per CU beat two
-  // blocks and one workgroup (128 rows, N = 4096 / 8192: 9.7 -> 8.9 / 10.6 -> 9.8 us); a longer K prefers
-  // the deeper ring (N = 4096, K = 14336, 96 rows: 18.4 against 19.0 us)
-  const bool shallow = !NV && K <= 4096;
   switch (mt) {
     case 1:
       // enough workgroups for three per CU: two blocks in flight per wave beat four by 3-5 %; with fewer
@@ -394,23 +471,11 @@ static int launch_stream(const void* xq, const void* xs, const void* wq, const v
       else FPQ_STREAM(1, 1, 4);
       break;
     case 2: FPQ_STREAM(1, 2, 2); break;
-    case 3:
-      // (NVFP4: whatever K is -- 96 rows, N = 6144 / 4096: 13.7 -> 12.6 / 13.3 -> 12.2 us, K = 12288: 28.1 -> 27.8)
-      if (shallow || NV) {
-        FPQ_STREAM(1, 3, 1);
-        break;
-      }
-      FPQ_STREAM(1, 3, 2);
-      break;
-    default:
-      if constexpr (!NV) {
-        if (shallow) {
-          FPQ_STREAM(1, 4, 1);
-          break;
-        }
-      }
-      FPQ_STREAM(1, 4, 2);
-      break;
+    // (65-128 rows: one block in flight per wave, which fits two workgroups into a CU, measured 1-2 %
+    // slower for MXFP4 and 6-12 % slower for NVFP4 than two blocks -- 96 rows of NVFP4, N = 4096:
+    // K = 4096 12.4 against 11.5 us, K = 14336 33.7 against 29.5 us)
+    case 3: FPQ_STREAM(1, 3, 2); break;
+    default: FPQ_STREAM(1, 4, 2); break;
   }
 #undef FPQ_STREAM
   return (int)hipGetLastError();
