@@ -11,7 +11,9 @@
 //     K = 4096 and 32 rows the whole weight tile is requested at once;
 //   * activations (at most four 32-row tiles, padded rows are zero) are re-read by every workgroup
 //     and come from the L2;
-//   * the four partial tiles meet in LDS and are summed in the fixed order (w0 + w2) + (w1 + w3).
+//   * the four partial tiles meet in LDS and are summed in the fixed order (w0 + w2) + (w1 + w3), every
+//     wave a quarter of each tile; the rounded tile goes through LDS once more so that a store writes 64
+//     contiguous bytes per row, and the four waves share the stores.
 // Shapes with few weight tiles (N = 4096: 128 workgroups for 256 CUs) or long K also split K
 // ACROSS workgroups: each stores its fp32 partial tile into a workspace, a per-tile counter tells
 // the last one to arrive, and that one adds the partials of all splits in split order (its own
@@ -48,8 +50,12 @@ __global__ __launch_bounds__(64 * NW, NT == 2 ? 2 : 1) void gemm_fp4_stream_kern
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias,
     const uint16_t* residual, uint16_t* y, int M, int N, int K, int bps, int ksplit,
     float* partial, unsigned* counters, const OutSegments seg) {
-  static_assert(NW == 4, "three waves hand their partial sums to the first");
-  __shared__ v4f part[3][NT * MT][4][64];
+  static_assert(NW == 4, "a wave owns a quarter of every tile");
+  __shared__ v4f part[4][NT * MT][3][64];   // [owning wave][tile][the other waves in order][lane]
+  constexpr int kStageRow = 20;             // dwords: 16 of a row's 32 bf16 + 4, rows stay 16-byte aligned
+  constexpr int kStageTile = 32 * kStageRow;
+  __shared__ __attribute__((aligned(16))) uint32_t stage[NT * MT][kStageTile];
+  __shared__ unsigned arrival;
   constexpr int kSB = NV ? 512 : 256;    // scale bytes per row tile and 256-K block
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int nu = K >> 6, nkb = K >> 8;
@@ -225,168 +231,143 @@ __global__ __launch_bounds__(64 * NW, NT == 2 ? 2 : 1) void gemm_fp4_stream_kern
     });
   }
 
-  // ---- the four K parts of the workgroup, summed in the fixed order (w0 + w2) + (w1 + w3)
-  auto put = [&](int slot) __attribute__((always_inline)) {
+  // ---- the four K parts of the workgroup, summed in the fixed order (w0 + w2) + (w1 + w3).
+  // Whatever follows the last matrix instruction delays the workgroup's end, so all four waves share it:
+  // wave g owns quarter g of every tile (registers 4g .. 4g + 3: columns 8g .. 8g + 7), gets that
+  // quarter from the three others through LDS and carries it through the rest of the kernel.
 #pragma unroll
-    for (int j = 0; j < NT * MT; ++j)
+  for (int g = 0; g < 4; ++g) {
+    if (g == wave) continue;
+    const int from = wave < g ? wave : wave - 1;
 #pragma unroll
-      for (int g = 0; g < 4; ++g)
-        part[slot][j][g][lane] = v4f{acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]};
-  };
-  // waves 1-3 hand their partial tiles to wave 0 through LDS (one barrier); wave 0 adds them as stated
-  if (wave != 0) put(wave - 1);
-  __syncthreads();
-  if (wave != 0) return;
+    for (int t = 0; t < NT * MT; ++t)
+      part[g][t][from][lane] = v4f{acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
+  }
   // The rows of the residual this wave will add are asked for now: they arrive during the reduction.
-  uint4 rv[NT][MT][2];
+  // (Store pass 2 t + p -- rows 16 p .. 16 p + 15 of tile t -- belongs to wave (2 t + p) % 4.)
+  uint4 rv[(2 * NT * MT + 3) / 4];
   if (res_rows) {
 #pragma unroll
-    for (int i = 0; i < NT; ++i)
-#pragma unroll
-      for (int j = 0; j < MT; ++j)
-#pragma unroll
-        for (int p = 0; p < 2; ++p) {
-          const int m = j * 32 + 16 * p + row16, n = (rtg * NT + i) * 32 + 8 * c;
-          rv[i][j][p] = m < M && n < N ? *(const uint4*)(res_src + (size_t)(j * 32 + 16 * p) * N + 32 * i)
-                                       : make_uint4(0, 0, 0, 0);
-        }
-  }
-#pragma unroll
-  for (int j = 0; j < NT * MT; ++j)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const v4f p1 = part[0][j][g][lane], p2 = part[1][j][g][lane], p3 = part[2][j][g][lane];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) acc[j][4 * g + q] = (acc[j][4 * g + q] + p2[q]) + (p1[q] + p3[q]);
+    for (int pass = 0; pass < 2 * NT * MT; ++pass) {
+      if ((pass & 3) != wave) continue;
+      const int i = (pass >> 1) / MT, j = (pass >> 1) % MT, p = pass & 1;
+      const int m = j * 32 + 16 * p + row16, n = (rtg * NT + i) * 32 + 8 * c;
+      rv[pass >> 2] = m < M && n < N ? *(const uint4*)(res_src + (size_t)(j * 32 + 16 * p) * N + 32 * i)
+                                     : make_uint4(0, 0, 0, 0);
     }
+  }
+  __syncthreads();
+  v4f sum[NT * MT];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    if (g != wave) continue;
+#pragma unroll
+    for (int t = 0; t < NT * MT; ++t) {
+      v4f k[4];   // the quarter as each wave computed it
+#pragma unroll
+      for (int w = 0; w < 4; ++w)
+        k[w] = w == g ? v4f{acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]}
+                      : part[g][t][w < g ? w : w - 1][lane];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) sum[t][q] = (k[0][q] + k[2][q]) + (k[1][q] + k[3][q]);
+    }
+  }
 
   // ---- K split across workgroups: partial tiles through the workspace, last arrival finishes
   if (ksplit > 1) {
     // The parts of a tile run on different XCDs, whose L2 caches are not coherent with each other
     // for ordinary accesses.  Device-scope fences would write back and invalidate whole caches
     // (measured: 55 us for a 6 us kernel); instead every access to the workspace is a relaxed
-    // device-scope atomic, which the hardware performs at the point all XCDs agree on, and the
-    // wave waits for its stores to be acknowledged before it moves the counter.
-    constexpr int kTile = NT * MT * 16 * 64;  // floats per partial
-    float* mine = partial + ((size_t)rtg * ksplit + split) * kTile + lane;
-#pragma unroll
-    for (int j = 0; j < NT * MT; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v)
-        __hip_atomic_store(mine + (j * 16 + v) * 64, acc[j][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    unsigned arrived = 0;
-    if (lane == 0) arrived = __hip_atomic_fetch_add(counters + rtg, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    arrived = __builtin_amdgcn_readfirstlane(arrived);
-    if (arrived != (unsigned)(ksplit - 1)) return;
-    const float* all = partial + (size_t)rtg * ksplit * kTile + lane;
-    for (int s = 0; s < ksplit; ++s) {
-#pragma unroll
-      for (int j = 0; j < NT * MT; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const float p = __hip_atomic_load(all + (size_t)s * kTile + (j * 16 + v) * 64, __ATOMIC_RELAXED,
-                                            __HIP_MEMORY_SCOPE_AGENT);
-          acc[j][v] = s == 0 ? p : acc[j][v] + p;
-        }
-    }
-    if (lane == 0) __hip_atomic_store(counters + rtg, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-
-  // ---- y[m][n] = bf16(alpha * acc) (+ bias) (+ residual, a further bf16 add): register 4g + q of
-  // tile (i, j) is m = 32 j + lane % 32, n = 32 (NT rtg + i) + 8 g + 4 (lane / 32) + q.  Stored from
-  // there, an instruction would write 16 bytes into each of 32 rows; so many small pieces cost 5-8 %
-  // of the whole kernel (M = 16, N = 14336: 8.0 -> 7.6 us; M = 64: 11.3 -> 10.4 us).  The rounded tile
-  // goes through LDS instead -- the buffer of the partial sums, which only this wave still uses --
-  // and comes back with a lane holding 8 consecutive columns: 64 contiguous bytes per row and store.
-  const int r32 = lane & 31, kh = lane >> 5;
-  constexpr int kStageRow = 20;   // dwords: 16 of a row's 32 bf16 + 4, rows stay 16-byte aligned
-  uint32_t* stage = (uint32_t*)&part[0][0][0][0];
-  static_assert(sizeof(part[0][0]) >= 32 * kStageRow * 4, "a staged tile fits a partial tile's place");
-  constexpr int kStageTile = sizeof(part[0][0]) / 4;
-  // (this wave alone is what the workgroup still waits for, so every instruction here is on the critical
-  // path: the case without a bias is a code path of its own rather than a select after the additions)
-  uint32_t* lane_stage = stage + r32 * kStageRow + 2 * kh;
-  if (!bias) {
+    // device-scope atomic, which the hardware performs at the point all XCDs agree on, and every
+    // wave waits for its stores to be acknowledged before the workgroup moves the counter.
+    constexpr int kTile = NT * MT * 16 * 64;  // floats per partial: register v of tile t at (16 t + v) * 64 + lane
+    float* mine = partial + ((size_t)rtg * ksplit + split) * kTile + wave * 256 + lane;
 #pragma unroll
     for (int t = 0; t < NT * MT; ++t)
 #pragma unroll
-      for (int g = 0; g < 4; ++g)
-        *(uint2*)(lane_stage + t * kStageTile + 4 * g) =
-            make_uint2(pack_bf16x2(acc[t][4 * g + 0] * alpha, acc[t][4 * g + 1] * alpha),
-                       pack_bf16x2(acc[t][4 * g + 2] * alpha, acc[t][4 * g + 3] * alpha));
+      for (int q = 0; q < 4; ++q)
+        __hip_atomic_store(mine + (t * 16 + q) * 64, sum[t][q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();   // (ksplit is the same for the whole grid: every wave of the workgroup is here)
+    // One arrival per workgroup: a counter that every wave moved made the exchange 1.5 us slower (its
+    // updates from different XCDs are served one after the other).
+    if (threadIdx.x == 0)
+      arrival = __hip_atomic_fetch_add(counters + rtg, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    // (one value for the workgroup: all its waves leave or all stay for the barrier further down)
+    if (__builtin_amdgcn_readfirstlane(arrival) != (unsigned)(ksplit - 1)) return;
+    const float* all = partial + (size_t)rtg * ksplit * kTile + wave * 256 + lane;
+    for (int s = 0; s < ksplit; ++s) {
+#pragma unroll
+      for (int t = 0; t < NT * MT; ++t)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float p = __hip_atomic_load(all + (size_t)s * kTile + (t * 16 + q) * 64, __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT);
+          sum[t][q] = s == 0 ? p : sum[t][q] + p;
+        }
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(counters + rtg, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+
+  // ---- y[m][n] = bf16(alpha * sum) (+ bias) (+ residual, a further bf16 add): element q of this wave's
+  // quarter of tile (i, j) is m = 32 j + lane % 32, n = 32 (NT rtg + i) + 8 wave + 4 (lane / 32) + q.
+  // Stored from there, an instruction would write 16 bytes into each of 32 rows; so many small pieces
+  // cost 5-8 % of the whole kernel (M = 16, N = 14336: 8.0 -> 7.6 us; M = 64: 11.3 -> 10.4 us).  The
+  // rounded tile goes through LDS instead and comes back with a lane holding 8 consecutive columns: 64
+  // contiguous bytes per row and store.
+  const int r32 = lane & 31, kh = lane >> 5;
+  uint32_t* lane_stage = &stage[0][r32 * kStageRow + 4 * wave + 2 * kh];
+  if (!bias) {   // (a code path of its own rather than a select after the additions)
+#pragma unroll
+    for (int t = 0; t < NT * MT; ++t)
+      *(uint2*)(lane_stage + t * kStageTile) = make_uint2(pack_bf16x2(sum[t][0] * alpha, sum[t][1] * alpha),
+                                                          pack_bf16x2(sum[t][2] * alpha, sum[t][3] * alpha));
   } else {
 #pragma unroll
-    for (int ig = 0; ig < NT * 4; ++ig) {
-      const int i = ig >> 2, g = ig & 3;
-      const int n = (rtg * NT + i) * 32 + 8 * g + 4 * kh;   // bias is indexed by the product's column
+    for (int i = 0; i < NT; ++i) {
+      const int n = (rtg * NT + i) * 32 + 8 * wave + 4 * kh;   // bias is indexed by the product's column
       float bv[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q) bv[q] = n + q < N ? __uint_as_float((uint32_t)bias[n + q] << 16) : 0.f;
 #pragma unroll
       for (int j = 0; j < MT; ++j) {
-        const v16f& t = acc[i * MT + j];
-        const uint32_t lo = pack_bf16x2(t[4 * g + 0] * alpha, t[4 * g + 1] * alpha);
-        const uint32_t hi = pack_bf16x2(t[4 * g + 2] * alpha, t[4 * g + 3] * alpha);
-        *(uint2*)(lane_stage + (i * MT + j) * kStageTile + 4 * g) =
+        const v4f& t = sum[i * MT + j];
+        const uint32_t lo = pack_bf16x2(t[0] * alpha, t[1] * alpha), hi = pack_bf16x2(t[2] * alpha, t[3] * alpha);
+        *(uint2*)(lane_stage + (i * MT + j) * kStageTile) =
             make_uint2(pack_bf16x2(__uint_as_float(lo << 16) + bv[0], __uint_as_float(lo & 0xffff0000u) + bv[1]),
                        pack_bf16x2(__uint_as_float(hi << 16) + bv[2], __uint_as_float(hi & 0xffff0000u) + bv[3]));
       }
     }
   }
-  // (the wave reads back what other lanes of it wrote: LDS serves one wave's accesses in order)
+  __syncthreads();
 #pragma unroll
-  for (int i = 0; i < NT; ++i) {
-    const int tn0 = (rtg * NT + i) * 32, n = tn0 + 8 * c;
-    if (tn0 >= N) continue;
-    const int ldy = out_ld[i];
-    const uint32_t* tile = stage + i * MT * kStageTile + row16 * kStageRow + 4 * c;
-    uint16_t* dst = out_dst[i];
-    // The same for every lane, so the common case is branch-free: all staged rows are asked for at once
-    // and the stores follow.
-    const bool whole = out_whole[i];
-    if (whole) {
-      uint4 v[MT][2];
-#pragma unroll
-      for (int j = 0; j < MT; ++j)
-#pragma unroll
-        for (int p = 0; p < 2; ++p) v[j][p] = *(const uint4*)(tile + j * kStageTile + 16 * p * kStageRow);
+  for (int pass = 0; pass < 2 * NT * MT; ++pass) {
+    if ((pass & 3) != wave) continue;
+    const int i = (pass >> 1) / MT, j = (pass >> 1) % MT, p = pass & 1;
+    const int n = (rtg * NT + i) * 32 + 8 * c, m = j * 32 + 16 * p + row16;
+    if (m >= M || n >= N) continue;
+    const uint4 v = *(const uint4*)&stage[pass >> 1][(16 * p + row16) * kStageRow + 4 * c];
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint16_t* dst = out_dst[i] + (size_t)(j * 32 + 16 * p) * out_ld[i];
+    if (out_whole[i]) {   // the same for every lane
       if (residual) {
+        const uint32_t r[4] = {rv[pass >> 2].x, rv[pass >> 2].y, rv[pass >> 2].z, rv[pass >> 2].w};
 #pragma unroll
-        for (int j = 0; j < MT; ++j)
-#pragma unroll
-          for (int p = 0; p < 2; ++p) {
-            const uint32_t w[4] = {v[j][p].x, v[j][p].y, v[j][p].z, v[j][p].w};
-            const uint32_t r[4] = {rv[i][j][p].x, rv[i][j][p].y, rv[i][j][p].z, rv[i][j][p].w};
-            uint32_t o[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-              o[q] = pack_bf16x2(__uint_as_float(w[q] << 16) + __uint_as_float(r[q] << 16),
-                                 __uint_as_float(w[q] & 0xffff0000u) + __uint_as_float(r[q] & 0xffff0000u));
-            v[j][p] = make_uint4(o[0], o[1], o[2], o[3]);
-          }
+        for (int q = 0; q < 4; ++q)
+          w[q] = pack_bf16x2(__uint_as_float(w[q] << 16) + __uint_as_float(r[q] << 16),
+                             __uint_as_float(w[q] & 0xffff0000u) + __uint_as_float(r[q] & 0xffff0000u));
       }
-#pragma unroll
-      for (int j = 0; j < MT; ++j)
-#pragma unroll
-        for (int p = 0; p < 2; ++p)
-          if (j * 32 + 16 * p + row16 < M) *(uint4*)(dst + (size_t)(j * 32 + 16 * p) * ldy) = v[j][p];
+      *(uint4*)dst = make_uint4(w[0], w[1], w[2], w[3]);
       continue;
     }
-    if (n >= N) continue;
-    for (int jp = 0; jp < 2 * MT; ++jp) {   // N's last tile, or an unaligned output: element by element
-      const int m = 16 * jp + row16;
-      if (m >= M) continue;
-      const uint4 v = *(const uint4*)(tile + (jp >> 1) * kStageTile + 16 * (jp & 1) * kStageRow);
-      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        if (n + q >= N) continue;
-        uint32_t h = (w[q >> 1] >> (16 * (q & 1))) & 0xffffu;
-        if (residual)
-          h = pack_bf16x2(__uint_as_float(h << 16) + __uint_as_float((uint32_t)residual[(size_t)m * N + n + q] << 16), 0.0f) & 0xffffu;
-        dst[(size_t)16 * jp * ldy + q] = (uint16_t)h;
-      }
+    for (int q = 0; q < 8; ++q) {   // N's last tile, or an unaligned output: element by element
+      if (n + q >= N) continue;
+      uint32_t h = (w[q >> 1] >> (16 * (q & 1))) & 0xffffu;
+      if (residual)
+        h = pack_bf16x2(__uint_as_float(h << 16) + __uint_as_float((uint32_t)residual[(size_t)m * N + n + q] << 16), 0.0f) & 0xffffu;
+      dst[q] = (uint16_t)h;
     }
   }
 }
