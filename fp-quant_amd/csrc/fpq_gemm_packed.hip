@@ -420,7 +420,7 @@ static int launch_packed(const void* xq, const void* xs, const void* wq, const v
 }
 
 // fpq_gemm_stream.hip: the weight-streaming kernel for at most 128 activation rows
-bool stream_eligible(int64_t M, int64_t N, int64_t K);
+bool stream_eligible(bool nv, int64_t M, int64_t N, int64_t K);
 int64_t gemm_mxf4_stream_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int gemm_fp4_stream(bool nv, const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                     const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
@@ -479,7 +479,7 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
       ((uintptr_t)y & 15u) || ((uintptr_t)residual & 15u))
     return FPQ_E_ALIGN;
   if ((uintptr_t)workspace & 255u) return FPQ_E_ALIGN;
-  if (stream_eligible(M, N, K) && (!NV || M <= FPQ_NV_STREAM_ROWS))
+  if (stream_eligible(NV, M, N, K) && (!NV || M <= FPQ_NV_STREAM_ROWS))
     return gemm_fp4_stream(NV, xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, workspace, workspace_bytes,
                            seg, (hipStream_t)stream);
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);

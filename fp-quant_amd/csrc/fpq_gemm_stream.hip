@@ -381,8 +381,12 @@ struct StreamPlan {
 
 // Which shapes run here and how (all thresholds are measured break-even points on Llama-3-8B and
 // Qwen3-8B layer shapes).  Up to 64 activation rows: always, one weight tile per workgroup.  More
-// rows: while the weight tiles fit one round of the 256 CUs; beyond that the 128x128 tile kernel,
-// which shares activations through LDS.  (Two weight tiles per workgroup halve what the L2 has to
+// rows: up to a number of weight tiles beyond which the 128x128 tile kernel, which shares activations
+// through LDS, is faster -- 65-96 rows: 1024 tiles for MXFP4 (N = 14336: 11.9 against 13.5 us, N =
+// 28672: 20.5 against 22.3, N = 57344: 36.3 against 27.7), any number for NVFP4 (N = 14336: 22.1
+// against 35.9 us, N = 128256: 165 against 215); 97-128 rows (276-346 registers, one workgroup per
+// CU): one round of the 256 CUs for MXFP4, two for NVFP4 (N = 16384: 28.1 against 35.1 us, N = 20480:
+// 39.9 against 35.2).  (Two weight tiles per workgroup halve what the L2 has to
 // deliver for 33-64 rows, but need so many registers that one workgroup fills a CU; one tile per
 // workgroup with two blocks in flight, two workgroups per CU, measured 5-13 % faster -- except from
 // 768 weight tiles on, where two tiles per workgroup with ONE block in flight, held to 256 registers,
@@ -394,7 +398,8 @@ static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace
   StreamPlan plan{false, 1, 1, 0};
   if (M < 1 || M > kStreamMaxRows || N < 1 || K < 256 || K % 256 != 0) return plan;
   const int64_t rt_m = (M + 31) / 32, tiles = (N + 31) / 32, nkb = K / 256;
-  if (rt_m > 2 && tiles > 256) return plan;
+  if (rt_m == 3 && !nv && tiles > 1024) return plan;
+  if (rt_m == 4 && tiles > (nv ? 512 : 256)) return plan;
   plan.use = true;
   if (rt_m == 2 && tiles >= 768 && !nv) plan.nt = 2;
   const int64_t groups = (tiles + plan.nt - 1) / plan.nt;
@@ -411,7 +416,7 @@ static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace
   return plan;
 }
 
-bool stream_eligible(int64_t M, int64_t N, int64_t K) { return stream_plan(M, N, K, 0).use; }
+bool stream_eligible(bool nv, int64_t M, int64_t N, int64_t K) { return stream_plan(M, N, K, 0, nv).use; }
 
 int64_t gemm_mxf4_stream_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   const StreamPlan plan = stream_plan(M, N, K, (int64_t)1 << 62);

@@ -163,11 +163,12 @@ def test_pack_nv_kernel_matches_definition(rows, k):
     assert torch.equal(ps, ws)
 
 
-# up to 128 rows: the weight-streaming kernel (one to four activation row tiles, ragged rows and columns, odd
-# tile counts, long K); 65-128 rows with more than 256 weight tiles and everything above: the tile kernels
+# up to 96 rows, and 97-128 rows with at most 512 weight tiles: the weight-streaming kernel (one to four
+# activation row tiles, ragged rows and columns, odd tile counts, long K); everything else: the tile kernels
 @pytest.mark.parametrize("m,n,k", [(1, 64, 256), (32, 32, 256), (65, 100, 512), (256, 256, 768), (300, 520, 1024),
                                    (512, 256, 4096), (16, 1024, 1024), (48, 515, 768), (64, 14336, 256),
-                                   (96, 2048, 4096), (128, 1000, 2304), (5, 257, 12288), (100, 8290, 256)])
+                                   (96, 2048, 4096), (128, 1000, 2304), (5, 257, 12288), (100, 8290, 256),
+                                   (96, 40000, 256), (128, 16384, 256), (128, 16400, 256), (97, 14339, 512)])
 @pytest.mark.parametrize("bias", [False, True])
 def test_gemm_nv_packed_matches_oracle(m, n, k, bias):
     g = torch.Generator().manual_seed(m + 2 * n + k)

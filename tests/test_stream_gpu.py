@@ -49,13 +49,16 @@ def _workspace(m, n, k, cap=None):
     return need, torch.zeros(max(size, 256), dtype=torch.uint8, device="cuda")
 
 
-# one to four activation row tiles (more than 64 rows only with at most 256 weight tiles), odd tile counts,
-# ragged rows and columns, one to 56 blocks of K
+# one to four activation row tiles (65-96 rows with at most 1024 weight tiles, 97-128 rows with at most 256;
+# the shapes just beyond run the tile kernels and meet the same oracle), odd tile counts, ragged rows and
+# columns, one to 56 blocks of K
 SHAPES = [(1, 32, 256), (1, 100, 512), (5, 257, 768), (16, 1024, 1024), (31, 64, 1280), (32, 4096, 4096),
           (33, 130, 2048), (64, 96, 3072), (70, 515, 1024), (96, 2048, 4096), (100, 36, 256), (128, 1000, 2304),
           (127, 4099, 1536), (8, 1024, 14336), (64, 8200, 512), (40, 8290, 768), (33, 16384, 256),
           # 768 weight tiles or more at 33-64 rows: two weight tiles per workgroup (an odd tile count, a ragged N)
-          (64, 24600, 512), (45, 28672, 256), (33, 24577, 256)]
+          (64, 24600, 512), (45, 28672, 256), (33, 24577, 256),
+          # three activation row tiles with more than 256 weight tiles, up to the limit and past it
+          (96, 8290, 512), (70, 14336, 256), (96, 32768, 256), (65, 32800, 256), (128, 8192, 256), (128, 8224, 256)]
 # shapes whose K is split when a workspace is given (few weight tiles, K of 8192 or more)
 SPLIT_SHAPES = [(1, 32, 8192), (5, 257, 12288), (16, 1024, 8192), (31, 64, 16384), (32, 4096, 8192),
                 (8, 1024, 14336), (17, 515, 9216)]
