@@ -482,6 +482,27 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
   if (stream_eligible(NV, M, N, K) && (!NV || M <= FPQ_NV_STREAM_ROWS))
     return gemm_fp4_stream(NV, xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, workspace, workspace_bytes,
                            seg, (hipStream_t)stream);
+  if constexpr (NV) {
+    // 129-256 rows of NVFP4 at up to 256 weight tiles (N <= 8192): the 128x128 tile kernel fills at most
+    // half of the 256 CUs with workgroups that take 34 us for K = 4096, so two passes of the weight-streaming
+    // kernel over one half of the rows each are faster although the second re-reads the weights (from the
+    // last-level cache): N = 6144, K = 4096: 192 rows 35.2 -> 23.1 us, 256 rows 34.8 -> 28.6; N = 4096, K =
+    // 12288: 97 -> 52 / 68 us.  (The tile kernel's time stays at one round up to N = 16384, where two passes
+    // take 44-55 us; three passes for more rows measured slower than the tiles as well.)
+    const int64_t half = ((M + 1) / 2 + 31) / 32 * 32;   // rows of the first pass, whole 32-row tiles
+    if (M > FPQ_NV_STREAM_ROWS && M <= 2 * FPQ_NV_STREAM_ROWS && (N + 31) / 32 <= 256 &&
+        stream_eligible(true, half, N, K)) {
+      const int rc = gemm_fp4_stream(true, xq, xs, wq, ws, alpha, bias, residual, y, half, N, K, nullptr, 0, seg,
+                                     (hipStream_t)stream);
+      if (rc != FPQ_OK) return rc;
+      OutSegments rest = seg;
+      for (int i = 0; i < seg.count; ++i)
+        rest.y[i] = seg.y[i] + (size_t)half * (seg.end[i] - (i ? seg.end[i - 1] : 0));
+      return gemm_fp4_stream(true, (const uint8_t*)xq + (size_t)half * (K / 2), (const uint8_t*)xs + (size_t)half * (K / 16),
+                             wq, ws, alpha, bias, residual ? (const uint16_t*)residual + (size_t)half * N : nullptr,
+                             (uint16_t*)y + (size_t)half * N, M - half, N, K, nullptr, 0, rest, (hipStream_t)stream);
+    }
+  }
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
   if (big_tiles < FPQ_PACKED_SMALL_BELOW)
     return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);

@@ -168,7 +168,9 @@ def test_pack_nv_kernel_matches_definition(rows, k):
 @pytest.mark.parametrize("m,n,k", [(1, 64, 256), (32, 32, 256), (65, 100, 512), (256, 256, 768), (300, 520, 1024),
                                    (512, 256, 4096), (16, 1024, 1024), (48, 515, 768), (64, 14336, 256),
                                    (96, 2048, 4096), (128, 1000, 2304), (5, 257, 12288), (100, 8290, 256),
-                                   (96, 40000, 256), (128, 16384, 256), (128, 16400, 256), (97, 14339, 512)])
+                                   (96, 40000, 256), (128, 16384, 256), (128, 16400, 256), (97, 14339, 512),
+                                   # 129-256 rows at up to 256 weight tiles: two passes of the weight-streaming kernel
+                                   (130, 515, 512), (192, 6144, 256), (256, 8192, 256), (255, 8200, 256), (161, 100, 1024)])
 @pytest.mark.parametrize("bias", [False, True])
 def test_gemm_nv_packed_matches_oracle(m, n, k, bias):
     g = torch.Generator().manual_seed(m + 2 * n + k)
@@ -335,11 +337,12 @@ def test_unpack_nv_is_the_inverse_of_the_layout_definition(rows, k):
 
 @pytest.mark.parametrize("m,splits,k", [(1, [512, 256, 256], 512), (48, [1024, 256], 1024), (96, [256, 512], 256),
                                         (128, [256, 256, 256, 256], 768), (300, [512, 256, 256], 512),
-                                        (2048, [2048, 1024, 256, 768], 256)])
+                                        (2048, [2048, 1024, 256, 768], 256), (200, [256, 512], 512),
+                                        (131, [1024, 256, 256], 256)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_nv_layers_end_to_end_get_their_own_outputs(m, splits, k, with_bias):
     """fpq_gemm_nvf4_packed_multi: every layer's matrix equals its column range of fpq_gemm_nvf4_packed on the
-    same operands bit for bit (weight-streaming kernel, 128x128 tiles, 256x256 tiles)."""
+    same operands bit for bit (weight-streaming kernel in one pass and in two, 128x128 tiles, 256x256 tiles)."""
     n = sum(splits)
     g = torch.Generator().manual_seed(900 + m + n)
     xq = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=g)
