@@ -152,6 +152,8 @@ __device__ __forceinline__ void barrier_lds() {
 //                    operand traffic costs (62.4 us against 66.1 us at M = 2048, N = 14336)
 //   <8, 8, 8, 2, 2>  256 x 256 tile, waves 128 x 128, one workgroup per CU: large M, NVFP4 (whose
 //                    limit is the register dequantization; half tiles measured mixed there)
+//   <2, 4, 4, 2, 2>  64 x 128 tile (weight rows x activation rows), waves 32 x 64: when even the 128 x 128
+//                    tiles would fill at most half of the CUs
 //   <4, 4, 4, 2, 2>  128 x 128 tile, waves 64 x 64, 80 KB of LDS: two workgroups per CU; used when
 //                    the big tiles would leave most CUs idle (M of a few hundred rows).  Its time
 //                    has a floor of about 12 us at K = 4096; two K steps per hand-over and a ring
@@ -457,6 +459,9 @@ static int pack_operand(const void* codes, const void* scales, int64_t scale_str
 #ifndef FPQ_PACKED_HALF_TILES
 #define FPQ_PACKED_HALF_TILES 1  // large M: 1 = 256x128 tiles for MXFP4, 2 = for NVFP4 too, 0 = 256x256
 #endif
+#ifndef FPQ_PACKED_NARROW_BELOW
+#define FPQ_PACKED_NARROW_BELOW 128  // up to this many 128x128 tiles: 64x128 tiles instead
+#endif
 #ifndef FPQ_PACKED_SMALL_BELOW
 #define FPQ_PACKED_SMALL_BELOW 100  // fewer 256x256 tiles than this (under about 200 of 256x128): 128x128 tiles
 #endif
@@ -503,6 +508,11 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
                              (uint16_t*)y + (size_t)half * N, M - half, N, K, nullptr, 0, rest, (hipStream_t)stream);
     }
   }
+  // At most 128 tiles of 128 x 128 would leave half of the CUs idle: 64 x 128 tiles (twice the workgroups, the
+  // same accumulation order and bits) take 25 instead of 34.5 us for NVFP4 at 257-512 rows, N = 4096, K = 4096
+  // (K = 12288: 69 instead of 97 us) and 4-7 % less for MXFP4; with more tiles they measured 14 % slower.
+  if (((M + 127) / 128) * ((N + 127) / 128) <= FPQ_PACKED_NARROW_BELOW)
+    return launch_packed<2, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
   if (big_tiles < FPQ_PACKED_SMALL_BELOW)
     return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);
