@@ -497,15 +497,17 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
     const int64_t half = ((M + 1) / 2 + 31) / 32 * 32;   // rows of the first pass, whole 32-row tiles
     if (M > FPQ_NV_STREAM_ROWS && M <= 2 * FPQ_NV_STREAM_ROWS && (N + 31) / 32 <= 256 &&
         stream_eligible(true, half, N, K)) {
-      const int rc = gemm_fp4_stream(true, xq, xs, wq, ws, alpha, bias, residual, y, half, N, K, nullptr, 0, seg,
-                                     (hipStream_t)stream);
+      // (both passes may split K through the caller's workspace: they run one after the other on the stream)
+      const int rc = gemm_fp4_stream(true, xq, xs, wq, ws, alpha, bias, residual, y, half, N, K, workspace,
+                                     workspace_bytes, seg, (hipStream_t)stream);
       if (rc != FPQ_OK) return rc;
       OutSegments rest = seg;
       for (int i = 0; i < seg.count; ++i)
         rest.y[i] = seg.y[i] + (size_t)half * (seg.end[i] - (i ? seg.end[i - 1] : 0));
       return gemm_fp4_stream(true, (const uint8_t*)xq + (size_t)half * (K / 2), (const uint8_t*)xs + (size_t)half * (K / 16),
                              wq, ws, alpha, bias, residual ? (const uint16_t*)residual + (size_t)half * N : nullptr,
-                             (uint16_t*)y + (size_t)half * N, M - half, N, K, nullptr, 0, rest, (hipStream_t)stream);
+                             (uint16_t*)y + (size_t)half * N, M - half, N, K, workspace, workspace_bytes, rest,
+                             (hipStream_t)stream);
     }
   }
   // At most 128 tiles of 128 x 128 would leave half of the CUs idle: 64 x 128 tiles (twice the workgroups, the

@@ -391,9 +391,11 @@ struct StreamPlan {
 // workgroup with two blocks in flight, two workgroups per CU, measured 5-13 % faster -- except from
 // 768 weight tiles on, where two tiles per workgroup with ONE block in flight, held to 256 registers,
 // are 12-16 % faster: MXFP4, N = 28672 at 64 rows 20.1 -> 17.0 us, N = 128256 73.5 -> 61.6 us.)
-// K is split across workgroups only for at most 32 rows, when the weight tiles leave at least half
-// of the CUs idle and every part keeps at least 4096 of K (the exchange of partial tiles through
-// the workspace costs about as much as streaming 16 blocks); fewer parts if the workspace is small.
+// K is split across workgroups when the weight tiles leave at least half of the CUs idle and every
+// part keeps at least 4096 of K (the exchange of partial tiles through the workspace costs about as
+// much as streaming 16 blocks); fewer parts if the workspace is small.  (While one wave did the
+// exchange alone the split paid for at most 32 rows; shared by the four waves it pays at every row
+// count: N = 4096, K = 14336: 64 rows 14.4 -> 11.7 us, 128 rows 19.8 -> 15.4 us, NVFP4 39.0 -> 24.6 us.)
 static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_bytes, bool nv = false) {
   StreamPlan plan{false, 1, 1, 0};
   if (M < 1 || M > kStreamMaxRows || N < 1 || K < 256 || K % 256 != 0) return plan;
@@ -404,11 +406,11 @@ static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace
   if (rt_m == 2 && tiles >= 768 && !nv) plan.nt = 2;
   const int64_t groups = (tiles + plan.nt - 1) / plan.nt;
   int64_t ksplit = 1;
-  if (rt_m == 1 && workspace_bytes > kStreamCounterBytes && groups <= kStreamCounters) {
+  if (workspace_bytes > kStreamCounterBytes && groups <= kStreamCounters) {
     ksplit = 256 / groups;
     if (ksplit > nkb / 16) ksplit = nkb / 16;
     if (ksplit < 1) ksplit = 1;
-    while (ksplit > 1 && kStreamCounterBytes + ksplit * groups * 4096 > workspace_bytes) --ksplit;
+    while (ksplit > 1 && kStreamCounterBytes + ksplit * groups * plan.nt * rt_m * 4096 > workspace_bytes) --ksplit;
   }
   const int64_t bps = (nkb + ksplit - 1) / ksplit;
   plan.ksplit = (int)((nkb + bps - 1) / bps);  // no empty part
@@ -482,8 +484,9 @@ int gemm_fp4_stream(bool nv, const void* xq, const void* xs, const void* wq, con
 // workspace.  Every GPU the library runs on holds its own copy at its own address until the process
 // ends; the array's name is only a host-side handle, the device address comes from
 // hipGetSymbolAddress, once per device, and that address is what kernels and host code use.
-// A split needs at most 256 partial tiles of 4 KB (stream_plan: parts x weight tiles <= 256).
-constexpr int64_t kScratchBytes = kStreamCounterBytes + 256 * 4096;
+// A split needs at most 1024 partial tiles of 4 KB (stream_plan: parts x weight tiles <= 256, times up
+// to four activation row tiles).
+constexpr int64_t kScratchBytes = kStreamCounterBytes + 1024 * 4096;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 constexpr int kMaxDevices = 64;

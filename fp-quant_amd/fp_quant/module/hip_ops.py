@@ -398,14 +398,15 @@ def packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False) -> Tu
 
 
 
-_splitk_need = {}   # (n, k) -> workspace bytes with which fpq_gemm_mxf4_packed_splitk splits K at up to 32 rows
+_splitk_need = {}   # (n, k) -> workspace bytes with which fpq_gemm_mxf4_packed_splitk splits K at up to SPLIT_K_ROWS rows
+SPLIT_K_ROWS = 128  # the rows the weight-streaming GEMM takes
 # FPQ_SPLIT_K=0: no layer keeps a split-K workspace (for callers that run ONE layer object on several streams at
 # the same time, whose kernels would share it)
 SPLIT_K = os.environ.get("FPQ_SPLIT_K", "1") != "0"
 
 
 def splitk_workspace(wq: torch.Tensor, n: int, k: int, create: bool) -> Optional[torch.Tensor]:
-    """The workspace with which the packed GEMM of a layer [n, k] (either format) splits K across workgroups at up to 32
+    """The workspace with which the packed GEMM of a layer [n, k] (either format) splits K across workgroups at up to 128
     activation rows (few weight rows and a long K: a Llama down-projection), or None where it would not
     split.  It belongs to the layer -- kept on its code tensor `wq`, zeroed once, left zeroed by every call --
     so that the layer takes the same kernel, and gives the same bits, on every stream, eagerly, traced or
@@ -415,7 +416,7 @@ def splitk_workspace(wq: torch.Tensor, n: int, k: int, create: bool) -> Optional
         return None
     need = _splitk_need.get((n, k))
     if need is None:
-        need = _splitk_need[(n, k)] = int(_engine.lib().fpq_gemm_mxf4_packed_workspace_bytes(32, n, k))
+        need = _splitk_need[(n, k)] = int(_engine.lib().fpq_gemm_mxf4_packed_workspace_bytes(SPLIT_K_ROWS, n, k))
     if need == 0:
         return None
     hit = getattr(wq, "_fpq_splitk", None)

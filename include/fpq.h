@@ -310,7 +310,9 @@ int fpq_gemm_mxf4_packed_splitk(const void* xq_packed, const void* xs_packed, co
                                 const void* residual, void* y, int64_t M, int64_t N, int64_t K,
                                 void* workspace, int64_t workspace_bytes, void* stream);
 /* The same for packed NVFP4 operands (fpq_gemm_nvf4_packed, with `residual` non-null fpq_gemm_nvf4_packed_residual);
- * workspace as above, sized by fpq_gemm_mxf4_packed_workspace_bytes (the split is the same for both formats). */
+ * workspace as above, sized by fpq_gemm_mxf4_packed_workspace_bytes (the split is the same for both formats;
+ * 129-256 rows of NVFP4 at N <= 8192 run as two passes over at most 128 rows each, and each pass may use it:
+ * size it for 128 rows). */
 int fpq_gemm_nvf4_packed_splitk(const void* xq_packed, const void* xs_packed, const void* wq_packed,
                                 const void* ws_packed, const float* alpha, const void* bias,
                                 const void* residual, void* y, int64_t M, int64_t N, int64_t K,
@@ -343,7 +345,7 @@ int fpq_gemm_nvf4_packed_multi(const void* xq_packed, const void* xs_packed, con
 /*
  * fpq_gemm_mxf4_packed_splitk for callers that cannot allocate or hold a workspace (code recorded
  * into a HIP graph, tight serving loops, harnesses that forbid hipMalloc): the counters and partial
- * tiles of a split K live in a file-scope device array of the library (1 064 960 bytes per GPU, held
+ * tiles of a split K live in a file-scope device array of the library (4 210 688 bytes per GPU, held
  * until the process ends) instead of a caller-provided buffer.  It has no counterpart in the
  * reference.  Same arguments, results and status codes as fpq_gemm_mxf4_packed_splitk called with a
  * workspace of that size, with these limits:

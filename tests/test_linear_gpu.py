@@ -99,9 +99,9 @@ def test_nvfp4_layer_with_a_long_k_owns_a_split_k_workspace():
 @pytest.mark.parametrize("bias", [False, True])
 def test_decode_rows_on_a_long_k_split_k_across_workgroups(bias):
     """A layer with few output features and a long K (a down-projection) owns a workspace with which its GEMM
-    splits K at up to 32 rows: oracle values, the same bits as the C entry point with a workspace of its own,
+    splits K at up to 128 rows: oracle values, the same bits as the C entry point with a workspace of its own,
     the same bits eagerly, under a graph capture on another stream and through the traced operator, the
-    residual taken inside the kernel, counters left at zero; more rows run the kernel that does not split."""
+    residual taken inside the kernel, counters left at zero; more rows run the tile kernel, which does not split."""
     import capi
     from fp_quant import _engine
     from fp_quant.module import eager, hip_ops
@@ -109,13 +109,13 @@ def test_decode_rows_on_a_long_k_split_k_across_workgroups(bias):
     k, n = 8192, 256
     lin = _quantized_linear("mxfp4", 128, k, n, seed=21, bias=bias)
     wsk = getattr(lin.qweight, "_fpq_splitk", None)
-    assert wsk is not None and wsk.numel() == _engine.lib().fpq_gemm_mxf4_packed_workspace_bytes(32, n, k) > 16384
+    assert wsk is not None and wsk.numel() == _engine.lib().fpq_gemm_mxf4_packed_workspace_bytes(128, n, k) > 16384
     norm = float(O.hadamard_matrix(128)[0, 0])
     alpha = O.alpha_from_global_scales(lin.weight_global_scale.cpu(), lin.act_global_scale.cpu())
     wq, ws = lin.qweight.cpu(), lin.scales.cpu()
     wp, wsp = pack_by_definition(wq, ws, k)
     b = lin.bias.detach().cpu() if bias else None
-    for m in (1, 20, 32):
+    for m in (1, 20, 32, 50, 128):
         x = torch.randn(m, k, generator=torch.Generator().manual_seed(m)).to(torch.bfloat16)
         xq, xs, _ = O.quantize_mx(x, O.ROT_HADAMARD, 128, norm)
         ref, mag = O.gemm_ref(xq, xs, wq, ws, alpha, "mxfp4")
@@ -146,10 +146,10 @@ def test_decode_rows_on_a_long_k_split_k_across_workgroups(bias):
             lin._fpq_residual = res
             assert torch.equal(lin(xd), y + res) and lin._fpq_residual is None
     with torch.no_grad():
-        x = torch.randn(33, k, generator=torch.Generator().manual_seed(33)).to(torch.bfloat16)
+        x = torch.randn(129, k, generator=torch.Generator().manual_seed(33)).to(torch.bfloat16)
         xq, xs, _ = O.quantize_mx(x, O.ROT_HADAMARD, 128, norm)
         xp, xsp = pack_by_definition(xq, xs, k)
-        assert torch.equal(lin(x.cuda()).cpu(), capi.gemm_packed(xp, xsp, wp, wsp, 33, n, k, alpha, bias=b))
+        assert torch.equal(lin(x.cuda()).cpu(), capi.gemm_packed(xp, xsp, wp, wsp, 129, n, k, alpha, bias=b))
         # the layer keeps a workspace when its weight changes hands (packed layout only and back)
         x = torch.randn(7, k, generator=torch.Generator().manual_seed(7)).to(torch.bfloat16).cuda()
         want = lin(x)

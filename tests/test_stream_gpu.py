@@ -59,9 +59,11 @@ SHAPES = [(1, 32, 256), (1, 100, 512), (5, 257, 768), (16, 1024, 1024), (31, 64,
           (64, 24600, 512), (45, 28672, 256), (33, 24577, 256),
           # three activation row tiles with more than 256 weight tiles, up to the limit and past it
           (96, 8290, 512), (70, 14336, 256), (96, 32768, 256), (65, 32800, 256), (128, 8192, 256), (128, 8224, 256)]
-# shapes whose K is split when a workspace is given (few weight tiles, K of 8192 or more)
+# shapes whose K is split when a workspace is given (few weight tiles, K of 8192 or more), one to four
+# activation row tiles
 SPLIT_SHAPES = [(1, 32, 8192), (5, 257, 12288), (16, 1024, 8192), (31, 64, 16384), (32, 4096, 8192),
-                (8, 1024, 14336), (17, 515, 9216)]
+                (8, 1024, 14336), (17, 515, 9216), (33, 4096, 8192), (64, 515, 9216), (96, 64, 16384),
+                (128, 1024, 8192), (100, 2050, 12288)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
@@ -143,7 +145,9 @@ def test_split_k_is_taken_for_few_weight_rows_and_long_k():
     assert need(16, 1024, 14336) == 16384 + 3 * 32 * 4096    # 32 weight tiles: three parts of 4864
     assert need(16, 4096, 4096) == 0                         # a part would be shorter than 4096
     assert need(16, 14336, 4096) == 0                        # 448 weight tiles fill the chip
-    assert need(33, 4096, 14336) == 0                        # more than 32 rows: never split
+    assert need(33, 4096, 14336) == 16384 + 2 * 128 * 2 * 4096   # two activation row tiles: partial tiles twice as many
+    assert need(128, 4096, 14336) == 16384 + 2 * 128 * 4 * 4096  # four: 4 MB, the most a split ever needs
+    assert need(96, 16384, 14336) == 0                       # 512 weight tiles: K stays whole at every row count
     assert need(129, 4096, 14336) == 0                       # tile kernels above 128 rows
     assert need(16, 4096, 256) == 0                          # one block of K: nothing to split
 

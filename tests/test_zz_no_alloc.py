@@ -44,10 +44,11 @@ def _with_workspace(ops, m, n, k, bias, res):
     return capi.gemm_packed_splitk(*ops, m, n, k, ALPHA, bias=bias, residual=res, workspace=wspace).cuda()
 
 
-# K split in two and in three, then smaller inputs on the same array: a split over fewer weight tiles,
+# K split in two and in three, the largest split the array holds (four activation row tiles, 4 MB of partial
+# tiles), then smaller inputs on the same array: a split over fewer weight tiles,
 # K whole (no scratch use), two activation row tiles, and the 128x128 tile kernel
-SEQUENCE = [(16, 4096, 14336), (8, 1024, 14336), (5, 257, 12288), (1, 32, 8192), (32, 2048, 4096),
-            (64, 8200, 512), (128, 8320, 256), (17, 515, 9216)]
+SEQUENCE = [(16, 4096, 14336), (8, 1024, 14336), (128, 4096, 8192), (5, 257, 12288), (1, 32, 8192), (32, 2048, 4096),
+            (64, 8200, 512), (128, 8320, 256), (17, 515, 9216), (64, 515, 9216)]
 
 
 def test_noalloc_equals_workspace_entry_on_calls_in_a_row():
