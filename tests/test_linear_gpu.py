@@ -65,13 +65,15 @@ def test_linear_matches_oracle_pipeline(fmt, g, bias):
     assert rel < 0.25, rel
 
 
-def test_nvfp4_layer_with_a_long_k_owns_a_split_k_workspace():
+@pytest.mark.parametrize("m", [9, 100, 200])
+def test_nvfp4_layer_with_a_long_k_owns_a_split_k_workspace(m):
     """The NVFP4 counterpart of the test below, in short: workspace made at priming, oracle values, eager ==
-    traced operator == C entry point with a workspace of its own."""
+    traced operator == C entry point with a workspace of its own -- at one and at four activation row tiles and
+    at 200 rows, which run as two passes of the kernel that splits K."""
     import capi
     from fp_quant.module import eager
     from test_packed_gpu import pack_nv_by_definition
-    k, n, m = 8192, 256, 9
+    k, n = 8192, 256
     lin = _quantized_linear("nvfp4", 16, k, n, seed=22, bias=True)
     wsk = getattr(lin.qweight, "_fpq_splitk", None)
     assert wsk is not None and wsk.numel() > 16384
@@ -94,6 +96,9 @@ def test_nvfp4_layer_with_a_long_k_owns_a_split_k_workspace():
     direct = capi.gemm_packed_splitk(xp, xsp, wp, wsp, m, n, k, alpha, bias=lin.bias.detach().cpu(), workspace=own,
                                      nv=True)
     assert torch.equal(y.cpu(), direct) and not wsk[:16384].any()
+    # the split is really taken: K whole (no workspace) sums in another order
+    whole = capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=lin.bias.detach().cpu())
+    assert ((whole.double() - want.double()).abs() <= 2.0 ** -6 * want.double().abs() + 1e-5 * mag + 1e-6).all()
 
 
 @pytest.mark.parametrize("bias", [False, True])
