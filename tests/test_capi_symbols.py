@@ -57,3 +57,17 @@ def test_argument_validation_needs_no_device():
     assert lib.fpq_gemm_mxf4_packed_multi(*args, ys, ns, 2, 0, 256, None) == 0
     with pytest.raises(ValueError):
         _engine.check(-2, "x")
+
+
+def test_split_k_workspace_sizes_are_host_arithmetic():
+    """fpq_gemm_mxf4_packed_workspace_bytes needs no device: 16 KB of counters plus 4 KB per part, weight tile
+    and activation row tile where K is split (few weight tiles, parts of at least 4096 of K), else 0."""
+    from fp_quant import _engine
+    need = _engine.lib().fpq_gemm_mxf4_packed_workspace_bytes
+    assert need(16, 4096, 14336) == 16384 + 2 * 128 * 4096
+    assert need(16, 1024, 14336) == 16384 + 3 * 32 * 4096
+    assert need(64, 4096, 14336) == 16384 + 2 * 128 * 2 * 4096
+    assert need(128, 4096, 8192) == 16384 + 2 * 128 * 4 * 4096 == 4210688   # the most a split ever needs
+    assert need(16, 4096, 4096) == need(16, 14336, 4096) == need(129, 4096, 14336) == need(16, 4096, 256) == 0
+    assert need(0, 4096, 14336) == need(16, 4096, 100) == 0                 # shapes the kernel does not take
+    assert _engine.lib().fpq_gemm_mxf4_packed_noalloc_max_rows() == 128
