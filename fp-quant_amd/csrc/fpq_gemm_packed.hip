@@ -427,6 +427,9 @@ int64_t gemm_mxf4_stream_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int gemm_fp4_stream(bool nv, const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                     const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
                     void* workspace, int64_t workspace_bytes, const OutSegments& seg, hipStream_t stream);
+int gemm_fp4_stream_slabs(bool nv, const void* xq, const void* xs, const void* wq, const void* ws,
+                          const float* alpha, const void* bias, const void* residual, void* y, int64_t M, int64_t N,
+                          int64_t K, int64_t slab_rows, const OutSegments& seg, hipStream_t stream);
 
 template <bool NV>
 static int gemm_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
@@ -459,6 +462,9 @@ static int pack_operand(const void* codes, const void* scales, int64_t scale_str
 #ifndef FPQ_PACKED_HALF_TILES
 #define FPQ_PACKED_HALF_TILES 1  // large M: 1 = 256x128 tiles for MXFP4, 2 = for NVFP4 too, 0 = 256x256
 #endif
+#ifndef FPQ_STREAM_SLAB_WGS
+#define FPQ_STREAM_SLAB_WGS 256   // more than 128 rows: slabs of the streaming kernel while they number at most this
+#endif
 #ifndef FPQ_PACKED_NARROW_BELOW
 #define FPQ_PACKED_NARROW_BELOW 128  // up to this many 128x128 tiles: 64x128 tiles instead
 #endif
@@ -487,6 +493,19 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
   if (stream_eligible(NV, M, N, K) && (!NV || M <= FPQ_NV_STREAM_ROWS))
     return gemm_fp4_stream(NV, xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, workspace, workspace_bytes,
                            seg, (hipStream_t)stream);
+  // More than 128 rows while slabs of at most 128 rows x weight tiles number at most 256: the weight-streaming
+  // kernel with one grid plane per slab fills the CUs with workgroups that neither share anything through LDS
+  // nor meet at barriers, where the tile kernels below would run 32-128 workgroups that do.  N = 4096: 129-256
+  // rows 9.9 -> 6.8-8.0 us at K = 4096, 27-32 -> 16-19 us at K = 14336 (NVFP4: 20-28 -> 11.7-14.1 us, K = 12288
+  // 44-67 -> 27-34 us); N = 2048, K = 8192 up to 512 rows 16 -> 11.8 us (NVFP4 47 -> 24); N = 1024 up to 1024 rows.
+  // (Slabs of 96 rows, two workgroups per CU and 512 in all, measured within +-10 % of the tile kernels.)
+  if (M > 128) {
+    const int64_t slabs = (M + 127) / 128;
+    const int64_t rows = ((M + slabs - 1) / slabs + 31) / 32 * 32;   // rows of a slab, whole 32-row tiles
+    if (slabs * ((N + 31) / 32) <= FPQ_STREAM_SLAB_WGS && rows < M && stream_eligible(NV, rows, N, K))
+      return gemm_fp4_stream_slabs(NV, xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, rows, seg,
+                                   (hipStream_t)stream);
+  }
   if constexpr (NV) {
     // 129-256 rows of NVFP4 at up to 256 weight tiles (N <= 8192): the 128x128 tile kernel fills at most
     // half of the 256 CUs with workgroups that take 34 us for K = 4096, so two passes of the weight-streaming

@@ -46,11 +46,19 @@ constexpr int kStreamMaxRows = 128;
 // of the unit on both sides, so the K order is permuted consistently and the sum is complete.
 template <int NT, int MT, int DB, int NW, bool NV = false>
 __global__ __launch_bounds__(64 * NW, NT == 2 ? 2 : 1) void gemm_fp4_stream_kernel(
-    const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
+    const uint8_t* __restrict__ xq_all, const uint8_t* __restrict__ xs_all, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias,
-    const uint16_t* residual, uint16_t* y, int M, int N, int K, int bps, int ksplit,
+    const uint16_t* residual_all, uint16_t* y, int M_all, int N, int K, int bps, int ksplit,
     float* partial, unsigned* counters, const OutSegments seg) {
   static_assert(NW == 4, "a wave owns a quarter of every tile");
+  // More than 32 MT activation rows: blockIdx.z numbers slabs of 32 MT rows, each a product of its own
+  // (the last may have fewer rows, even fewer row tiles).
+  const int slab = blockIdx.z, m0 = slab * (MT * 32);
+  const int M = min(M_all - m0, MT * 32);
+  const uint8_t* xq = xq_all + (size_t)slab * MT * (K >> 6) * 1024;
+  const uint8_t* xs = xs_all + (size_t)slab * MT * (K >> 8) * (NV ? 512 : 256);
+  const uint16_t* residual = residual_all ? residual_all + (size_t)m0 * N : nullptr;
+  const int tile_id = slab * gridDim.x + blockIdx.x;   // numbers the output tile groups for the K split
   __shared__ v4f part[4][NT * MT][3][64];   // [owning wave][tile][the other waves in order][lane]
   constexpr int kStageRow = 20;             // dwords: 16 of a row's 32 bf16 + 4, rows stay 16-byte aligned
   constexpr int kStageTile = 32 * kStageRow;
@@ -75,17 +83,17 @@ __global__ __launch_bounds__(64 * NW, NT == 2 ? 2 : 1) void gemm_fp4_stream_kern
     wcode[i] = wq + (size_t)rt * nu * 1024 + lane * 16;
     wscale[i] = ws + (size_t)rt * nkb * kSB + lane * (kSB / 64);
   }
-  // Lanes whose activation row lies past M (last row tile only) read what the lane of row 0 in
-  // their K half reads: no further cache line is touched for rows that are never stored.
-  const int rows_last = M - 32 * (MT - 1);
-  const int xl = (lane & 31) < rows_last ? lane : (lane & 32);
+  // Lanes whose activation row lies past M read what the lane of row 0 in their K half reads: no further
+  // cache line is touched for rows that are never stored.  A row tile past the last one (a short last
+  // slab) re-reads the last: the operand ends there.
   const uint8_t* xcode[MT];
   const uint8_t* xscale[MT];
 #pragma unroll
   for (int j = 0; j < MT; ++j) {
-    const int l = j == MT - 1 ? xl : lane;
-    xcode[j] = xq + (size_t)j * nu * 1024 + l * 16;
-    xscale[j] = xs + (size_t)j * nkb * kSB + l * (kSB / 64);
+    const int l = (lane & 31) < M - 32 * j ? lane : (lane & 32);
+    const int jt = min(j, (M - 1) >> 5);
+    xcode[j] = xq + (size_t)jt * nu * 1024 + l * 16;
+    xscale[j] = xs + (size_t)jt * nkb * kSB + l * (kSB / 64);
   }
 
   v16f acc[NT * MT];
@@ -203,7 +211,7 @@ __global__ __launch_bounds__(64 * NW, NT == 2 ? 2 : 1) void gemm_fp4_stream_kern
     const int tn0 = (rtg * NT + i) * 32;
     const OutView out = out_view(seg, y, nullptr, tn0, N);   // the matrix this tile's columns go to (unused past N)
     out_ld[i] = __builtin_amdgcn_readfirstlane(out.N);
-    out_dst[i] = out.y + (size_t)row16 * out.N + out.n0 + 8 * c;
+    out_dst[i] = out.y + (size_t)(m0 + row16) * out.N + out.n0 + 8 * c;
     out_whole[i] = __builtin_amdgcn_readfirstlane(tn0 + 32 <= N && (out.N & 7) == 0 && ((uintptr_t)out.y & 15) == 0 &&
                                                   (!residual || res_rows));
     // (values the compiler may not look through: it would otherwise move their computation, kernel
@@ -281,7 +289,7 @@ __global__ __launch_bounds__(64 * NW, NT == 2 ? 2 : 1) void gemm_fp4_stream_kern
     // device-scope atomic, which the hardware performs at the point all XCDs agree on, and every
     // wave waits for its stores to be acknowledged before the workgroup moves the counter.
     constexpr int kTile = NT * MT * 16 * 64;  // floats per partial: register v of tile t at (16 t + v) * 64 + lane
-    float* mine = partial + ((size_t)rtg * ksplit + split) * kTile + wave * 256 + lane;
+    float* mine = partial + ((size_t)tile_id * ksplit + split) * kTile + wave * 256 + lane;
 #pragma unroll
     for (int t = 0; t < NT * MT; ++t)
 #pragma unroll
@@ -292,11 +300,11 @@ __global__ __launch_bounds__(64 * NW, NT == 2 ? 2 : 1) void gemm_fp4_stream_kern
     // One arrival per workgroup: a counter that every wave moved made the exchange 1.5 us slower (its
     // updates from different XCDs are served one after the other).
     if (threadIdx.x == 0)
-      arrival = __hip_atomic_fetch_add(counters + rtg, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      arrival = __hip_atomic_fetch_add(counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     // (one value for the workgroup: all its waves leave or all stay for the barrier further down)
     if (__builtin_amdgcn_readfirstlane(arrival) != (unsigned)(ksplit - 1)) return;
-    const float* all = partial + (size_t)rtg * ksplit * kTile + wave * 256 + lane;
+    const float* all = partial + (size_t)tile_id * ksplit * kTile + wave * 256 + lane;
     for (int s = 0; s < ksplit; ++s) {
 #pragma unroll
       for (int t = 0; t < NT * MT; ++t)
@@ -307,7 +315,7 @@ __global__ __launch_bounds__(64 * NW, NT == 2 ? 2 : 1) void gemm_fp4_stream_kern
           sum[t][q] = s == 0 ? p : sum[t][q] + p;
         }
     }
-    if (threadIdx.x == 0) __hip_atomic_store(counters + rtg, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) __hip_atomic_store(counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
   // ---- y[m][n] = bf16(alpha * sum) (+ bias) (+ residual, a further bf16 add): element q of this wave's
@@ -428,13 +436,19 @@ int64_t gemm_mxf4_stream_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 }
 
 // Arguments are validated by the caller (gemm_packed); `workspace` is null or 256-byte aligned with
-// its first kStreamCounterBytes zero.  NV: NVFP4 operands.
+// its first kStreamCounterBytes zero.  NV: NVFP4 operands.  slab_rows > 0 (a multiple of 32, at most 128):
+// M exceeds what one workgroup takes and is cut into slabs of that many rows, one grid plane each, K whole.
 template <bool NV>
 static int launch_stream(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                          const void* bias, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
-                         void* workspace, int64_t workspace_bytes, const OutSegments& seg, hipStream_t stream) {
-  const StreamPlan plan = stream_plan(M, N, K, workspace ? workspace_bytes : 0, NV);
-  const dim3 grid((unsigned)(((N + 31) / 32 + plan.nt - 1) / plan.nt), (unsigned)plan.ksplit);
+                         void* workspace, int64_t workspace_bytes, const OutSegments& seg, hipStream_t stream,
+                         int64_t slab_rows = 0) {
+  if (slab_rows) workspace = nullptr;
+  const int64_t rows = slab_rows ? slab_rows : M;   // what one workgroup sees
+  const StreamPlan plan = stream_plan(rows, N, K, workspace ? workspace_bytes : 0, NV);
+  if (!plan.use) return FPQ_E_UNSUPPORTED;
+  const dim3 grid((unsigned)(((N + 31) / 32 + plan.nt - 1) / plan.nt), (unsigned)plan.ksplit,
+                  (unsigned)(slab_rows ? (M + slab_rows - 1) / slab_rows : 1));
   unsigned* counters = (unsigned*)workspace;
   float* partial = workspace ? (float*)((uint8_t*)workspace + kStreamCounterBytes) : nullptr;
 #define FPQ_STREAM(NTT, MTT, DBB)                                                                       \
@@ -442,7 +456,7 @@ static int launch_stream(const void* xq, const void* xs, const void* wq, const v
                      (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq, (const uint8_t*)ws, alpha, \
                      (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, (int)M, (int)N,    \
                      (int)K, plan.bps, plan.ksplit, partial, counters, seg)
-  const int mt = (int)((M + 31) / 32);
+  const int mt = (int)((rows + 31) / 32);
   if (plan.nt == 2) {   // MXFP4, 33-64 rows only
     if constexpr (!NV) {
       if (mt != 2) return FPQ_E_UNSUPPORTED;
@@ -476,6 +490,15 @@ int gemm_fp4_stream(bool nv, const void* xq, const void* xs, const void* wq, con
                                   stream)
             : launch_stream<false>(xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, workspace, workspace_bytes, seg,
                                    stream);
+}
+
+// M rows in slabs of slab_rows (a multiple of 32 for which stream_eligible holds), all in one launch.
+int gemm_fp4_stream_slabs(bool nv, const void* xq, const void* xs, const void* wq, const void* ws,
+                          const float* alpha, const void* bias, const void* residual, void* y, int64_t M, int64_t N,
+                          int64_t K, int64_t slab_rows, const OutSegments& seg, hipStream_t stream) {
+  if (slab_rows < 32 || slab_rows > kStreamMaxRows || slab_rows % 32 != 0 || M <= slab_rows) return FPQ_E_UNSUPPORTED;
+  return nv ? launch_stream<true>(xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, nullptr, 0, seg, stream, slab_rows)
+            : launch_stream<false>(xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, nullptr, 0, seg, stream, slab_rows);
 }
 
 

@@ -86,8 +86,12 @@ def test_quantize_packed_rejects():
         capi.quantize_packed(torch.zeros(32, 512, dtype=torch.bfloat16), rot="gsr", g=128)
 
 
+# more than 128 rows: slabs of the weight-streaming kernel while slabs x weight tiles stay within 256 (a short
+# last slab, one with fewer row tiles than the others, eight slabs), else 64x128 tiles (up to 128 tiles of
+# 128x128) or 128x128 tiles, both with ragged edges
 @pytest.mark.parametrize("m,n,k", [(32, 32, 256), (65, 100, 256), (256, 256, 512), (300, 520, 768),
-                                   (256, 512, 2304), (512, 256, 4096)])
+                                   (256, 512, 2304), (512, 256, 4096), (129, 4096, 512), (260, 100, 256),
+                                   (1000, 1000, 256), (300, 2790, 512), (300, 8300, 256), (257, 4100, 256)])
 @pytest.mark.parametrize("bias", [False, True])
 def test_gemm_packed_matches_oracle_and_row_major_kernel(m, n, k, bias):
     g = torch.Generator().manual_seed(m + n + k)
@@ -108,9 +112,14 @@ def test_gemm_packed_matches_oracle_and_row_major_kernel(m, n, k, bias):
     # fp32 accumulation in another order than the oracle's, then one bf16 rounding (two with bias)
     tol = 2.0 ** -7 * want.double().abs() + 1e-5 * mag + 1e-6
     assert ((y.double() - want.double()).abs() <= tol).all()
-    # the same MFMA sequence per output as the row-major kernel: identical bits
     y_rm = capi.gemm(xq, xs, wq, ws, alpha, "mxfp4", bias=b)
-    assert torch.equal(y.view(torch.int16), y_rm.view(torch.int16))
+    if k == 256 or (m > 128 and ((m + 127) // 128) * ((n + 31) // 32) > 256):
+        # the tile kernels (and any kernel on one block of K): the same MFMA sequence per output as the
+        # row-major kernel, identical bits
+        assert torch.equal(y.view(torch.int16), y_rm.view(torch.int16))
+    else:
+        # the weight-streaming kernel (also in slabs) adds four K parts: another order, the same tolerance
+        assert ((y.double() - y_rm.double()).abs() <= 2 * tol).all()
 
 
 def test_gemm_packed_rejects():
@@ -170,7 +179,9 @@ def test_pack_nv_kernel_matches_definition(rows, k):
                                    (96, 2048, 4096), (128, 1000, 2304), (5, 257, 12288), (100, 8290, 256),
                                    (96, 40000, 256), (128, 16384, 256), (128, 16400, 256), (97, 14339, 512),
                                    # 129-256 rows at up to 256 weight tiles: two passes of the weight-streaming kernel
-                                   (130, 515, 512), (192, 6144, 256), (256, 8192, 256), (255, 8200, 256), (161, 100, 1024)])
+                                   (130, 515, 512), (192, 6144, 256), (256, 8192, 256), (255, 8200, 256), (161, 100, 1024),
+                                   # more than 128 rows in slabs, and the tile kernels' ragged edges past them
+                                   (129, 4096, 512), (260, 100, 256), (1000, 1000, 256), (300, 2790, 512), (300, 8300, 256)])
 @pytest.mark.parametrize("bias", [False, True])
 def test_gemm_nv_packed_matches_oracle(m, n, k, bias):
     g = torch.Generator().manual_seed(m + 2 * n + k)
@@ -200,7 +211,8 @@ def test_gemm_nv_packed_matches_oracle(m, n, k, bias):
     assert torch.equal(capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=b, residual=res, in_place=True), yr)
 
 
-@pytest.mark.parametrize("m,n,k", [(32, 32, 256), (65, 100, 256), (300, 520, 768), (256, 4096, 512), (2048, 1024, 512)])
+@pytest.mark.parametrize("m,n,k", [(32, 32, 256), (65, 100, 256), (300, 520, 768), (256, 4096, 512), (2048, 1024, 512),
+                                   (300, 2790, 256), (300, 8300, 256), (129, 4096, 256)])
 @pytest.mark.parametrize("bias", [False, True])
 def test_gemm_packed_residual_equals_gemm_then_add(m, n, k, bias):
     """The residual epilogue is the separate bf16 addition, bit for bit, for every tile shape and at
