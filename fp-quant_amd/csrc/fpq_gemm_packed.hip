@@ -463,7 +463,7 @@ static int pack_operand(const void* codes, const void* scales, int64_t scale_str
 #define FPQ_PACKED_HALF_TILES 1  // large M: 1 = 256x128 tiles for MXFP4, 2 = for NVFP4 too, 0 = 256x256
 #endif
 #ifndef FPQ_STREAM_SLAB_WGS
-#define FPQ_STREAM_SLAB_WGS 256   // more than 128 rows: slabs of the streaming kernel while they number at most this
+#define FPQ_STREAM_SLAB_WGS 256   // row slabs of the streaming kernel x weight tiles: at most this many workgroups
 #endif
 #ifndef FPQ_PACKED_NARROW_BELOW
 #define FPQ_PACKED_NARROW_BELOW 128  // up to this many 128x128 tiles: 64x128 tiles instead
@@ -490,22 +490,32 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
       ((uintptr_t)y & 15u) || ((uintptr_t)residual & 15u))
     return FPQ_E_ALIGN;
   if ((uintptr_t)workspace & 255u) return FPQ_E_ALIGN;
+  // Few weight tiles: the rows are cut into slabs, one grid plane of the weight-streaming kernel each, as low as
+  // keeps slabs x weight tiles within one round of the 256 CUs -- more workgroups that each hold fewer
+  // activation row tiles (fewer registers, less to re-read per weight tile, a shorter tail) and that, unlike
+  // the tile kernels', share nothing through LDS and meet at no barrier in their K loop.  Slabs of 32 / 64 /
+  // 96 / 128 rows measured best exactly where they are the lowest that fit (us, K = 4096, against one
+  // workgroup per weight tile or the tile kernels): N = 4096: 64 rows 6.3 -> 5.3, 128 rows 8.0 -> 6.2, 256
+  // rows 9.9 -> 8.0; N = 2048: 128 rows 7.8 -> 5.1, 256 rows 7.6 -> 6.0 (tiles: 9.5), 384 rows 9.6 -> 6.9;
+  // N = 1024: 512 rows 9.5 -> 5.5; NVFP4 N = 4096: 128 rows 14.1 -> 9.3, 256 rows 28 -> 14.1; K = 14336, 256
+  // rows: 32 -> 19.  (More slabs than one round -- two or three workgroups per CU -- measured slower.)  K
+  // stays whole in slabs, so a shape whose K the caller's workspace lets split keeps the split.
+  {
+    const int64_t tiles = (N + 31) / 32;
+    const bool splits = workspace && workspace_bytes > 16384 && M <= 128 && gemm_mxf4_stream_workspace_bytes(M, N, K) > 0;
+    for (int64_t cap = 32; cap <= 128 && !splits; cap += 32) {
+      const int64_t slabs = (M + cap - 1) / cap;
+      if (slabs * tiles > FPQ_STREAM_SLAB_WGS) continue;
+      const int64_t rows = ((M + slabs - 1) / slabs + 31) / 32 * 32;   // rows of a slab, whole 32-row tiles
+      if (slabs > 1 && rows < M && stream_eligible(NV, rows, N, K))
+        return gemm_fp4_stream_slabs(NV, xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, rows, seg,
+                                     (hipStream_t)stream);
+      break;   // one slab, or a shape the kernel does not take: the paths below
+    }
+  }
   if (stream_eligible(NV, M, N, K) && (!NV || M <= FPQ_NV_STREAM_ROWS))
     return gemm_fp4_stream(NV, xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, workspace, workspace_bytes,
                            seg, (hipStream_t)stream);
-  // More than 128 rows while slabs of at most 128 rows x weight tiles number at most 256: the weight-streaming
-  // kernel with one grid plane per slab fills the CUs with workgroups that neither share anything through LDS
-  // nor meet at barriers, where the tile kernels below would run 32-128 workgroups that do.  N = 4096: 129-256
-  // rows 9.9 -> 6.8-8.0 us at K = 4096, 27-32 -> 16-19 us at K = 14336 (NVFP4: 20-28 -> 11.7-14.1 us, K = 12288
-  // 44-67 -> 27-34 us); N = 2048, K = 8192 up to 512 rows 16 -> 11.8 us (NVFP4 47 -> 24); N = 1024 up to 1024 rows.
-  // (Slabs of 96 rows, two workgroups per CU and 512 in all, measured within +-10 % of the tile kernels.)
-  if (M > 128) {
-    const int64_t slabs = (M + 127) / 128;
-    const int64_t rows = ((M + slabs - 1) / slabs + 31) / 32 * 32;   // rows of a slab, whole 32-row tiles
-    if (slabs * ((N + 31) / 32) <= FPQ_STREAM_SLAB_WGS && rows < M && stream_eligible(NV, rows, N, K))
-      return gemm_fp4_stream_slabs(NV, xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, rows, seg,
-                                   (hipStream_t)stream);
-  }
   if constexpr (NV) {
     // 129-256 rows of NVFP4 at up to 256 weight tiles (N <= 8192): the 128x128 tile kernel fills at most
     // half of the 256 CUs with workgroups that take 34 us for K = 4096, so two passes of the weight-streaming

@@ -469,7 +469,7 @@ static int launch_stream(const void* xq, const void* xs, const void* wq, const v
     case 1:
       // enough workgroups for three per CU: two blocks in flight per wave beat four by 3-5 %; with fewer
       // workgroups the deeper ring of each wave is what keeps the memory system busy
-      if ((int64_t)grid.x * grid.y >= 384) FPQ_STREAM(1, 1, 2);
+      if ((int64_t)grid.x * grid.y * grid.z >= 384) FPQ_STREAM(1, 1, 2);
       else FPQ_STREAM(1, 1, 4);
       break;
     case 2: FPQ_STREAM(1, 2, 2); break;
