@@ -499,10 +499,11 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
   // rows 9.9 -> 8.0; N = 2048: 128 rows 7.8 -> 5.1, 256 rows 7.6 -> 6.0 (tiles: 9.5), 384 rows 9.6 -> 6.9;
   // N = 1024: 512 rows 9.5 -> 5.5; NVFP4 N = 4096: 128 rows 14.1 -> 9.3, 256 rows 28 -> 14.1; K = 14336, 256
   // rows: 32 -> 19.  (More slabs than one round -- two or three workgroups per CU -- measured slower.)  K
-  // stays whole in slabs, so a shape whose K the caller's workspace lets split keeps the split.
+  // stays whole in slabs, so a shape whose K the caller's workspace lets split keeps the split up to 96 rows
+  // (N = 4096, K = 14336: 64 rows 11.7 split / 11.9 us in slabs, 96 rows 13.9 / 13.9, 128 rows 15.4 / 14.1).
   {
     const int64_t tiles = (N + 31) / 32;
-    const bool splits = workspace && workspace_bytes > 16384 && M <= 128 && gemm_mxf4_stream_workspace_bytes(M, N, K) > 0;
+    const bool splits = workspace && workspace_bytes > 16384 && M <= 96 && gemm_mxf4_stream_workspace_bytes(M, N, K) > 0;
     for (int64_t cap = 32; cap <= 128 && !splits; cap += 32) {
       const int64_t slabs = (M + cap - 1) / cap;
       if (slabs * tiles > FPQ_STREAM_SLAB_WGS) continue;

@@ -86,9 +86,9 @@ def test_quantize_packed_rejects():
         capi.quantize_packed(torch.zeros(32, 512, dtype=torch.bfloat16), rot="gsr", g=128)
 
 
-# more than 128 rows: slabs of the weight-streaming kernel while slabs x weight tiles stay within 256 (a short
-# last slab, one with fewer row tiles than the others, eight slabs), else 64x128 tiles (up to 128 tiles of
-# 128x128) or 128x128 tiles, both with ragged edges
+# row slabs of the weight-streaming kernel while slabs x weight tiles stay within 256 (a short last slab, one
+# with fewer row tiles than the others, eight slabs), else 64x128 tiles (up to 128 tiles of 128x128) or
+# 128x128 tiles, both with ragged edges
 @pytest.mark.parametrize("m,n,k", [(32, 32, 256), (65, 100, 256), (256, 256, 512), (300, 520, 768),
                                    (256, 512, 2304), (512, 256, 4096), (129, 4096, 512), (260, 100, 256),
                                    (1000, 1000, 256), (300, 2790, 512), (300, 8300, 256), (257, 4100, 256)])
