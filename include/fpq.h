@@ -311,7 +311,7 @@ int fpq_gemm_mxf4_packed_splitk(const void* xq_packed, const void* xs_packed, co
                                 void* workspace, int64_t workspace_bytes, void* stream);
 /* The same for packed NVFP4 operands (fpq_gemm_nvf4_packed, with `residual` non-null fpq_gemm_nvf4_packed_residual);
  * workspace as above, sized by fpq_gemm_mxf4_packed_workspace_bytes (the split is the same for both formats;
- * 129-256 rows of NVFP4 at N <= 8192 run as two passes over at most 128 rows each, and each pass may use it:
+ * 129-256 rows of NVFP4 at 4096 < N <= 8192 run as two passes over at most 128 rows each, and each pass may use it:
  * size it for 128 rows). */
 int fpq_gemm_nvf4_packed_splitk(const void* xq_packed, const void* xs_packed, const void* wq_packed,
                                 const void* ws_packed, const float* alpha, const void* bias,
