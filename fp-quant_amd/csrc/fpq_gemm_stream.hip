@@ -398,7 +398,8 @@ struct StreamPlan {
 // deliver for 33-64 rows, but need so many registers that one workgroup fills a CU; one tile per
 // workgroup with two blocks in flight, two workgroups per CU, measured 5-13 % faster -- except from
 // 768 weight tiles on, where two tiles per workgroup with ONE block in flight, held to 256 registers,
-// are 12-16 % faster: MXFP4, N = 28672 at 64 rows 20.1 -> 17.0 us, N = 128256 73.5 -> 61.6 us.)
+// are 12-16 % faster: MXFP4, N = 28672 at 64 rows 20.1 -> 17.0 us, N = 128256 73.5 -> 61.6 us; NVFP4 -- where the
+// two weight tiles also share the activations' conversion to fp16 -- N = 28672 26.2 -> 22.6 us, N = 57344 45.6 -> 40.8.)
 // K is split across workgroups when the weight tiles leave at least half of the CUs idle and every
 // part keeps at least 4096 of K (the exchange of partial tiles through the workspace costs about as
 // much as streaming 16 blocks); fewer parts if the workspace is small.  (While one wave did the
@@ -411,7 +412,7 @@ static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace
   if (rt_m == 3 && !nv && tiles > 1024) return plan;
   if (rt_m == 4 && tiles > (nv ? 512 : 256)) return plan;
   plan.use = true;
-  if (rt_m == 2 && tiles >= 768 && !nv) plan.nt = 2;
+  if (rt_m == 2 && tiles >= 768) plan.nt = 2;
   const int64_t groups = (tiles + plan.nt - 1) / plan.nt;
   int64_t ksplit = 1;
   if (workspace_bytes > kStreamCounterBytes && groups <= kStreamCounters) {
@@ -457,13 +458,10 @@ static int launch_stream(const void* xq, const void* xs, const void* wq, const v
                      (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, (int)M, (int)N,    \
                      (int)K, plan.bps, plan.ksplit, partial, counters, seg)
   const int mt = (int)((rows + 31) / 32);
-  if (plan.nt == 2) {   // MXFP4, 33-64 rows only
-    if constexpr (!NV) {
-      if (mt != 2) return FPQ_E_UNSUPPORTED;
-      FPQ_STREAM(2, 2, 1);
-      return (int)hipGetLastError();
-    }
-    return FPQ_E_UNSUPPORTED;
+  if (plan.nt == 2) {   // 33-64 rows only
+    if (mt != 2) return FPQ_E_UNSUPPORTED;
+    FPQ_STREAM(2, 2, 1);
+    return (int)hipGetLastError();
   }
   switch (mt) {
     case 1:

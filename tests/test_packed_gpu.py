@@ -181,7 +181,9 @@ def test_pack_nv_kernel_matches_definition(rows, k):
                                    # 129-256 rows at up to 256 weight tiles: two passes of the weight-streaming kernel
                                    (130, 515, 512), (192, 6144, 256), (256, 8192, 256), (255, 8200, 256), (161, 100, 1024),
                                    # more than 128 rows in slabs, and the tile kernels' ragged edges past them
-                                   (129, 4096, 512), (260, 100, 256), (1000, 1000, 256), (300, 2790, 512), (300, 8300, 256)])
+                                   (129, 4096, 512), (260, 100, 256), (1000, 1000, 256), (300, 2790, 512), (300, 8300, 256),
+                                   # 33-64 rows at 768 weight tiles or more: two weight tiles per workgroup (odd count, ragged N)
+                                   (64, 24600, 256), (45, 28672, 256)])
 @pytest.mark.parametrize("bias", [False, True])
 def test_gemm_nv_packed_matches_oracle(m, n, k, bias):
     g = torch.Generator().manual_seed(m + 2 * n + k)
