@@ -399,7 +399,7 @@ struct StreamPlan {
 // workgroup with two blocks in flight, two workgroups per CU, measured 5-13 % faster -- except from
 // 768 weight tiles on, where two tiles per workgroup with ONE block in flight, held to 256 registers,
 // are 12-16 % faster: MXFP4, N = 28672 at 64 rows 20.1 -> 17.0 us, N = 128256 73.5 -> 61.6 us; NVFP4 -- where the
-// two weight tiles also share the activations' conversion to fp16 -- N = 28672 26.2 -> 22.6 us, N = 57344 45.6 -> 40.8.)
+// two weight tiles also share the activations' conversion to fp16 -- N = 28672 26.2 -> 22.6 us, N = 57344 45.6 -> 40.8, and already from 384 tiles on 1-4 %.)
 // K is split across workgroups when the weight tiles leave at least half of the CUs idle and every
 // part keeps at least 4096 of K (the exchange of partial tiles through the workspace costs about as
 // much as streaming 16 blocks); fewer parts if the workspace is small.  (While one wave did the
@@ -412,7 +412,7 @@ static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace
   if (rt_m == 3 && !nv && tiles > 1024) return plan;
   if (rt_m == 4 && tiles > (nv ? 512 : 256)) return plan;
   plan.use = true;
-  if (rt_m == 2 && tiles >= 768) plan.nt = 2;
+  if (rt_m == 2 && tiles >= (nv ? 384 : 768)) plan.nt = 2;
   const int64_t groups = (tiles + plan.nt - 1) / plan.nt;
   int64_t ksplit = 1;
   if (workspace_bytes > kStreamCounterBytes && groups <= kStreamCounters) {
