@@ -123,8 +123,9 @@ template <int G, int ROT, int PRO = kProNone>
 __device__ __forceinline__ void lane8_load_rotate(const uint4* __restrict__ x, uint32_t chunk, bool active,
                                                   uint32_t lane, float norm, float* __restrict__ stage,
                                                   const uint16_t* __restrict__ hmat, float (&p)[8],
-                                                  const Prologue& pro = Prologue{}, float row_scale = -1.0f) {
-  // row_scale >= 0: the row's 1 / rms, computed by the caller in this launch (else pro.row_scale[row])
+                                                  const Prologue& pro = Prologue{}, float row_scale = 0.0f) {
+  // kProRmsNorm: the row's 1 / rms is pro.row_scale[row]; a caller that computed it in this launch leaves
+  // pro.row_scale null and passes the value as row_scale (any value, NaN and infinity included, is data)
   uint4 raw = make_uint4(0u, 0u, 0u, 0u);
   if (PRO == kProNone) {
     if (active) raw = x[chunk];
@@ -137,7 +138,7 @@ __device__ __forceinline__ void lane8_load_rotate(const uint4* __restrict__ x, u
       raw = x[(size_t)row * pro.ld_first + cc];
       if (PRO == kProRmsNorm) {
         aux = pro.col_scale[cc];
-        rs = row_scale >= 0.0f ? row_scale : pro.row_scale[row];
+        rs = pro.row_scale ? pro.row_scale[row] : row_scale;
       } else {
         aux = pro.second[(size_t)row * pro.ld_second + cc];
       }
@@ -241,7 +242,7 @@ __device__ __forceinline__ void lane8_process(const uint4* __restrict__ x, uint3
                                               uint32_t scale_stride, float norm, float gscale, float rg,
                                               float* __restrict__ stage, const uint16_t* __restrict__ hmat,
                                               uint8_t* __restrict__ mask = nullptr,
-                                              const Prologue& pro = Prologue{}, float row_scale = -1.0f) {
+                                              const Prologue& pro = Prologue{}, float row_scale = 0.0f) {
   static_assert(!QUEST || FMT == kFmtMx, "the quest rule exists for MXFP4 only");
   constexpr int GROUP = FMT == kFmtMx ? 32 : 16;
   float p[8];

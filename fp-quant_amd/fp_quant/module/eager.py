@@ -39,15 +39,26 @@ from .hip_ops import (
 )
 
 
-def cached_on(t: torch.Tensor, slot: str, key, make, remember: bool = True):
+def cached_on(t: torch.Tensor, slot: str, key, make, remember: bool = True, refresh: bool = False):
     """`make()` remembered on tensor `t` under attribute `slot` while `key` stays the same.
     `remember=False` uses what is remembered but stores nothing new: for callers that may be running
-    inside a compiler's graph memory pool, where a tensor that outlives the call is an error."""
+    inside a compiler's graph memory pool, where a tensor that outlives the call is an error.
+    `refresh`: make it anew whatever the key says.  A remembered tensor that is outdated is overwritten
+    in place where that is possible, so that a recorded graph, which holds its address, reads the new value."""
     hit = getattr(t, slot, None)
-    if hit is not None and hit[0] == key:
+    if hit is not None and hit[0] == key and not refresh:
         return hit[1]
     val = make()
     if remember:
+        old = hit[1] if hit is not None else None
+        if (isinstance(old, torch.Tensor) and isinstance(val, torch.Tensor) and old.shape == val.shape
+                and old.dtype == val.dtype and old.device == val.device and old is not val
+                and not torch.cuda.is_current_stream_capturing()):
+            try:
+                old.copy_(val)
+                val = old
+            except RuntimeError:   # (an inference tensor outside inference mode: replaced instead)
+                pass
         try:
             setattr(t, slot, (key, val))
         except (AttributeError, RuntimeError):
@@ -56,20 +67,21 @@ def cached_on(t: torch.Tensor, slot: str, key, make, remember: bool = True):
 
 
 def linear_alpha(weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor,
-                 remember: bool = True) -> torch.Tensor:
+                 remember: bool = True, refresh: bool = False) -> torch.Tensor:
     """fp32 one-element `1 / (wgs * ags)` evaluated in the buffers' dtype as the reference does
     (linear_fns.py:505; bf16 buffers round 1/9 to 0.111328125), cached until a buffer changes."""
     key = (_version(weight_global_scale), _version(act_global_scale), act_global_scale.data_ptr(),
            weight_global_scale.data_ptr())
     return cached_on(weight_global_scale, "_fpq_alpha", key,
                      lambda: (1.0 / (weight_global_scale * act_global_scale)).float().reshape(1).contiguous(),
-                     remember)
+                     remember, refresh)
 
 
-def as_f32_scalar(t: torch.Tensor, remember: bool = True) -> torch.Tensor:
+def as_f32_scalar(t: torch.Tensor, remember: bool = True, refresh: bool = False) -> torch.Tensor:
     if t.dtype == torch.float32 and t.is_contiguous():
         return t
-    return cached_on(t, "_fpq_f32", (_version(t), t.data_ptr()), lambda: t.detach().float().contiguous(), remember)
+    return cached_on(t, "_fpq_f32", (_version(t), t.data_ptr()), lambda: t.detach().float().contiguous(), remember,
+                     refresh)
 
 
 # Several layers that consume one tensor (q/k/v projections, gate/up projections) would rotate and
@@ -282,7 +294,8 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
             if packed is None:
                 wp, wsp = packed_weight(wq, ws, True)
             # (NVFP4 runs 129-256 rows as two passes of the kernel that can split K: each may use the workspace)
-            workspace = splitk_workspace(wq, n, k, remember) if (m <= 2 * SPLIT_K_ROWS and packed is None) else None
+            workspace = (splitk_workspace(wq, n, k, remember, stream)
+                         if (m <= 2 * SPLIT_K_ROWS and packed is None) else None)
             if workspace is not None:
                 st = lib.fpq_gemm_nvf4_packed_splitk(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
                                                      alpha.data_ptr(), b_ptr,
@@ -312,7 +325,7 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
         pc, ps = qa.packed()
         if packed is None:
             wp, wsp = packed_weight(wq, ws)
-        workspace = splitk_workspace(wq, n, k, remember) if (m <= SPLIT_K_ROWS and packed is None) else None
+        workspace = splitk_workspace(wq, n, k, remember, stream) if (m <= SPLIT_K_ROWS and packed is None) else None
         if workspace is not None:
             # few weight rows and a long K at decode sizes: K split across workgroups (deterministic sum)
             st = lib.fpq_gemm_mxf4_packed_splitk(pc.data_ptr(), ps.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
@@ -416,16 +429,21 @@ def _member_key(wq: torch.Tensor, ws: torch.Tensor, bias: Optional[torch.Tensor]
             None if bias is None else (bias.data_ptr(), _version(bias)))
 
 
-def weight_group(members, create: bool = False, nvfp4: bool = False) -> Optional[WeightGroup]:
+def weight_group(members, create: bool = False, nvfp4: bool = False,
+                 previous: Optional["WeightGroup"] = None) -> Optional[WeightGroup]:
     """The WeightGroup of `members` = [(qweight, scales, bias or None, in_features), ...] (one format, same K,
     every N a multiple of 32, biases all absent or all contiguous bf16; weights row-major, or all in the packed
     layout only), remembered on the first member's qweight until a member is written to; built now if
-    `create`, else None when there is none."""
+    `create`, else None when there is none.  A group built in place of an outdated one of the same shape
+    (`previous`, or the one remembered) is written into that one's buffers, so that the addresses a recorded
+    graph holds stay those of the current weights."""
     first = members[0][0]
     key = tuple(_member_key(*m[:3]) for m in members)
     hit = getattr(first, "_fpq_group", None)
     if hit is not None and hit.key == key and hit.nvfp4 == nvfp4:
         return hit
+    if previous is None:
+        previous = hit
     if not create or not packed_weights_enabled():
         return None
     k = members[0][3]
@@ -456,30 +474,43 @@ def weight_group(members, create: bool = False, nvfp4: bool = False) -> Optional
     group.n, group.splits, group.k, group.nvfp4 = n, splits, k, nvfp4
     scales_bytes = lib.fpq_packed_scales_bytes_nv if nvfp4 else lib.fpq_packed_scales_bytes
     pack = lib.fpq_pack_nvf4 if nvfp4 else lib.fpq_pack_mxf4
+    reuse = previous
+    if (reuse is not None and (reuse.nvfp4 != nvfp4 or reuse.k != k or reuse.splits != splits or reuse.wp.device != dev
+                               or torch.cuda.is_current_stream_capturing())):
+        reuse = None
     with on_device(dev):
         stream = _current_stream(dev.index)
+        bounds, row = [], 0
+        for rows in splits:
+            bounds.append((lib.fpq_packed_codes_bytes(row, k), lib.fpq_packed_codes_bytes(row + rows, k),
+                           scales_bytes(row, k), scales_bytes(row + rows, k)))
+            row += rows
         if packed_only:
-            # the members' buffers laid end to end; the members then live in the new buffers (views) and
-            # their own are freed, so the weights are still held once
-            group.wp = torch.cat([m[0] for m in members])
-            group.wsp = torch.cat([m[1] for m in members])
+            in_place = reuse is not None and all(
+                m[0].data_ptr() == reuse.wp.data_ptr() + b[0] and m[1].data_ptr() == reuse.wsp.data_ptr() + b[2]
+                for m, b in zip(members, bounds))
+            if in_place:     # the members already live in the outdated group's buffers (re-packed there)
+                group.wp, group.wsp = reuse.wp, reuse.wsp
+            else:
+                # the members' buffers laid end to end; the members then live in the new buffers (views) and
+                # their own are freed, so the weights are still held once
+                group.wp = torch.cat([m[0] for m in members])
+                group.wsp = torch.cat([m[1] for m in members])
+        elif reuse is not None:
+            group.wp, group.wsp = reuse.wp, reuse.wsp
         else:
             group.wp = torch.empty(lib.fpq_packed_codes_bytes(n, k), dtype=torch.uint8, device=dev)
             group.wsp = torch.empty(scales_bytes(n, k), dtype=torch.uint8, device=dev)
-        row = 0
-        for wq, ws, _, _ in members:
-            rows = weight_rows(wq, k)
-            c0, c1 = lib.fpq_packed_codes_bytes(row, k), lib.fpq_packed_codes_bytes(row + rows, k)
-            s0, s1 = scales_bytes(row, k), scales_bytes(row + rows, k)
+        for (wq, ws, _, _), rows, (c0, c1, s0, s1) in zip(members, splits, bounds):
             pc, ps = group.wp[c0:c1], group.wsp[s0:s1]
             if packed_only:
-                wq.data, ws.data = pc, ps
+                if wq.data_ptr() != pc.data_ptr() or ws.data_ptr() != ps.data_ptr():
+                    wq.data, ws.data = pc, ps
             else:
                 st = pack(wq.data_ptr(), ws.data_ptr(), ws.shape[1], rows, k, pc.data_ptr(), ps.data_ptr(), stream)
                 _engine.check(st, "fpq_pack")
                 # the member's own packed copy: these views (same key as hip_ops.packed_weight uses)
                 wq._fpq_packed = ((wq.data_ptr(), _version(wq), ws.data_ptr(), _version(ws), tuple(wq.shape), nvfp4), pc, ps)
-            row += rows
     group.key = tuple(_member_key(*m[:3]) for m in members)   # (packed-only members have just moved)
     group.bias = torch.cat([m[2] for m in members]).contiguous() if all(have_bias) else None
     try:
@@ -645,14 +676,17 @@ def _(gate, up, hadamard_matrix, wq, ws, weight_global_scale, act_global_scale, 
     return gate.new_empty((rows, weight_rows(wq, gate.shape[-1])), dtype=torch.bfloat16)
 
 
-def prime(hadamard_matrix: torch.Tensor, weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor) -> None:
+def prime(hadamard_matrix: torch.Tensor, weight_global_scale: torch.Tensor, act_global_scale: torch.Tensor,
+          refresh: bool = False) -> None:
     """Compute and remember a layer's per-call constants (rotation kind, alpha, fp32 global scale) now,
-    in ordinary memory: afterwards neither a traced call nor a graph capture has to create them."""
+    in ordinary memory: afterwards neither a traced call nor a graph capture has to create them.
+    `refresh`: the buffers may have been rewritten behind their modification counters; alpha and the fp32
+    scale are computed anew (into the tensors that held them)."""
     if not weight_global_scale.is_cuda or hadamard_matrix.device != weight_global_scale.device:
         return
     classify_rotation(as_bf16(hadamard_matrix))
-    linear_alpha(weight_global_scale, act_global_scale)
-    as_f32_scalar(act_global_scale)
+    linear_alpha(weight_global_scale, act_global_scale, refresh=refresh)
+    as_f32_scalar(act_global_scale, refresh=refresh)
     prepare_device(weight_global_scale.device)
 
 

@@ -37,13 +37,14 @@ _TENSOR_CACHES = ("_fpq_rotation", "_fpq_bf16", "_fpq_packed", "_fpq_group", "_f
                   "_fpq_splitk")
 
 
-def drop_tensor_caches(*tensors) -> None:
-    """Forget everything remembered on these tensors (packed weights, alpha, converted copies): for
-    callers that rewrote their storage in a way the modification counter does not see."""
+def drop_tensor_caches(*tensors, keep=()) -> None:
+    """Forget everything remembered on these tensors (packed weights, alpha, converted copies) but the
+    attributes named in `keep`: for callers that rewrote their storage in a way the modification counter does
+    not see."""
     for t in tensors:
         if isinstance(t, torch.Tensor):
             for name in _TENSOR_CACHES:
-                if hasattr(t, name):
+                if name not in keep and hasattr(t, name):
                     try:
                         delattr(t, name)
                     except AttributeError:
@@ -306,24 +307,35 @@ def packed_weights_enabled() -> bool:
     return os.environ.get("FPQ_PACKED_WEIGHTS", "1") != "0"
 
 
-def pack_mxf4(codes: torch.Tensor, scales: torch.Tensor, rows: int, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+def _pack_buffers(into, codes_bytes: int, scales_bytes: int, device) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Output buffers of a pack: `into` = (codes, scales) of exactly these sizes (written in place, so that
+    raw pointers to them stay valid), or new ones."""
+    if into is not None:
+        pc, ps = into
+        if (pc.numel() == codes_bytes and ps.numel() == scales_bytes and pc.device == device and ps.device == device
+                and pc.dtype == torch.uint8 and ps.dtype == torch.uint8 and pc.is_contiguous() and ps.is_contiguous()):
+            return pc, ps
+    return (torch.empty(codes_bytes, dtype=torch.uint8, device=device),
+            torch.empty(scales_bytes, dtype=torch.uint8, device=device))
+
+
+def pack_mxf4(codes: torch.Tensor, scales: torch.Tensor, rows: int, k: int, into=None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Row-major codes [rows, k/2] and E8M0 scales [>=rows, >=k/32] -> the packed layout of
     fpq_gemm_mxf4_packed (rows padded to a multiple of 32)."""
     lib = _engine.lib()
-    pc = torch.empty(lib.fpq_packed_codes_bytes(rows, k), dtype=torch.uint8, device=codes.device)
-    ps = torch.empty(lib.fpq_packed_scales_bytes(rows, k), dtype=torch.uint8, device=codes.device)
+    pc, ps = _pack_buffers(into, lib.fpq_packed_codes_bytes(rows, k), lib.fpq_packed_scales_bytes(rows, k), codes.device)
     st = lib.fpq_pack_mxf4(codes.data_ptr(), scales.data_ptr(), scales.shape[1], rows, k,
                            pc.data_ptr(), ps.data_ptr(), _stream(codes))
     _engine.check(st, "fpq_pack_mxf4")
     return pc, ps
 
 
-def pack_nvf4(codes: torch.Tensor, scales: torch.Tensor, rows: int, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+def pack_nvf4(codes: torch.Tensor, scales: torch.Tensor, rows: int, k: int, into=None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Row-major codes [rows, k/2] and E4M3 scales [>=rows, >=k/16] -> the packed layout of
     fpq_gemm_nvf4_packed."""
     lib = _engine.lib()
-    pc = torch.empty(lib.fpq_packed_codes_bytes(rows, k), dtype=torch.uint8, device=codes.device)
-    ps = torch.empty(lib.fpq_packed_scales_bytes_nv(rows, k), dtype=torch.uint8, device=codes.device)
+    pc, ps = _pack_buffers(into, lib.fpq_packed_codes_bytes(rows, k), lib.fpq_packed_scales_bytes_nv(rows, k),
+                           codes.device)
     st = lib.fpq_pack_nvf4(codes.data_ptr(), scales.data_ptr(), scales.shape[1], rows, k,
                            pc.data_ptr(), ps.data_ptr(), _stream(codes))
     _engine.check(st, "fpq_pack_nvf4")
@@ -380,16 +392,20 @@ def packed_weight_ready(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False)
     return hit is not None and hit[0] == _packed_weight_key(wq, ws, nvfp4)
 
 
-def packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+def packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False, into=None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Packed copy of a weight, cached on the code tensor until either tensor is written to (a weight
-    held in the packed layout only is its own packed copy)."""
+    held in the packed layout only is its own packed copy).  A copy that has gone stale is re-packed into the
+    buffers it already has, and a new one into `into` = (codes, scales) if those have the right sizes: the
+    addresses a recorded graph holds stay those of the layer's current weight."""
     if wq.dim() == 1:
         return wq, ws
     key = _packed_weight_key(wq, ws, nvfp4)
     hit = getattr(wq, "_fpq_packed", None)
     if hit is not None and hit[0] == key:
         return hit[1], hit[2]
-    pc, ps = (pack_nvf4 if nvfp4 else pack_mxf4)(wq, ws, wq.shape[0], wq.shape[1] * 2)
+    if hit is not None and into is None and not torch.cuda.is_current_stream_capturing():
+        into = (hit[1], hit[2])
+    pc, ps = (pack_nvf4 if nvfp4 else pack_mxf4)(wq, ws, wq.shape[0], wq.shape[1] * 2, into)
     try:
         wq._fpq_packed = (key, pc, ps)
     except (AttributeError, RuntimeError):
@@ -398,20 +414,53 @@ def packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool = False) -> Tu
 
 
 
+def adopt_packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool, pc: torch.Tensor, ps: torch.Tensor) -> None:
+    """Declare (pc, ps) the packed copy of the row-major weight (wq, ws), as packed_weight would have made it."""
+    try:
+        wq._fpq_packed = (_packed_weight_key(wq, ws, nvfp4), pc, ps)
+    except (AttributeError, RuntimeError):
+        pass
+
+
 _splitk_need = {}   # (n, k) -> workspace bytes with which fpq_gemm_mxf4_packed_splitk splits K at up to SPLIT_K_ROWS rows
 SPLIT_K_ROWS = 128  # the rows the weight-streaming GEMM takes
-# FPQ_SPLIT_K=0: no layer keeps a split-K workspace (for callers that run ONE layer object on several streams at
-# the same time, whose kernels would share it)
+# FPQ_SPLIT_K=0: no split-K workspace anywhere; every GEMM walks the whole of K in one workgroup
 SPLIT_K = os.environ.get("FPQ_SPLIT_K", "1") != "0"
 
+# Eager calls: ONE workspace per (device, stream), shared by every layer called on that stream.  Kernels on a
+# stream run one after the other and each leaves the workspace zeroed, so layers may share it, while calls of
+# one layer on different streams (host threads with a stream each) never meet in one.  Created, and grown, by
+# the call that needs it, on the stream it is for; at most _STREAM_WORKSPACES_MAX per device (the oldest goes
+# first: PyTorch's allocator hands its memory out again in the order of the stream that used it).
+_stream_workspaces = {}
+_STREAM_WORKSPACES_MAX = 16
 
-def splitk_workspace(wq: torch.Tensor, n: int, k: int, create: bool) -> Optional[torch.Tensor]:
-    """The workspace with which the packed GEMM of a layer [n, k] (either format) splits K across workgroups at up to 128
-    activation rows (few weight rows and a long K: a Llama down-projection), or None where it would not
-    split.  It belongs to the layer -- kept on its code tensor `wq`, zeroed once, left zeroed by every call --
-    so that the layer takes the same kernel, and gives the same bits, on every stream, eagerly, traced or
-    under a graph capture; `create`: make it now if it does not exist (never during a capture, where the
-    memory would belong to the graph).  Two calls of the SAME layer must not overlap in time on the GPU."""
+
+def _stream_workspace(device: torch.device, stream: int, need: int) -> torch.Tensor:
+    per_device = _stream_workspaces.setdefault(device.index, {})
+    hit = per_device.get(stream)
+    if hit is not None and hit.numel() >= need:
+        return hit
+    per_device.pop(stream, None)
+    while len(per_device) >= _STREAM_WORKSPACES_MAX:
+        per_device.pop(next(iter(per_device)))
+    workspace = per_device[stream] = torch.zeros(need, dtype=torch.uint8, device=device)
+    return workspace
+
+
+def splitk_workspace(wq: torch.Tensor, n: int, k: int, create: bool, stream: Optional[int] = None) -> Optional[torch.Tensor]:
+    """The workspace with which the packed GEMM of a layer [n, k] (either format) splits K across workgroups at
+    up to 128 activation rows (few weight rows and a long K: a Llama down-projection), or None where it would
+    not split.  Always zeroed between calls.  Which one:
+
+    * an eager call (`create` and the current stream `stream` given, no capture running): the stream's own
+      workspace (_stream_workspace), so calls on different streams share nothing;
+    * a call recorded into a graph capture, or a traced call (which may not create anything): the LAYER's
+      workspace, kept on its code tensor `wq`, made when the layer is primed (`create` without `stream`) and
+      kept for the layer's lifetime, so that a recorded graph's pointers stay valid.  Two graphs that hold the
+      same layer must not be replayed at the same time on different streams.
+
+    Either way the layer takes the same kernel and gives the same bits."""
     if not SPLIT_K:
         return None
     need = _splitk_need.get((n, k))
@@ -419,10 +468,13 @@ def splitk_workspace(wq: torch.Tensor, n: int, k: int, create: bool) -> Optional
         need = _splitk_need[(n, k)] = int(_engine.lib().fpq_gemm_mxf4_packed_workspace_bytes(SPLIT_K_ROWS, n, k))
     if need == 0:
         return None
+    capturing = torch.cuda.is_current_stream_capturing()
+    if create and stream is not None and not capturing:
+        return _stream_workspace(wq.device, stream, need)
     hit = getattr(wq, "_fpq_splitk", None)
     if hit is not None and hit.numel() >= need and hit.device == wq.device:
         return hit
-    if not create or torch.cuda.is_current_stream_capturing():
+    if not create or capturing:
         return None
     workspace = torch.zeros(need, dtype=torch.uint8, device=wq.device)
     try:

@@ -146,13 +146,23 @@ class FPQuantLinear(nn.Module):
 
     def _prime(self, *_):
         """Per-call constants (rotation kind, alpha, fp32 global scale) computed now rather than inside
-        the first forward, which may be a traced one or a graph capture; also run after load_state_dict."""
+        the first forward, which may be a traced one or a graph capture; also run after load_state_dict.
+        What a recorded graph may point at keeps its address when the weight was rewritten in place: the
+        split-K workspace stays, and a packed copy of the old weight is re-packed into its own buffers."""
         h, wgs, ags = self.forward_hadamard_matrix, self.weight_global_scale, self.act_global_scale
+        q, s = getattr(self, "qweight", None), getattr(self, "scales", None)
+        stale = getattr(q, "_fpq_packed", None) if isinstance(q, torch.Tensor) else None
         # whatever was remembered about the old contents goes (in-place copies under torch.inference_mode()
         # leave no trace in a tensor's modification counter)
-        hip_ops.drop_tensor_caches(h, wgs, ags, getattr(self, "qweight", None), getattr(self, "scales", None))
+        hip_ops.drop_tensor_caches(h, wgs, ags, q, s, keep=("_fpq_splitk", "_fpq_alpha", "_fpq_f32"))
         if all(isinstance(t, torch.Tensor) and t.is_cuda for t in (h, wgs, ags)):
-            eager.prime(h, wgs, ags)
+            eager.prime(h, wgs, ags, refresh=True)   # alpha and the fp32 scale: new values in the old tensors
+        else:
+            hip_ops.drop_tensor_caches(wgs, ags)
+        if (stale is not None and isinstance(s, torch.Tensor) and q.is_cuda and q.dim() == 2 and s.dim() == 2
+                and q.dtype == torch.uint8 and s.dtype == torch.uint8 and q.is_contiguous() and s.is_contiguous()
+                and hip_ops.packed_weights_enabled() and not torch.cuda.is_current_stream_capturing()):
+            hip_ops.packed_weight(q, s, self.config.forward_dtype == FPQuantDtype.NVFP4, into=(stale[1], stale[2]))
         if self._fpq_single_copy or os.environ.get("FPQ_SINGLE_WEIGHT_COPY", "0") == "1":
             self.release_row_major()
         self._ensure_splitk_workspace()
@@ -196,9 +206,12 @@ class FPQuantLinear(nn.Module):
                 or tuple(s.shape) != (self.out_features, self.in_features // self.config.forward_dtype.scale_group)):
             return False
         pc, ps = hip_ops.packed_weight(q.contiguous(), s.contiguous(), nvfp4)
+        workspace = getattr(q, "_fpq_splitk", None)
         hip_ops.drop_tensor_caches(q, s)
         self.qweight = nn.Parameter(pc, requires_grad=False)
         self.scales = nn.Parameter(ps, requires_grad=False)
+        if workspace is not None:
+            self.qweight._fpq_splitk = workspace   # the layer's, whichever tensor holds its weight
         self._fpq_single_copy = True
         self._ensure_splitk_workspace()
         return True
@@ -208,10 +221,17 @@ class FPQuantLinear(nn.Module):
         """Undo release_row_major: `qweight` [out, in/2] and `scales` [out, in/32] as the reference holds them."""
         if not self.weights_packed_only:
             return
-        codes, scales = hip_ops.unpack_fp4(self.qweight, self.scales, self.out_features, self.in_features,
-                                           self.config.forward_dtype == FPQuantDtype.NVFP4)
+        nvfp4 = self.config.forward_dtype == FPQuantDtype.NVFP4
+        pc, ps = self.qweight.detach(), self.scales.detach()
+        workspace = getattr(self.qweight, "_fpq_splitk", None)
+        codes, scales = hip_ops.unpack_fp4(pc, ps, self.out_features, self.in_features, nvfp4)
         self.qweight = nn.Parameter(codes, requires_grad=False)
         self.scales = nn.Parameter(scales, requires_grad=False)
+        # the packed buffers stay the row-major tensors' packed copy (same addresses; re-packed in place when
+        # the weight is rewritten)
+        hip_ops.adopt_packed_weight(self.qweight, self.scales, nvfp4, pc, ps)
+        if workspace is not None:
+            self.qweight._fpq_splitk = workspace
         self._fpq_single_copy = False
         self._ensure_splitk_workspace()
 

@@ -95,7 +95,7 @@ def _quantize_alike(layers) -> bool:
     return True
 
 
-def _weight_group(layers, create: bool = False):
+def _weight_group(layers, create: bool = False, previous=None):
     """The layers' packed weights laid end to end (eager.WeightGroup), if they can be multiplied as one:
     abs-max layers (MXFP4 or NVFP4) that quantize alike with equal alpha.  Built when the model is patched
     (`create`), looked up afterwards (None: the layers were rewritten since, or never qualified)."""
@@ -110,7 +110,7 @@ def _weight_group(layers, create: bool = False):
             if not torch.equal(layer.weight_global_scale.float(), first.weight_global_scale.float()):
                 return None
     return _eager().weight_group([(l.qweight, l.scales, l.bias, l.in_features) for l in layers], create,
-                                 first.config.forward_dtype == FPQuantDtype.NVFP4)
+                                 first.config.forward_dtype == FPQuantDtype.NVFP4, previous)
 
 
 def _attach_weight_group(module: nn.Module, names) -> None:
@@ -119,7 +119,9 @@ def _attach_weight_group(module: nn.Module, names) -> None:
     addresses and counters, never multiplies by weights that have been replaced."""
     def build(*_):
         layers = [getattr(module, n) for n in names]
-        module._fpq_weight_group = (_weight_group(layers, create=True)
+        # (built into the buffers of the group it replaces where the shapes allow: a recorded graph keeps
+        # pointing at the current weights)
+        module._fpq_weight_group = (_weight_group(layers, create=True, previous=getattr(module, "_fpq_weight_group", None))
                                     if all(_is_real_quant_linear(l) for l in layers) else None)
 
     build()
@@ -383,7 +385,7 @@ def _eager_group_linear(owner: nn.Module, layers, x: torch.Tensor):
         return None
     first = layers[0]
     if group.key != tuple(_eager()._member_key(l.qweight, l.scales, l.bias) for l in layers):
-        group = owner._fpq_weight_group = _weight_group(layers, create=True)
+        group = owner._fpq_weight_group = _weight_group(layers, create=True, previous=group)
         if group is None:
             return None
     eager = _eager()

@@ -6,6 +6,7 @@ import pytest
 import torch
 
 from oracle import fpq_oracle as O
+from tests.conftest import row_major_weights
 
 pytestmark = pytest.mark.gpu
 
@@ -47,10 +48,11 @@ def _check_linear(lin, x2d, rows=24, cols=160, seed=0):
     y = lin(x2d)
     gen = torch.Generator().manual_seed(seed)
     ri = torch.randperm(x2d.shape[0], generator=gen)[:rows].sort().values
-    ci = torch.randperm(lin.qweight.shape[0], generator=gen)[:cols].sort().values
+    ci = torch.randperm(lin.out_features, generator=gen)[:cols].sort().values
+    wq, ws = row_major_weights(lin)      # (never index `lin.qweight` by output feature: a layer may hold 1-D packed buffers)
     xq, xs, _ = O.quantize_mx(x2d[ri.cuda()].cpu(), O.ROT_HADAMARD, 128)
     alpha = O.alpha_from_global_scales(lin.weight_global_scale.cpu(), lin.act_global_scale.cpu())
-    ref, mag = O.gemm_ref(xq, xs, lin.qweight[ci.cuda()].cpu(), lin.scales[ci.cuda()].cpu(), alpha, "mxfp4")
+    ref, mag = O.gemm_ref(xq, xs, wq[ci], ws[ci], alpha, "mxfp4")
     got = y[ri.cuda()][:, ci.cuda()].cpu()
     tol = 2.0 ** -8 * ref.abs() + 1e-5 * mag + 1e-6
     assert ((got.double() - ref).abs() <= tol).all()

@@ -5,7 +5,7 @@ import torch
 
 from oracle import fpq_oracle as O
 from tests import capi
-from tests.conftest import make_outlier_normal, make_student_t
+from tests.conftest import make_outlier_normal, make_student_t, needs_packed, packed_copy
 
 pytestmark = pytest.mark.gpu
 
@@ -200,6 +200,30 @@ def test_fused_quantize_packed_nvfp4_bit_exact(kind, rot, g, rows, cols):
     assert torch.equal(pc, want_c) and torch.equal(ps, want_s)
     pc2, ps2, none = capi.fused_quantize_packed(kind, a, b, g=g, rot=rot, want_out=False, global_scale=777.0)
     assert none is None and torch.equal(pc2, want_c) and torch.equal(ps2, want_s)
+
+
+@pytest.mark.parametrize("gs", [None, 777.0])
+def test_rmsnorm_rows_in_one_launch_non_finite_rows_are_data(gs):
+    """A row holding NaN (its 1 / rms is NaN) or infinity (1 / rms = 0) goes through the one-launch kernel as
+    data, as the reference's RMSNorm propagates it: every byte equals what fpq_row_inv_rms followed by
+    fpq_rmsnorm_quantize_*_packed writes, the NaN row's by-product is NaN, and the finite rows keep the
+    oracle's bits."""
+    rows, cols, g = 6, 1024, 128 if gs is None else 16
+    x = make_student_t(rows, cols, seed=11) * 2
+    x[1, 100] = float("nan")
+    x[4, 7] = float("inf")
+    gen = torch.Generator().manual_seed(cols)
+    w = (1 + 0.3 * torch.randn(cols, generator=gen)).to(torch.bfloat16)
+    pc, ps, out, inv = capi.rmsnorm_rows_quantize_packed(x, w, g=g, global_scale=gs)
+    pc2, ps2, out2 = capi.fused_quantize_packed("rmsnorm", x, w, g=g, global_scale=gs)
+    assert torch.equal(pc, pc2) and torch.equal(ps, ps2)
+    assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
+    assert torch.isnan(inv[1]) and inv[4] == 0.0
+    assert torch.isnan(out[1]).all() and torch.isnan(out[4, 7])
+    finite = [0, 2, 3, 5]
+    want_v = O.rmsnorm(x[finite], w, 1e-5)
+    assert torch.equal(out[finite], want_v)
+    assert torch.equal(inv[finite], O.row_inv_rms(x[finite], 1e-5))
 
 
 def test_fused_quantize_packed_nvfp4_needs_a_global_scale():
@@ -557,7 +581,7 @@ def test_fused_decoder_block_with_residual_epilogues_is_graph_capturable(tokens)
 
 @pytest.mark.parametrize("fmt,g,arch,held_once", [("mxfp4", 128, "llama", False), ("nvfp4", 16, "llama", False),
                                                   ("mxfp4", 128, "qwen3", False), ("nvfp4", 16, "qwen3", False),
-                                                  ("mxfp4", 128, "llama", True)])
+                                                  pytest.param("mxfp4", 128, "llama", True, marks=needs_packed)])
 def test_compiled_decode_with_grouped_operators_matches_eager(fmt, g, arch, held_once):
     """fuse_producers before torch.compile: the traced attention calls one operator for q/k/v and the
     traced MLP two (gate/up; SiLU*up -> down) instead of seven layer operators and an elementwise kernel.
@@ -613,6 +637,7 @@ def test_compiled_decode_with_grouped_operators_matches_eager(fmt, g, arch, held
         assert torch.equal(a, b), i
 
 
+@needs_packed
 @pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])
 @pytest.mark.parametrize("tokens", [1, 3, 40, 300])
 def test_grouped_projections_run_as_one_gemm_on_concatenated_packed_weights(tokens, fmt, g):
@@ -636,7 +661,7 @@ def test_grouped_projections_run_as_one_gemm_on_concatenated_packed_weights(toke
         assert group is not None and group.n == sum(w.shape[-1] for w in want) and mlp._fpq_weight_group is not None
         lo, hi = group.wp.data_ptr(), group.wp.data_ptr() + group.wp.numel()
         for layer in (attn.q_proj, attn.k_proj, attn.v_proj):
-            assert lo <= layer.qweight._fpq_packed[1].data_ptr() < hi        # no further copy of the weights
+            assert lo <= packed_copy(layer)[0].data_ptr() < hi        # no further copy of the weights
         got = attn._fpq_qkv(x)
         # k and v have 128 output features here: column ranges of one output matrix
         assert (got[0].data_ptr() + 2 * want[0].shape[-1] == got[1].data_ptr()) == grouped
@@ -660,10 +685,12 @@ def test_grouped_projections_run_as_one_gemm_on_concatenated_packed_weights(toke
         # new weights: the hook rebuilds the group
         attn.load_state_dict(block2.self_attn.state_dict())
         assert attn._fpq_weight_group is not group
+        assert attn._fpq_weight_group.wp.data_ptr() == lo      # ... in the buffers of the one it replaces
         for a, b in zip(attn._fpq_qkv(x), want2):
             assert torch.equal(a, b)
 
 
+@needs_packed
 @pytest.mark.parametrize("order,fmt,g", [("fuse_then_release", "mxfp4", 128), ("release_then_fuse", "mxfp4", 128),
                                          ("fuse_then_release", "nvfp4", 16), ("release_then_fuse", "nvfp4", 16)])
 def test_model_with_weights_held_once_keeps_its_logits(order, fmt, g):

@@ -5,6 +5,8 @@ import torch
 from torch import nn
 
 from oracle import fpq_oracle as O
+from tests.conftest import (PACKED_WEIGHTS, SINGLE_WEIGHT_COPY, needs_packed, needs_row_major_parameters, packed_copy,
+                            row_major_weights)
 
 pytestmark = pytest.mark.gpu
 
@@ -30,9 +32,12 @@ def test_linear_matches_oracle_pipeline(fmt, g, bias):
         lin.bias.data = b.cuda()
     lin.pre_forward()
     assert lin.weight is None and lin.dqweight is None
-    assert lin.qweight.dtype == torch.uint8 and lin.qweight.shape == (n, k // 2)
     group = 32 if fmt == "mxfp4" else 16
-    assert lin.scales.dtype == torch.uint8 and lin.scales.shape == (n, k // group)
+    if not SINGLE_WEIGHT_COPY:
+        assert lin.qweight.dtype == torch.uint8 and lin.qweight.shape == (n, k // 2)
+        assert lin.scales.dtype == torch.uint8 and lin.scales.shape == (n, k // group)
+    got_q, got_s = row_major_weights(lin)
+    assert got_q.dtype == torch.uint8 and got_q.shape == (n, k // 2) and got_s.shape == (n, k // group)
     # linear.py:190-200: the abs_max branch (3.0) is tested before the NVFP4 branch (10.0), and
     # NVFP4 only validates with abs_max, so every real-quant layer gets 3.0
     gsv = 3.0
@@ -47,7 +52,7 @@ def test_linear_matches_oracle_pipeline(fmt, g, bias):
     else:
         wq, ws, _ = O.quantize_nv(w, gsv, O.ROT_HADAMARD, g, norm)
         xq, xs, _ = O.quantize_nv(x.view(-1, k), gsv, O.ROT_HADAMARD, g, norm)
-    assert torch.equal(lin.qweight.cpu(), wq) and torch.equal(lin.scales.cpu(), ws)
+    assert torch.equal(got_q, wq) and torch.equal(got_s, ws)
 
     y = lin(x.cuda())
     assert y.shape == (2, 9, n) and y.dtype == torch.bfloat16
@@ -65,6 +70,7 @@ def test_linear_matches_oracle_pipeline(fmt, g, bias):
     assert rel < 0.25, rel
 
 
+@needs_packed
 @pytest.mark.parametrize("m", [9, 100, 200])
 def test_nvfp4_layer_with_a_long_k_owns_a_split_k_workspace(m):
     """The NVFP4 counterpart of the test below, in short: workspace made at priming, oracle values, eager ==
@@ -81,7 +87,7 @@ def test_nvfp4_layer_with_a_long_k_owns_a_split_k_workspace(m):
     alpha = O.alpha_from_global_scales(lin.weight_global_scale.cpu(), lin.act_global_scale.cpu())
     x = torch.randn(m, k, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16)
     xq, xs, _ = O.quantize_nv(x, float(lin.act_global_scale), O.ROT_HADAMARD, 16, norm)
-    wq, ws = lin.qweight.cpu(), lin.scales.cpu()
+    wq, ws = row_major_weights(lin)
     ref, mag = O.gemm_ref(xq, xs, wq, ws, alpha, "nvfp4")
     want = ref.to(torch.bfloat16) + lin.bias.detach().cpu()
     with torch.no_grad():
@@ -101,6 +107,7 @@ def test_nvfp4_layer_with_a_long_k_owns_a_split_k_workspace(m):
     assert ((whole.double() - want.double()).abs() <= 2.0 ** -6 * want.double().abs() + 1e-5 * mag + 1e-6).all()
 
 
+@needs_packed
 @pytest.mark.parametrize("bias", [False, True])
 def test_decode_rows_on_a_long_k_split_k_across_workgroups(bias):
     """A layer with few output features and a long K (a down-projection) owns a workspace with which its GEMM
@@ -117,7 +124,7 @@ def test_decode_rows_on_a_long_k_split_k_across_workgroups(bias):
     assert wsk is not None and wsk.numel() == _engine.lib().fpq_gemm_mxf4_packed_workspace_bytes(128, n, k) > 16384
     norm = float(O.hadamard_matrix(128)[0, 0])
     alpha = O.alpha_from_global_scales(lin.weight_global_scale.cpu(), lin.act_global_scale.cpu())
-    wq, ws = lin.qweight.cpu(), lin.scales.cpu()
+    wq, ws = row_major_weights(lin)
     wp, wsp = pack_by_definition(wq, ws, k)
     b = lin.bias.detach().cpu() if bias else None
     for m in (1, 20, 32, 50, 128):
@@ -181,7 +188,8 @@ def test_other_transform_inits(init):
     assert hip_ops.classify_rotation(lin.forward_hadamard_matrix)[0] == kind
     okind = {"identity": O.ROT_IDENTITY, "gsr": O.ROT_GSR}[init]
     wq, ws, _ = O.quantize_mx(w, okind, 64)
-    assert torch.equal(lin.qweight.cpu(), wq) and torch.equal(lin.scales.cpu(), ws)
+    got_q, got_s = row_major_weights(lin)
+    assert torch.equal(got_q, wq) and torch.equal(got_s, ws)
     xq, xs, _ = O.quantize_mx(x, okind, 64)
     ref, mag = O.gemm_ref(xq, xs, wq, ws, 0.111328125, "mxfp4")
     y = lin(x.cuda()).cpu()
@@ -394,6 +402,8 @@ def _quantized_linear(fmt, g, k, n, seed, bias=False):
     return lin
 
 
+@needs_packed
+@needs_row_major_parameters
 @pytest.mark.parametrize("fmt,g,m", [("mxfp4", 128, 5), ("mxfp4", 32, 200), ("nvfp4", 16, 8), ("nvfp4", 16, 300)])
 def test_activations_quantized_into_one_layout_serve_the_other(fmt, g, m):
     """Quantized activations held in the packed layout only feed a GEMM on row-major operands (they are
@@ -528,6 +538,30 @@ def test_layers_called_from_two_threads_on_their_own_streams():
         lin.pre_forward()
         lins.append(lin)
     inputs = [[torch.randn(m, 512, device="cuda", dtype=torch.bfloat16) for m in (1, 30, 70, 300)] for _ in range(2)]
+    _run_on_two_streams(lins, inputs)
+
+
+@needs_packed
+def test_layers_that_split_k_called_from_two_threads_on_their_own_streams():
+    """The same with layers whose GEMM splits K through a workspace (few output features, K = 8192) at 1 and 70
+    rows: the two threads' calls of ONE layer overlap on the GPU, each stream has a workspace of its own, and
+    both get the single-stream bits (FPQ_SPLIT_K at its default)."""
+    from fp_quant.module import hip_ops
+    assert hip_ops.SPLIT_K
+    lins = [_quantized_linear(fmt, g, 8192, 1024, seed=31, bias=True) for fmt, g in (("mxfp4", 128), ("nvfp4", 16))]
+    for lin in lins:
+        assert getattr(lin.qweight, "_fpq_splitk", None) is not None       # the shape splits
+    inputs = [[torch.randn(m, 8192, device="cuda", dtype=torch.bfloat16) for m in (1, 70)] for _ in range(2)]
+    before = {k: v.data_ptr() for k, v in hip_ops._stream_workspaces.get(torch.cuda.current_device(), {}).items()}
+    _run_on_two_streams(lins, inputs, rounds=60, sync_every_call=False)
+    after = hip_ops._stream_workspaces[torch.cuda.current_device()]
+    assert len(set(v.data_ptr() for v in after.values()) - set(before.values())) >= 2   # one per worker stream
+    torch.cuda.synchronize()
+    assert not any(bool(v[:16384].any()) for v in after.values())      # counters left at zero
+
+
+def _run_on_two_streams(lins, inputs, rounds=25, sync_every_call=True):
+    import threading
     with torch.no_grad():
         want = [[[lin(x) for x in xs] for lin in lins] for xs in inputs]
     torch.cuda.synchronize()
@@ -537,13 +571,17 @@ def test_layers_called_from_two_threads_on_their_own_streams():
         try:
             stream = torch.cuda.Stream()
             with torch.cuda.stream(stream), torch.no_grad():
-                for _ in range(25):
+                for _ in range(rounds):
+                    got = []
                     for li, lin in enumerate(lins):
                         for xi, x in enumerate(inputs[t]):
-                            y = lin(x)
-                            stream.synchronize()
-                            if not torch.equal(y, want[t][li][xi]):
-                                errors.append((t, li, xi))
+                            got.append((li, xi, lin(x)))
+                            if sync_every_call:
+                                stream.synchronize()
+                    stream.synchronize()
+                    for li, xi, y in got:
+                        if not torch.equal(y, want[t][li][xi]):
+                            errors.append((t, li, xi))
         except Exception as exc:   # surfaced below
             errors.append(repr(exc))
 
@@ -633,6 +671,47 @@ def test_load_state_dict_onto_tensors_without_a_modification_counter(fmt, g, m):
             assert torch.equal(a(x), c(x))
 
 
+@needs_packed
+@needs_row_major_parameters
+@pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])
+@pytest.mark.parametrize("released", [False, True])
+def test_recorded_graph_follows_an_in_place_load_state_dict(fmt, g, released):
+    """A HIP graph recorded around a layer holds raw pointers to the packed weight and the layer's split-K
+    workspace.  load_state_dict (in place) keeps both where they are -- the packed copy is re-packed into its own
+    buffers -- so a replay afterwards multiplies by the NEW weights, as the reference, which reads `qweight` in
+    place, would."""
+    k, n = 8192, 256
+    lin = _quantized_linear(fmt, g, k, n, seed=51, bias=True)
+    other = _quantized_linear(fmt, g, k, n, seed=52, bias=True)
+    sd = {key: v.clone() for key, v in other.state_dict().items()}
+    sd["act_global_scale"] = sd["act_global_scale"] * 2          # another alpha (and NVFP4 activation scale) too
+    other.load_state_dict(sd)
+    if released:
+        assert lin.release_row_major()
+    x = torch.randn(5, k, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        y_old, y_new = lin(x), other(x)
+        assert not torch.equal(y_old, y_new)
+        graph = torch.cuda.CUDAGraph()
+        static_x = x.clone()
+        with torch.cuda.graph(graph):
+            static_y = lin(static_x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y, y_old)
+        workspace = lin.qweight._fpq_splitk.data_ptr()
+        packed = (lin.qweight if released else lin.qweight._fpq_packed[1]).data_ptr()
+        lin.load_state_dict(other.state_dict())
+        assert lin.weights_packed_only == released
+        assert lin.qweight._fpq_splitk.data_ptr() == workspace
+        assert (lin.qweight if released else lin.qweight._fpq_packed[1]).data_ptr() == packed
+        for _ in range(2):
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_y, y_new)
+        assert torch.equal(lin(x), y_new)
+
+
 def test_prepare_device_entry_point():
     from fp_quant import _engine
     lib = _engine.lib()
@@ -644,6 +723,8 @@ def test_prepare_device_entry_point():
         assert lib.fpq_prepare_device(s.cuda_stream) == _engine.E_UNSUPPORTED   # must run, not be recorded
 
 
+@needs_packed
+@needs_row_major_parameters
 @pytest.mark.parametrize("fmt,g", [("mxfp4", 128), ("nvfp4", 16)])
 @pytest.mark.parametrize("bias", [False, True])
 def test_release_row_major_keeps_results_and_the_reference_state_dict(bias, fmt, g):
@@ -701,6 +782,7 @@ def test_release_row_major_declines_what_the_packed_layout_cannot_hold():
         assert nv(x).shape == (5, 48) and ragged(x).shape == (5, 48)
 
 
+@needs_packed
 def test_single_weight_copy_by_environment(monkeypatch):
     """FPQ_SINGLE_WEIGHT_COPY=1: every eligible layer releases its row-major tensors as soon as it is quantized."""
     monkeypatch.setenv("FPQ_SINGLE_WEIGHT_COPY", "1")
@@ -723,6 +805,6 @@ def test_empty_batch(fmt, g):
         for shape in ((0, 256), (2, 0, 256), (0, 5, 256)):
             y = lin(torch.empty(*shape, device="cuda", dtype=torch.bfloat16))
             assert y.shape == (*shape[:-1], 96) and y.dtype == torch.bfloat16
-        if fmt == "mxfp4":
+        if fmt == "mxfp4" and PACKED_WEIGHTS:
             assert lin.release_row_major()
             assert lin(torch.empty(0, 256, device="cuda", dtype=torch.bfloat16)).shape == (0, 96)

@@ -6,7 +6,7 @@ import torch
 from oracle import fpq_oracle as O
 from fp_quant import _engine
 import capi
-from conftest import make_outlier_normal
+from conftest import make_outlier_normal, needs_packed, needs_row_major_parameters, packed_copy
 
 pytestmark = pytest.mark.gpu
 
@@ -128,6 +128,7 @@ def test_gemm_packed_rejects():
         capi.gemm_packed(z, z, z, z, 32, 32, 128, 1.0)       # K % 256 != 0
 
 
+@needs_packed
 def test_linear_uses_packed_path_and_matches_row_major(monkeypatch):
     """FPQuantLinear above the row threshold runs quantize-to-packed + packed GEMM; the result is
     bit-identical to the row-major kernels (FPQ_PACKED_WEIGHTS=0)."""
@@ -143,7 +144,7 @@ def test_linear_uses_packed_path_and_matches_row_major(monkeypatch):
     x = torch.randn(3, 100, 512, device="cuda", dtype=torch.bfloat16)
     assert x.shape[0] * x.shape[1] >= hip_ops.PACKED_LINEAR_MIN_M
     y_packed = lin(x)
-    assert getattr(lin.qweight, "_fpq_packed", None) is not None
+    assert packed_copy(lin) is not None
     monkeypatch.setenv("FPQ_PACKED_WEIGHTS", "0")
     y_rm = lin(x)
     assert torch.equal(y_packed, y_rm)
@@ -291,6 +292,7 @@ def test_quantize_nv_packed_large_matches_row_major_path():
         capi.quantize_nv_packed(torch.zeros(32, 384, dtype=torch.bfloat16), 1.0)   # cols % 256 != 0
 
 
+@needs_packed
 def test_nvfp4_linear_mid_m_runs_packed_and_matches_oracle(monkeypatch):
     import fp_quant
     from fp_quant.module import hip_ops
@@ -305,7 +307,7 @@ def test_nvfp4_linear_mid_m_runs_packed_and_matches_oracle(monkeypatch):
     lin.pre_forward()
     assert hip_ops.nv_packed_eligible(m, n, k)
     y = lin(x.cuda()).cpu()
-    assert getattr(lin.qweight, "_fpq_packed", None) is not None
+    assert packed_copy(lin) is not None
     gs = float(lin.act_global_scale)
     norm = float(O.hadamard_matrix(16)[0, 0])
     wq, ws, _ = O.quantize_nv(w, gs, O.ROT_HADAMARD, 16, norm)

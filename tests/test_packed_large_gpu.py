@@ -12,6 +12,7 @@ import torch
 
 from oracle import fpq_oracle as O
 import capi
+from conftest import needs_packed, packed_copy, row_major_weights
 from test_packed_gpu import pack_by_definition, pack_nv_by_definition
 
 pytestmark = pytest.mark.gpu
@@ -87,6 +88,7 @@ def test_c3_m2048_packed_residual_epilogue(c3_operands, bias):
     assert torch.equal(got.view(torch.int16), (plain + c["res"]).view(torch.int16))
 
 
+@needs_packed
 def test_c3_m2048_through_module(c3_operands, monkeypatch):
     """FPQuantLinear.forward on the shape the headline is measured on: packed weights, packed
     activations, big-tile kernel; against the oracle's quantizers + fp64 GEMM and against the module
@@ -100,9 +102,9 @@ def test_c3_m2048_through_module(c3_operands, monkeypatch):
     lin.weight.data = c["w"].cuda()
     lin.bias.data = c["bias"].cuda()
     lin.pre_forward()
-    assert torch.equal(lin.qweight.cpu(), c["wq"])
+    assert torch.equal(row_major_weights(lin)[0], c["wq"])
     y = lin(c["x"].cuda()).cpu()
-    assert getattr(lin.qweight, "_fpq_packed", None) is not None
+    assert packed_copy(lin) is not None
     alpha = O.alpha_from_global_scales(lin.weight_global_scale.cpu(), lin.act_global_scale.cpu())
     ri, ci = _sample(torch.Generator().manual_seed(18), m, n, rows=32, cols=256)
     norm = float(O.hadamard_matrix(128)[0, 0])

@@ -6,7 +6,7 @@ import torch
 from oracle import fpq_oracle as O
 from fp_quant import _engine
 import capi
-from conftest import make_outlier_normal, make_student_t
+from conftest import make_outlier_normal, make_student_t, row_major_weights
 
 pytestmark = pytest.mark.gpu
 
@@ -76,7 +76,8 @@ def test_quest_operator_and_linear():
     lin.pre_forward()
     assert float(lin.weight_global_scale) == 1.0 and float(lin.act_global_scale) == 1.0   # linear.py:190-192
     wq, wsc, _, _ = O.quantize_mx_quest(w, O.ROT_HADAMARD, 64)
-    assert torch.equal(lin.qweight.cpu(), wq) and torch.equal(lin.scales.cpu(), wsc)
+    got_q, got_s = row_major_weights(lin)
+    assert torch.equal(got_q, wq) and torch.equal(got_s, wsc)
     y = lin(x).cpu()
     ref, mag = O.gemm_ref(wc, ws, wq, wsc, 1.0, "mxfp4")
     assert ((y.double() - ref).abs() <= 2.0 ** -8 * ref.abs() + 1e-5 * mag).all()
@@ -108,7 +109,8 @@ def test_quest_module_equals_the_operator_chain(m):
         codes, scales, _ = hip_ops.fused_quantize_mx_op(x, layers[0].forward_hadamard_matrix, "quest", False)
         alpha = torch.ones(1, dtype=torch.float32, device="cuda")
         for lin in layers:                      # called one after the other with the same tensor: shared
-            want = hip_ops.matmul_mxf4_bf16_tn_op(codes, lin.qweight, scales, lin.scales.view(torch.float8_e8m0fnu), alpha)
+            wq, ws = (t.cuda() for t in row_major_weights(lin))
+            want = hip_ops.matmul_mxf4_bf16_tn_op(codes, wq, scales, ws.view(torch.float8_e8m0fnu), alpha)
             if lin.bias is not None:
                 want = want + lin.bias
             assert torch.equal(lin(x), want)
