@@ -127,9 +127,12 @@ def bench_quantize(torch, fmt, rows, cols, g, steps, warmup, seed, packed=False)
     norm = float(torch.tensor(g ** -0.5, dtype=torch.bfloat16))
     gs = torch.tensor([1.0], dtype=torch.float32, device=dev)
     if fmt == "nvfp4":
-        from fp_quant.module import hip_ops  # noqa: F401
-        amax = float(x_cpu.float().abs().max()) * (g ** 0.5)  # bound of the rotated abs-max
-        gs.fill_(2688.0 / amax)
+        # the tracked global scale of the configuration: 2688 * fl(1 / max|rotated x|), two fp32 roundings as
+        # src/quantization/quantizer.py:145-150 writes it (outside the timed region)
+        amax = torch.zeros(1, dtype=torch.float32, device=dev)
+        _engine.check(lib.fpq_rotated_absmax(xs[0].data_ptr(), rows, cols, 0, g, norm, None, amax.data_ptr(),
+                                             torch.cuda.current_stream().cuda_stream), "fpq_rotated_absmax")
+        gs.copy_(torch.tensor(2688.0, dtype=torch.float32, device=dev) * (1.0 / amax))
     stream = torch.cuda.current_stream().cuda_stream
     ptrs = [(xs[i].data_ptr(), codes[i].data_ptr(), scales[i].data_ptr()) for i in range(n_buf)]
 

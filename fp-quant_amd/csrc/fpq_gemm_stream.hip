@@ -544,10 +544,23 @@ extern "C" int fpq_gemm_mxf4_packed_noalloc(const void* xq, const void* xs, cons
                                             const float* alpha, const void* bias, const void* residual,
                                             void* y, int64_t M, int64_t N, int64_t K, void* stream) {
   if (M > fpq::kStreamMaxRows) return FPQ_E_LIMIT;
+  // (defensive: stream_plan keeps parts x weight tiles within 256, so no shape asks for more today)
   if (fpq::gemm_mxf4_stream_workspace_bytes(M, N, K) > fpq::kScratchBytes) return FPQ_E_LIMIT;
   void* ptr = nullptr;
   const int st = fpq::scratch_address(&ptr);
   if (st != FPQ_OK) return st;
   return fpq::gemm_mxf4_packed_any(xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, ptr, fpq::kScratchBytes,
                                    stream);
+}
+
+// Test hook: the split-K counters at the head of the current device's scratch array (16 KB), copied to
+// `out` (device memory) in stream order; they must read zero between calls.
+extern "C" int fpq_test_noalloc_counters(void* out, int64_t bytes, void* stream) {
+  if (!out) return FPQ_E_NULL;
+  if (bytes < 0 || bytes > fpq::kStreamCounterBytes) return FPQ_E_SHAPE;
+  void* ptr = nullptr;
+  const int st = fpq::scratch_address(&ptr);
+  if (st != FPQ_OK) return st;
+  if (bytes == 0) return FPQ_OK;
+  return (int)hipMemcpyAsync(out, ptr, (size_t)bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream);
 }

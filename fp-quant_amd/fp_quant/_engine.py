@@ -66,6 +66,7 @@ _SIGNATURES = {
     "fpq_silu_mul_quantize_nv_packed": ([_P, _I64, _P, _I64, _I64, _I64, _I, _I, _F, _P, _P, _P, _P, _I, _P], _I),
     "fpq_prepare_device": ([_P], _I),
     "fpq_gemm_mxf4_packed_noalloc_max_rows": ([], _I64),
+    "fpq_test_noalloc_counters": ([_P, _I64, _P], _I),
     "fpq_gemm_mxf4_packed_noalloc": ([_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _I),
 }
 

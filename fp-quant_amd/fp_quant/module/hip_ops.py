@@ -493,15 +493,23 @@ def _gemm(entry: str, x, w, xs, ws, alpha, bias: Optional[torch.Tensor], group: 
     xq = x.contiguous().view(-1, x.shape[-1])
     wq = w.contiguous()
     m, kb = xq.shape
-    n = wq.shape[0]
     k = kb * 2
-    if wq.shape[1] != kb:
-        raise ValueError(f"inner dimensions differ: x has K={k}, w has K={wq.shape[1] * 2}")
     xs_b = xs.contiguous().view(torch.uint8)
-    ws_b = ws.contiguous().view(torch.uint8)
     xs_b = xs_b.view(-1, xs_b.shape[-1])
-    ws_b = ws_b.view(-1, ws_b.shape[-1])
-    if xs_b.shape[0] < m or ws_b.shape[0] < n or xs_b.shape[1] < k // group or ws_b.shape[1] < k // group:
+    ws_b = ws.contiguous().view(torch.uint8)
+    packed_only = is_packed_only(wq)   # a layer that holds its weight in the packed layout only
+    if packed_only:
+        n = weight_rows(wq, k)
+        if ws_b.numel() * (group // 2) != wq.numel():
+            raise ValueError("packed scales do not match the packed codes")
+    else:
+        n = wq.shape[0]
+        if wq.shape[1] != kb:
+            raise ValueError(f"inner dimensions differ: x has K={k}, w has K={wq.shape[1] * 2}")
+        ws_b = ws_b.view(-1, ws_b.shape[-1])
+        if ws_b.shape[0] < n or ws_b.shape[1] < k // group:
+            raise ValueError("scale tensors are smaller than the operands they describe")
+    if xs_b.shape[0] < m or xs_b.shape[1] < k // group:
         raise ValueError("scale tensors are smaller than the operands they describe")
     y = torch.empty(*x.shape[:-1], n, dtype=torch.bfloat16, device=x.device)
     b_ptr = None
@@ -511,7 +519,7 @@ def _gemm(entry: str, x, w, xs, ws, alpha, bias: Optional[torch.Tensor], group: 
         bias = bias.contiguous()
         b_ptr = bias.data_ptr()
     a = alpha.contiguous()
-    if entry == "fpq_gemm_mxf4" and m >= PACKED_MIN_M and k % 256 == 0 and packed_weights_enabled():
+    if entry == "fpq_gemm_mxf4" and (packed_only or (m >= PACKED_MIN_M and k % 256 == 0 and packed_weights_enabled())):
         with on_device(x.device):
             wp, wsp = packed_weight(wq, ws_b)
             xp, xsp = pack_mxf4(xq, xs_b, m, k)
@@ -520,7 +528,7 @@ def _gemm(entry: str, x, w, xs, ws, alpha, bias: Optional[torch.Tensor], group: 
                 y.data_ptr(), m, n, k, _stream(x))
         _engine.check(st, "fpq_gemm_mxf4_packed")
         return y
-    if entry == "fpq_gemm_nvf4" and nv_packed_eligible(m, n, k):
+    if entry == "fpq_gemm_nvf4" and (packed_only or nv_packed_eligible(m, n, k)):
         with on_device(x.device):
             wp, wsp = packed_weight(wq, ws_b, True)
             xp, xsp = pack_nvf4(xq, xs_b, m, k)
@@ -546,7 +554,7 @@ def matmul_mxf4_bf16_tn_op(
 
 @matmul_mxf4_bf16_tn_op.register_fake
 def _(x, w, xs, ws, alpha):
-    return x.new_empty(*x.shape[:-1], w.shape[0], dtype=torch.bfloat16)
+    return x.new_empty(*x.shape[:-1], weight_rows(w, x.shape[-1] * 2), dtype=torch.bfloat16)
 
 
 @torch.library.custom_op("fp_quant::matmul_ada_mxf4_bf16_tn_op", mutates_args=())
@@ -560,7 +568,7 @@ def matmul_ada_mxf4_bf16_tn_op(
 
 @matmul_ada_mxf4_bf16_tn_op.register_fake
 def _(x, w, xs, ws, alpha):
-    return x.new_empty(*x.shape[:-1], w.shape[0], dtype=torch.bfloat16)
+    return x.new_empty(*x.shape[:-1], weight_rows(w, x.shape[-1] * 2), dtype=torch.bfloat16)
 
 
 @torch.library.custom_op("fp_quant::matmul_nvf4_bf16_tn_op", mutates_args=())
@@ -572,7 +580,7 @@ def matmul_nvf4_bf16_tn_op(
 
 @matmul_nvf4_bf16_tn_op.register_fake
 def _(x, w, xs, ws, alpha):
-    return x.new_empty(*x.shape[:-1], w.shape[0], dtype=torch.bfloat16)
+    return x.new_empty(*x.shape[:-1], weight_rows(w, x.shape[-1] * 2), dtype=torch.bfloat16)
 
 
 ### Fused epilogue variants (bias added inside the GEMM; not part of the reference op set)
@@ -588,7 +596,7 @@ def matmul_mxf4_bf16_tn_bias_op(
 
 @matmul_mxf4_bf16_tn_bias_op.register_fake
 def _(x, w, xs, ws, alpha, bias):
-    return x.new_empty(*x.shape[:-1], w.shape[0], dtype=torch.bfloat16)
+    return x.new_empty(*x.shape[:-1], weight_rows(w, x.shape[-1] * 2), dtype=torch.bfloat16)
 
 
 @torch.library.custom_op("fp_quant::matmul_nvf4_bf16_tn_bias_op", mutates_args=())
@@ -601,4 +609,4 @@ def matmul_nvf4_bf16_tn_bias_op(
 
 @matmul_nvf4_bf16_tn_bias_op.register_fake
 def _(x, w, xs, ws, alpha, bias):
-    return x.new_empty(*x.shape[:-1], w.shape[0], dtype=torch.bfloat16)
+    return x.new_empty(*x.shape[:-1], weight_rows(w, x.shape[-1] * 2), dtype=torch.bfloat16)

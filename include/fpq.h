@@ -364,6 +364,13 @@ int fpq_gemm_mxf4_packed_noalloc(const void* xq_packed, const void* xs_packed, c
                                  void* stream);
 
 /*
+ * Test hook: copies the first `bytes` (at most 16384) of the current device's scratch array -- the split-K
+ * counters of fpq_gemm_mxf4_packed_noalloc -- to `out` (device memory) in stream order.  They read zero
+ * between calls.
+ */
+int fpq_test_noalloc_counters(void* out, int64_t bytes, void* stream);
+
+/*
  * Test hook: E2M1 codes of n fp32 values exactly as the quantize kernels round them
  * (out[i] in 0..15, one byte per value).  Used to check the device rounding exhaustively.
  */
