@@ -973,7 +973,8 @@ def main():
         with open(tpath) as f:
             traffic = json.load(f)  # HBM bytes per launch from an earlier rocprofv3 --pmc run (see profiles/)
     traffic_source = ("profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, run by the "
-                      "builder and scaled by a 256 MiB copy; a constant, not measured in this run")
+                      "builder on the library built from commit " + str(traffic.get("source_commit", "?")) +
+                      " and scaled by a 256 MiB copy; a constant, not measured in this run")
     line = {
         "metric": METRIC,
         "value": round(head["linear_tflops_over_steps"], 2),
