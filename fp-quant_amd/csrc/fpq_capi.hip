@@ -29,10 +29,38 @@ extern "C" int fpq_device_supported(int device) {
   return strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 0;
 }
 
+#include <atomic>
+
 namespace fpq {
+// Compute units of the current device, asked once per device; 256 (one MI355X) where no device answers, so
+// that the size helpers stay host arithmetic.  Every shape threshold of the GEMM dispatch that stands for
+// "one round of workgroups" or a fraction of it is derived from this number.
+int device_cus() {
+  constexpr int kDefault = 256, kMaxDevices = 64;
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) {
+    (void)hipGetLastError();
+    return kDefault;
+  }
+  if (dev < kMaxDevices) {
+    const int hit = cached[dev].load(std::memory_order_acquire);
+    if (hit > 0) return hit;
+  }
+  int cus = 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+    (void)hipGetLastError();
+    return kDefault;
+  }
+  if (dev < kMaxDevices) cached[dev].store(cus, std::memory_order_release);
+  return cus;
+}
+
 int ensure_silu_table(hipStream_t stream);   // fpq_quantize.hip
 int scratch_address(void** out);             // fpq_gemm_stream.hip
 }  // namespace fpq
+
+extern "C" int fpq_compute_units(void) { return fpq::device_cus(); }
 
 extern "C" int fpq_prepare_device(void* stream) {
   hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;

@@ -11,6 +11,8 @@ namespace fpq {
 // Raises a kernel's dynamic-LDS limit once per device (the attribute is per device; one
 // function-local static instance per kernel lives in the launcher).  Safe from any host thread: a
 // race only repeats the idempotent call.
+int device_cus();   // fpq_capi.hip: compute units of the current device (256 where none answers)
+
 struct LdsLimitOnce {
   std::atomic<uint64_t> done{0};  // bit d: set for device d (devices >= 64 set it on every call)
   int ensure(const void* kernel, int bytes) {

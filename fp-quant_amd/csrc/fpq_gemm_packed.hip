@@ -462,15 +462,14 @@ static int pack_operand(const void* codes, const void* scales, int64_t scale_str
 #ifndef FPQ_PACKED_HALF_TILES
 #define FPQ_PACKED_HALF_TILES 1  // large M: 1 = 256x128 tiles for MXFP4, 2 = for NVFP4 too, 0 = 256x256
 #endif
-#ifndef FPQ_STREAM_SLAB_WGS
-#define FPQ_STREAM_SLAB_WGS 256   // row slabs of the streaming kernel x weight tiles: at most this many workgroups
-#endif
-#ifndef FPQ_PACKED_NARROW_BELOW
-#define FPQ_PACKED_NARROW_BELOW 128  // up to this many 128x128 tiles: 64x128 tiles instead
-#endif
-#ifndef FPQ_PACKED_SMALL_BELOW
-#define FPQ_PACKED_SMALL_BELOW 100  // fewer 256x256 tiles than this (under about 200 of 256x128): 128x128 tiles
-#endif
+// Shape thresholds that stand for a share of the chip are multiples of the device's compute-unit count
+// (measured on the 256 CUs of an MI355X, where they come to the figures in the comments):
+//   row slabs of the streaming kernel x weight tiles: at most one workgroup per CU (256)
+//   up to CUs / 2 tiles of 128 x 128 (128): 64 x 128 tiles instead
+//   fewer than 25/64 CUs tiles of 256 x 256 (100; under about 200 of 256 x 128): 128 x 128 tiles
+static inline int64_t slab_workgroups(int cus) { return cus; }
+static inline int64_t narrow_below(int cus) { return cus / 2; }
+static inline int64_t small_below(int cus) { return (int64_t)cus * 25 / 64; }
 
 namespace fpq {
 template <bool NV>
@@ -501,12 +500,13 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
   // rows: 32 -> 19.  (More slabs than one round -- two or three workgroups per CU -- measured slower.)  K
   // stays whole in slabs, so a shape whose K the caller's workspace lets split keeps the split up to 96 rows
   // (N = 4096, K = 14336: 64 rows 11.7 split / 11.9 us in slabs, 96 rows 13.9 / 13.9, 128 rows 15.4 / 14.1).
+  const int cus = device_cus();
   {
     const int64_t tiles = (N + 31) / 32;
     const bool splits = workspace && workspace_bytes > 16384 && M <= 96 && gemm_mxf4_stream_workspace_bytes(M, N, K) > 0;
     for (int64_t cap = 32; cap <= 128 && !splits; cap += 32) {
       const int64_t slabs = (M + cap - 1) / cap;
-      if (slabs * tiles > FPQ_STREAM_SLAB_WGS) continue;
+      if (slabs * tiles > slab_workgroups(cus)) continue;
       const int64_t rows = ((M + slabs - 1) / slabs + 31) / 32 * 32;   // rows of a slab, whole 32-row tiles
       if (slabs > 1 && rows < M && stream_eligible(NV, rows, N, K))
         return gemm_fp4_stream_slabs(NV, xq, xs, wq, ws, alpha, bias, residual, y, M, N, K, rows, seg,
@@ -525,7 +525,7 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
     // 12288: 97 -> 52 / 68 us.  (The tile kernel's time stays at one round up to N = 16384, where two passes
     // take 44-55 us; three passes for more rows measured slower than the tiles as well.)
     const int64_t half = ((M + 1) / 2 + 31) / 32 * 32;   // rows of the first pass, whole 32-row tiles
-    if (M > FPQ_NV_STREAM_ROWS && M <= 2 * FPQ_NV_STREAM_ROWS && (N + 31) / 32 <= 256 &&
+    if (M > FPQ_NV_STREAM_ROWS && M <= 2 * FPQ_NV_STREAM_ROWS && (N + 31) / 32 <= cus &&
         stream_eligible(true, half, N, K)) {
       // (both passes may split K through the caller's workspace: they run one after the other on the stream)
       const int rc = gemm_fp4_stream(true, xq, xs, wq, ws, alpha, bias, residual, y, half, N, K, workspace,
@@ -543,10 +543,10 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
   // At most 128 tiles of 128 x 128 would leave half of the CUs idle: 64 x 128 tiles (twice the workgroups, the
   // same accumulation order and bits) take 25 instead of 34.5 us for NVFP4 at 257-512 rows, N = 4096, K = 4096
   // (K = 12288: 69 instead of 97 us) and 4-7 % less for MXFP4; with more tiles they measured 14 % slower.
-  if (((M + 127) / 128) * ((N + 127) / 128) <= FPQ_PACKED_NARROW_BELOW)
+  if (((M + 127) / 128) * ((N + 127) / 128) <= narrow_below(cus))
     return launch_packed<2, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  if (big_tiles < FPQ_PACKED_SMALL_BELOW)
+  if (big_tiles < small_below(cus))
     return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);
 #if FPQ_PACKED_HALF_TILES
   if (!NV || FPQ_PACKED_HALF_TILES > 1)

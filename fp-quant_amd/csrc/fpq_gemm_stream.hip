@@ -409,14 +409,16 @@ static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace
   StreamPlan plan{false, 1, 1, 0};
   if (M < 1 || M > kStreamMaxRows || N < 1 || K < 256 || K % 256 != 0) return plan;
   const int64_t rt_m = (M + 31) / 32, tiles = (N + 31) / 32, nkb = K / 256;
-  if (rt_m == 3 && !nv && tiles > 1024) return plan;
-  if (rt_m == 4 && tiles > (nv ? 512 : 256)) return plan;
+  // (weight-tile counts in units of the device's compute units: 256 on the part the figures above were measured on)
+  const int64_t cus = device_cus();
+  if (rt_m == 3 && !nv && tiles > 4 * cus) return plan;
+  if (rt_m == 4 && tiles > (nv ? 2 * cus : cus)) return plan;
   plan.use = true;
-  if (rt_m == 2 && tiles >= (nv ? 384 : 768)) plan.nt = 2;
+  if (rt_m == 2 && tiles >= (nv ? 3 * cus / 2 : 3 * cus)) plan.nt = 2;
   const int64_t groups = (tiles + plan.nt - 1) / plan.nt;
   int64_t ksplit = 1;
   if (workspace_bytes > kStreamCounterBytes && groups <= kStreamCounters) {
-    ksplit = 256 / groups;
+    ksplit = cus / groups;
     if (ksplit > nkb / 16) ksplit = nkb / 16;
     if (ksplit < 1) ksplit = 1;
     while (ksplit > 1 && kStreamCounterBytes + ksplit * groups * plan.nt * rt_m * 4096 > workspace_bytes) --ksplit;
@@ -467,7 +469,7 @@ static int launch_stream(const void* xq, const void* xs, const void* wq, const v
     case 1:
       // enough workgroups for three per CU: two blocks in flight per wave beat four by 3-5 %; with fewer
       // workgroups the deeper ring of each wave is what keeps the memory system busy
-      if ((int64_t)grid.x * grid.y * grid.z >= 384) FPQ_STREAM(1, 1, 2);
+      if ((int64_t)grid.x * grid.y * grid.z >= 3 * device_cus() / 2) FPQ_STREAM(1, 1, 2);
       else FPQ_STREAM(1, 1, 4);
       break;
     case 2: FPQ_STREAM(1, 2, 2); break;
@@ -505,8 +507,8 @@ int gemm_fp4_stream_slabs(bool nv, const void* xq, const void* xs, const void* w
 // workspace.  Every GPU the library runs on holds its own copy at its own address until the process
 // ends; the array's name is only a host-side handle, the device address comes from
 // hipGetSymbolAddress, once per device, and that address is what kernels and host code use.
-// A split needs at most 1024 partial tiles of 4 KB (stream_plan: parts x weight tiles <= 256, times up
-// to four activation row tiles).
+// A split needs at most 1024 partial tiles of 4 KB on a device of 256 compute units (stream_plan: parts x
+// weight tiles <= compute units, times up to four activation row tiles).
 constexpr int64_t kScratchBytes = kStreamCounterBytes + 1024 * 4096;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
@@ -544,8 +546,8 @@ extern "C" int fpq_gemm_mxf4_packed_noalloc(const void* xq, const void* xs, cons
                                             const float* alpha, const void* bias, const void* residual,
                                             void* y, int64_t M, int64_t N, int64_t K, void* stream) {
   if (M > fpq::kStreamMaxRows) return FPQ_E_LIMIT;
-  // (defensive: stream_plan keeps parts x weight tiles within 256, so no shape asks for more today)
-  if (fpq::gemm_mxf4_stream_workspace_bytes(M, N, K) > fpq::kScratchBytes) return FPQ_E_LIMIT;
+  // (a shape that could use more than the array holds -- none on a device of 256 compute units -- splits K
+  // into as many parts as fit: stream_plan sizes the split to the workspace it is given)
   void* ptr = nullptr;
   const int st = fpq::scratch_address(&ptr);
   if (st != FPQ_OK) return st;

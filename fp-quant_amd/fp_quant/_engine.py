@@ -67,6 +67,7 @@ _SIGNATURES = {
     "fpq_prepare_device": ([_P], _I),
     "fpq_gemm_mxf4_packed_noalloc_max_rows": ([], _I64),
     "fpq_test_noalloc_counters": ([_P, _I64, _P], _I),
+    "fpq_compute_units": ([], _I),
     "fpq_gemm_mxf4_packed_noalloc": ([_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _I),
 }
 

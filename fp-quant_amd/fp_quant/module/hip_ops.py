@@ -342,11 +342,24 @@ def pack_nvf4(codes: torch.Tensor, scales: torch.Tensor, rows: int, k: int, into
     return pc, ps
 
 
+_nv_big_tiles = {}   # device index -> tiles of 256 x 256 from which NVFP4 runs on row-major operands
+
+
+def _nv_packed_below() -> int:
+    """25/64 of the device's compute units (100 on the 256 of an MI355X): the library's own border between its
+    128 x 128 and its large tiles."""
+    dev = torch.cuda.current_device() if torch.cuda.is_available() else -1
+    hit = _nv_big_tiles.get(dev)
+    if hit is None:
+        hit = _nv_big_tiles[dev] = int(_engine.lib().fpq_compute_units()) * 25 // 64
+    return hit
+
+
 def nv_packed_eligible(m: int, n: int, k: int, fused_linear: bool = False) -> bool:
     """NVFP4: the packed kernels win for few and mid-sized M (weight-streaming kernel, 128x128 tiles);
     large M runs at the same speed on row-major operands."""
     return ((NV_PACKED_LINEAR_MIN_M if fused_linear else NV_PACKED_MIN_M) <= m and k % 256 == 0
-            and packed_weights_enabled() and ((m + 255) // 256) * ((n + 255) // 256) < 100)
+            and packed_weights_enabled() and ((m + 255) // 256) * ((n + 255) // 256) < _nv_packed_below())
 
 
 def unpack_fp4(pc: torch.Tensor, ps: torch.Tensor, rows: int, k: int, nvfp4: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:

@@ -57,6 +57,10 @@ const char* fpq_status_string(int status);
 /* 1 if `device` is a gfx950 GPU this library has code for, 0 if not, <0 / >0 on error. */
 int fpq_device_supported(int device);
 
+/* Compute units of the current device (256 on an MI355X; 256 also where no device answers).  The GEMM
+ * entry points choose their kernels by problem size relative to this number. */
+int fpq_compute_units(void);
+
 /*
  * Sets up the per-device state described at the top for the current device, on `stream`, and waits
  * for it: call it once per device before capturing graphs or entering a loop that must not block.
@@ -351,7 +355,8 @@ int fpq_gemm_nvf4_packed_multi(const void* xq_packed, const void* xs_packed, con
  * workspace of that size, with these limits:
  *   M <= fpq_gemm_mxf4_packed_noalloc_max_rows() (128), the weight-streaming regime; more rows
  *   return FPQ_E_LIMIT (the tile kernels of fpq_gemm_mxf4_packed use no scratch memory at all);
- *   a shape whose split would need more than the array holds returns FPQ_E_LIMIT.
+ *   K is split into at most as many parts as the array holds partial tiles for (on a device of 256
+ *   compute units that is every split fpq_gemm_mxf4_packed_splitk would make).
  * The call makes no hipMalloc/hipFree and launches the same kernels.  All calls on one GPU share
  * that GPU's array: calls that may overlap on one GPU (different streams without an ordering
  * event) race on it and must use fpq_gemm_mxf4_packed_splitk with their own workspaces.  The
