@@ -111,6 +111,14 @@ __global__ __launch_bounds__(256) void unpack_fp4_kernel(const uint8_t* __restri
 }
 
 // ---------------------------------------------------------------------------------------------
+constexpr int kTileCounters = 4096;                          // as the weight-streaming kernel's: they open the workspace
+constexpr int64_t kTileCounterBytes = kTileCounters * 4;
+#ifndef FPQ_TILE_SPLIT_MIN_BLOCKS
+#define FPQ_TILE_SPLIT_MIN_BLOCKS 16     // a part of a K split keeps at least this many 256-K blocks
+#endif
+#ifndef FPQ_TILE_SPLIT_OVER_SLABS
+#define FPQ_TILE_SPLIT_OVER_SLABS 1      // a tile kernel that splits K comes before row slabs of the streaming kernel
+#endif
 constexpr int kRing = 8;                 // 64-K units resident or in flight
 // Scales of a 256-K block: 256 bytes per row tile for MXFP4 (one E8M0 byte per lane and K step), 512
 // for NVFP4 (two E4M3 bytes per lane and K step).  They travel with the first unit of their block,
@@ -170,7 +178,8 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int tiles_m,
-    const uint16_t* __restrict__ residual, const OutSegments seg) {
+    const uint16_t* __restrict__ residual, const OutSegments seg, int ksplit, int bps, float* partial,
+    unsigned* counters) {
   constexpr int BN = NT * 32, BM = MT * 32;
   constexpr int NW = WN * WM;           // waves
   static_assert(NW == 4 && NT <= KW && KW % 4 == 0 && MT % 4 == 0 && NT % WN == 0 && MT % WM == 0,
@@ -204,7 +213,13 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
   const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
   const int n_blk = tile_n * BN, m_blk = tile_m * BM;
   const int wn = wave % WN, wm = wave / WN;
-  const int nu = K >> 6, nkb = K >> 8;          // units, scale blocks
+  const int nu = K >> 6, nkb_all = K >> 8;      // units, scale blocks of a whole row tile
+  // K split across workgroups (ksplit > 1, grid plane blockIdx.y): this one multiplies the 256-K blocks
+  // [kb_begin, kb_begin + nkb) only, and the parts of a tile meet in the workspace after the loop.
+  // Only the kernels for few tiles are ever launched that way (the large tiles have no register to spare).
+  constexpr bool kCanSplit = NT * MT <= 16;
+  const int kb_begin = kCanSplit ? blockIdx.y * bps : 0;
+  const int nkb = kCanSplit ? min(nkb_all - kb_begin, bps) : nkb_all;
   const int rt_n = (N + 31) >> 5, rt_m = (M + 31) >> 5;
 
   // ---- loads.  Operand b of a unit: b < KW weight row tile tile_n*NT + b, else activation row tile
@@ -217,10 +232,10 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
     const int b = wave * kPer + j;
     if (b < KW) {
       const int rt = min(tile_n * NT + b, rt_n - 1);
-      op_base[j] = wq + (size_t)rt * nu * 1024;
+      op_base[j] = wq + ((size_t)rt * nu + kb_begin * 4) * 1024;
     } else {
       const int rt = min(tile_m * MT + b - KW, rt_m - 1);
-      op_base[j] = xq + (size_t)rt * nu * 1024;
+      op_base[j] = xq + ((size_t)rt * nu + kb_begin * 4) * 1024;
     }
   }
   // Scale piece p of a block: one load instruction for kRpp row tiles (unit operand order), lane L
@@ -236,8 +251,8 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
     constexpr int kLpr = 64 / kRpp;                            // lanes per row tile
     const int rt = min((is_w ? tile_n * NT + fb : tile_m * MT + fb - KW) + (int)(lane / kLpr),
                        (is_w ? rt_n : rt_m) - 1);
-    sc_base[j] = is_w ? ws : xs;
-    sc_off[j] = (uint32_t)rt * (uint32_t)nkb * (uint32_t)kSB + (lane % kLpr) * 16;
+    sc_base[j] = (is_w ? ws : xs) + (size_t)kb_begin * kSB;
+    sc_off[j] = (uint32_t)rt * (uint32_t)nkb_all * (uint32_t)kSB + (lane % kLpr) * 16;
   }
   const uint32_t lane16 = lane * 16;
 
@@ -294,7 +309,7 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
   };
 
   // ---- prologue: the first RING units (scales of blocks 0 and 1 with units 0 and 4)
-  const int n_pro = min(nu, RING);
+  const int n_pro = min(nkb * 4, RING);
   for (int u = 0; u < n_pro; ++u) issue_unit(u, (u & 3) == 0);
   // Loads complete in order: unit 0 and scale block 0 have landed once at most the loads of the
   // younger units are outstanding (a wave issues kPer per unit, one more with scales).
@@ -398,6 +413,49 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
 #undef FPQ_MFMA_ROW
 #undef FPQ_TAKE_SCALES
 
+  if (kCanSplit && ksplit > 1) {
+    // The parts of a tile run on different XCDs, whose L2 caches are not coherent with each other for
+    // ordinary accesses: every access to the workspace is a relaxed device-scope atomic, every wave waits
+    // for its stores to be acknowledged before the workgroup moves the tile's counter, and the workgroup
+    // that arrives last adds all parts in part order (its own read back like the others), so the sum does
+    // not depend on the order of arrival.  Register v of accumulator tile t of wave w: float
+    // ((w * TN * TM + t) * 16 + v) * 64 + lane of the part.  The counter is left at zero.  (Sixteen-byte
+    // accesses with the same cache policy measured no faster than these four-byte ones: the exchange is
+    // bound by its volume, M x N x 4 bytes per part written and read.)
+    constexpr int kPart = NW * TN * TM * 16 * 64;   // floats per part
+    float* mine = partial + ((size_t)logical * ksplit + blockIdx.y) * kPart + wave * (TN * TM * 16 * 64) + lane;
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < TM; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          __hip_atomic_store(mine + ((i * TM + j) * 16 + v) * 64, acc[i][j][v], __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();   // (every wave is past its last LDS read as well: the first word may be reused)
+    unsigned* arrival = (unsigned*)smem;
+    if (threadIdx.x == 0)
+      *arrival = __hip_atomic_fetch_add(counters + logical, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    // (one value for the workgroup: all its waves leave or all stay for the barriers of the epilogue)
+    if (__builtin_amdgcn_readfirstlane(*arrival) != (unsigned)(ksplit - 1)) return;
+    const float* all = partial + (size_t)logical * ksplit * kPart + wave * (TN * TM * 16 * 64) + lane;
+    for (int part = 0; part < ksplit; ++part) {
+#pragma unroll
+      for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const float p = __hip_atomic_load(all + (size_t)part * kPart + ((i * TM + j) * 16 + v) * 64,
+                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            acc[i][j][v] = part == 0 ? p : acc[i][j][v] + p;
+          }
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(counters + logical, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+
   const OutView out = out_view(seg, y, bias, n_blk + wn * TN * 32, N);
   wave_tile_store<TN, TM, packed_lds_alloc(kBlocks, NV, RING, TN * 32, TM * 32), NW>(
       acc, smem, out.y, out.bias, alpha_p, out.n0, m_blk + wm * TM * 32, wave, lane, M, out.N, residual);
@@ -405,20 +463,101 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
 
 }  // namespace fpq
 
+#ifndef FPQ_NV_STREAM_ROWS
+#define FPQ_NV_STREAM_ROWS 128  // NVFP4: up to this many rows the weight-streaming kernel (where its plan applies)
+#endif
+#ifndef FPQ_PACKED_HALF_TILES
+#define FPQ_PACKED_HALF_TILES 1  // large M: 1 = 256x128 tiles for MXFP4, 2 = for NVFP4 too, 0 = 256x256
+#endif
+// Shape thresholds that stand for a share of the chip are multiples of the device's compute-unit count
+// (measured on the 256 CUs of an MI355X, where they come to the figures in the comments):
+//   row slabs of the streaming kernel x weight tiles: at most one workgroup per CU (256)
+//   up to CUs / 2 tiles of 128 x 128 (128): 64 x 128 tiles instead
+//   fewer than 25/64 CUs tiles of 256 x 256 (100; under about 200 of 256 x 128): 128 x 128 tiles
+static inline int64_t slab_workgroups(int cus) { return cus; }
+static inline int64_t narrow_below(int cus) { return cus / 2; }
+static inline int64_t small_below(int cus) { return (int64_t)cus * 25 / 64; }
+
 namespace fpq {
+// A K split of a tile kernel (ksplit > 1): `workspace` = kStreamCounterBytes of counters, all zero, then
+// one fp32 part of the workgroup tile per (tile, split).
+struct TileSplit {
+  int ksplit = 1;   // parts of K, one grid plane each
+  int bps = 0;      // 256-K blocks per part (the last part may have fewer, never none)
+};
+
 template <int NT, int KW, int MT, int WN, int WM, bool NV, int RING = kRing>
 static int launch_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                          const void* bias, void* y, int64_t M, int64_t N, int64_t K, hipStream_t stream,
-                         const void* residual, const OutSegments& seg) {
+                         const void* residual, const OutSegments& seg, TileSplit split = TileSplit{},
+                         void* workspace = nullptr) {
   constexpr int kLds = packed_lds_alloc(KW + MT, NV, RING, NT / WN * 32, MT / WM * 32);
   const int tiles_m = (int)((M + MT * 32 - 1) / (MT * 32)), tiles_n = (int)((N + NT * 32 - 1) / (NT * 32));
+  if (split.ksplit <= 1 || !workspace || NT * MT > 16) split = TileSplit{1, (int)(K / 256)};
   static LdsLimitOnce lds_limit;
   if (const int st = lds_limit.ensure((const void*)gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV, RING>, kLds)) return st;
-  hipLaunchKernelGGL((gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV, RING>), dim3((unsigned)(tiles_m * tiles_n)),
-                     dim3(256), kLds, stream, (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq,
-                     (const uint8_t*)ws, alpha, (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K,
-                     tiles_m, (const uint16_t*)residual, seg);
+  hipLaunchKernelGGL((gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV, RING>),
+                     dim3((unsigned)(tiles_m * tiles_n), (unsigned)split.ksplit), dim3(256), kLds, stream,
+                     (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq, (const uint8_t*)ws, alpha,
+                     (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K, tiles_m,
+                     (const uint16_t*)residual, seg, split.ksplit, split.bps,
+                     workspace ? (float*)((uint8_t*)workspace + kTileCounterBytes) : nullptr, (unsigned*)workspace);
   return (int)hipGetLastError();
+}
+
+// Which shapes split K in the tile kernels, and how.  Shapes of a few hundred rows on few weight rows and a
+// long K (a down-projection at 257-512 rows: 64-256 workgroups, each walking all of K, against a few
+// microseconds of arithmetic) get up to two workgroups per CU by cutting K, every part keeping at least
+// kTileSplitMinBlocks blocks of 256; fewer parts if the workspace is small.  `part_bytes`: one fp32 part of the
+// kernel's workgroup tile.  The exchange moves M x N x 4 bytes per part each way, about as much as the
+// operands themselves, so the split only pays where the main loop is slow for other reasons -- NVFP4, whose
+// loop is bound by the in-register dequantization (N = 4096: K = 14336, 384 rows 79.6 -> 69.8 us; K = 12288,
+// 512 rows 69.2 -> 65.2).  MXFP4 measured slower with it (N = 4096, K = 14336: 256 rows 19.5 -> 21.5 us,
+// 512 rows 29.0 -> 29.8; doubling the workgroups and halving their K left the time where it was: these tiles
+// are bound by what a CU can have in flight from the L2, not by the length of a workgroup's loop) and does not split.
+constexpr int64_t kTileSplitMinBlocks = FPQ_TILE_SPLIT_MIN_BLOCKS;
+static TileSplit tile_split_plan(int64_t tiles, int64_t K, int64_t part_bytes, int64_t workspace_bytes, int cus) {
+  TileSplit plan{1, (int)(K / 256)};
+  const int64_t nkb = K / 256;
+  if (tiles < 1 || tiles > kTileCounters || tiles > cus) return plan;
+  int64_t ksplit = 2 * (int64_t)cus / tiles;
+  if (ksplit > nkb / kTileSplitMinBlocks) ksplit = nkb / kTileSplitMinBlocks;
+  while (ksplit > 1 && kTileCounterBytes + ksplit * tiles * part_bytes > workspace_bytes) --ksplit;
+  if (ksplit <= 1) return plan;
+  const int64_t bps = (nkb + ksplit - 1) / ksplit;
+  plan.ksplit = (int)((nkb + bps - 1) / bps);   // no empty part
+  plan.bps = (int)bps;
+  return plan;
+}
+
+// The tile kernel a shape beyond the weight-streaming kernel's reach runs, and its K split.
+struct TilePlan {
+  int kind;          // 0: 64 x 128 tiles, 1: 128 x 128, 2: 256 x 128 (MXFP4), 3: 256 x 256
+  int64_t tiles;
+  int64_t part_bytes;
+  TileSplit split;
+};
+template <bool NV>
+static TilePlan tile_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_bytes, int cus) {
+  TilePlan plan{};
+  const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  if (((M + 127) / 128) * ((N + 127) / 128) <= narrow_below(cus)) {
+    plan.kind = 0;
+    plan.tiles = ((M + 127) / 128) * ((N + 63) / 64);
+    plan.part_bytes = 4 * 64 * 32 * 4;     // four waves of 32 x 64: two accumulator tiles per lane
+  } else if (big_tiles < small_below(cus)) {
+    plan.kind = 1;
+    plan.tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    plan.part_bytes = 4 * 64 * 64 * 4;     // four waves of 64 x 64
+  } else {
+    plan.kind = (!NV || FPQ_PACKED_HALF_TILES > 1) && FPQ_PACKED_HALF_TILES ? 2 : 3;
+    plan.split = TileSplit{1, (int)(K / 256)};
+    return plan;
+  }
+  plan.split = TileSplit{1, (int)(K / 256)};
+  // (NVFP4 beyond the 256 rows that two passes of the weight-streaming kernel serve better)
+  if (NV && M > 2 * FPQ_NV_STREAM_ROWS) plan.split = tile_split_plan(plan.tiles, K, plan.part_bytes, workspace_bytes, cus);
+  return plan;
 }
 
 // fpq_gemm_stream.hip: the weight-streaming kernel for at most 128 activation rows
@@ -456,21 +595,6 @@ static int pack_operand(const void* codes, const void* scales, int64_t scale_str
 }
 }  // namespace fpq
 
-#ifndef FPQ_NV_STREAM_ROWS
-#define FPQ_NV_STREAM_ROWS 128  // NVFP4: up to this many rows the weight-streaming kernel (where its plan applies)
-#endif
-#ifndef FPQ_PACKED_HALF_TILES
-#define FPQ_PACKED_HALF_TILES 1  // large M: 1 = 256x128 tiles for MXFP4, 2 = for NVFP4 too, 0 = 256x256
-#endif
-// Shape thresholds that stand for a share of the chip are multiples of the device's compute-unit count
-// (measured on the 256 CUs of an MI355X, where they come to the figures in the comments):
-//   row slabs of the streaming kernel x weight tiles: at most one workgroup per CU (256)
-//   up to CUs / 2 tiles of 128 x 128 (128): 64 x 128 tiles instead
-//   fewer than 25/64 CUs tiles of 256 x 256 (100; under about 200 of 256 x 128): 128 x 128 tiles
-static inline int64_t slab_workgroups(int cus) { return cus; }
-static inline int64_t narrow_below(int cus) { return cus / 2; }
-static inline int64_t small_below(int cus) { return (int64_t)cus * 25 / 64; }
-
 namespace fpq {
 template <bool NV>
 static int gemm_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
@@ -501,9 +625,13 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
   // stays whole in slabs, so a shape whose K the caller's workspace lets split keeps the split up to 96 rows
   // (N = 4096, K = 14336: 64 rows 11.7 split / 11.9 us in slabs, 96 rows 13.9 / 13.9, 128 rows 15.4 / 14.1).
   const int cus = device_cus();
+  // A tile kernel that splits K through the caller's workspace comes before the row slabs.
+  const TilePlan plan = tile_plan<NV>(M, N, K, workspace ? workspace_bytes : 0, cus);
+  const bool tile_splits = FPQ_TILE_SPLIT_OVER_SLABS && plan.split.ksplit > 1;
   {
     const int64_t tiles = (N + 31) / 32;
-    const bool splits = workspace && workspace_bytes > 16384 && M <= 96 && gemm_mxf4_stream_workspace_bytes(M, N, K) > 0;
+    const bool splits = tile_splits || (workspace && workspace_bytes > 16384 && M <= 96 &&
+                                        gemm_mxf4_stream_workspace_bytes(M, N, K) > 0);
     for (int64_t cap = 32; cap <= 128 && !splits; cap += 32) {
       const int64_t slabs = (M + cap - 1) / cap;
       if (slabs * tiles > slab_workgroups(cus)) continue;
@@ -525,7 +653,7 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
     // 12288: 97 -> 52 / 68 us.  (The tile kernel's time stays at one round up to N = 16384, where two passes
     // take 44-55 us; three passes for more rows measured slower than the tiles as well.)
     const int64_t half = ((M + 1) / 2 + 31) / 32 * 32;   // rows of the first pass, whole 32-row tiles
-    if (M > FPQ_NV_STREAM_ROWS && M <= 2 * FPQ_NV_STREAM_ROWS && (N + 31) / 32 <= cus &&
+    if (!tile_splits && M > FPQ_NV_STREAM_ROWS && M <= 2 * FPQ_NV_STREAM_ROWS && (N + 31) / 32 <= cus &&
         stream_eligible(true, half, N, K)) {
       // (both passes may split K through the caller's workspace: they run one after the other on the stream)
       const int rc = gemm_fp4_stream(true, xq, xs, wq, ws, alpha, bias, residual, y, half, N, K, workspace,
@@ -543,15 +671,15 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
   // At most 128 tiles of 128 x 128 would leave half of the CUs idle: 64 x 128 tiles (twice the workgroups, the
   // same accumulation order and bits) take 25 instead of 34.5 us for NVFP4 at 257-512 rows, N = 4096, K = 4096
   // (K = 12288: 69 instead of 97 us) and 4-7 % less for MXFP4; with more tiles they measured 14 % slower.
-  if (((M + 127) / 128) * ((N + 127) / 128) <= narrow_below(cus))
-    return launch_packed<2, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);
-  const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
-  if (big_tiles < small_below(cus))
-    return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);
-#if FPQ_PACKED_HALF_TILES
-  if (!NV || FPQ_PACKED_HALF_TILES > 1)
+  // Either of these two kernels splits K through the caller's workspace where that fills the CUs (tile_split_plan).
+  if (plan.kind == 0)
+    return launch_packed<2, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg,
+                                            plan.split, workspace);
+  if (plan.kind == 1)
+    return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg,
+                                            plan.split, workspace);
+  if (plan.kind == 2)
     return launch_packed<8, 8, 4, 2, 2, NV, 4>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);
-#endif
   return launch_packed<8, 8, 8, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);
 }
 }  // namespace fpq
@@ -632,6 +760,21 @@ int gemm_mxf4_packed_any(const void* xq, const void* xs, const void* wq, const v
 
 extern "C" int64_t fpq_gemm_mxf4_packed_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return fpq::gemm_mxf4_stream_workspace_bytes(M, N, K);
+}
+
+extern "C" int64_t fpq_gemm_nvf4_packed_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M < 1 || N < 1 || K < 256 || K % 256 != 0) return 0;
+  int64_t need = 0;
+  if (M <= FPQ_NV_STREAM_ROWS) {
+    need = fpq::gemm_mxf4_stream_workspace_bytes(M, N, K);
+  } else if (M <= 2 * FPQ_NV_STREAM_ROWS) {   // two passes, the first over `half` rows
+    need = fpq::gemm_mxf4_stream_workspace_bytes(((M + 1) / 2 + 31) / 32 * 32, N, K);
+  }
+  // a tile kernel: what its K split, if it makes one, exchanges
+  const fpq::TilePlan plan = fpq::tile_plan<true>(M, N, K, (int64_t)1 << 62, fpq::device_cus());
+  const int64_t tile = plan.split.ksplit > 1
+                           ? fpq::kTileCounterBytes + plan.split.ksplit * plan.tiles * plan.part_bytes : 0;
+  return tile > need ? tile : need;
 }
 
 extern "C" int fpq_gemm_mxf4_packed_splitk(const void* xq, const void* xs, const void* wq, const void* ws,

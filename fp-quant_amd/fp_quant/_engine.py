@@ -51,6 +51,7 @@ _SIGNATURES = {
     "fpq_gemm_nvf4_packed": ([_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _I),
     "fpq_gemm_mxf4_packed": ([_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _I),
     "fpq_gemm_mxf4_packed_workspace_bytes": ([_I64, _I64, _I64], _I64),
+    "fpq_gemm_nvf4_packed_workspace_bytes": ([_I64, _I64, _I64], _I64),
     "fpq_gemm_mxf4_packed_splitk": ([_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P, _I64, _P], _I),
     "fpq_gemm_nvf4_packed_splitk": ([_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P, _I64, _P], _I),
     "fpq_gemm_mxf4_packed_residual": ([_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _I),

@@ -33,6 +33,7 @@ from .hip_ops import (
     packed_weights_enabled,
     quantize_mx_packed,
     splitk_workspace,
+    SPLIT_K_MAX_ROWS,
     SPLIT_K_ROWS,
     unpack_fp4,
     weight_rows,
@@ -293,9 +294,10 @@ def linear_on(qa: QuantizedActivations, wq: torch.Tensor, ws: torch.Tensor, alph
             xp, xsp = qa.packed()
             if packed is None:
                 wp, wsp = packed_weight(wq, ws, True)
-            # (NVFP4 runs 129-256 rows as two passes of the kernel that can split K: each may use the workspace)
-            workspace = (splitk_workspace(wq, n, k, remember, stream)
-                         if (m <= 2 * SPLIT_K_ROWS and packed is None) else None)
+            # (NVFP4 runs 129-256 rows as two passes of the kernel that can split K: each may use the workspace;
+            # beyond, the tile kernels split K where that fills the CUs)
+            workspace = (splitk_workspace(wq, n, k, remember, stream, True)
+                         if (m <= SPLIT_K_MAX_ROWS and packed is None) else None)
             if workspace is not None:
                 st = lib.fpq_gemm_nvf4_packed_splitk(xp.data_ptr(), xsp.data_ptr(), wp.data_ptr(), wsp.data_ptr(),
                                                      alpha.data_ptr(), b_ptr,

@@ -435,8 +435,13 @@ def adopt_packed_weight(wq: torch.Tensor, ws: torch.Tensor, nvfp4: bool, pc: tor
         pass
 
 
-_splitk_need = {}   # (n, k) -> workspace bytes with which fpq_gemm_mxf4_packed_splitk splits K at up to SPLIT_K_ROWS rows
-SPLIT_K_ROWS = 128  # the rows the weight-streaming GEMM takes
+_splitk_need = {}   # (n, k, nvfp4) -> workspace bytes with which fpq_gemm_*_packed_splitk splits K at any row count it does
+SPLIT_K_ROWS = 128  # the rows the weight-streaming GEMM takes (MXFP4 splits nowhere else)
+# NVFP4: beyond them come two passes of that kernel (up to 256 rows) and the tile kernels' K split (a few
+# hundred rows on few weight rows and a long K); the row counts probed for the workspace a layer may need,
+# and the row count up to which a call hands its workspace to the library
+_SPLIT_K_PROBE_ROWS = (32, 64, 96, 128, 192, 256, 384, 512, 768, 1024)
+SPLIT_K_MAX_ROWS = 1024
 # FPQ_SPLIT_K=0: no split-K workspace anywhere; every GEMM walks the whole of K in one workgroup
 SPLIT_K = os.environ.get("FPQ_SPLIT_K", "1") != "0"
 
@@ -461,7 +466,8 @@ def _stream_workspace(device: torch.device, stream: int, need: int) -> torch.Ten
     return workspace
 
 
-def splitk_workspace(wq: torch.Tensor, n: int, k: int, create: bool, stream: Optional[int] = None) -> Optional[torch.Tensor]:
+def splitk_workspace(wq: torch.Tensor, n: int, k: int, create: bool, stream: Optional[int] = None,
+                     nvfp4: bool = False) -> Optional[torch.Tensor]:
     """The workspace with which the packed GEMM of a layer [n, k] (either format) splits K across workgroups at
     up to 128 activation rows (few weight rows and a long K: a Llama down-projection), or None where it would
     not split.  Always zeroed between calls.  Which one:
@@ -476,9 +482,12 @@ def splitk_workspace(wq: torch.Tensor, n: int, k: int, create: bool, stream: Opt
     Either way the layer takes the same kernel and gives the same bits."""
     if not SPLIT_K:
         return None
-    need = _splitk_need.get((n, k))
+    need = _splitk_need.get((n, k, nvfp4))
     if need is None:
-        need = _splitk_need[(n, k)] = int(_engine.lib().fpq_gemm_mxf4_packed_workspace_bytes(SPLIT_K_ROWS, n, k))
+        lib = _engine.lib()
+        size = lib.fpq_gemm_nvf4_packed_workspace_bytes if nvfp4 else lib.fpq_gemm_mxf4_packed_workspace_bytes
+        rows = _SPLIT_K_PROBE_ROWS if nvfp4 else _SPLIT_K_PROBE_ROWS[:4]
+        need = _splitk_need[(n, k, nvfp4)] = max(int(size(m, n, k)) for m in rows)
     if need == 0:
         return None
     capturing = torch.cuda.is_current_stream_capturing()

@@ -174,7 +174,8 @@ class FPQuantLinear(nn.Module):
         if (isinstance(qweight, torch.Tensor) and qweight.is_cuda and hip_ops.packed_weights_enabled()
                 and self.config.forward_dtype in (FPQuantDtype.MXFP4, FPQuantDtype.NVFP4)
                 and self.in_features % 256 == 0):
-            hip_ops.splitk_workspace(qweight, self.out_features, self.in_features, True)
+            hip_ops.splitk_workspace(qweight, self.out_features, self.in_features, True,
+                                     nvfp4=self.config.forward_dtype == FPQuantDtype.NVFP4)
 
     # True once release_row_major has been asked for: the layer goes back to the packed layout after
     # every load_state_dict

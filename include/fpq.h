@@ -314,9 +314,13 @@ int fpq_gemm_mxf4_packed_splitk(const void* xq_packed, const void* xs_packed, co
                                 const void* residual, void* y, int64_t M, int64_t N, int64_t K,
                                 void* workspace, int64_t workspace_bytes, void* stream);
 /* The same for packed NVFP4 operands (fpq_gemm_nvf4_packed, with `residual` non-null fpq_gemm_nvf4_packed_residual);
- * workspace as above, sized by fpq_gemm_mxf4_packed_workspace_bytes (the split is the same for both formats;
- * 129-256 rows of NVFP4 at 4096 < N <= 8192 run as two passes over at most 128 rows each, and each pass may use it:
- * size it for 128 rows). */
+ * workspace as above, sized by fpq_gemm_nvf4_packed_workspace_bytes(M, N, K).  Up to 128 rows the split is
+ * that of the MXFP4 entry; 129-256 rows on few weight rows run as two passes over at most 128 rows each, and
+ * each pass may use the workspace; from 257 rows on the tile kernels split K the same way (fp32 parts of
+ * their workgroup tiles, a counter per tile, parts added in part order) where few tiles and a long K would
+ * leave CUs idle -- the NVFP4 loop is bound by its in-register dequantization, so more workgroups pay there
+ * although the parts are as many bytes as the operands (MXFP4 measured slower with it and never does). */
+int64_t fpq_gemm_nvf4_packed_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int fpq_gemm_nvf4_packed_splitk(const void* xq_packed, const void* xs_packed, const void* wq_packed,
                                 const void* ws_packed, const float* alpha, const void* bias,
                                 const void* residual, void* y, int64_t M, int64_t N, int64_t K,
