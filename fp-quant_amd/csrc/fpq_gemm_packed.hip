@@ -150,6 +150,11 @@ __device__ __forceinline__ void wait_vmem_le() {
 __device__ __forceinline__ void barrier_lds() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
+// The same with this wave's N newest LDS reads left outstanding (LDS operations complete in order).
+template <int N>
+__device__ __forceinline__ void barrier_lds_but() {
+  asm volatile("s_waitcnt lgkmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
 
 // One workgroup of four waves (WN x WM) computes a tile of NT*32 weight rows (n) x MT*32 activation
 // rows (m); a wave owns TN x TM accumulator tiles of 32 x 32.  A unit holds KW >= NT weight and MT
@@ -280,8 +285,22 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   // operand registers of the current and the next unit; scales of the current block and, read
-  // ahead, of the next one
-  uint4 aq[2][TN], bq[2][TM];
+  // ahead, of the next one.
+  // kDeep (one row of MFMAs per unit, MXFP4): a wave has only TM matrix instructions per unit to cover the
+  // LDS reads of the next one, the wait for them and the barrier, which left the matrix pipes idle three
+  // quarters of the time.  There the registers run TWO units ahead (four sets, indexed by the unit's place in
+  // its 256-K block): at the hand-over of unit u the reads of unit u + 2 are issued, those of unit u + 1 may
+  // stay outstanding across the barrier, and the matrix instructions of unit u follow at once (64 x 128
+  // tiles, N = 4096, K = 14336: 384 / 512 rows 28.9 / 29.0 -> 26.5 / 26.8 us; N = 14336, K = 4096, 128 rows
+  // 10.1 -> 9.7 us; a ring of sixteen units instead of eight changed nothing, and with every load, LDS read
+  // and barrier compiled out the matrix instructions alone take 16.3 us at 512 rows).  NVFP4 and the tiles
+  // with two rows of matrix instructions per unit measured slower that way and keep one unit ahead.
+#ifndef FPQ_DEEP_SMALL
+#define FPQ_DEEP_SMALL 1
+#endif
+  constexpr bool kDeep = FPQ_DEEP_SMALL && TN == 1 && !NV;
+  constexpr int kSets = kDeep ? 4 : 2;
+  uint4 aq[kSets][TN], bq[kSets][TM];
   uint2 sa[TN], sb[TM], sa_next[TN], sb_next[TM];   // MXFP4 uses .x only
   const int a_off = (wn * TN) * 1024 + lane * 16, b_off = (KW + wm * TM) * 1024 + lane * 16;
   const int sa_off = kScaleBase + (wn * TN) * kSB + lane * (kSB / 64);
@@ -313,11 +332,18 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
   for (int u = 0; u < n_pro; ++u) issue_unit(u, (u & 3) == 0);
   // Loads complete in order: unit 0 and scale block 0 have landed once at most the loads of the
   // younger units are outstanding (a wave issues kPer per unit, one more with scales).
-  if (n_pro == RING) wait_vmem_le<(RING - 1) * kPer>();
+  if (n_pro == RING) wait_vmem_le<(RING - (kDeep ? 2 : 1)) * kPer>();
   else wait_vmem();
   barrier_lds();
   read_unit(0, 0);
+  if constexpr (kDeep) read_unit(1, 1);   // (a K range holds at least four units)
   read_scales(0);
+  if constexpr (kDeep) {   // (the first block's scales move into place here, the others' behind the block before)
+#pragma unroll
+    for (int i = 0; i < TN; ++i) sa[i] = sa_next[i];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) sb[j] = sb_next[j];
+  }
 
   // One 64-K unit: 16 MFMAs per wave.  After the first row of MFMAs comes the hand-over: every
   // wave holds unit u in registers, so its ring slot is free for unit u + RING, and unit u + 1
@@ -335,10 +361,10 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
     }                                                                                               \
     __builtin_amdgcn_sched_barrier(0);                                                              \
   } else {                                                                                          \
-    const uint4 av = aq[(Q) & 1][I];                                                                \
+    const uint4 av = aq[(Q) & (kSets - 1)][I];                                                      \
     const v8i a = v8i{(int)av.x, (int)av.y, (int)av.z, (int)av.w, 0, 0, 0, 0};                      \
     _Pragma("unroll") for (int j = 0; j < TM; ++j) {                                                \
-      const uint4 bv = bq[(Q) & 1][j];                                                              \
+      const uint4 bv = bq[(Q) & (kSets - 1)][j];                                                    \
       const v8i b = v8i{(int)bv.x, (int)bv.y, (int)bv.z, (int)bv.w, 0, 0, 0, 0};                    \
       acc[I][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[I][j], 4, 4, Q,        \
                                                                   (int)sa[I].x, Q, (int)sb[j].x);   \
@@ -358,23 +384,46 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
     }                                                                                               \
   }
   constexpr int kHand = (TM >= 4 || TN <= 2) ? 1 : 2;  // rows of MFMAs ahead of the hand-over
-  // ALLOWED: loads of this wave that may still be outstanding while unit u + 1 is complete
-#define FPQ_UNIT(Q, U, ALLOWED, ISSUE, READ, READ_SCALES)                                           \
-  {                                                                                                 \
+  // ALLOWED: loads of this wave that may still be outstanding while unit u + 1 is complete; READ / READ2: unit
+  // u + 1 / u + 2 exists; NEXT_BLOCK: so does the 256-K block after this unit's, whose scales are read into
+  // registers at the block's last hand-over (kDeep: at the one before, so that the reads of unit u + 1 are
+  // the newest at the start of a block and taking the scales does not wait for them)
+#define FPQ_UNIT(Q, U, ALLOWED, ISSUE, READ, NEXT_BLOCK, READ2)                                     \
+  if constexpr (kDeep) {                                                                            \
+    wait_vmem_le<((ALLOWED) >= kPer ? (ALLOWED) - kPer : 0)>();   /* unit u + 2 is complete */     \
+    barrier_lds_but<TN + TM>();                                                                     \
+    if (ISSUE) issue_unit((U) + RING, (Q) == 0);                                                   \
+    if ((Q) == 2 && (NEXT_BLOCK)) read_scales(((U) + 2) >> 2);                                      \
+    if (READ2) read_unit((U) + 2, ((Q) + 2) & 3);                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                                              \
+    _Pragma("unroll") for (int i1 = 0; i1 < TN; ++i1) FPQ_MFMA_ROW(Q, i1)                           \
+  } else {                                                                                          \
     FPQ_PREP_B(Q)                                                                                   \
     _Pragma("unroll") for (int i0 = 0; i0 < kHand; ++i0) FPQ_MFMA_ROW(Q, i0)                        \
     wait_vmem_le<(ALLOWED)>();                                                                      \
     barrier_lds();                                                                                  \
     if (ISSUE) issue_unit((U) + RING, (Q) == 0);                                                   \
     if (READ) read_unit((U) + 1, ((Q) + 1) & 1);                                                    \
-    if (READ_SCALES) read_scales(((U) + 1) >> 2);                                                   \
+    if ((Q) == 3 && (NEXT_BLOCK)) read_scales(((U) + 1) >> 2);                                      \
     __builtin_amdgcn_sched_barrier(0);                                                              \
     _Pragma("unroll") for (int i1 = kHand; i1 < TN; ++i1) FPQ_MFMA_ROW(Q, i1)                       \
   }
-#define FPQ_TAKE_SCALES()                                                                           \
+#define FPQ_TAKE_SCALES_NOW()                                                                       \
   {                                                                                                 \
     _Pragma("unroll") for (int i = 0; i < TN; ++i) sa[i] = sa_next[i];                              \
     _Pragma("unroll") for (int j = 0; j < TM; ++j) sb[j] = sb_next[j];                              \
+  }
+  // The scales of a block move into place at its start; kDeep: at the end of the block before (behind its last
+  // matrix instructions, in straight-line code, where the compiler sees that only the operand reads issued
+  // since may still be outstanding: at the head of the loop it waits for every LDS read instead)
+#define FPQ_TAKE_SCALES()                                                                           \
+  if constexpr (!kDeep) FPQ_TAKE_SCALES_NOW()
+#define FPQ_TAKE_SCALES_AFTER()                                                                     \
+  if constexpr (kDeep) {   /* (moves the compiler may not turn into copies at the head of the loop) */ \
+    _Pragma("unroll") for (int i = 0; i < TN; ++i)                                                  \
+      asm volatile("v_mov_b32 %0, %1" : "=v"(sa[i].x) : "v"(sa_next[i].x));                         \
+    _Pragma("unroll") for (int j = 0; j < TM; ++j)                                                  \
+      asm volatile("v_mov_b32 %0, %1" : "=v"(sb[j].x) : "v"(sb_next[j].x));                         \
   }
 
   // steady state: every unit of these blocks still has a unit RING ahead of it to issue
@@ -383,35 +432,38 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
   for (int kb = 0; kb < kb_tail; ++kb) {
     const int u0 = kb * 4;
     FPQ_TAKE_SCALES()
-    FPQ_UNIT(0, u0 + 0, (RING - 2) * kPer, true, true, false)
-    FPQ_UNIT(1, u0 + 1, (RING - 2) * kPer, true, true, false)
-    FPQ_UNIT(2, u0 + 2, (RING - 2) * kPer, true, true, false)
-    FPQ_UNIT(3, u0 + 3, (RING - 2) * kPer, true, true, true)
+    FPQ_UNIT(0, u0 + 0, (RING - 2) * kPer, true, true, true, true)
+    FPQ_UNIT(1, u0 + 1, (RING - 2) * kPer, true, true, true, true)
+    FPQ_UNIT(2, u0 + 2, (RING - 2) * kPer, true, true, true, true)
+    FPQ_UNIT(3, u0 + 3, (RING - 2) * kPer, true, true, true, true)
+    FPQ_TAKE_SCALES_AFTER()
   }
   // drain: the last ring of units (fewer if K is short); nothing is issued any more, and with t
-  // units to go after unit u + 1 exactly t * kPer loads may stay outstanding
-  if constexpr (RING == 8) {
-    if (nkb >= 2) {
-      const int u0 = (nkb - 2) * 4;
-      FPQ_TAKE_SCALES()
-      FPQ_UNIT(0, u0 + 0, 6 * kPer, false, true, false)
-      FPQ_UNIT(1, u0 + 1, 5 * kPer, false, true, false)
-      FPQ_UNIT(2, u0 + 2, 4 * kPer, false, true, false)
-      FPQ_UNIT(3, u0 + 3, 3 * kPer, false, true, true)
-    }
+  // units to go after unit u + 1 exactly t * kPer loads may stay outstanding.  Block D of the kDrain last ones:
+#define FPQ_DRAIN_BLOCK(D)                                                                          \
+  if constexpr (kDrain > (D)) {                                                                     \
+    constexpr int kLeft = 4 * (kDrain - 1 - (D));   /* units behind this block */                   \
+    if (kLeft == 0 || nkb >= kDrain - (D)) {   /* (the last block always exists) */                 \
+      const int u0 = (nkb - (kDrain - (D))) * 4;                                                    \
+      FPQ_TAKE_SCALES()                                                                             \
+      FPQ_UNIT(0, u0 + 0, (kLeft + 2) * kPer, false, true, kLeft > 0, true)                         \
+      FPQ_UNIT(1, u0 + 1, (kLeft + 1) * kPer, false, true, kLeft > 0, true)                         \
+      FPQ_UNIT(2, u0 + 2, kLeft * kPer, false, true, kLeft > 0, kLeft > 0)                          \
+      FPQ_UNIT(3, u0 + 3, (kLeft > 0 ? kLeft - 1 : 0) * kPer, false, kLeft > 0, kLeft > 0, kLeft > 0) \
+      if constexpr (kLeft > 0) FPQ_TAKE_SCALES_AFTER()                                              \
+    }                                                                                               \
   }
-  {
-    const int u0 = (nkb - 1) * 4;
-    FPQ_TAKE_SCALES()
-    FPQ_UNIT(0, u0 + 0, 2 * kPer, false, true, false)
-    FPQ_UNIT(1, u0 + 1, 1 * kPer, false, true, false)
-    FPQ_UNIT(2, u0 + 2, 0, false, true, false)
-    FPQ_UNIT(3, u0 + 3, 0, false, false, false)
-  }
+  FPQ_DRAIN_BLOCK(0)
+  FPQ_DRAIN_BLOCK(1)
+  FPQ_DRAIN_BLOCK(2)
+  FPQ_DRAIN_BLOCK(3)
+#undef FPQ_DRAIN_BLOCK
 #undef FPQ_UNIT
 #undef FPQ_PREP_B
 #undef FPQ_MFMA_ROW
 #undef FPQ_TAKE_SCALES
+#undef FPQ_TAKE_SCALES_NOW
+#undef FPQ_TAKE_SCALES_AFTER
 
   if (kCanSplit && ksplit > 1) {
     // The parts of a tile run on different XCDs, whose L2 caches are not coherent with each other for
