@@ -292,7 +292,8 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
   // its 256-K block): at the hand-over of unit u the reads of unit u + 2 are issued, those of unit u + 1 may
   // stay outstanding across the barrier, and the matrix instructions of unit u follow at once (64 x 128
   // tiles, N = 4096, K = 14336: 384 / 512 rows 28.9 / 29.0 -> 26.5 / 26.8 us; N = 14336, K = 4096, 128 rows
-  // 10.1 -> 9.7 us; a ring of sixteen units instead of eight changed nothing, and with every load, LDS read
+  // 10.1 -> 9.7 us, 14.0 -> 13.4 with the weights streamed from HBM; a ring of sixteen units instead of eight
+  // changed nothing from the caches and cost 3 % from HBM, and with every load, LDS read
   // and barrier compiled out the matrix instructions alone take 16.3 us at 512 rows).  NVFP4 and the tiles
   // with two rows of matrix instructions per unit measured slower that way and keep one unit ahead.
 #ifndef FPQ_DEEP_SMALL
