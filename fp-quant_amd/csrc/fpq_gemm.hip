@@ -408,12 +408,8 @@ __global__ __launch_bounds__(128 * WM) void gemm_mxf4_lds_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   // Consecutive workgroup ids land on different XCDs (8 of them, each with its own L2), so
   // give every XCD a contiguous run of the tile list: its tiles then share weight row-panels.
-  int logical = blockIdx.x;
-  {
-    const int nb = gridDim.x, per = nb / 8;
-    if (blockIdx.x < (unsigned)(per * 8)) logical = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
-  }
-  const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
+  int tile_m, tile_n;
+  banded_tile<BM>(tiles_m, tile_m, tile_n);
   const int n_blk = tile_n * BN, m_blk = tile_m * BM;
   const int wn = wave & 1, wm = wave >> 1;
   const int kbytes = K >> 1;
@@ -722,12 +718,8 @@ __global__ __launch_bounds__(256) void gemm_nvf4_lds_kernel(
   const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  int logical = blockIdx.x;
-  {
-    const int nb = gridDim.x, per = nb / 8;
-    if (blockIdx.x < (unsigned)(per * 8)) logical = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
-  }
-  const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
+  int tile_m, tile_n;
+  banded_tile<BM>(tiles_m, tile_m, tile_n);
   const int n_blk = tile_n * BN, m_blk = tile_m * BM;
   const int wn = wave & 1, wm = wave >> 1;
   const int kbytes = K >> 1;

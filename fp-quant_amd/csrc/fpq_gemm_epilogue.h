@@ -28,6 +28,35 @@ struct LdsLimitOnce {
   }
 };
 
+// Which output tile a workgroup of a large-M kernel computes, and its number in the tile list (returned).
+// Consecutive workgroup ids land on different XCDs (8 of them, each with its own L2), so every XCD gets a
+// contiguous run of the list.  The list walks bands of kBandRows activation rows: inside a band the
+// activation row tiles run fastest, then the weight strips, so the workgroups an XCD holds at a time (32 or
+// 64) form a block that shares about as many weight strips as activation tiles through the XCD's L2, and a
+// band's activations stay there while its strips stream past.  Measured against activation tiles fastest
+// over the whole of M (256 x 128 tiles, K = 4096): 4096 rows, N = 14336 127.1 -> 120.0 us; 8192 rows, N = 4096 /
+// 14336 / 28672 75.1 -> 70.3 / 245.1 -> 232.2 / 493.9 -> 463.0 us; 2048 rows unchanged; bands of 512 or 2048 rows
+// 1-2 % behind 1024.  The row-major NVFP4 kernel (256 x 256 tiles) gains 2.4 % at 8192 rows, nothing at 4096.
+constexpr int kBandRows = 1024;
+template <int BM>
+__device__ __forceinline__ int banded_tile(int tiles_m, int& tile_m, int& tile_n) {
+  int logical = blockIdx.x;
+  const int nb = gridDim.x, per = nb / 8;
+  if (blockIdx.x < (unsigned)(per * 8)) logical = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+  constexpr int kBand = kBandRows / BM > 0 ? kBandRows / BM : 1;   // activation row tiles per band
+  if (tiles_m > kBand) {
+    const int tiles_n = nb / tiles_m;
+    const int band = logical / (kBand * tiles_n), within = logical - band * (kBand * tiles_n);
+    const int first_m = band * kBand, rows = min(tiles_m - first_m, kBand);
+    tile_m = first_m + within % rows;
+    tile_n = within / rows;
+  } else {
+    tile_m = logical % tiles_m;
+    tile_n = logical / tiles_m;
+  }
+  return logical;
+}
+
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));

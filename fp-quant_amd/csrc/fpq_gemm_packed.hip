@@ -206,16 +206,10 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
   static_assert(kScaleBase + kSlots * kSlotBytes == kPackedLds, "LDS map does not match the allocation");
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  // Consecutive workgroup ids land on different XCDs (8 of them, each with its own L2): give
-  // every XCD a contiguous run of the tile list so that its tiles share operand panels.  (One
-  // workgroup per tile: a persistent variant that walked several tiles per CU measured slower,
-  // the hardware's own dispatch balances the XCDs better.)
-  int logical = blockIdx.x;
-  {
-    const int nb = gridDim.x, per = nb / 8;
-    if (blockIdx.x < (unsigned)(per * 8)) logical = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
-  }
-  const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
+  // (One workgroup per tile: a persistent variant that walked several tiles per CU measured slower, the
+  // hardware's own dispatch balances the XCDs better.)
+  int tile_m, tile_n;
+  const int logical = banded_tile<BM>(tiles_m, tile_m, tile_n);
   const int n_blk = tile_n * BN, m_blk = tile_m * BM;
   const int wn = wave % WN, wm = wave / WN;
   const int nu = K >> 6, nkb_all = K >> 8;      // units, scale blocks of a whole row tile
