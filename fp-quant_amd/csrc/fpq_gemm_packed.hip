@@ -129,16 +129,17 @@ constexpr int scale_block_bytes(bool nv) { return nv ? 512 : 256; }
 constexpr int scale_slot_bytes(int blocks, bool nv) {
   return (blocks * scale_block_bytes(nv) > 4096 ? blocks * scale_block_bytes(nv) : 4096);
 }
-constexpr int scale_slots(bool nv) { return nv ? 2 : kScaleSlots; }
-// LDS of a workgroup whose unit holds `blocks` operand kilobytes (weight + activation row tiles)
-constexpr int packed_lds_bytes(int blocks, bool nv = false, int ring = kRing) {
-  return ring * blocks * 1024 + scale_slots(nv) * scale_slot_bytes(blocks, nv);
+constexpr int scale_slots(bool nv, int groups = 1) { return nv || groups > 1 ? 2 : kScaleSlots; }
+// LDS of a group of four waves whose unit holds `blocks` operand kilobytes (weight + activation row tiles)
+constexpr int packed_lds_bytes(int blocks, bool nv = false, int ring = kRing, int groups = 1) {
+  return ring * blocks * 1024 + scale_slots(nv, groups) * scale_slot_bytes(blocks, nv);
 }
 // ... and what is allocated: at least the epilogue's staging area (four waves, each WT_M rows of
 // WT_N bf16 + 16 bytes)
-constexpr int packed_lds_alloc(int blocks, bool nv, int ring, int wt_n, int wt_m) {
-  return packed_lds_bytes(blocks, nv, ring) > 4 * wt_m * (wt_n * 2 + 16) ? packed_lds_bytes(blocks, nv, ring)
-                                                                         : 4 * wt_m * (wt_n * 2 + 16);
+constexpr int packed_lds_alloc(int blocks, bool nv, int ring, int wt_n, int wt_m, int groups = 1) {
+  return groups * packed_lds_bytes(blocks, nv, ring, groups) > 4 * wt_m * (wt_n * 2 + 16)
+             ? groups * packed_lds_bytes(blocks, nv, ring, groups)
+             : 4 * wt_m * (wt_n * 2 + 16);
 }
 
 template <int N>
@@ -178,8 +179,14 @@ __device__ __forceinline__ void barrier_lds_but() {
 // scale blocks): codes are dequantized in registers to exact fp16 and fed to the fp16 MFMA; a lane's
 // dword s of a block goes to MFMA s of the unit on both operands, so the K order is permuted
 // consistently and the sum is complete.
-template <int NT, int KW, int MT, int WN, int WM, bool NV = false, int RING = kRing>
-__global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_kernel(
+// GR = 2 (the 64 x 128 and 128 x 128 tiles when every workgroup has a CU to itself): a workgroup of eight
+// waves in two groups of four, each group the kernel described above on one half of K with a ring of its
+// own; the second group hands its accumulators to the first through LDS after the loop.  A wave of these
+// small tiles spends most of a unit waiting -- for its loads, for the barrier, for its two or four matrix
+// instructions to drain -- and alone on its SIMD nothing fills that time; with a second wave there, working
+// on the other half of K, something does, and each group's loop is half as long.
+template <int NT, int KW, int MT, int WN, int WM, bool NV = false, int RING = kRing, int GR = 1>
+__global__ __launch_bounds__(256 * GR, (NT * MT <= 32 && GR == 1 ? 2 : 1)) void gemm_fp4_packed_kernel(
     const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p,
     const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, int M, int N, int K, int tiles_m,
@@ -196,16 +203,19 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
   constexpr int kRpp = 1024 / kSB;                      // row tiles per 1 KB scale piece
   constexpr int kPieces = kBlocks / kRpp;               // scale pieces per 256-K block
   constexpr int kScLoads = kPieces >= NW ? kPieces / NW : 1;  // scale loads per wave per block
-  constexpr int kSlots = scale_slots(NV), kSlotBytes = scale_slot_bytes(kBlocks, NV);
+  constexpr int kSlots = scale_slots(NV, GR), kSlotBytes = scale_slot_bytes(kBlocks, NV);
   constexpr int kUnitBytes = kBlocks * 1024;
   static_assert(RING == 4 || RING == 8, "the ring holds one or two 256-K blocks");
-  constexpr int kPackedLds = packed_lds_bytes(kBlocks, NV, RING);
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  constexpr int kPackedLds = packed_lds_bytes(kBlocks, NV, RING, GR);
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_all[];
+  static_assert(GR == 1 || GR == 2, "one or two groups of four waves");
+  const int grp = GR > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 8) : 0;
+  uint8_t* const smem = smem_all + grp * kPackedLds;   // this group's ring and scale slots
   const uint32_t smem_base = (uint32_t)(uintptr_t)smem;
   constexpr int kScaleBase = RING * kUnitBytes;
   static_assert(kScaleBase + kSlots * kSlotBytes == kPackedLds, "LDS map does not match the allocation");
 
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((threadIdx.x >> 6) & 3), lane = threadIdx.x & 63;
   // (One workgroup per tile: a persistent variant that walked several tiles per CU measured slower, the
   // hardware's own dispatch balances the XCDs better.)
   int tile_m, tile_n;
@@ -217,7 +227,8 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
   // [kb_begin, kb_begin + nkb) only, and the parts of a tile meet in the workspace after the loop.
   // Only the kernels for few tiles are ever launched that way (the large tiles have no register to spare).
   constexpr bool kCanSplit = NT * MT <= 16;
-  const int kb_begin = kCanSplit ? blockIdx.y * bps : 0;
+  static_assert(GR == 1 || kCanSplit, "groups split K");
+  const int kb_begin = kCanSplit ? (blockIdx.y * GR + grp) * bps : 0;   // (GR = 2: both halves hold bps blocks)
   const int nkb = kCanSplit ? min(nkb_all - kb_begin, bps) : nkb_all;
   const int rt_n = (N + 31) >> 5, rt_m = (M + 31) >> 5;
 
@@ -463,7 +474,33 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
 #undef FPQ_TAKE_SCALES_NOW
 #undef FPQ_TAKE_SCALES_AFTER
 
-  if (kCanSplit && ksplit > 1) {
+  if constexpr (GR == 2) {
+    // The second group's accumulators go to the first through LDS (the rings are idle: every wave has waited
+    // for its last loads and read its last unit), added in a fixed order; then the second group only keeps
+    // the first company at the one barrier of the epilogue.  (Launched with K whole per workgroup: ksplit = 1.)
+    __syncthreads();
+    float* xch = (float*)smem_all + wave * (TN * TM * 16 * 64) + lane;
+    if (grp == 1) {
+#pragma unroll
+      for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) xch[((i * TM + j) * 16 + v) * 64] = acc[i][j][v];
+    }
+    __syncthreads();
+    if (grp == 1) {
+      __syncthreads();
+      return;
+    }
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < TM; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] += xch[((i * TM + j) * 16 + v) * 64];
+  }
+  if (GR == 1 && kCanSplit && ksplit > 1) {
     // The parts of a tile run on different XCDs, whose L2 caches are not coherent with each other for
     // ordinary accesses: every access to the workspace is a relaxed device-scope atomic, every wave waits
     // for its stores to be acknowledged before the workgroup moves the tile's counter, and the workgroup
@@ -507,8 +544,8 @@ __global__ __launch_bounds__(256, (NT * MT <= 32 ? 2 : 1)) void gemm_fp4_packed_
   }
 
   const OutView out = out_view(seg, y, bias, n_blk + wn * TN * 32, N);
-  wave_tile_store<TN, TM, packed_lds_alloc(kBlocks, NV, RING, TN * 32, TM * 32), NW>(
-      acc, smem, out.y, out.bias, alpha_p, out.n0, m_blk + wm * TM * 32, wave, lane, M, out.N, residual);
+  wave_tile_store<TN, TM, packed_lds_alloc(kBlocks, NV, RING, TN * 32, TM * 32, GR), NW>(
+      acc, smem_all, out.y, out.bias, alpha_p, out.n0, m_blk + wm * TM * 32, wave, lane, M, out.N, residual);
 }
 
 }  // namespace fpq
@@ -536,18 +573,23 @@ struct TileSplit {
   int bps = 0;      // 256-K blocks per part (the last part may have fewer, never none)
 };
 
-template <int NT, int KW, int MT, int WN, int WM, bool NV, int RING = kRing>
+template <int NT, int KW, int MT, int WN, int WM, bool NV, int RING = kRing, int GR = 1>
 static int launch_packed(const void* xq, const void* xs, const void* wq, const void* ws, const float* alpha,
                          const void* bias, void* y, int64_t M, int64_t N, int64_t K, hipStream_t stream,
                          const void* residual, const OutSegments& seg, TileSplit split = TileSplit{},
                          void* workspace = nullptr) {
-  constexpr int kLds = packed_lds_alloc(KW + MT, NV, RING, NT / WN * 32, MT / WM * 32);
+  constexpr int kLds = packed_lds_alloc(KW + MT, NV, RING, NT / WN * 32, MT / WM * 32, GR);
+  static_assert(kLds <= 160 * 1024, "more LDS than a CU has");
   const int tiles_m = (int)((M + MT * 32 - 1) / (MT * 32)), tiles_n = (int)((N + NT * 32 - 1) / (NT * 32));
-  if (split.ksplit <= 1 || !workspace || NT * MT > 16) split = TileSplit{1, (int)(K / 256)};
+  if (split.ksplit <= 1 || !workspace || NT * MT > 16 || GR > 1) split = TileSplit{1, (int)(K / 256)};
+  if (GR > 1) {   // the two groups of a workgroup take one half of K each (the caller checked that K / 256 is even)
+    if ((K / 256) % GR != 0) return FPQ_E_UNSUPPORTED;
+    split.bps = (int)(K / 256) / GR;
+  }
   static LdsLimitOnce lds_limit;
-  if (const int st = lds_limit.ensure((const void*)gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV, RING>, kLds)) return st;
-  hipLaunchKernelGGL((gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV, RING>),
-                     dim3((unsigned)(tiles_m * tiles_n), (unsigned)split.ksplit), dim3(256), kLds, stream,
+  if (const int st = lds_limit.ensure((const void*)gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV, RING, GR>, kLds)) return st;
+  hipLaunchKernelGGL((gemm_fp4_packed_kernel<NT, KW, MT, WN, WM, NV, RING, GR>),
+                     dim3((unsigned)(tiles_m * tiles_n), (unsigned)split.ksplit), dim3(256 * GR), kLds, stream,
                      (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq, (const uint8_t*)ws, alpha,
                      (const uint16_t*)bias, (uint16_t*)y, (int)M, (int)N, (int)K, tiles_m,
                      (const uint16_t*)residual, seg, split.ksplit, split.bps,
@@ -586,10 +628,12 @@ struct TilePlan {
   int64_t tiles;
   int64_t part_bytes;
   TileSplit split;
+  int groups;        // 2: workgroups of eight waves, K halved inside the workgroup (no K split across workgroups then)
 };
 template <bool NV>
 static TilePlan tile_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_bytes, int cus) {
   TilePlan plan{};
+  plan.groups = 1;
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
   if (((M + 127) / 128) * ((N + 127) / 128) <= narrow_below(cus)) {
     plan.kind = 0;
@@ -605,6 +649,16 @@ static TilePlan tile_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_byt
     return plan;
   }
   plan.split = TileSplit{1, (int)(K / 256)};
+  // NVFP4 with at most one workgroup per CU: two groups of four waves per workgroup, one half of K each (the
+  // in-register conversions of one wave overlap the matrix instructions of the other on its SIMD, and the halves
+  // meet in LDS): 300-512 rows, N = 4096, K = 4096 25.9 -> 23.4 us; 640-1024 rows 34.9-37.3 -> 32.2-35.6;
+  // N = 12288, 129-256 rows 35.1 -> 32.9; K = 12288, 384 / 512 rows 69 / 70 -> 59.3 / 62.7 (a K split across two
+  // workgroups through the caller's workspace: 61.1 / 65.3).  MXFP4, whose waves wait on what the CU receives
+  // from the L2, measured the same with 64 x 128 tiles and 8 % slower with 128 x 128: it keeps four waves.
+  if (NV && plan.tiles <= cus && (K / 256) % 2 == 0 && K >= 2048) {
+    plan.groups = 2;
+    return plan;
+  }
   // (NVFP4 beyond the 256 rows that two passes of the weight-streaming kernel serve better)
   if (NV && M > 2 * FPQ_NV_STREAM_ROWS) plan.split = tile_split_plan(plan.tiles, K, plan.part_bytes, workspace_bytes, cus);
   return plan;
@@ -722,6 +776,14 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
   // same accumulation order and bits) take 25 instead of 34.5 us for NVFP4 at 257-512 rows, N = 4096, K = 4096
   // (K = 12288: 69 instead of 97 us) and 4-7 % less for MXFP4; with more tiles they measured 14 % slower.
   // Either of these two kernels splits K through the caller's workspace where that fills the CUs (tile_split_plan).
+  if constexpr (NV) {
+    if (plan.groups == 2 && plan.kind == 0)
+      return launch_packed<2, 4, 4, 2, 2, true, kRing, 2>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream,
+                                                          residual, seg);
+    if (plan.groups == 2 && plan.kind == 1)
+      return launch_packed<4, 4, 4, 2, 2, true, kRing, 2>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream,
+                                                          residual, seg);
+  }
   if (plan.kind == 0)
     return launch_packed<2, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg,
                                             plan.split, workspace);

@@ -316,10 +316,12 @@ int fpq_gemm_mxf4_packed_splitk(const void* xq_packed, const void* xs_packed, co
 /* The same for packed NVFP4 operands (fpq_gemm_nvf4_packed, with `residual` non-null fpq_gemm_nvf4_packed_residual);
  * workspace as above, sized by fpq_gemm_nvf4_packed_workspace_bytes(M, N, K).  Up to 128 rows the split is
  * that of the MXFP4 entry; 129-256 rows on few weight rows run as two passes over at most 128 rows each, and
- * each pass may use the workspace; from 257 rows on the tile kernels split K the same way (fp32 parts of
- * their workgroup tiles, a counter per tile, parts added in part order) where few tiles and a long K would
- * leave CUs idle -- the NVFP4 loop is bound by its in-register dequantization, so more workgroups pay there
- * although the parts are as many bytes as the operands (MXFP4 measured slower with it and never does). */
+ * each pass may use the workspace.  Beyond, where the tile kernels have at most one workgroup tile per CU, a
+ * K with an even number of 256-blocks is halved INSIDE the workgroups (eight waves, the halves meet in LDS:
+ * no workspace, the size function returns 0); with an odd number and a long K the tile kernels split K across
+ * workgroups the way the weight-streaming kernel does (fp32 parts of their workgroup tiles, a counter per tile,
+ * parts added in part order) -- the NVFP4 loop is bound by its in-register dequantization, so more waves pay
+ * there (MXFP4 measured slower with either and never does). */
 int64_t fpq_gemm_nvf4_packed_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int fpq_gemm_nvf4_packed_splitk(const void* xq_packed, const void* xs_packed, const void* wq_packed,
                                 const void* ws_packed, const float* alpha, const void* bias,

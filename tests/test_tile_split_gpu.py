@@ -1,9 +1,11 @@
-"""K split inside the tile kernels (fpq_gemm_nvf4_packed_splitk beyond 256 rows): a few hundred rows on few
-weight rows and a long K -- a down-projection at prefill-chunk sizes -- run the 64 x 128 or 128 x 128 tile
-kernel with K cut across workgroups; fp32 parts of the workgroup tiles meet in the caller's workspace and the
-workgroup that arrives last adds them in part order.  Checked: the oracle's values (bias and residual
-included), the same bits on every repetition, counters left at zero, a smaller workspace only means fewer
-parts, and the layer takes the same kernel eagerly, through the traced operator and under a graph capture.
+"""K split inside the NVFP4 tile kernels (a few hundred rows on few weight rows: at most one 64 x 128 or
+128 x 128 workgroup tile per CU).  With an even number of 256-K blocks the workgroup has eight waves in two
+groups, each multiplying one half of K, and the halves meet in LDS (no workspace).  With an odd number and a
+long K (fpq_gemm_nvf4_packed_splitk beyond 256 rows) K is cut across workgroups: fp32 parts of the workgroup
+tiles meet in the caller's workspace and the workgroup that arrives last adds them in part order.  Checked: the
+oracle's values (bias and residual included), the same bits on every repetition, counters left at zero, a
+smaller workspace only means fewer parts, and the layer takes the same kernel eagerly, through the traced
+operator and under a graph capture.
 Reference contract: matmul_nvf4_bf16_tn_op (inference_lib/src/fp_quant/module/qutlass_ops.py:149-168)."""
 import pytest
 import torch
@@ -30,9 +32,14 @@ def _operands(m, n, k, seed):
     return xq, xs, wq, ws, bias, res, g
 
 
-# (rows, N, K): 64 x 128 tiles in two and three parts, 128 x 128 tiles, ragged edges in both directions
-SHAPES = [(300, 1024, 8192), (512, 4096, 12288), (384, 2048, 14336), (257, 200, 8192), (700, 520, 8448),
-          (1000, 1024, 8192)]
+# (rows, N, K), an odd number of 256-K blocks: 64 x 128 tiles in two and three parts, 128 x 128 tiles, ragged
+# edges in both directions
+SHAPES = [(300, 1024, 8448), (512, 4096, 12544), (384, 2048, 14592), (257, 200, 8448), (700, 520, 8448),
+          (1000, 1024, 8448)]
+# an even number of blocks: two groups of four waves per workgroup -- 64 x 128 and 128 x 128 tiles, one block per
+# group up to 28, ragged edges, 129-256 rows on many weight rows
+GROUP_SHAPES = [(512, 4096, 12288), (300, 4100, 8192), (1000, 1100, 2560), (384, 4096, 14336), (640, 4096, 4096),
+                (200, 12288, 2048), (129, 16384, 2560), (513, 8190, 3072)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
@@ -69,11 +76,44 @@ def test_tile_kernel_split_matches_the_oracle(m, n, k):
     assert ((fewer[ri][:, ci].double() - want.double()).abs() <= tol).all() and not small[:16384].any()
 
 
+@pytest.mark.parametrize("m,n,k", GROUP_SHAPES)
+def test_two_groups_per_workgroup_match_the_oracle(m, n, k):
+    lib = _engine.lib()
+    xq, xs, wq, ws, bias, res, g = _operands(m, n, k, m + n + k)
+    xp, xsp = pack_nv_by_definition(xq, xs, k)
+    wp, wsp = pack_nv_by_definition(wq, ws, k)
+    y = capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, ALPHA, bias=bias, residual=res)
+    ri = torch.cat([torch.tensor([0, 127, 128, m - 1]), torch.randperm(m, generator=g)[:40]]).unique()
+    ci = torch.cat([torch.tensor([0, 63, 64, 127, 128, n - 1]), torch.randperm(n, generator=g)[:160]]).unique()
+    ref, mag = O.gemm_ref(xq[ri], xs[ri], wq[ci], ws[ci], ALPHA, "nvfp4")
+    want = (ref.to(torch.bfloat16) + bias[ci]) + res[ri][:, ci]
+    got = y[ri][:, ci]
+    tol = 2.0 ** -7 * torch.maximum(want.double().abs(), ref.abs()) + 2.0 ** -7 * res[ri][:, ci].double().abs() + 1e-5 * mag + 1e-6
+    assert ((got.double() - want.double()).abs() <= tol).all()
+    assert (got.view(torch.int16) == want.view(torch.int16)).double().mean() > 0.95
+    for _ in range(3):   # the halves are added in a fixed order
+        again = capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, ALPHA, bias=bias, residual=res)
+        assert torch.equal(again.view(torch.int16), y.view(torch.int16))
+    # a workspace changes nothing: these shapes need none
+    if m > 256:
+        assert int(lib.fpq_gemm_nvf4_packed_workspace_bytes(m, n, k)) == 0
+    workspace = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    same = capi.gemm_packed_splitk(xp, xsp, wp, wsp, m, n, k, ALPHA, bias=bias, residual=res, workspace=workspace, nv=True)
+    if m > 256:
+        assert torch.equal(same.view(torch.int16), y.view(torch.int16)) and not workspace.any()
+    # without bias and residual as well
+    plain = capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, ALPHA)
+    want0 = ref.to(torch.bfloat16)
+    assert ((plain[ri][:, ci].double() - ref).abs() <= 2.0 ** -8 * ref.abs() + 1e-5 * mag + 1e-6).all()
+    assert (plain[ri][:, ci] == want0).double().mean() > 0.97
+
+
 def test_workspace_size_function():
     lib = _engine.lib()
     size = lib.fpq_gemm_nvf4_packed_workspace_bytes
-    assert size(512, 4096, 12288) == 16384 + 2 * 256 * 32768       # 4 x 64 tiles of 64 x 128, K in two parts
-    assert size(512, 4096, 4096) == 0                              # K too short to cut
+    assert size(512, 4096, 12544) == 16384 + 2 * 256 * 32768       # 4 x 64 tiles of 64 x 128, 49 blocks of K in two parts
+    assert size(512, 4096, 12288) == 0                             # 48 blocks: halved inside the workgroups
+    assert size(512, 4096, 4096) == 0                              # K too short to cut across workgroups
     assert size(4096, 4096, 12288) == 0                            # enough tiles without
     assert size(64, 4096, 12288) == lib.fpq_gemm_mxf4_packed_workspace_bytes(64, 4096, 12288) > 0
     assert size(200, 4096, 12288) == lib.fpq_gemm_mxf4_packed_workspace_bytes(128, 4096, 12288)   # two passes of 128 / 72 rows
@@ -87,7 +127,7 @@ def test_layer_takes_the_split_on_every_call_path():
     bits, which are those of the C entry point with a workspace of its own."""
     import fp_quant
     from fp_quant.module import eager
-    k, n, m = 8192, 512, 300
+    k, n, m = 8448, 512, 300
     cfg = fp_quant.FPQuantConfig(forward_dtype=fp_quant.FPQuantDtype.NVFP4, forward_method="abs_max",
                                  backward_dtype=fp_quant.FPQuantDtype.BF16, hadamard_group_size=16)
     torch.manual_seed(3)
