@@ -37,6 +37,11 @@ constexpr int kStreamCounters = 4096;                        // one per weight t
 constexpr int64_t kStreamCounterBytes = kStreamCounters * 4;  // they open the workspace
 constexpr int kStreamMaxRows = 128;
 
+// Dynamic LDS of a workgroup with more than four output tiles (0: the kernel's own arrays hold them)
+constexpr int stream_dynamic_lds(int nt, int mt) {
+  return nt * mt > 4 ? 4 * nt * mt * 3 * 64 * 16 + nt * mt * 32 * 20 * 4 : 0;
+}
+
 // NT weight row tiles per workgroup, MT activation row tiles (exactly ceil(M / 32)), DB 256-K blocks
 // of loads in flight per wave, NW waves.  Every workgroup re-reads all activations (NT = 2 halves
 // that, at a register cost that stream_plan explains).  Two weight tiles per workgroup are compiled for
@@ -45,7 +50,7 @@ constexpr int kStreamMaxRows = 128;
 // of a 64-K unit, times its group's scale, is its fp16 operand of the s-th 32x32x16 matrix instruction
 // of the unit on both sides, so the K order is permuted consistently and the sum is complete.
 template <int NT, int MT, int DB, int NW, bool NV = false>
-__global__ __launch_bounds__(64 * NW, NT == 2 ? 2 : 1) void gemm_fp4_stream_kernel(
+__global__ __launch_bounds__(64 * NW, NT == 2 && NT * MT <= 4 ? 2 : 1) void gemm_fp4_stream_kernel(
     const uint8_t* __restrict__ xq_all, const uint8_t* __restrict__ xs_all, const uint8_t* __restrict__ wq,
     const uint8_t* __restrict__ ws, const float* __restrict__ alpha_p, const uint16_t* __restrict__ bias,
     const uint16_t* residual_all, uint16_t* y, int M_all, int N, int K, int bps, int ksplit,
@@ -59,10 +64,19 @@ __global__ __launch_bounds__(64 * NW, NT == 2 ? 2 : 1) void gemm_fp4_stream_kern
   const uint8_t* xs = xs_all + (size_t)slab * MT * (K >> 8) * (NV ? 512 : 256);
   const uint16_t* residual = residual_all ? residual_all + (size_t)m0 * N : nullptr;
   const int tile_id = slab * gridDim.x + blockIdx.x;   // numbers the output tile groups for the K split
-  __shared__ v4f part[4][NT * MT][3][64];   // [owning wave][tile][the other waves in order][lane]
   constexpr int kStageRow = 20;             // dwords: 16 of a row's 32 bf16 + 4, rows stay 16-byte aligned
   constexpr int kStageTile = 32 * kStageRow;
-  __shared__ __attribute__((aligned(16))) uint32_t stage[NT * MT][kStageTile];
+  // part: [owning wave][tile][the other waves in order][lane]; stage: the rounded tiles on their way out.  More
+  // than four tiles per workgroup need more than the 64 KB a kernel may declare: those take them from the
+  // launch's dynamic LDS.
+  typedef v4f PartOf[NT * MT][3][64];
+  typedef uint32_t StageOf[kStageTile];
+  constexpr bool kDynLds = stream_dynamic_lds(NT, MT) > 0;
+  __shared__ v4f part_fixed[kDynLds ? 1 : 4][kDynLds ? 1 : NT * MT][3][64];
+  __shared__ __attribute__((aligned(16))) uint32_t stage_fixed[kDynLds ? 1 : NT * MT][kStageTile];
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds_dynamic[];
+  PartOf* const part = kDynLds ? (PartOf*)lds_dynamic : (PartOf*)part_fixed;
+  StageOf* const stage = kDynLds ? (StageOf*)(lds_dynamic + 4 * sizeof(PartOf)) : (StageOf*)stage_fixed;
   __shared__ unsigned arrival;
   constexpr int kSB = NV ? 512 : 256;    // scale bytes per row tile and 256-K block
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -415,6 +429,10 @@ static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace
   if (rt_m == 4 && tiles > (nv ? 2 * cus : cus)) return plan;
   plan.use = true;
   if (rt_m == 2 && tiles >= (nv ? 3 * cus / 2 : 3 * cus)) plan.nt = 2;
+  // NVFP4, 33-64 rows, between two and three weight tiles per CU: three per workgroup, one workgroup per CU in
+  // a single round instead of a round and a half of pairs (N = 24576: K = 4096 22.2 -> 21.2 us, K = 12288 56.0 ->
+  // 48.0; N = 20480 21.0 -> 19.7; four tiles per workgroup for the next range measured 4 % slower than pairs)
+  if (nv && rt_m == 2 && tiles > 2 * cus && tiles <= 3 * cus) plan.nt = 3;
   const int64_t groups = (tiles + plan.nt - 1) / plan.nt;
   int64_t ksplit = 1;
   if (workspace_bytes > kStreamCounterBytes && groups <= kStreamCounters) {
@@ -460,6 +478,22 @@ static int launch_stream(const void* xq, const void* xs, const void* wq, const v
                      (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, (int)M, (int)N,    \
                      (int)K, plan.bps, plan.ksplit, partial, counters, seg)
   const int mt = (int)((rows + 31) / 32);
+#define FPQ_STREAM_BIG(NTT, MTT, DBB)                                                                   \
+  {                                                                                                     \
+    constexpr int kLds = stream_dynamic_lds(NTT, MTT);                                                  \
+    static LdsLimitOnce lds_limit;                                                                      \
+    if (const int st = lds_limit.ensure((const void*)gemm_fp4_stream_kernel<NTT, MTT, DBB, 4, NV>, kLds)) return st; \
+    hipLaunchKernelGGL((gemm_fp4_stream_kernel<NTT, MTT, DBB, 4, NV>), grid, dim3(256), kLds, stream,   \
+                       (const uint8_t*)xq, (const uint8_t*)xs, (const uint8_t*)wq, (const uint8_t*)ws, alpha, \
+                       (const uint16_t*)bias, (const uint16_t*)residual, (uint16_t*)y, (int)M, (int)N,  \
+                       (int)K, plan.bps, plan.ksplit, partial, counters, seg);                          \
+    return (int)hipGetLastError();                                                                      \
+  }
+  if constexpr (NV) {
+    if (plan.nt == 3 && mt == 2) FPQ_STREAM_BIG(3, 2, 1)
+  }
+#undef FPQ_STREAM_BIG
+  if (plan.nt > 2) return FPQ_E_UNSUPPORTED;
   if (plan.nt == 2) {   // 33-64 rows only
     if (mt != 2) return FPQ_E_UNSUPPORTED;
     FPQ_STREAM(2, 2, 1);

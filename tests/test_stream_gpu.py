@@ -139,6 +139,32 @@ def test_nvfp4_split_k_matches_oracle_and_is_deterministic(m, n, k):
     assert torch.equal(y0, capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha))
 
 
+@pytest.mark.parametrize("m,n,k", [(64, 24576, 512), (40, 17000, 768), (33, 20480, 256), (64, 16416, 1280)])
+def test_nvfp4_three_weight_tiles_per_workgroup(m, n, k):
+    """NVFP4 at 33-64 rows with 513-768 weight tiles (a whole number of groups of three, a ragged N whose last
+    group holds one tile, one block of K so that three of the four waves have nothing to multiply): rows sampled
+    against the oracle, bias and residual as separate bf16 additions, the same bits on a second call."""
+    from test_packed_gpu import pack_nv_by_definition
+    g = torch.Generator().manual_seed(m + n + k)
+    xq = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=g)
+    wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=g)
+    xs = torch.randint(0x20, 0x50, (m, k // 16), dtype=torch.uint8, generator=g)
+    ws = torch.randint(0x20, 0x50, (n, k // 16), dtype=torch.uint8, generator=g)
+    alpha = 2.0 ** -6
+    xp, xsp = pack_nv_by_definition(xq, xs, k)
+    wp, wsp = pack_nv_by_definition(wq, ws, k)
+    y = capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha)
+    assert not torch.isnan(y.float()).any()
+    ci = torch.cat([torch.tensor([0, 31, 32, 95, 96, n - 97, n - 33, n - 1]), torch.randperm(n, generator=g)[:600]]).unique()
+    ref, mag = O.gemm_ref(xq, xs, wq[ci], ws[ci], alpha, "nvfp4")
+    assert ((y[:, ci].double() - ref).abs() <= 2.0 ** -8 * ref.abs() + 1e-5 * mag + 1e-6).all()
+    assert (y[:, ci] == ref.to(torch.bfloat16)).float().mean() > 0.98
+    assert torch.equal(capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha).view(torch.int16), y.view(torch.int16))
+    b = torch.randn(n, generator=g).to(torch.bfloat16)
+    res = (torch.randn(m, n, generator=g) * 8).to(torch.bfloat16)
+    assert torch.equal(capi.gemm_nv_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=b, residual=res), (y + b) + res)
+
+
 def test_split_k_is_taken_for_few_weight_rows_and_long_k():
     need = _engine.lib().fpq_gemm_mxf4_packed_workspace_bytes
     assert need(16, 4096, 14336) == 16384 + 2 * 128 * 4096   # 128 weight tiles, 56 blocks: two parts
