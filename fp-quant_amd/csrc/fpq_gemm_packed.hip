@@ -561,7 +561,7 @@ __global__ __launch_bounds__(256 * GR, (NT * MT <= 32 && GR == 1 ? 2 : 1)) void 
 // (measured on the 256 CUs of an MI355X, where they come to the figures in the comments):
 //   row slabs of the streaming kernel x weight tiles: at most one workgroup per CU (256)
 //   up to CUs / 2 tiles of 128 x 128 (128): 64 x 128 tiles instead
-//   fewer than 25/64 CUs tiles of 256 x 256 (100; under about 200 of 256 x 128): 128 x 128 tiles
+//   MXFP4: up to CUs tiles of 128 x 128 (256), NVFP4: fewer than 25/64 CUs tiles of 256 x 256 (100): 128 x 128 tiles
 static inline int64_t slab_workgroups(int cus) { return cus; }
 static inline int64_t narrow_below(int cus) { return cus / 2; }
 static inline int64_t small_below(int cus) { return (int64_t)cus * 25 / 64; }
@@ -640,7 +640,11 @@ static TilePlan tile_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_byt
     plan.kind = 0;
     plan.tiles = ((M + 127) / 128) * ((N + 63) / 64);
     plan.part_bytes = 4 * 64 * 32 * 4;     // four waves of 32 x 64: two accumulator tiles per lane
-  } else if (big_tiles < small_below(cus)) {
+  } else if (NV ? big_tiles < small_below(cus) : ((M + 127) / 128) * ((N + 127) / 128) <= cus) {
+    // MXFP4: 128 x 128 tiles while every workgroup has a CU to itself -- two of them on a CU wait on its LDS, and
+    // with the weights from HBM the 256 x 128 tiles are faster from there on (us, K = 4096: 256 rows, N = 20480 /
+    // 24576 23.0 / 23.9 -> 20.3 / 21.2; 512 rows, N = 12288 22.0 -> 20.0; 768 rows, N = 8192 21.4 -> 19.0; 1024 rows,
+    // N = 6144 21.1 -> 19.4; at exactly one tile per CU the small tiles win: 1024 rows, N = 4096 13.6 against 18.6)
     plan.kind = 1;
     plan.tiles = ((M + 127) / 128) * ((N + 127) / 128);
     plan.part_bytes = 4 * 64 * 64 * 4;     // four waves of 64 x 64
