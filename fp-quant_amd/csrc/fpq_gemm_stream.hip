@@ -404,8 +404,9 @@ struct StreamPlan {
 // Which shapes run here and how (all thresholds are measured break-even points on Llama-3-8B and
 // Qwen3-8B layer shapes).  Up to 64 activation rows: always, one weight tile per workgroup.  More
 // rows: up to a number of weight tiles beyond which the 128x128 tile kernel, which shares activations
-// through LDS, is faster -- 65-96 rows: 1024 tiles for MXFP4 (N = 14336: 11.9 against 13.5 us, N =
-// 28672: 20.5 against 22.3, N = 57344: 36.3 against 27.7), any number for NVFP4 (N = 14336: 22.1
+// through LDS, is faster -- 65-96 rows: 512 tiles for MXFP4, one round of this kernel's workgroups (with the
+// weights from HBM, this kernel against the tiles: N = 14336 12.0 / 12.3 us, N = 16384 12.5 / 12.5, N = 18432
+// 15.6 / 14.3, N = 24576 17.1 / 15.3, N = 28672 20.7 / 16.5, N = 32768 21.9 / 18.0), any number for NVFP4 (N = 14336: 22.1
 // against 35.9 us, N = 128256: 165 against 215); 97-128 rows (276-346 registers, one workgroup per
 // CU): one round of the 256 CUs for MXFP4, two for NVFP4 (N = 16384: 28.1 against 35.1 us, N = 20480:
 // 39.9 against 35.2).  (Two weight tiles per workgroup halve what the L2 has to
@@ -425,7 +426,7 @@ static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace
   const int64_t rt_m = (M + 31) / 32, tiles = (N + 31) / 32, nkb = K / 256;
   // (weight-tile counts in units of the device's compute units: 256 on the part the figures above were measured on)
   const int64_t cus = device_cus();
-  if (rt_m == 3 && !nv && tiles > 4 * cus) return plan;
+  if (rt_m == 3 && !nv && tiles > 2 * cus) return plan;
   if (rt_m == 4 && tiles > (nv ? 2 * cus : cus)) return plan;
   plan.use = true;
   if (rt_m == 2 && tiles >= (nv ? 3 * cus / 2 : 3 * cus)) plan.nt = 2;

@@ -49,7 +49,7 @@ def _workspace(m, n, k, cap=None):
     return need, torch.zeros(max(size, 256), dtype=torch.uint8, device="cuda")
 
 
-# one to four activation row tiles (65-96 rows with at most 1024 weight tiles, 97-128 rows with at most 256;
+# one to four activation row tiles (65-96 rows with at most 512 weight tiles, 97-128 rows with at most 256;
 # the shapes just beyond run the tile kernels and meet the same oracle), odd tile counts, ragged rows and
 # columns, one to 56 blocks of K
 SHAPES = [(1, 32, 256), (1, 100, 512), (5, 257, 768), (16, 1024, 1024), (31, 64, 1280), (32, 4096, 4096),
@@ -58,7 +58,7 @@ SHAPES = [(1, 32, 256), (1, 100, 512), (5, 257, 768), (16, 1024, 1024), (31, 64,
           # 768 weight tiles or more at 33-64 rows: two weight tiles per workgroup (an odd tile count, a ragged N)
           (64, 24600, 512), (45, 28672, 256), (33, 24577, 256),
           # three activation row tiles with more than 256 weight tiles, up to the limit and past it
-          (96, 8290, 512), (70, 14336, 256), (96, 32768, 256), (65, 32800, 256), (128, 8192, 256), (128, 8224, 256)]
+          (96, 8290, 512), (70, 14336, 256), (96, 16384, 256), (65, 16416, 256), (96, 32768, 256), (128, 8192, 256), (128, 8224, 256)]
 # shapes whose K is split when a workspace is given (few weight tiles, K of 8192 or more), one to four
 # activation row tiles
 SPLIT_SHAPES = [(1, 32, 8192), (5, 257, 12288), (16, 1024, 8192), (31, 64, 16384), (32, 4096, 8192),
