@@ -408,8 +408,8 @@ struct StreamPlan {
 // weights from HBM, this kernel against the tiles: N = 14336 12.0 / 12.3 us, N = 16384 12.5 / 12.5, N = 18432
 // 15.6 / 14.3, N = 24576 17.1 / 15.3, N = 28672 20.7 / 16.5, N = 32768 21.9 / 18.0), any number for NVFP4 (N = 14336: 22.1
 // against 35.9 us, N = 128256: 165 against 215); 97-128 rows (276-346 registers, one workgroup per
-// CU): one round of the 256 CUs for MXFP4, two for NVFP4 (N = 16384: 28.1 against 35.1 us, N = 20480:
-// 39.9 against 35.2).  (Two weight tiles per workgroup halve what the L2 has to
+// CU): one round of the 256 CUs for both formats (NVFP4 took two until its tile kernels ran eight waves per
+// workgroup: N = 8192 15.0 against 22.9 us for the tiles, N = 10240 26.7 against 22.7, N = 16384 27.7 against 23.9).  (Two weight tiles per workgroup halve what the L2 has to
 // deliver for 33-64 rows, but need so many registers that one workgroup fills a CU; one tile per
 // workgroup with two blocks in flight, two workgroups per CU, measured 5-13 % faster -- except from
 // 768 weight tiles on, where two tiles per workgroup with ONE block in flight, held to 256 registers,
@@ -427,7 +427,7 @@ static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace
   // (weight-tile counts in units of the device's compute units: 256 on the part the figures above were measured on)
   const int64_t cus = device_cus();
   if (rt_m == 3 && !nv && tiles > 2 * cus) return plan;
-  if (rt_m == 4 && tiles > (nv ? 2 * cus : cus)) return plan;
+  if (rt_m == 4 && tiles > cus) return plan;
   plan.use = true;
   if (rt_m == 2 && tiles >= (nv ? 3 * cus / 2 : 3 * cus)) plan.nt = 2;
   // NVFP4, 33-64 rows, between two and three weight tiles per CU: three per workgroup, one workgroup per CU in
