@@ -760,9 +760,14 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
     // kernel over one half of the rows each are faster although the second re-reads the weights (from the
     // last-level cache): N = 6144, K = 4096: 192 rows 35.2 -> 23.1 us, 256 rows 34.8 -> 28.6; N = 4096, K =
     // 12288: 97 -> 52 / 68 us.  (The tile kernel's time stays at one round up to N = 16384, where two passes
-    // take 44-55 us; three passes for more rows measured slower than the tiles as well.)
+    // take 44-55 us; three passes for more rows measured slower than the tiles as well.)  Where the tile
+    // kernels halve K inside their workgroups they take 23 us for K = 4096 at any of these row counts and the
+    // two passes are ahead up to 192 rows only (weights from HBM; N = 6144: 144 rows 22.5 two passes / 25.8 us
+    // tiles, 192 rows 23.7 / 23.6, 224 rows 26.7 / 23.5, 256 rows 28.7 / 22.9; N = 8192, K = 8192: 35.7 / 43.4,
+    // 39.5 / 42.6, 45.5 / 43.1, 49.7 / 42.8).
     const int64_t half = ((M + 1) / 2 + 31) / 32 * 32;   // rows of the first pass, whole 32-row tiles
-    if (!tile_splits && M > FPQ_NV_STREAM_ROWS && M <= 2 * FPQ_NV_STREAM_ROWS && (N + 31) / 32 <= cus &&
+    const int64_t two_pass_rows = plan.groups == 2 ? 192 : 2 * FPQ_NV_STREAM_ROWS;
+    if (!tile_splits && M > FPQ_NV_STREAM_ROWS && M <= two_pass_rows && (N + 31) / 32 <= cus &&
         stream_eligible(true, half, N, K)) {
       // (both passes may split K through the caller's workspace: they run one after the other on the stream)
       const int rc = gemm_fp4_stream(true, xq, xs, wq, ws, alpha, bias, residual, y, half, N, K, workspace,
