@@ -126,8 +126,11 @@ constexpr int kRing = 8;                 // 64-K units resident or in flight
 // slot a block lands in was last read several hand-overs (barriers) earlier: 2 slots would do.
 constexpr int kScaleSlots = 4;
 constexpr int scale_block_bytes(bool nv) { return nv ? 512 : 256; }
+// (one kilobyte piece per load instruction, the same number of loads for each of the four waves: with six
+// pieces -- NVFP4, 256 x 128 tiles -- two each, the last two kilobytes copies that are never read)
+constexpr int scale_loads_per_wave(int blocks, bool nv) { return (blocks * scale_block_bytes(nv) / 1024 + 3) / 4; }
 constexpr int scale_slot_bytes(int blocks, bool nv) {
-  return (blocks * scale_block_bytes(nv) > 4096 ? blocks * scale_block_bytes(nv) : 4096);
+  return (scale_loads_per_wave(blocks, nv) > 1 ? scale_loads_per_wave(blocks, nv) : 1) * 4096;
 }
 constexpr int scale_slots(bool nv, int groups = 1) { return nv || groups > 1 ? 2 : kScaleSlots; }
 // LDS of a group of four waves whose unit holds `blocks` operand kilobytes (weight + activation row tiles)
@@ -137,9 +140,10 @@ constexpr int packed_lds_bytes(int blocks, bool nv = false, int ring = kRing, in
 // ... and what is allocated: at least the epilogue's staging area (four waves, each WT_M rows of
 // WT_N bf16 + 16 bytes)
 constexpr int packed_lds_alloc(int blocks, bool nv, int ring, int wt_n, int wt_m, int groups = 1) {
-  return groups * packed_lds_bytes(blocks, nv, ring, groups) > 4 * wt_m * (wt_n * 2 + 16)
-             ? groups * packed_lds_bytes(blocks, nv, ring, groups)
-             : 4 * wt_m * (wt_n * 2 + 16);
+  const int rings = groups * packed_lds_bytes(blocks, nv, ring, groups), staging = 4 * wt_m * (wt_n * 2 + 16);
+  const int exchange = groups > 1 ? 4 * (wt_n / 32) * (wt_m / 32) * 4096 : 0;   // four waves' accumulators
+  const int most = rings > staging ? rings : staging;
+  return most > exchange ? most : exchange;
 }
 
 template <int N>
@@ -165,7 +169,8 @@ __device__ __forceinline__ void barrier_lds_but() {
 //                    the other keeps the matrix pipes busy, which is worth more than the 1.5x
 //                    operand traffic costs (62.4 us against 66.1 us at M = 2048, N = 14336)
 //   <8, 8, 8, 2, 2>  256 x 256 tile, waves 128 x 128, one workgroup per CU: large M, NVFP4 (whose
-//                    limit is the register dequantization; half tiles measured mixed there)
+//                    limit is the register dequantization), where whole rounds of them cost less than
+//                    the 256 x 128 tiles' finer rounds (tile_plan)
 //   <2, 4, 4, 2, 2>  64 x 128 tile (weight rows x activation rows), waves 32 x 64: when even the 128 x 128
 //                    tiles would fill at most half of the CUs
 //   <4, 4, 4, 2, 2>  128 x 128 tile, waves 64 x 64, 80 KB of LDS: two workgroups per CU; used when
@@ -203,7 +208,7 @@ __global__ __launch_bounds__(256 * GR, (NT * MT <= 32 && GR == 1 ? 2 : 1)) void 
   constexpr int kSB = scale_block_bytes(NV);            // scale bytes per row tile and 256-K block
   constexpr int kRpp = 1024 / kSB;                      // row tiles per 1 KB scale piece
   constexpr int kPieces = kBlocks / kRpp;               // scale pieces per 256-K block
-  constexpr int kScLoads = kPieces >= NW ? kPieces / NW : 1;  // scale loads per wave per block
+  constexpr int kScLoads = kPieces >= NW ? (kPieces + NW - 1) / NW : 1;  // scale loads per wave per block
   constexpr int kSlots = scale_slots(NV, GR), kSlotBytes = scale_slot_bytes(kBlocks, NV);
   constexpr int kUnitBytes = kBlocks * 1024;
   static_assert(RING == 4 || RING == 8, "the ring holds one or two 256-K blocks");
@@ -561,10 +566,9 @@ __global__ __launch_bounds__(256 * GR, (NT * MT <= 32 && GR == 1 ? 2 : 1)) void 
 // (measured on the 256 CUs of an MI355X, where they come to the figures in the comments):
 //   row slabs of the streaming kernel x weight tiles: at most one workgroup per CU (256)
 //   up to CUs / 2 tiles of 128 x 128 (128): 64 x 128 tiles instead
-//   MXFP4: up to CUs tiles of 128 x 128 (256), NVFP4: fewer than 25/64 CUs tiles of 256 x 256 (100): 128 x 128 tiles
+//   up to CUs tiles of 128 x 128 (256): those; beyond, tiles of 256 x 128 or (NVFP4, by round counts) 256 x 256
 static inline int64_t slab_workgroups(int cus) { return cus; }
 static inline int64_t narrow_below(int cus) { return cus / 2; }
-static inline int64_t small_below(int cus) { return (int64_t)cus * 25 / 64; }
 
 namespace fpq {
 // A K split of a tile kernel (ksplit > 1): `workspace` = kStreamCounterBytes of counters, all zero, then
@@ -636,20 +640,35 @@ static TilePlan tile_plan(int64_t M, int64_t N, int64_t K, int64_t workspace_byt
   TilePlan plan{};
   plan.groups = 1;
   const int64_t big_tiles = ((M + 255) / 256) * ((N + 255) / 256);
+  const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+  const bool ragged = ((M + 127) / 128) % 2 == 1;   // the last 256 activation rows of the large tiles would be half empty
   if (((M + 127) / 128) * ((N + 127) / 128) <= narrow_below(cus)) {
     plan.kind = 0;
     plan.tiles = ((M + 127) / 128) * ((N + 63) / 64);
     plan.part_bytes = 4 * 64 * 32 * 4;     // four waves of 32 x 64: two accumulator tiles per lane
-  } else if (NV ? big_tiles < small_below(cus) : ((M + 127) / 128) * ((N + 127) / 128) <= cus) {
+  } else if (tiles128 <= cus) {
     // MXFP4: 128 x 128 tiles while every workgroup has a CU to itself -- two of them on a CU wait on its LDS, and
     // with the weights from HBM the 256 x 128 tiles are faster from there on (us, K = 4096: 256 rows, N = 20480 /
     // 24576 23.0 / 23.9 -> 20.3 / 21.2; 512 rows, N = 12288 22.0 -> 20.0; 768 rows, N = 8192 21.4 -> 19.0; 1024 rows,
-    // N = 6144 21.1 -> 19.4; at exactly one tile per CU the small tiles win: 1024 rows, N = 4096 13.6 against 18.6)
+    // N = 6144 21.1 -> 19.4; at exactly one tile per CU the small tiles win: 1024 rows, N = 4096 13.6 against 18.6).
+    // NVFP4 likewise (the small tiles ran up to 400 of them before): K = 4096, 512 rows, N = 12288 60.3 -> 56.2 us;
+    // 768 rows, N = 8192 59.9 -> 54.9; 256 rows, N = 24576 61.1 -> 55.9; K = 12288, 512 rows, N = 12288 170 -> 153.
     plan.kind = 1;
     plan.tiles = ((M + 127) / 128) * ((N + 127) / 128);
     plan.part_bytes = 4 * 64 * 64 * 4;     // four waves of 64 x 64
   } else {
-    plan.kind = (!NV || FPQ_PACKED_HALF_TILES > 1) && FPQ_PACKED_HALF_TILES ? 2 : 3;
+    // MXFP4: 256 x 128 tiles.  NVFP4: 256 x 256 tiles (one workgroup per CU) do a given amount of work 4 % faster,
+    // 256 x 128 tiles (two per CU; alone on a CU one takes 0.54 of a large tile's time) waste less of the last
+    // round and of a row count that is an odd number of 128s -- whichever the round counts favour (K = 4096:
+    // 4096 rows, N = 6144 197 -> 164 us; 128 rows, N = 28672 97 -> 41, now 128 x 128 tiles; 384 rows, N = 14336
+    // 96 -> 54; 896 rows, N = 8192 98 -> 57; 4096 rows, N = 24576 633 / 625 and K = 12288, N = 4096 302 / 314
+    // stay with the large tiles).
+    const int64_t half_tiles = ((M + 127) / 128) * ((N + 255) / 256);
+    const int64_t rounds = half_tiles / (2 * cus), rest = half_tiles % (2 * cus);
+    const int64_t cost_half = rounds * 104 + (rest == 0 ? 0 : rest <= cus ? 54 : 104);
+    const int64_t cost_large = (big_tiles + cus - 1) / cus * 100;
+    const bool half = !NV || FPQ_PACKED_HALF_TILES > 1 || cost_half + (ragged ? 0 : 4) <= cost_large;
+    plan.kind = half && FPQ_PACKED_HALF_TILES ? 2 : 3;
     plan.split = TileSplit{1, (int)(K / 256)};
     return plan;
   }

@@ -191,6 +191,70 @@ __global__ __launch_bounds__(64 * NW, NT == 2 && NT * MT <= 4 ? 2 : 1) void gemm
     FPQ_STREAM_STEP(3)
 #undef FPQ_STREAM_STEP
   };
+  // NVFP4 with three activation row tiles: the 16 K steps of a block (one 32x32x16 matrix instruction per output
+  // tile each) as a software pipeline -- while the matrix instructions of step t issue, the operands of step
+  // t + 1 are converted, and the instruction order is pinned to one matrix instruction followed by its share of
+  // the conversions.  Only a step's operands are held as fp16 (32 registers, not the 48 of a whole unit's
+  // activations), which brings the kernel under 256 registers: two workgroups per CU, whose waves fill each
+  // other's gaps (a wave alone on its SIMD issues a conversion every 8 cycles, measured).  96 rows, K = 4096,
+  // weights from HBM: N = 14336 22.5 -> 20.5 us, N = 24576 33.7 -> 28.9, N = 28672 44.7 -> 36.0.  One, two and
+  // four row tiles measured the same or up to 5 % slower this way and keep the unit-by-unit order above.
+  constexpr bool kPipelined = NV && MT == 3;
+  auto a_op = [&](auto slot, int t, int i) __attribute__((always_inline)) {
+    constexpr int s = decltype(slot)::value;
+    const int U = t >> 2, s4 = t & 3;
+    const uint4 q = a[s][U][i];
+    const uint32_t cd = s4 == 0 ? q.x : s4 == 1 ? q.y : s4 == 2 ? q.z : q.w;
+    const uint32_t sc = (U < 2 ? sa[s][i].x : sa[s][i].y) >> (16 * (U & 1) + 8 * (s4 >> 1));
+    return dequant8_f16_s(cd, e4m3_pair_f16(sc));
+  };
+  auto b_op = [&](auto slot, int t, int j) __attribute__((always_inline)) {
+    constexpr int s = decltype(slot)::value;
+    const int U = t >> 2, s4 = t & 3;
+    const uint4 q = b[s][U][j];
+    const uint32_t cd = s4 == 0 ? q.x : s4 == 1 ? q.y : s4 == 2 ? q.z : q.w;
+    const uint32_t sc = (U < 2 ? sb[s][j].x : sb[s][j].y) >> (16 * (U & 1) + 8 * (s4 >> 1));
+    return dequant8_f16_s(cd, e4m3_pair_f16(sc));
+  };
+  auto compute_block_nv = [&](auto slot) __attribute__((always_inline)) {
+    v8h ah[NT], bh[MT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) ah[i] = a_op(slot, 0, i);
+#pragma unroll
+    for (int j = 0; j < MT; ++j) bh[j] = b_op(slot, 0, j);
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      v8h an[NT], bn[MT];
+      if (t < 15) {
+#pragma unroll
+        for (int i = 0; i < NT; ++i) an[i] = a_op(slot, t + 1, i);
+#pragma unroll
+        for (int j = 0; j < MT; ++j) bn[j] = b_op(slot, t + 1, j);
+      }
+#pragma unroll
+      for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+          acc[i * MT + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[i], bh[j], acc[i * MT + j], 0, 0, 0);
+      constexpr int kValu = ((NT + MT) * 9 + NT * MT - 1) / (NT * MT);   // 8 conversions + the scale's share, per operand
+#pragma unroll
+      for (int m = 0; m < NT * MT; ++m) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (t < 15) {
+#pragma unroll
+        for (int i = 0; i < NT; ++i) ah[i] = an[i];
+#pragma unroll
+        for (int j = 0; j < MT; ++j) bh[j] = bn[j];
+      }
+    }
+  };
+  auto run_block = [&](auto slot) __attribute__((always_inline)) {
+    if constexpr (kPipelined) compute_block_nv(slot);
+    else compute_block(slot);
+  };
   auto for_slots = [&](auto&& f) __attribute__((always_inline)) {
     f(std::integral_constant<int, 0>{});
     if constexpr (DB > 1) f(std::integral_constant<int, 1>{});
@@ -236,20 +300,20 @@ __global__ __launch_bounds__(64 * NW, NT == 2 && NT * MT <= 4 ? 2 : 1) void gemm
   int t0 = 0;
   for (; t0 + 2 * DB <= nblk; t0 += DB) {   // steady state: the block DB ahead exists
     for_slots([&](auto slot) {
-      compute_block(slot);
+      run_block(slot);
       if constexpr (kOrdered) __builtin_amdgcn_sched_barrier(0);
       load_block(slot, t0 + DB + decltype(slot)::value);
       if constexpr (kOrdered) __builtin_amdgcn_sched_barrier(0);
     });
   }
   for_slots([&](auto slot) {                // the ring's last full or partial content
-    if (t0 + decltype(slot)::value < nblk) compute_block(slot);
+    if (t0 + decltype(slot)::value < nblk) run_block(slot);
     if constexpr (kOrdered) __builtin_amdgcn_sched_barrier(0);
   });
   if (nblk - t0 > DB) {                     // up to DB - 1 blocks more
     for_slots([&](auto slot) { load_block(slot, t0 + DB + decltype(slot)::value); });
     for_slots([&](auto slot) {
-      if (t0 + DB + decltype(slot)::value < nblk) compute_block(slot);
+      if (t0 + DB + decltype(slot)::value < nblk) run_block(slot);
     });
   }
 
@@ -432,7 +496,9 @@ static StreamPlan stream_plan(int64_t M, int64_t N, int64_t K, int64_t workspace
   if (rt_m == 2 && tiles >= (nv ? 3 * cus / 2 : 3 * cus)) plan.nt = 2;
   // NVFP4, 33-64 rows, between two and three weight tiles per CU: three per workgroup, one workgroup per CU in
   // a single round instead of a round and a half of pairs (N = 24576: K = 4096 22.2 -> 21.2 us, K = 12288 56.0 ->
-  // 48.0; N = 20480 21.0 -> 19.7; four tiles per workgroup for the next range measured 4 % slower than pairs)
+  // 48.0; N = 20480 21.0 -> 19.7; four tiles per workgroup for the next range measured 4 % slower than pairs).
+  // With one workgroup per CU anyway it keeps two blocks in flight per wave (N = 24576: 20.9 -> 20.1 us, K = 12288
+  // 48.2 -> 45.2; N = 20480 19.8 -> 18.8; three measured 15-20 % slower).
   if (nv && rt_m == 2 && tiles > 2 * cus && tiles <= 3 * cus) plan.nt = 3;
   const int64_t groups = (tiles + plan.nt - 1) / plan.nt;
   int64_t ksplit = 1;
@@ -491,7 +557,7 @@ static int launch_stream(const void* xq, const void* xs, const void* wq, const v
     return (int)hipGetLastError();                                                                      \
   }
   if constexpr (NV) {
-    if (plan.nt == 3 && mt == 2) FPQ_STREAM_BIG(3, 2, 1)
+    if (plan.nt == 3 && mt == 2) FPQ_STREAM_BIG(3, 2, 2)
   }
 #undef FPQ_STREAM_BIG
   if (plan.nt > 2) return FPQ_E_UNSUPPORTED;

@@ -184,7 +184,11 @@ def test_pack_nv_kernel_matches_definition(rows, k):
                                    # more than 128 rows in slabs, and the tile kernels' ragged edges past them
                                    (129, 4096, 512), (260, 100, 256), (1000, 1000, 256), (300, 2790, 512), (300, 8300, 256),
                                    # 33-64 rows at 768 weight tiles or more: two weight tiles per workgroup (odd count, ragged N)
-                                   (64, 24600, 256), (45, 28672, 256)])
+                                   (64, 24600, 256), (45, 28672, 256),
+                                   # more than 256 tiles of 128 x 128: 256 x 128 tiles (six scale pieces per block; an odd
+                                   # and an even number of 128-row tiles, ragged rows and columns), 256 x 256 tiles where
+                                   # they fill whole rounds
+                                   (384, 11010, 256), (300, 11100, 512), (512, 8450, 512), (1024, 16384, 256)])
 @pytest.mark.parametrize("bias", [False, True])
 def test_gemm_nv_packed_matches_oracle(m, n, k, bias):
     g = torch.Generator().manual_seed(m + 2 * n + k)
