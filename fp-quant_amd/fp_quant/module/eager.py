@@ -772,7 +772,7 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
 
 _ROWS_KERNEL_MAX_ROWS = 64   # fpq_rmsnorm_rows_max_rows()
 # NVFP4 layers take the packed GEMM up to mid-sized batches (nv_packed_eligible: fewer than 100 tiles of
-# 256 x 256) and the row-major one beyond; a fused producer does not know its consumers' widths, so it
+# 256 x 256, or a last round that half tiles fill better) and the row-major one beyond; a fused producer does not know its consumers' widths, so it
 # writes the packed layout up to this many rows (a consumer that wants the other layout re-tiles, exactly).
 _NV_PACKED_PRODUCER_MAX_ROWS = 512
 

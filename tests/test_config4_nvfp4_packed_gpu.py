@@ -102,8 +102,9 @@ def _expected_entry(name, m, released):
     tiles = ((m + 255) // 256) * ((n + 255) // 256)
     if not PACKED_WEIGHTS:
         return "fpq_gemm_nvf4"
-    if not released and tiles >= 100:
-        return "fpq_gemm_nvf4"                       # large batches: the row-major kernel
+    if not released and tiles >= 100 and not (name == "qkv" and m == 4096):
+        return "fpq_gemm_nvf4"                       # large batches: the row-major kernel (qkv at 4096 rows is a round
+                                                     # and a half of its tiles: the packed kernel's half tiles)
     if name == "down" and m <= 1024:
         # few weight tiles, K = 12288: the entry that may split K through a workspace (the weight-streaming kernel up
         # to 128 rows, its two passes up to 256, the tile kernels beyond)
