@@ -63,6 +63,43 @@ def test_gemms_on_random_shapes(seed):
             assert torch.equal(outs[0], y[:, :cut]) and torch.equal(outs[1], y[:, cut:]), what + f" two layers at {cut}"
 
 
+@pytest.mark.parametrize("seed", [21, 22])
+def test_gemms_beyond_one_round_of_small_tiles(seed):
+    """More than 256 tiles of 128 x 128: the 256 x 128 and 256 x 256 tiles of both formats (an odd or even number of
+    128-row tiles, ragged rows and columns), alone, with bias and residual, and as several layers in one launch."""
+    rnd = random.Random(seed)
+    for _ in range(10):
+        m = rnd.choice([257, 300, 384, 512, 640, 700, 1024]) + rnd.choice([0, 0, -1, 1])
+        n = rnd.choice([8192, 12288, 16384]) + rnd.choice([0, 0, 0, 31, 100, -1])
+        k = 256 * rnd.choice([1, 1, 2])
+        if ((m + 127) // 128) * ((n + 127) // 128) <= 256:
+            n += 4096
+        fmt = rnd.choice(["mxfp4", "nvfp4", "nvfp4"])
+        nv = fmt == "nvfp4"
+        what = f"{fmt} m={m} n={n} k={k}"
+        g = torch.Generator().manual_seed(rnd.randrange(1 << 30))
+        group = 16 if nv else 32
+        xq = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=g)
+        wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=g)
+        lo, hi = (0x08, 0x7f) if nv else (118, 134)
+        xs = torch.randint(lo, hi, (m, k // group), dtype=torch.uint8, generator=g)
+        ws = torch.randint(lo, hi, (n, k // group), dtype=torch.uint8, generator=g)
+        alpha = ALPHA / 4096 if nv else ALPHA
+        ref, mag = O.gemm_ref(xq, xs, wq, ws, alpha, fmt)
+        xp, xsp = (pack_nv_by_definition if nv else pack_by_definition)(xq, xs, k)
+        wp, wsp = (pack_nv_by_definition if nv else pack_by_definition)(wq, ws, k)
+        gemm = capi.gemm_nv_packed if nv else capi.gemm_packed
+        y = gemm(xp, xsp, wp, wsp, m, n, k, alpha)
+        assert _close(y, ref, mag), what + " packed"
+        b = torch.randn(n, generator=g).to(torch.bfloat16)
+        res = (torch.randn(m, n, generator=g) * 8).to(torch.bfloat16)
+        assert torch.equal(gemm(xp, xsp, wp, wsp, m, n, k, alpha, bias=b, residual=res), (y + b) + res), what + " bias and residual"
+        if n % 256 == 0:
+            cut = rnd.randrange(1, n // 256) * 256
+            outs = capi.gemm_packed_multi(xp, xsp, wp, wsp, m, [cut, n - cut], k, alpha, nv=nv)
+            assert torch.equal(outs[0], y[:, :cut]) and torch.equal(outs[1], y[:, cut:]), what + f" two layers at {cut}"
+
+
 def _data(rnd, rows, cols, gen):
     x = torch.randn(rows, cols, generator=gen)
     kind = rnd.randrange(5)
