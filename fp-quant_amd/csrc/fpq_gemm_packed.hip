@@ -819,6 +819,16 @@ static int gemm_packed(const void* xq, const void* xs, const void* wq, const voi
   if (plan.kind == 1)
     return launch_packed<4, 4, 4, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg,
                                             plan.split, workspace);
+  // 256 x 128 tiles that have a CU to themselves and a long K: a ring of eight units.  Four units are 48 KB in
+  // flight per CU, less than the weights' way from HBM takes at the rate one workgroup consumes them (two
+  // workgroups per CU have 96 KB); weights from HBM, N = 4096, K = 14336: 1280 rows 59.6 -> 56.4 us, 1536 rows
+  // 58.1 -> 53.6; N = 8192, K = 8192, 640 rows 35.3 -> 32.8 (from the caches 4-10 % slower; K = 4096 and NVFP4
+  // measured the same either way and keep four).
+  if constexpr (!NV) {
+    if (plan.kind == 2 && K >= 8192 && ((M + 127) / 128) * ((N + 255) / 256) <= cus)
+      return launch_packed<8, 8, 4, 2, 2, false, 8>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream,
+                                                    residual, seg);
+  }
   if (plan.kind == 2)
     return launch_packed<8, 8, 4, 2, 2, NV, 4>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);
   return launch_packed<8, 8, 8, 2, 2, NV>(xq, xs, wq, ws, alpha, bias, y, M, N, K, (hipStream_t)stream, residual, seg);

@@ -122,6 +122,29 @@ def test_gemm_packed_matches_oracle_and_row_major_kernel(m, n, k, bias):
         assert ((y.double() - y_rm.double()).abs() <= 2 * tol).all()
 
 
+@pytest.mark.parametrize("m,n,k", [(257, 11008, 8192), (700, 5400, 8448)])
+def test_long_k_half_tiles_with_a_cu_to_themselves(m, n, k):
+    """More than 256 tiles of 128 x 128, at most 256 of 256 x 128 and K >= 8192: the 256 x 128 MXFP4 tiles with a
+    ring of eight units.  Bit for bit the row-major kernel's result (the same MFMA sequence per output), and within
+    tolerance of the oracle on a sample of the columns."""
+    g = torch.Generator().manual_seed(m + n + k)
+    xq = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, generator=g)
+    wq = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, generator=g)
+    xs = torch.randint(118, 134, (m, k // 32), dtype=torch.uint8, generator=g)
+    ws = torch.randint(118, 134, (n, k // 32), dtype=torch.uint8, generator=g)
+    b = torch.randn(n, generator=g).to(torch.bfloat16)
+    alpha = 0.111328125
+    xp, xsp = pack_by_definition(xq, xs, k)
+    wp, wsp = pack_by_definition(wq, ws, k)
+    y = capi.gemm_packed(xp, xsp, wp, wsp, m, n, k, alpha, bias=b)
+    assert torch.equal(y.view(torch.int16), capi.gemm(xq, xs, wq, ws, alpha, "mxfp4", bias=b).view(torch.int16))
+    cols = torch.randperm(n, generator=g)[:300]
+    ref, mag = O.gemm_ref(xq, xs, wq[cols], ws[cols], alpha, "mxfp4")
+    want = ref.to(torch.bfloat16) + b[cols]
+    tol = 2.0 ** -7 * want.double().abs() + 1e-5 * mag + 1e-6
+    assert ((y[:, cols].double() - want.double()).abs() <= tol).all()
+
+
 def test_gemm_packed_rejects():
     z = torch.zeros(4096, dtype=torch.uint8)
     with pytest.raises(ValueError):
