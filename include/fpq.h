@@ -315,8 +315,8 @@ int fpq_gemm_mxf4_packed_splitk(const void* xq_packed, const void* xs_packed, co
                                 void* workspace, int64_t workspace_bytes, void* stream);
 /* The same for packed NVFP4 operands (fpq_gemm_nvf4_packed, with `residual` non-null fpq_gemm_nvf4_packed_residual);
  * workspace as above, sized by fpq_gemm_nvf4_packed_workspace_bytes(M, N, K).  Up to 128 rows the split is
- * that of the MXFP4 entry; 129-256 rows on few weight rows run as two passes over at most 128 rows each, and
- * each pass may use the workspace.  Beyond, where the tile kernels have at most one workgroup tile per CU, a
+ * that of the MXFP4 entry; 129-256 rows on few weight rows (129-192 where the tile kernels can halve K inside
+ * their workgroups, below) run as two passes over at most 128 rows each, and each pass may use the workspace.  Beyond, where the tile kernels have at most one workgroup tile per CU, a
  * K with an even number of 256-blocks is halved INSIDE the workgroups (eight waves, the halves meet in LDS:
  * no workspace, the size function returns 0); with an odd number and a long K the tile kernels split K across
  * workgroups the way the weight-streaming kernel does (fp32 parts of their workgroup tiles, a counter per tile,
