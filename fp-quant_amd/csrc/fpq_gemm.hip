@@ -799,12 +799,12 @@ __global__ __launch_bounds__(256) void gemm_nvf4_lds_kernel(
   auto a_half = [&](int set, int sub, int i) {
     const uint4 c = aq[set][i];
     const uint32_t cd = sub == 0 ? c.x : sub == 1 ? c.y : sub == 2 ? c.z : c.w;
-    return dequant8_f16_s(cd, e4m3_pair_f16(sa[set][i] >> (8 * (sub >> 1))));
+    return dequant8_f16_h(cd, e4m3_byte_f16(sa[set][i], sub >> 1));
   };
   auto b_half = [&](int set, int sub, int j) {
     const uint4 c = bq[set][j];
     const uint32_t cd = sub == 0 ? c.x : sub == 1 ? c.y : sub == 2 ? c.z : c.w;
-    return dequant8_f16_s(cd, e4m3_pair_f16(sb[set][j] >> (8 * (sub >> 1))));
+    return dequant8_f16_h(cd, e4m3_byte_f16(sb[set][j], sub >> 1));
   };
 
   issue_loads(0, 0);

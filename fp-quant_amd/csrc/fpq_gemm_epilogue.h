@@ -82,6 +82,25 @@ __device__ __forceinline__ v8h dequant8_f16_s(uint32_t codes, v2h s2) {
   return v8h{p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
 }
 
+// The four E4M3 bytes of a dword at once: bytes 0 and 2 (low / high half of `even`) and bytes 1 and 3 (of `odd`)
+// as fp16 (value * 2^-8), two instructions each; a multiply then takes one half for both of its lanes.
+// (The empty asm keeps the compiler from splitting the dword operation into one 16-bit pair per half.)
+__device__ __forceinline__ v2h e4m3_even_f16(uint32_t d) {
+  uint32_t e = (d << 7) & 0x3f803f80u;
+  asm("" : "+v"(e));
+  return __builtin_bit_cast(v2h, e);
+}
+__device__ __forceinline__ v2h e4m3_odd_f16(uint32_t d) {
+  uint32_t e = (d >> 1) & 0x3f803f80u;
+  asm("" : "+v"(e));
+  return __builtin_bit_cast(v2h, e);
+}
+__device__ __forceinline__ _Float16 e4m3_byte_f16(uint32_t d, int byte) {   // byte: a constant once unrolled
+  const v2h h = (byte & 1) ? e4m3_odd_f16(d) : e4m3_even_f16(d);
+  return (byte & 2) ? h.y : h.x;
+}
+__device__ __forceinline__ v8h dequant8_f16_h(uint32_t codes, _Float16 s) { return dequant8_f16_s(codes, v2h{s, s}); }
+
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 

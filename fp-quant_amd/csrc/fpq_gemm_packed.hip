@@ -368,9 +368,9 @@ __global__ __launch_bounds__(256 * GR, (NT * MT <= 32 && GR == 1 ? 2 : 1)) void 
   if constexpr (NV) {                                                                               \
     const uint4 av = aq[(Q) & 1][I];                                                                \
     const uint32_t aw[4] = {av.x, av.y, av.z, av.w};                                                \
-    const uint32_t asc = ((Q) < 2 ? sa[I].x : sa[I].y) >> (16 * ((Q) & 1));                         \
+    const uint32_t asc = (Q) < 2 ? sa[I].x : sa[I].y;                                               \
     _Pragma("unroll") for (int s4 = 0; s4 < 4; ++s4) {                                              \
-      const v8h ah = dequant8_f16_s(aw[s4], e4m3_pair_f16(asc >> (8 * (s4 >> 1))));                 \
+      const v8h ah = dequant8_f16_h(aw[s4], e4m3_byte_f16(asc, 2 * ((Q) & 1) + (s4 >> 1)));         \
       _Pragma("unroll") for (int j = 0; j < TM; ++j)                                                \
         acc[I][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[j][s4], acc[I][j], 0, 0, 0);      \
     }                                                                                               \
@@ -393,9 +393,9 @@ __global__ __launch_bounds__(256 * GR, (NT * MT <= 32 && GR == 1 ? 2 : 1)) void 
     _Pragma("unroll") for (int j = 0; j < TM; ++j) {                                                \
       const uint4 bv = bq[(Q) & 1][j];                                                              \
       const uint32_t bw[4] = {bv.x, bv.y, bv.z, bv.w};                                              \
-      const uint32_t bsc = ((Q) < 2 ? sb[j].x : sb[j].y) >> (16 * ((Q) & 1));                       \
+      const uint32_t bsc = (Q) < 2 ? sb[j].x : sb[j].y;                                             \
       _Pragma("unroll") for (int s4 = 0; s4 < 4; ++s4)                                              \
-        bh[j][s4] = dequant8_f16_s(bw[s4], e4m3_pair_f16(bsc >> (8 * (s4 >> 1))));                  \
+        bh[j][s4] = dequant8_f16_h(bw[s4], e4m3_byte_f16(bsc, 2 * ((Q) & 1) + (s4 >> 1)));          \
     }                                                                                               \
   }
   constexpr int kHand = (TM >= 4 || TN <= 2) ? 1 : 2;  // rows of MFMAs ahead of the hand-over

@@ -157,16 +157,18 @@ __global__ __launch_bounds__(64 * NW, NT == 2 && NT * MT <= 4 ? 2 : 1) void gemm
       _Pragma("unroll") for (int j = 0; j < kJB; ++j) {                                                 \
         const uint4 bq = b[s][U][j0 + j];                                                               \
         const uint32_t bw[4] = {bq.x, bq.y, bq.z, bq.w};                                                \
-        const uint32_t bsc = ((U) < 2 ? sb[s][j0 + j].x : sb[s][j0 + j].y) >> (16 * ((U) & 1));         \
+        const uint32_t bsc = (U) < 2 ? sb[s][j0 + j].x : sb[s][j0 + j].y;                               \
+        const _Float16 bsh[2] = {e4m3_byte_f16(bsc, 2 * ((U) & 1)), e4m3_byte_f16(bsc, 2 * ((U) & 1) + 1)};   \
         _Pragma("unroll") for (int s4 = 0; s4 < 4; ++s4)                                                \
-          bh[j][s4] = dequant8_f16_s(bw[s4], e4m3_pair_f16(bsc >> (8 * (s4 >> 1))));                    \
+          bh[j][s4] = dequant8_f16_h(bw[s4], bsh[s4 >> 1]);                                             \
       }                                                                                                 \
       _Pragma("unroll") for (int i = 0; i < NT; ++i) {                                                  \
         const uint4 aq = a[s][U][i];                                                                    \
         const uint32_t aw[4] = {aq.x, aq.y, aq.z, aq.w};                                                \
-        const uint32_t asc = ((U) < 2 ? sa[s][i].x : sa[s][i].y) >> (16 * ((U) & 1));                   \
+        const uint32_t asc = (U) < 2 ? sa[s][i].x : sa[s][i].y;                                         \
+        const _Float16 ash[2] = {e4m3_byte_f16(asc, 2 * ((U) & 1)), e4m3_byte_f16(asc, 2 * ((U) & 1) + 1)};   \
         _Pragma("unroll") for (int s4 = 0; s4 < 4; ++s4) {                                              \
-          const v8h ah = dequant8_f16_s(aw[s4], e4m3_pair_f16(asc >> (8 * (s4 >> 1))));                 \
+          const v8h ah = dequant8_f16_h(aw[s4], ash[s4 >> 1]);                                          \
           _Pragma("unroll") for (int j = 0; j < kJB; ++j)                                               \
             acc[i * MT + j0 + j] =                                                                      \
                 __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[j][s4], acc[i * MT + j0 + j], 0, 0, 0);   \
@@ -205,16 +207,14 @@ __global__ __launch_bounds__(64 * NW, NT == 2 && NT * MT <= 4 ? 2 : 1) void gemm
     const int U = t >> 2, s4 = t & 3;
     const uint4 q = a[s][U][i];
     const uint32_t cd = s4 == 0 ? q.x : s4 == 1 ? q.y : s4 == 2 ? q.z : q.w;
-    const uint32_t sc = (U < 2 ? sa[s][i].x : sa[s][i].y) >> (16 * (U & 1) + 8 * (s4 >> 1));
-    return dequant8_f16_s(cd, e4m3_pair_f16(sc));
+    return dequant8_f16_h(cd, e4m3_byte_f16(U < 2 ? sa[s][i].x : sa[s][i].y, 2 * (U & 1) + (s4 >> 1)));
   };
   auto b_op = [&](auto slot, int t, int j) __attribute__((always_inline)) {
     constexpr int s = decltype(slot)::value;
     const int U = t >> 2, s4 = t & 3;
     const uint4 q = b[s][U][j];
     const uint32_t cd = s4 == 0 ? q.x : s4 == 1 ? q.y : s4 == 2 ? q.z : q.w;
-    const uint32_t sc = (U < 2 ? sb[s][j].x : sb[s][j].y) >> (16 * (U & 1) + 8 * (s4 >> 1));
-    return dequant8_f16_s(cd, e4m3_pair_f16(sc));
+    return dequant8_f16_h(cd, e4m3_byte_f16(U < 2 ? sb[s][j].x : sb[s][j].y, 2 * (U & 1) + (s4 >> 1)));
   };
   auto compute_block_nv = [&](auto slot) __attribute__((always_inline)) {
     v8h ah[NT], bh[MT];
