@@ -777,7 +777,7 @@ __global__ __launch_bounds__(256) void gemm_nvf4_lds_kernel(
   // Raw codes and scales are read from LDS one K step ahead, and dequantized operands run one MFMA
   // group ahead: while the four MFMAs of weight tile i (K sub-step `sub`) execute, the wave
   // converts weight tile i + 1 and activation tile i of the following sub-step, and the
-  // instruction order is pinned to one MFMA followed by five or six conversion instructions, which
+  // instruction order is pinned to one MFMA followed by four or five conversion instructions, which
   // is what fits under the 32 cycles of a 32x32x16 MFMA.  (Issue is in order: conversions written
   // in a block ahead of the MFMAs leave the matrix pipe idle; pinned this way the pipe's duty rose
   // from 52 % to 64 %.  Carrying the pipeline across the stage barrier as well measured no faster.)
@@ -836,13 +836,13 @@ __global__ __launch_bounds__(256) void gemm_nvf4_lds_kernel(
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah_cur, bh_cur[j], acc[i][j], 0, 0, 0);
           static_assert(TM == 4, "the instruction pattern below is written for four MFMAs per weight tile");
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA ...
-          __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);  // ... conversions behind it
+          __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);  // ... conversions behind it
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
           ah_cur = ah_next;
         }
 #pragma unroll
