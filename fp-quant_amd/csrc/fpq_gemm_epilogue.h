@@ -100,6 +100,16 @@ __device__ __forceinline__ _Float16 e4m3_byte_f16(uint32_t d, int byte) {   // b
   return (byte & 2) ? h.y : h.x;
 }
 __device__ __forceinline__ v8h dequant8_f16_h(uint32_t codes, _Float16 s) { return dequant8_f16_s(codes, v2h{s, s}); }
+// ... and one half of that: codes 4 part .. 4 part + 3
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ v4h dequant4_f16_h(uint32_t codes, _Float16 s, int part) {
+  const v2h s2 = {s, s};
+  const v2h p0 = (part ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 2)
+                       : __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 0)) * s2;
+  const v2h p1 = (part ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 3)
+                       : __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, 256.0f, 1)) * s2;
+  return v4h{p0.x, p0.y, p1.x, p1.y};
+}
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));

@@ -388,6 +388,45 @@ __global__ __launch_bounds__(256 * GR, (NT * MT <= 32 && GR == 1 ? 2 : 1)) void 
   }
   // NVFP4: the activation operands of the unit, dequantized once for all rows of MFMAs
   v8h bh[NV ? TM : 1][4];
+  // NVFP4 on the large tiles (four rows of matrix instructions per wave): a software pipeline over the K steps of 16
+  // instead -- while the matrix instructions of step (unit, s4) issue, row by row, the operands of the next step
+  // are converted (row i: weight tile i and its share of the activation tiles' halves), and the instruction
+  // order is pinned to one matrix instruction followed by its share of the conversions.  The step after a
+  // unit's last one belongs to the next unit, whose registers were read at this unit's hand-over (the next
+  // block's scales with them); after the last unit of all the conversions run on stale registers and nothing
+  // consumes them.  Against converting a unit's activation operands in one block ahead of its matrix instructions
+  // (K = 4096, weights from HBM): 256 x 256 tiles, 4096 x 24576 618 -> 570 us (the row-major kernel: 610), 2048 x
+  // 14336 197 -> 178; 256 x 128 tiles 52-55 -> 44-48; 128 x 128 tiles with eight waves 2-5 % (640-1024 rows, N =
+  // 4096: 30.4-35.4 -> 29.2-34.8); the 64 x 128 tiles measured 1-2 % slower this way and keep the block.
+  constexpr bool kNvPipe = NV && TN >= 2 && (2 * TM) % TN == 0;
+  constexpr int kHpr = kNvPipe ? 2 * TM / TN : 1;   // halves of activation tiles converted per row
+  // conversion instructions behind each matrix instruction of a row (a row converts 9 + 4.5 kHpr for its TM; one
+  // more or less measured 1-3 % slower)
+  constexpr int kPinValu = TN == 4 ? (TM == 4 ? 5 : 6) : 8;
+  v8h ah_c[kNvPipe ? TN : 1], ah_n[kNvPipe ? TN : 1];
+  v4h bh_c[kNvPipe ? TM : 1][2], bh_n[kNvPipe ? TM : 1][2];
+  auto nv_scale = [&](const uint2& cur, const uint2& next, int qn, int sn, bool nxt) __attribute__((always_inline)) {
+    const uint2 sc = nxt ? next : cur;
+    return e4m3_byte_f16(qn < 2 ? sc.x : sc.y, 2 * (qn & 1) + (sn >> 1));
+  };
+  auto nv_dword = [&](const uint4& c, int sn) __attribute__((always_inline)) {
+    return sn == 0 ? c.x : sn == 1 ? c.y : sn == 2 ? c.z : c.w;
+  };
+  auto nv_a = [&](int qn, int sn, int i, bool nxt) __attribute__((always_inline)) {
+    return dequant8_f16_h(nv_dword(aq[qn & 1][i], sn), nv_scale(sa[i], sa_next[i], qn, sn, nxt));
+  };
+  auto nv_b = [&](int qn, int sn, int j, int part, bool nxt) __attribute__((always_inline)) {
+    return dequant4_f16_h(nv_dword(bq[qn & 1][j], sn), nv_scale(sb[j], sb_next[j], qn, sn, nxt), part);
+  };
+  if constexpr (kNvPipe) {   // the first step's operands (block 0's scales are still where they were read ahead)
+#pragma unroll
+    for (int i = 0; i < TN; ++i) ah_c[i] = nv_a(0, 0, i, true);
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      bh_c[j][0] = nv_b(0, 0, j, 0, true);
+      bh_c[j][1] = nv_b(0, 0, j, 1, true);
+    }
+  }
 #define FPQ_PREP_B(Q)                                                                               \
   if constexpr (NV) {                                                                               \
     _Pragma("unroll") for (int j = 0; j < TM; ++j) {                                                \
@@ -412,6 +451,37 @@ __global__ __launch_bounds__(256 * GR, (NT * MT <= 32 && GR == 1 ? 2 : 1)) void 
     if (READ2) read_unit((U) + 2, ((Q) + 2) & 3);                                                   \
     __builtin_amdgcn_sched_barrier(0);                                                              \
     _Pragma("unroll") for (int i1 = 0; i1 < TN; ++i1) FPQ_MFMA_ROW(Q, i1)                           \
+  } else if constexpr (kNvPipe) {                                                                   \
+    _Pragma("unroll") for (int s4 = 0; s4 < 4; ++s4) {                                              \
+      const int qn = s4 == 3 ? ((Q) + 1) & 3 : (Q), sn = s4 == 3 ? 0 : s4 + 1;                      \
+      const bool nxt = s4 == 3 && (Q) == 3;   /* the next block's scales */                         \
+      _Pragma("unroll") for (int i = 0; i < TN; ++i) {                                              \
+        ah_n[i] = nv_a(qn, sn, i, nxt);                                                             \
+        _Pragma("unroll") for (int h = i * kHpr; h < (i + 1) * kHpr; ++h)                           \
+          bh_n[h >> 1][h & 1] = nv_b(qn, sn, h >> 1, h & 1, nxt);                                   \
+        _Pragma("unroll") for (int j = 0; j < TM; ++j)                                              \
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(                                       \
+              ah_c[i], __builtin_shufflevector(bh_c[j][0], bh_c[j][1], 0, 1, 2, 3, 4, 5, 6, 7), acc[i][j], 0, 0, 0); \
+        _Pragma("unroll") for (int j = 0; j < TM; ++j) {                                            \
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                        \
+          __builtin_amdgcn_sched_group_barrier(0x002, kPinValu, 0);                                 \
+        }                                                                                           \
+        __builtin_amdgcn_sched_barrier(0);                                                          \
+      }                                                                                             \
+      if (s4 == 0) {                                                                                \
+        wait_vmem_le<(ALLOWED)>();                                                                  \
+        barrier_lds();                                                                              \
+        if (ISSUE) issue_unit((U) + RING, (Q) == 0);                                               \
+        if (READ) read_unit((U) + 1, ((Q) + 1) & 1);                                                \
+        if ((Q) == 3 && (NEXT_BLOCK)) read_scales(((U) + 1) >> 2);                                  \
+        __builtin_amdgcn_sched_barrier(0);                                                          \
+      }                                                                                             \
+      _Pragma("unroll") for (int i = 0; i < TN; ++i) ah_c[i] = ah_n[i];                             \
+      _Pragma("unroll") for (int j = 0; j < TM; ++j) {                                              \
+        bh_c[j][0] = bh_n[j][0];                                                                    \
+        bh_c[j][1] = bh_n[j][1];                                                                    \
+      }                                                                                             \
+    }                                                                                               \
   } else {                                                                                          \
     FPQ_PREP_B(Q)                                                                                   \
     _Pragma("unroll") for (int i0 = 0; i0 < kHand; ++i0) FPQ_MFMA_ROW(Q, i0)                        \

@@ -740,8 +740,7 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
         qa = QuantizedActivations(rows, cols, nvfp4)
         qa.mx_packed = (pc, ps)
         return qa
-    if (allow_packed and nvfp4 and rows <= _NV_PACKED_PRODUCER_MAX_ROWS and cols % 256 == 0
-            and nv_packed_eligible(rows, 32, cols, fused_linear=True)):
+    if allow_packed and nvfp4 and cols % 256 == 0 and nv_packed_eligible(rows, 32, cols, fused_linear=True):
         # the row counts whose consumers run the packed NVFP4 GEMM: straight into its layout
         gs = as_f32_scalar(act_global_scale, remember)
         pc = torch.empty(lib.fpq_packed_codes_bytes(rows, cols), dtype=torch.uint8, device=dev)
@@ -771,10 +770,6 @@ def _fused_quantize(entry: str, head: tuple, rows: int, cols: int, h: torch.Tens
 
 
 _ROWS_KERNEL_MAX_ROWS = 64   # fpq_rmsnorm_rows_max_rows()
-# NVFP4 layers take the packed GEMM up to mid-sized batches (nv_packed_eligible: fewer than 100 tiles of
-# 256 x 256, or a last round that half tiles fill better) and the row-major one beyond; a fused producer does not know its consumers' widths, so it
-# writes the packed layout up to this many rows (a consumer that wants the other layout re-tiles, exactly).
-_NV_PACKED_PRODUCER_MAX_ROWS = 512
 
 
 def rmsnorm_quantize(x: torch.Tensor, weight: torch.Tensor, eps: float, hadamard_matrix: torch.Tensor,

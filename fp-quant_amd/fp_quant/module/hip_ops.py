@@ -342,43 +342,12 @@ def pack_nvf4(codes: torch.Tensor, scales: torch.Tensor, rows: int, k: int, into
     return pc, ps
 
 
-_compute_units = {}   # device index -> compute units
-
-
-def _device_cus() -> int:
-    dev = torch.cuda.current_device() if torch.cuda.is_available() else -1
-    hit = _compute_units.get(dev)
-    if hit is None:
-        hit = _compute_units[dev] = int(_engine.lib().fpq_compute_units())
-    return hit
-
-
-def _nv_packed_below() -> int:
-    """25/64 of the device's compute units (100 on the 256 of an MI355X): tiles of 256 x 256 from which the
-    row-major NVFP4 kernel, whose large tiles are 7 % faster than the packed kernel's, takes whole rounds."""
-    return _device_cus() * 25 // 64
-
-
-def _nv_half_tiles_cheaper(m: int, n: int) -> bool:
-    """Large shapes whose 256 x 256 tiles fill their last round badly: the packed kernel's 256 x 128 tiles (two
-    workgroups per CU; one alone on a CU takes 0.54 of a large tile's time) finish sooner than whole rounds of the
-    row-major kernel's 256 x 256 tiles.  The same round count as the library's own choice between its two packed
-    tile shapes (tile_plan, csrc/fpq_gemm_packed.hip), with the row-major kernel's large tile at 0.93 of the packed
-    one (K = 4096: 4096 x 6144 200 -> 172 us, 3072 x 6144 179 -> 151, 1024 x 24576 179 -> 163; K = 12288, 2048 x 4096
-    230 -> 177; 2048 x 14336, 186 against 201, stays row-major)."""
-    cus = _device_cus()
-    big = ((m + 255) // 256) * ((n + 255) // 256)
-    rounds, rest = divmod(((m + 127) // 128) * ((n + 255) // 256), 2 * cus)
-    cost_half = rounds * 104 + (0 if rest == 0 else 54 if rest <= cus else 104)
-    return cost_half < -(-big // cus) * 93
-
-
 def nv_packed_eligible(m: int, n: int, k: int, fused_linear: bool = False) -> bool:
-    """NVFP4: the packed kernels win for few and mid-sized M (weight-streaming kernel, 128 x 128 and 256 x 128
-    tiles) and where half tiles fill the last round better; other large M runs faster on row-major operands."""
+    """NVFP4: the packed kernels at every row count from the smallest they take (the weight-streaming kernel,
+    the tile kernels, whose large tiles convert the operands of the next K step behind the matrix instructions
+    of the current one and are 6-7 % faster than the row-major kernel: 4096 x 24576 x 4096 570 against 610 us)."""
     return ((NV_PACKED_LINEAR_MIN_M if fused_linear else NV_PACKED_MIN_M) <= m and k % 256 == 0
-            and packed_weights_enabled()
-            and (((m + 255) // 256) * ((n + 255) // 256) < _nv_packed_below() or _nv_half_tiles_cheaper(m, n)))
+            and packed_weights_enabled())
 
 
 def unpack_fp4(pc: torch.Tensor, ps: torch.Tensor, rows: int, k: int, nvfp4: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:

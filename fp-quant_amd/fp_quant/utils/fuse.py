@@ -129,22 +129,12 @@ def _attach_weight_group(module: nn.Module, names) -> None:
     module._fpq_weight_group_hook = module.register_load_state_dict_post_hook(build)
 
 
-# NVFP4: the one GEMM pays for decode-sized batches (weight-streaming and 128x128-tile kernels on packed
-# operands, the same kernels the layers run one by one there); large batches are faster on the row-major
-# kernel, layer by layer.
-_NV_GROUP_MAX_ROWS = 128
-
-
-def _group_serves(group, x: torch.Tensor) -> bool:
-    return not group.nvfp4 or x.numel() // x.shape[-1] <= _NV_GROUP_MAX_ROWS
-
-
 def _group_linear(layers, x: torch.Tensor, group=None):
     """The outputs of `layers` on `x` from ONE operator: one quantization and, where the layers' packed
     weights lie end to end (`group`, a WeightGroup), one GEMM whose column ranges are the outputs; else
     one GEMM each."""
     first = layers[0]
-    if group is not None and _group_serves(group, x):
+    if group is not None:
         outs = _eager().linear_cat_w4a4_op(x.reshape(-1, x.shape[-1]), first.forward_hadamard_matrix, group.wp,
                                            group.wsp, group.splits, first.weight_global_scale,
                                            first.act_global_scale, group.bias, group.nvfp4)
@@ -381,7 +371,7 @@ def _eager_group_linear(owner: nn.Module, layers, x: torch.Tensor):
     `x` is taken from, or left in, the sharing slot); None if there is no group.  The group kept on
     `owner` is checked against the layers' tensors as they are now and rebuilt if they were written to."""
     group = getattr(owner, "_fpq_weight_group", None)
-    if group is None or not _group_serves(group, x):
+    if group is None:
         return None
     first = layers[0]
     if group.key != tuple(_eager()._member_key(l.qweight, l.scales, l.bias) for l in layers):

@@ -1,7 +1,7 @@
 """NVFP4 linears of the Qwen3-8B shapes (qkv 6144x4096, o 4096x4096, gate_up 24576x4096, down 4096x12288) at
 1, 64, 512 and 4096 rows ON THE KERNELS FPQuantLinear DISPATCHES THERE: the packed-operand kernels
-(fpq_gemm_nvf4_packed, and fpq_gemm_nvf4_packed_splitk on the long-K down-projection) up to mid-sized
-batches, the row-major kernel beyond.  Reference contract: matmul_nvf4_bf16_tn_op
+(fpq_gemm_nvf4_packed, and fpq_gemm_nvf4_packed_splitk on the long-K down-projection) at every row
+count.  Reference contract: matmul_nvf4_bf16_tn_op
 (inference_lib/src/fp_quant/module/qutlass_ops.py:149-168) as forward_gemm calls it (linear_fns.py:53-64).
 
 Every case is checked against the oracle (quantizers + fp64 dequantize-then-matmul, tolerance of
@@ -99,12 +99,8 @@ class _Calls:
 
 def _expected_entry(name, m, released):
     n, k = SHAPES[name]
-    tiles = ((m + 255) // 256) * ((n + 255) // 256)
     if not PACKED_WEIGHTS:
         return "fpq_gemm_nvf4"
-    if not released and tiles >= 100 and not (name == "qkv" and m == 4096):
-        return "fpq_gemm_nvf4"                       # large batches: the row-major kernel (qkv at 4096 rows is a round
-                                                     # and a half of its tiles: the packed kernel's half tiles)
     if name == "down" and m <= 1024:
         # few weight tiles, K = 12288: the entry that may split K through a workspace (the weight-streaming kernel up
         # to 128 rows, its two passes up to 256, the tile kernels beyond)
@@ -162,8 +158,8 @@ def test_released_layer_runs_the_packed_kernels_at_every_row_count(name, m, monk
     oxq, oxs, _ = O.quantize_nv(x[ri], 10.0, O.ROT_HADAMARD, G, NORM)
     ref, mag = O.gemm_ref(oxq, oxs, owq, ows, 0.010009765625, "nvfp4")
     _assert_close(y.cpu()[ri][:, ci], ref, mag, f"released {name} M={m}")
-    # (the row-major kernel, which ran before the release, sums K in another order: same tolerance, other bits)
-    _assert_close(want.cpu()[ri][:, ci], ref, mag, f"row-major {name} M={m}")
+    # (the same kernel ran before the release: the same bits)
+    assert torch.equal(want, y)
 
 
 @pytest.fixture(scope="module")

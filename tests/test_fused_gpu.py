@@ -648,7 +648,7 @@ def test_grouped_projections_run_as_one_gemm_on_concatenated_packed_weights(toke
     from fp_quant.utils import fuse_producers
     model = _tiny_llama(fmt, g, seed=3)
     other = _tiny_llama(fmt, g, seed=4)
-    grouped = fmt == "mxfp4" or tokens <= 128      # NVFP4: one GEMM for decode-sized batches only
+    grouped = True      # both formats, every row count
     block, block2 = model.model.layers[0], other.model.layers[0]
     attn, mlp = block.self_attn, block.mlp
     x = (torch.randn(1, tokens, 256, device="cuda") * 1.5).to(torch.bfloat16)
